@@ -1,0 +1,200 @@
+/*
+ * merak_tp_gfx950 — C ABI of the gfx950 (MI355X) kernels behind Merak's
+ * Megatron-style tensor-parallel layers.
+ *
+ * Every entry point takes raw device pointers, sizes and a HIP stream
+ * (hipStream_t passed as void*; NULL = the null stream).  Nothing here
+ * allocates, frees or synchronises: the caller owns every buffer, and
+ * the kernels are enqueued on `stream` and return immediately.
+ *
+ * Return value: 0 on success, a negative MTP_E* code otherwise.  After a
+ * failure mtp_last_error() returns a thread-local, human readable reason.
+ * The library is re-entrant: it keeps no mutable global state apart from
+ * that thread-local error string (backward passes call it from PyTorch's
+ * autograd worker thread while forward runs on the main thread).
+ *
+ * File:line citations name the interface in the reference tree
+ * (HPDL-Group/Merak) that each entry point stands in for.
+ */
+#ifndef MERAK_TP_GFX950_H
+#define MERAK_TP_GFX950_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MTP_ABI_VERSION 1
+
+/* element types */
+#define MTP_F32  0
+#define MTP_BF16 1
+
+/* error codes */
+#define MTP_OK            0
+#define MTP_EINVAL       -1   /* bad argument (null pointer, negative size, unknown enum) */
+#define MTP_EUNSUPPORTED -2   /* shape/alignment the kernels do not cover */
+#define MTP_EDEVICE      -3   /* current device is not gfx950, or a HIP call failed */
+#define MTP_EWORKSPACE   -4   /* workspace too small */
+
+/* epilogues of mtp_linear_fwd / mtp_gemv */
+#define MTP_EPI_NONE      0   /* Y = X W^T                                   */
+#define MTP_EPI_BIAS      1   /* Y = X W^T + b                               */
+#define MTP_EPI_BIAS_GELU 2   /* Y = X W^T + b ; ACT = gelu_new(Y)           */
+#define MTP_EPI_SWIGLU    3   /* Y = X W^T (+ b); ACT = silu(Y[:, :N/2]) * Y[:, N/2:] */
+#define MTP_EPI_GELU      4   /* Y = X W^T ; ACT = gelu_new(Y)               */
+
+int         mtp_abi_version(void);
+const char* mtp_last_error(void);
+
+/* Name of the gfx architecture of the current HIP device ("gfx950"), written
+ * into buf (NUL terminated, truncated to len).  MTP_EDEVICE if no device. */
+int mtp_device_arch(char* buf, int len);
+
+/* ------------------------------------------------------------------------
+ * Linear layers.  All matrices are row-major and dense (leading dimension
+ * = number of columns).  dtype is the element type of X, W, Y, dY, dX and
+ * bias; accumulation is always fp32.
+ * ------------------------------------------------------------------------ */
+
+/* Y[M,N] = X[M,K] W[N,K]^T (+ bias[N]) with an optional fused activation.
+ * Replaces F.linear in ColumnParallelLinear.forward
+ * (Merak/core/mpu/layers.py:251-252) and RowParallelLinear.forward
+ * (layers.py:354 and the "+ bias" of :357-358, which at tensor-parallel
+ * world size 1 follows an identity reduce), plus the elementwise activation
+ * HF applies between the two (gelu_new for GPT-2, silu(gate)*up for Llama).
+ *
+ *  y   : [M,N] pre-activation output; may be NULL when an activation
+ *        epilogue is selected and the caller does not need it.
+ *  act : activation output, required for *_GELU ([M,N]) and SWIGLU
+ *        ([M,N/2]); must be NULL otherwise.
+ *  bias: [N] or NULL (required for MTP_EPI_BIAS, MTP_EPI_BIAS_GELU). */
+int mtp_linear_fwd(const void* x, const void* w, const void* bias,
+                   void* y, void* act,
+                   int64_t M, int64_t N, int64_t K,
+                   int dtype, int epilogue, void* stream);
+
+/* dX[M,K] = dY[M,N] W[N,K]  — the input gradient autograd derives for
+ * F.linear (entered from loss.backward(), Merak/core/merak_engine.py:926;
+ * at world size 1 the all-reduce of _CopyToModelParallelRegion.backward,
+ * Merak/core/mpu/mappings.py:320, is the identity). */
+int mtp_linear_dgrad(const void* dy, const void* w, void* dx,
+                     int64_t M, int64_t N, int64_t K,
+                     int dtype, void* stream);
+
+/* dW[N,K] (+)= dY[M,N]^T X[M,K]; db[N] (+)= sum_m dY[m,:]  — the weight and
+ * bias gradients of F.linear.  dw_dtype selects the element type of dW and
+ * db (MTP_F32 lets the caller keep an fp32 main gradient); accumulate != 0
+ * adds into the existing contents instead of overwriting.  db may be NULL. */
+int mtp_linear_wgrad(const void* dy, const void* x, void* dw, void* db,
+                     int64_t M, int64_t N, int64_t K,
+                     int dtype, int dw_dtype, int accumulate, void* stream);
+
+/* Backward of the fused activations: given dACT and the saved
+ * pre-activation Y, writes dY.
+ *   MTP_EPI_BIAS_GELU / MTP_EPI_GELU: dY[M,N]   = dACT[M,N] * gelu_new'(Y)
+ *   MTP_EPI_SWIGLU:                   dY[M,N]   from dACT[M,N/2], Y=[gate|up]
+ * dy may alias dact only for the GELU forms. */
+int mtp_activation_bwd(const void* dact, const void* y, void* dy,
+                       int64_t M, int64_t N, int dtype, int epilogue,
+                       void* stream);
+
+/* ------------------------------------------------------------------------
+ * Vocab-parallel embedding (Merak/core/mpu/layers.py:145-165).
+ * out[i,:] = table[ids[i]-vocab_start,:] if vocab_start <= ids[i] < vocab_end
+ *            else 0                         (layers.py:148-152,162)
+ * row_bytes = embedding_dim * element size; any value >= 1 is accepted
+ * (wider vector copies are used when table, out and row_bytes are 16/8/4
+ * byte aligned).  oob_count (device int32, may be NULL) is incremented once
+ * per id outside [vocab_start, vocab_end).
+ * ------------------------------------------------------------------------ */
+int mtp_embedding_gather(const int64_t* ids, const void* table, void* out,
+                         int64_t n_ids, int64_t row_bytes,
+                         int64_t vocab_start, int64_t vocab_end,
+                         int32_t* oob_count, void* stream);
+
+/* Dense gradient of the lookup: dtable[ids[i]-vocab_start,:] += dout[i,:]
+ * for in-range ids, accumulated in fp32 (dtable is fp32 [rows,dim]).  This is
+ * the embedding_dense_backward ATen runs behind F.embedding (layers.py:156).
+ * The caller zeroes dtable first unless it wants accumulation. */
+int mtp_embedding_bwd(const int64_t* ids, const void* dout, float* dtable,
+                      int64_t n_ids, int64_t dim, int dtype,
+                      int64_t vocab_start, int64_t vocab_end, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Vocab-parallel cross entropy (Merak/core/mpu/cross_entropy.py:29-106).
+ * logits: [n_rows, vocab] contiguous, this rank's vocab slice
+ * [vocab_start, vocab_start+vocab).  One pass, fp32 arithmetic.
+ *
+ *   row_max[i]    = max_j logits[i,j]                       (:32)
+ *   row_sumexp[i] = sum_j exp(logits[i,j] - row_max[i])     (:70-71)
+ *   pred[i]       = logits[i, t_i - vocab_start] if t_i in range else 0
+ *                   (raw logit, not max-subtracted)          (:48-62)
+ *   loss[i]       = log(row_sumexp[i]) - (pred[i]-row_max[i]) in range,
+ *                   log(row_sumexp[i]) otherwise             (:77)
+ * loss is the single-rank result; the three partials are what ranks would
+ * exchange (MAX, SUM, SUM; :33,64,72).  Targets outside the range — -100
+ * included — get no one-hot term, exactly as the reference's mask does.
+ * The logits are NOT modified by the forward.
+ * ------------------------------------------------------------------------ */
+int mtp_vocab_ce_fwd(const void* logits, const int64_t* target,
+                     float* loss, float* row_max, float* row_sumexp,
+                     float* pred,
+                     int64_t n_rows, int64_t vocab, int64_t vocab_start,
+                     int dtype, void* stream);
+
+/* In place: logits[i,j] <- (exp(logits[i,j]-row_max[i]) / row_sumexp[i]
+ *                           - [j == t_i - vocab_start]) * grad_out[i]
+ * (cross_entropy.py:86-106).  row_max / row_sumexp are the (globally
+ * combined) values from the forward.  grad_out may be NULL (= 1 for every
+ * row), which together with out-of-range targets yields the softmax the
+ * reference leaves in the caller's logits after forward (:80). */
+int mtp_vocab_ce_bwd(void* logits, const int64_t* target,
+                     const float* row_max, const float* row_sumexp,
+                     const float* grad_out,
+                     int64_t n_rows, int64_t vocab, int64_t vocab_start,
+                     int dtype, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Decode step (Merak/inference/text_generation_inference.py:223,226-227):
+ * a handful of single-token activation rows through a linear layer, and the
+ * greedy pick over the LM-head row.  bf16 only, B <= 32, K % 8 == 0.
+ * ------------------------------------------------------------------------ */
+
+/* Y[B,N] = X[B,K] W[N,K]^T (+bias) ; epilogue NONE, BIAS or SWIGLU
+ * (SWIGLU: y is [B,N/2] = silu(gate)*up with W = [gate rows | up rows]). */
+int mtp_gemv(const void* x, const void* w, const void* bias, void* y,
+             int64_t B, int64_t N, int64_t K, int epilogue, void* stream);
+
+/* Bytes of device scratch mtp_gemv_argmax needs for this shape. */
+int64_t mtp_gemv_argmax_workspace_bytes(int64_t B, int64_t N, int64_t K);
+
+/* idx[b] = argmax_n (X[b,:] . W[n,:]) — first index among equal maxima, NaN
+ * counts as the maximum (torch.argmax semantics, :227); maxval[b] (may be
+ * NULL) receives the winning fp32 logit.  The [B,N] logits are never
+ * written to memory. */
+int mtp_gemv_argmax(const void* x, const void* w,
+                    int64_t* idx, float* maxval,
+                    void* workspace, int64_t workspace_bytes,
+                    int64_t B, int64_t N, int64_t K, void* stream);
+
+/* Row-wise argmax of materialised logits [B,V] (dtype f32 or bf16): the
+ * literal torch.argmax(logits, dim=-1) of :227. */
+int mtp_argmax_rows(const void* logits, int64_t* idx,
+                    int64_t B, int64_t V, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Measurement helpers (used by bench.py to state what this GPU can do).
+ * ------------------------------------------------------------------------ */
+/* dst[0:bytes] = src[0:bytes] with 16-byte accesses; bytes % 16 == 0. */
+int mtp_stream_copy(const void* src, void* dst, int64_t bytes, void* stream);
+/* Register-resident bf16 MFMA loop: iters x 32x32x16 MFMAs per wave on
+ * `waves_per_cu * cu_count` waves; writes one float per lane to sink
+ * (>= 64*waves floats).  Reports nothing itself: time it with events. */
+int mtp_mfma_peak(float* sink, int64_t n_waves, int64_t iters, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MERAK_TP_GFX950_H */

@@ -1,0 +1,212 @@
+// Bandwidth-bound helpers around the GEMMs: backward of the fused
+// activations, the bias gradient (column sum of dY), and two measurement
+// kernels (streaming copy, register-resident MFMA loop).
+#include "mtp_common.h"
+
+namespace {
+
+// ---- activation backward ---------------------------------------------------
+// T = float or uint16_t (bf16 bits); one thread handles one 16-byte vector.
+template <typename T> struct Io;
+template <> struct Io<float> {
+  static constexpr int EPV = 4;
+  __device__ static __forceinline__ void unpack(const u32x4_t& v, float* f) {
+    f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y);
+    f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+  }
+  __device__ static __forceinline__ u32x4_t pack(const float* f) {
+    return u32x4_t{__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
+  }
+  __device__ static __forceinline__ float ld(const float* p) { return *p; }
+  __device__ static __forceinline__ void st(float* p, float v) { *p = v; }
+};
+template <> struct Io<uint16_t> {
+  static constexpr int EPV = 8;
+  __device__ static __forceinline__ void unpack(const u32x4_t& v, float* f) {
+    f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x); f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
+    f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z); f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
+  }
+  __device__ static __forceinline__ u32x4_t pack(const float* f) {
+    return u32x4_t{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                   pack_bf16x2(f[6], f[7])};
+  }
+  __device__ static __forceinline__ float ld(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+  __device__ static __forceinline__ void st(uint16_t* p, float v) { *p = f32_to_bf16_bits(v); }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_bwd_kernel(const T* __restrict__ dact, const T* __restrict__ y,
+                                                       T* __restrict__ dy, int64_t n) {
+  constexpr int EPV = Io<T>::EPV;
+  const int64_t nvec = n / EPV;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const int64_t t0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (int64_t i = t0; i < nvec; i += stride) {
+    u32x4_t a = reinterpret_cast<const u32x4_t*>(dact)[i];
+    u32x4_t b = reinterpret_cast<const u32x4_t*>(y)[i];
+    float fa[EPV], fb[EPV];
+    Io<T>::unpack(a, fa);
+    Io<T>::unpack(b, fb);
+#pragma unroll
+    for (int e = 0; e < EPV; e++) fa[e] *= gelu_new_grad_f(fb[e]);
+    reinterpret_cast<u32x4_t*>(dy)[i] = Io<T>::pack(fa);
+  }
+  for (int64_t j = nvec * EPV + t0; j < n; j += stride) Io<T>::st(dy + j, Io<T>::ld(dact + j) * gelu_new_grad_f(Io<T>::ld(y + j)));
+}
+
+// y = [gate | up] of width N = 2H per row; dact has width H.
+//   dgate = dact * up * silu'(gate),  dup = dact * silu(gate)
+// VEC: rows are 16-byte aligned and H % EPV == 0
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ dact, const T* __restrict__ y,
+                                                         T* __restrict__ dy, int64_t M, int64_t H) {
+  constexpr int EPV = VEC ? Io<T>::EPV : 1;
+  const int64_t hv = H / EPV;
+  const int64_t total = M * hv;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int64_t m = i / hv, c = (i - m * hv) * EPV;
+    const T* pg = y + m * 2 * H + c;
+    const T* pu = pg + H;
+    const T* pd = dact + m * H + c;
+    T* og = dy + m * 2 * H + c;
+    T* ou = og + H;
+    float g[EPV], u[EPV], d[EPV], rg[EPV], ru[EPV];
+    if constexpr (VEC) {
+      Io<T>::unpack(*reinterpret_cast<const u32x4_t*>(pg), g);
+      Io<T>::unpack(*reinterpret_cast<const u32x4_t*>(pu), u);
+      Io<T>::unpack(*reinterpret_cast<const u32x4_t*>(pd), d);
+    } else {
+      g[0] = Io<T>::ld(pg); u[0] = Io<T>::ld(pu); d[0] = Io<T>::ld(pd);
+    }
+#pragma unroll
+    for (int e = 0; e < EPV; e++) {
+      const float s = 1.0f / (1.0f + __expf(-g[e]));  // sigmoid(gate)
+      const float silu = g[e] * s;
+      rg[e] = d[e] * u[e] * (s + silu * (1.0f - s));
+      ru[e] = d[e] * silu;
+    }
+    if constexpr (VEC) {
+      *reinterpret_cast<u32x4_t*>(og) = Io<T>::pack(rg);
+      *reinterpret_cast<u32x4_t*>(ou) = Io<T>::pack(ru);
+    } else {
+      Io<T>::st(og, rg[0]); Io<T>::st(ou, ru[0]);
+    }
+  }
+}
+
+// ---- measurement -------------------------------------------------------------
+__global__ __launch_bounds__(256) void stream_copy_kernel(const u32x4_t* __restrict__ src, u32x4_t* __restrict__ dst,
+                                                          int64_t nvec) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i + 3 * stride < nvec; i += 4 * stride) {
+    u32x4_t a = __builtin_nontemporal_load(src + i);
+    u32x4_t b = __builtin_nontemporal_load(src + i + stride);
+    u32x4_t c = __builtin_nontemporal_load(src + i + 2 * stride);
+    u32x4_t d = __builtin_nontemporal_load(src + i + 3 * stride);
+    __builtin_nontemporal_store(a, dst + i);
+    __builtin_nontemporal_store(b, dst + i + stride);
+    __builtin_nontemporal_store(c, dst + i + 2 * stride);
+    __builtin_nontemporal_store(d, dst + i + 3 * stride);
+  }
+  for (; i < nvec; i += stride) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+__global__ __launch_bounds__(256) void mfma_peak_kernel(float* __restrict__ sink, int64_t iters) {
+  const int lane = threadIdx.x & 63;
+  bf16x8_t a, b;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    a[i] = (__bf16)(0.001f * (lane + i));
+    b[i] = (__bf16)(0.002f * (lane - i));
+  }
+  f32x16_t c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
+  for (int64_t it = 0; it < iters; it += 4) {
+    c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c0, 0, 0, 0);
+    c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c1, 0, 0, 0);
+    c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c2, 0, 0, 0);
+    c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c3, 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; i++) s += c0[i] + c1[i] + c2[i] + c3[i];
+  sink[(int64_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+unsigned grid_for(int64_t work_items) {
+  int64_t b = (work_items + 255) / 256;
+  if (b > 256 * 32) b = 256 * 32;
+  if (b < 1) b = 1;
+  return (unsigned)b;
+}
+
+}  // namespace
+
+extern "C" int mtp_activation_bwd(const void* dact, const void* y, void* dy, int64_t M, int64_t N, int dtype,
+                                  int epilogue, void* stream) {
+  MTP_REQUIRE(M >= 0 && N >= 1, MTP_EINVAL, "activation_bwd: M=%lld N=%lld", (long long)M, (long long)N);
+  MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16, MTP_EINVAL, "activation_bwd: unknown dtype %d", dtype);
+  if (M == 0) return MTP_OK;
+  MTP_REQUIRE(dact && y && dy, MTP_EINVAL, "activation_bwd: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  const uintptr_t al = reinterpret_cast<uintptr_t>(dact) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(dy);
+  if (epilogue == MTP_EPI_BIAS_GELU || epilogue == MTP_EPI_GELU) {
+    MTP_REQUIRE((al & 15) == 0, MTP_EUNSUPPORTED, "activation_bwd: buffers must be 16-byte aligned");
+    const int64_t n = M * N;
+    if (dtype == MTP_F32)
+      hipLaunchKernelGGL(gelu_bwd_kernel<float>, dim3(grid_for(n / 4 + 1)), dim3(256), 0, s, (const float*)dact,
+                         (const float*)y, (float*)dy, n);
+    else
+      hipLaunchKernelGGL(gelu_bwd_kernel<uint16_t>, dim3(grid_for(n / 8 + 1)), dim3(256), 0, s,
+                         (const uint16_t*)dact, (const uint16_t*)y, (uint16_t*)dy, n);
+  } else if (epilogue == MTP_EPI_SWIGLU) {
+    MTP_REQUIRE(N % 2 == 0, MTP_EINVAL, "activation_bwd: SwiGLU needs an even N, got %lld", (long long)N);
+    MTP_REQUIRE(dy != dact, MTP_EINVAL, "activation_bwd: SwiGLU output may not alias dact");
+    const int64_t H = N / 2;
+    const int epv = dtype == MTP_F32 ? 4 : 8;
+    const bool vec = (al & 15) == 0 && H % epv == 0;
+    if (dtype == MTP_F32) {
+      if (vec)
+        hipLaunchKernelGGL((swiglu_bwd_kernel<float, true>), dim3(grid_for(M * H / 4)), dim3(256), 0, s,
+                           (const float*)dact, (const float*)y, (float*)dy, M, H);
+      else
+        hipLaunchKernelGGL((swiglu_bwd_kernel<float, false>), dim3(grid_for(M * H)), dim3(256), 0, s,
+                           (const float*)dact, (const float*)y, (float*)dy, M, H);
+    } else {
+      if (vec)
+        hipLaunchKernelGGL((swiglu_bwd_kernel<uint16_t, true>), dim3(grid_for(M * H / 8)), dim3(256), 0, s,
+                           (const uint16_t*)dact, (const uint16_t*)y, (uint16_t*)dy, M, H);
+      else
+        hipLaunchKernelGGL((swiglu_bwd_kernel<uint16_t, false>), dim3(grid_for(M * H)), dim3(256), 0, s,
+                           (const uint16_t*)dact, (const uint16_t*)y, (uint16_t*)dy, M, H);
+    }
+  } else {
+    MTP_REQUIRE(false, MTP_EINVAL, "activation_bwd: epilogue %d has no activation", epilogue);
+  }
+  MTP_CHECK_LAUNCH("activation_bwd");
+  return MTP_OK;
+}
+
+extern "C" int mtp_stream_copy(const void* src, void* dst, int64_t bytes, void* stream) {
+  MTP_REQUIRE(bytes >= 0 && bytes % 16 == 0, MTP_EINVAL, "stream_copy: bytes=%lld not a multiple of 16", (long long)bytes);
+  if (bytes == 0) return MTP_OK;
+  MTP_REQUIRE(src && dst, MTP_EINVAL, "stream_copy: null pointer");
+  MTP_REQUIRE(((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0, MTP_EINVAL,
+              "stream_copy: buffers must be 16-byte aligned");
+  const int64_t nvec = bytes / 16;
+  int64_t blocks = (nvec + 256 * 4 - 1) / (256 * 4);
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const u32x4_t*)src, (u32x4_t*)dst, nvec);
+  MTP_CHECK_LAUNCH("stream_copy");
+  return MTP_OK;
+}
+
+extern "C" int mtp_mfma_peak(float* sink, int64_t n_waves, int64_t iters, void* stream) {
+  MTP_REQUIRE(sink && n_waves >= 4 && n_waves % 4 == 0 && iters >= 4 && iters % 4 == 0, MTP_EINVAL,
+              "mfma_peak: n_waves and iters must be positive multiples of 4");
+  hipLaunchKernelGGL(mfma_peak_kernel, dim3((unsigned)(n_waves / 4)), dim3(256), 0, (hipStream_t)stream, sink, iters);
+  MTP_CHECK_LAUNCH("mfma_peak");
+  return MTP_OK;
+}

@@ -1,0 +1,104 @@
+// Entry points of the linear layers: argument checks and the choice between
+// the bf16 MFMA kernel, and the general fp32-MFMA kernel that serves fp32
+// tensors and every bf16 shape the fast kernel does not take.
+#include "mtp_common.h"
+
+int mtp_gemm_bf16_nt(const void* A, const void* B, const void* bias, void* C, void* C2, int64_t M, int64_t N,
+                     int64_t K, int epilogue, hipStream_t s);
+int mtp_gemm_bf16_dgrad(const void* dy, const void* w, void* dx, int64_t M, int64_t N, int64_t K, hipStream_t s);
+int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
+                        int dw_dtype, int accumulate, hipStream_t s);
+int mtp_gemm_generic(const void* A, int64_t sam, int64_t sak, const void* B, int64_t sbn, int64_t sbk,
+                     const void* bias, void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, int out_dtype,
+                     int accumulate, hipStream_t s);
+int mtp_colsum(const void* dy, void* db, int64_t M, int64_t N, int dtype, int out_dtype, int accumulate,
+               hipStream_t s);
+int mtp_act_fwd(const void* y, void* act, int64_t M, int64_t N, int dtype, int swiglu, hipStream_t s);
+
+namespace {
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_dims(const char* what, int64_t M, int64_t N, int64_t K, int dtype) {
+  MTP_REQUIRE(M >= 0 && N >= 1 && K >= 1, MTP_EINVAL, "%s: M=%lld N=%lld K=%lld", what, (long long)M, (long long)N,
+              (long long)K);
+  MTP_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), MTP_EUNSUPPORTED,
+              "%s: a dimension exceeds 2^31-1", what);
+  MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16, MTP_EINVAL, "%s: unknown dtype %d", what, dtype);
+  return MTP_OK;
+}
+
+// The bf16 MFMA kernel needs 16-byte aligned rows, and tile-relative byte offsets below 2^31.
+bool fast_ok(int64_t rows_ld_a, int64_t rows_ld_b, const void* a, const void* b) {
+  return rows_ld_a % 8 == 0 && rows_ld_b % 8 == 0 && aligned16(a) && aligned16(b) && rows_ld_a * 2 * 256 < (1ll << 31) &&
+         rows_ld_b * 2 * 256 < (1ll << 31);
+}
+
+}  // namespace
+
+extern "C" int mtp_linear_fwd(const void* x, const void* w, const void* bias, void* y, void* act, int64_t M,
+                              int64_t N, int64_t K, int dtype, int epilogue, void* stream) {
+  int rc = check_dims("linear_fwd", M, N, K, dtype);
+  if (rc) return rc;
+  MTP_REQUIRE(epilogue >= MTP_EPI_NONE && epilogue <= MTP_EPI_GELU, MTP_EINVAL, "linear_fwd: unknown epilogue %d",
+              epilogue);
+  const bool has_act = epilogue == MTP_EPI_BIAS_GELU || epilogue == MTP_EPI_SWIGLU || epilogue == MTP_EPI_GELU;
+  MTP_REQUIRE(has_act ? act != nullptr : act == nullptr, MTP_EINVAL,
+              "linear_fwd: act must be given exactly for the activation epilogues");
+  MTP_REQUIRE(has_act || y, MTP_EINVAL, "linear_fwd: null output");
+  MTP_REQUIRE((epilogue != MTP_EPI_BIAS && epilogue != MTP_EPI_BIAS_GELU) || bias, MTP_EINVAL,
+              "linear_fwd: bias epilogue without bias");
+  MTP_REQUIRE(epilogue != MTP_EPI_SWIGLU || N % 2 == 0, MTP_EINVAL, "linear_fwd: SwiGLU needs an even N");
+  if (M == 0) return MTP_OK;
+  MTP_REQUIRE(x && w, MTP_EINVAL, "linear_fwd: null input");
+  hipStream_t s = (hipStream_t)stream;
+  const void* use_bias = (epilogue == MTP_EPI_NONE || epilogue == MTP_EPI_GELU) ? nullptr : bias;
+
+  if (dtype == MTP_BF16 && fast_ok(K, K, x, w) && N * K * 2 < (1ll << 31)) {
+    int epi = epilogue;
+    if (epilogue == MTP_EPI_SWIGLU && !use_bias) use_bias = nullptr;
+    return mtp_gemm_bf16_nt(x, w, use_bias, y, act, M, N, K, epi, s);
+  }
+  // general path: GEMM (+bias) into y, then the activation as a second pass
+  MTP_REQUIRE(y, MTP_EUNSUPPORTED, "linear_fwd: this shape needs the pre-activation buffer y");
+  rc = mtp_gemm_generic(x, K, 1, w, K, 1, use_bias, y, N, M, N, K, dtype, dtype, 0, s);
+  if (rc) return rc;
+  if (has_act) return mtp_act_fwd(y, act, M, N, dtype, epilogue == MTP_EPI_SWIGLU, s);
+  return MTP_OK;
+}
+
+extern "C" int mtp_linear_dgrad(const void* dy, const void* w, void* dx, int64_t M, int64_t N, int64_t K, int dtype,
+                                void* stream) {
+  int rc = check_dims("linear_dgrad", M, N, K, dtype);
+  if (rc) return rc;
+  if (M == 0) return MTP_OK;
+  MTP_REQUIRE(dy && w && dx, MTP_EINVAL, "linear_dgrad: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == MTP_BF16 && fast_ok(N, K, dy, w) && aligned16(dx)) {
+    rc = mtp_gemm_bf16_dgrad(dy, w, dx, M, N, K, s);
+    if (rc != MTP_EUNSUPPORTED) return rc;
+  }
+  // dX[m,k] = sum_n dY[m,n] W[n,k]: A = dY (N,1), B(k,n) = W[n*K + k]
+  return mtp_gemm_generic(dy, N, 1, w, 1, K, nullptr, dx, K, M, K, N, dtype, dtype, 0, s);
+}
+
+extern "C" int mtp_linear_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
+                                int dtype, int dw_dtype, int accumulate, void* stream) {
+  int rc = check_dims("linear_wgrad", M, N, K, dtype);
+  if (rc) return rc;
+  MTP_REQUIRE(dw_dtype == MTP_F32 || dw_dtype == MTP_BF16, MTP_EINVAL, "linear_wgrad: unknown dw_dtype %d", dw_dtype);
+  MTP_REQUIRE(!(dtype == MTP_F32 && dw_dtype == MTP_BF16), MTP_EUNSUPPORTED,
+              "linear_wgrad: fp32 inputs with bf16 gradients are not supported");
+  MTP_REQUIRE(dw, MTP_EINVAL, "linear_wgrad: null dw");
+  MTP_REQUIRE(M == 0 || (dy && x), MTP_EINVAL, "linear_wgrad: null input");
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == MTP_BF16 && M > 0 && fast_ok(N, K, dy, x) && aligned16(dw)) {
+    rc = mtp_gemm_bf16_wgrad(dy, x, dw, db, M, N, K, dw_dtype, accumulate, s);
+    if (rc != MTP_EUNSUPPORTED) return rc;
+  }
+  // dW[n,k] = sum_m dY[m,n] X[m,k]: A(n,m) = dY[m*N + n], B(k,m) = X[m*K + k]; M == 0 writes zeros
+  rc = mtp_gemm_generic(dy, 1, N, x, 1, K, nullptr, dw, K, N, K, M, dtype, dw_dtype, accumulate, s);
+  if (rc) return rc;
+  if (db) return mtp_colsum(dy, db, M, N, dtype, dw_dtype, accumulate, s);
+  return MTP_OK;
+}

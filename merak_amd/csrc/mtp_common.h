@@ -1,0 +1,87 @@
+// Shared device helpers for the gfx950 kernels: wave64 reductions, bf16
+// conversion, 16-byte vector types, and the host-side error plumbing.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/merak_tp_gfx950.h"
+
+#define MTP_WAVE 64
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+
+#define LDS_PTR(p) ((void __attribute__((address_space(3)))*)(p))
+
+// ---- bf16 <-> f32 --------------------------------------------------------
+__device__ __forceinline__ float bf16_lo(uint32_t packed) {  // element 0 of a pair
+  return __uint_as_float(packed << 16);
+}
+__device__ __forceinline__ float bf16_hi(uint32_t packed) {  // element 1 of a pair
+  return __uint_as_float(packed & 0xffff0000u);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
+  return __uint_as_float(((uint32_t)b) << 16);
+}
+// round-to-nearest-even, NaN kept quiet
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+
+// ---- wave64 reductions (butterfly over ds_bpermute-free shuffles) ---------
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// ---- activations -----------------------------------------------------------
+// gelu_new(x) = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
+// written as x * sigmoid(2u) with u the tanh argument (tanh(u) = 2 sigmoid(2u) - 1)
+__device__ __forceinline__ float gelu_new_f(float x) {
+  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+  float u = k0 * (x + k1 * x * x * x);
+  return x / (1.0f + __expf(-2.0f * u));
+}
+__device__ __forceinline__ float gelu_new_grad_f(float x) {
+  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+  float u = k0 * (x + k1 * x * x * x);
+  float s = 1.0f / (1.0f + __expf(-2.0f * u));        // sigmoid(2u)
+  float du = k0 * (1.0f + 3.0f * k1 * x * x);
+  return s + x * 2.0f * s * (1.0f - s) * du;
+}
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+
+// ---- host side -------------------------------------------------------------
+void mtp_set_error(const char* fmt, ...);
+
+#define MTP_REQUIRE(cond, code, ...)        \
+  do {                                      \
+    if (!(cond)) {                          \
+      mtp_set_error(__VA_ARGS__);           \
+      return (code);                        \
+    }                                       \
+  } while (0)
+
+#define MTP_CHECK_LAUNCH(what)                                              \
+  do {                                                                      \
+    hipError_t e_ = hipGetLastError();                                      \
+    if (e_ != hipSuccess) {                                                 \
+      mtp_set_error("%s: launch failed: %s", what, hipGetErrorString(e_));  \
+      return MTP_EDEVICE;                                                   \
+    }                                                                       \
+  } while (0)

@@ -1,0 +1,290 @@
+// Vocab-parallel cross entropy for gfx950: one workgroup per logits row.
+//
+// Forward  : one pass over the row with an online (max, sum-exp) pair per
+//            lane, combined across the wave by shuffles and across waves
+//            through LDS.  Reads N*V elements, writes 4 floats per row.
+// Backward : one pass that rewrites the row in place with
+//            (softmax - onehot) * grad_out.  Reads N*V, writes N*V.
+//
+// Rows are streamed with 16-byte loads.  A row need not start on a 16-byte
+// boundary (V=50257 fp32 rows do not): the few elements before the first
+// aligned address and after the last full vector are handled by scalar code.
+//
+// Follows Merak/core/mpu/cross_entropy.py:29-106 (see the C header for the
+// exact correspondence of outputs to reference lines).
+#include "mtp_common.h"
+
+namespace {
+
+constexpr int CE_THREADS = 256;
+constexpr int CE_WAVES = CE_THREADS / MTP_WAVE;
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float NEG_BIG = -3.0e38f;  // finite stand-in for -inf: keeps (-inf) - m well defined
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+  static constexpr int EPV = 4;  // elements per 16-byte vector
+  __device__ static __forceinline__ float ld(const float* p) { return *p; }
+  __device__ static __forceinline__ void st(float* p, float v) { *p = v; }
+  __device__ static __forceinline__ void unpack(const u32x4_t& v, float* f) {
+    f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y);
+    f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+  }
+  __device__ static __forceinline__ u32x4_t pack(const float* f) {
+    u32x4_t v;
+    v.x = __float_as_uint(f[0]); v.y = __float_as_uint(f[1]);
+    v.z = __float_as_uint(f[2]); v.w = __float_as_uint(f[3]);
+    return v;
+  }
+};
+template <> struct Elem<uint16_t> {  // bf16 bits
+  static constexpr int EPV = 8;
+  __device__ static __forceinline__ float ld(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+  __device__ static __forceinline__ void st(uint16_t* p, float v) { *p = f32_to_bf16_bits(v); }
+  __device__ static __forceinline__ void unpack(const u32x4_t& v, float* f) {
+    f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x); f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
+    f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z); f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
+  }
+  __device__ static __forceinline__ u32x4_t pack(const float* f) {
+    u32x4_t v;
+    v.x = pack_bf16x2(f[0], f[1]); v.y = pack_bf16x2(f[2], f[3]);
+    v.z = pack_bf16x2(f[4], f[5]); v.w = pack_bf16x2(f[6], f[7]);
+    return v;
+  }
+};
+
+// Split a row of V elements starting at p into [0,head) scalar, nvec aligned
+// 16-byte vectors, and a scalar tail.
+template <typename T>
+__device__ __forceinline__ void row_split(const T* p, int64_t V, int& head, int64_t& nvec) {
+  constexpr int EPV = Elem<T>::EPV;
+  uintptr_t mis = reinterpret_cast<uintptr_t>(p) & 15u;
+  int h = mis ? (int)((16u - mis) / sizeof(T)) : 0;
+  if (h > V) h = (int)V;
+  head = h;
+  nvec = (V - h) / EPV;
+}
+
+struct MaxSum {
+  float m, s;
+};
+__device__ __forceinline__ MaxSum ms_combine(MaxSum a, MaxSum b) {
+  float m = fmaxf(a.m, b.m);
+  MaxSum r;
+  r.m = m;
+  r.s = a.s * __builtin_amdgcn_exp2f((a.m - m) * LOG2E) + b.s * __builtin_amdgcn_exp2f((b.m - m) * LOG2E);
+  return r;
+}
+
+template <int N>
+__device__ __forceinline__ void ms_accumulate(MaxSum& acc, const float* f) {
+  float lm = f[0];
+#pragma unroll
+  for (int i = 1; i < N; i++) lm = fmaxf(lm, f[i]);
+  float m = fmaxf(acc.m, lm);
+  float mc = m * LOG2E;
+  float s = acc.s * __builtin_amdgcn_exp2f(acc.m * LOG2E - mc);
+#pragma unroll
+  for (int i = 0; i < N; i++) s += __builtin_amdgcn_exp2f(__builtin_fmaf(f[i], LOG2E, -mc));
+  acc.m = m;
+  acc.s = s;
+}
+
+template <typename T>
+__global__ __launch_bounds__(CE_THREADS) void vocab_ce_fwd_kernel(
+    const T* __restrict__ logits, const int64_t* __restrict__ target, float* __restrict__ loss,
+    float* __restrict__ row_max, float* __restrict__ row_sumexp, float* __restrict__ pred, int64_t V,
+    int64_t vocab_start) {
+  constexpr int EPV = Elem<T>::EPV;
+  constexpr int UNROLL = 4;
+  const int64_t row = blockIdx.x;
+  const T* rp = logits + row * V;
+  const int tid = threadIdx.x;
+
+  int head;
+  int64_t nvec;
+  row_split(rp, V, head, nvec);
+  const u32x4_t* vp = reinterpret_cast<const u32x4_t*>(rp + head);
+
+  MaxSum acc{NEG_BIG, 0.0f};
+
+  int64_t i = tid;
+  for (; i + (UNROLL - 1) * CE_THREADS < nvec; i += UNROLL * CE_THREADS) {
+    u32x4_t v[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) v[u] = __builtin_nontemporal_load(vp + i + u * CE_THREADS);
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+      float f[EPV];
+      Elem<T>::unpack(v[u], f);
+      ms_accumulate<EPV>(acc, f);
+    }
+  }
+  for (; i < nvec; i += CE_THREADS) {
+    u32x4_t v = __builtin_nontemporal_load(vp + i);
+    float f[EPV];
+    Elem<T>::unpack(v, f);
+    ms_accumulate<EPV>(acc, f);
+  }
+  // scalar head and tail (fewer than 2*EPV elements in total)
+  {
+    const int64_t tail0 = head + nvec * EPV;
+    const int n_edge = head + (int)(V - tail0);
+    if (tid < n_edge) {
+      int64_t j = tid < head ? tid : tail0 + (tid - head);
+      float f = Elem<T>::ld(rp + j);
+      ms_accumulate<1>(acc, &f);
+    }
+  }
+
+  // wave butterfly, then across waves through LDS
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    MaxSum other;
+    other.m = __shfl_xor(acc.m, o, 64);
+    other.s = __shfl_xor(acc.s, o, 64);
+    acc = ms_combine(acc, other);
+  }
+  __shared__ float sm[CE_WAVES], ss[CE_WAVES];
+  if ((tid & 63) == 0) {
+    sm[tid >> 6] = acc.m;
+    ss[tid >> 6] = acc.s;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    MaxSum t{sm[0], ss[0]};
+#pragma unroll
+    for (int w = 1; w < CE_WAVES; w++) t = ms_combine(t, MaxSum{sm[w], ss[w]});
+    const int64_t tl = target[row] - vocab_start;
+    const bool in_range = tl >= 0 && tl < V;
+    const float x_t = in_range ? Elem<T>::ld(rp + tl) : 0.0f;
+    row_max[row] = t.m;
+    row_sumexp[row] = t.s;
+    pred[row] = x_t;
+    loss[row] = logf(t.s) - (in_range ? (x_t - t.m) : 0.0f);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(CE_THREADS) void vocab_ce_bwd_kernel(
+    T* __restrict__ logits, const int64_t* __restrict__ target, const float* __restrict__ row_max,
+    const float* __restrict__ row_sumexp, const float* __restrict__ grad_out, int64_t V, int64_t vocab_start) {
+  constexpr int EPV = Elem<T>::EPV;
+  constexpr int UNROLL = 4;
+  const int64_t row = blockIdx.x;
+  T* rp = logits + row * V;
+  const int tid = threadIdx.x;
+
+  int head;
+  int64_t nvec;
+  row_split(rp, V, head, nvec);
+  u32x4_t* vp = reinterpret_cast<u32x4_t*>(rp + head);
+
+  const float g = grad_out ? grad_out[row] : 1.0f;
+  const float mc = row_max[row] * LOG2E;
+  const float scale = g / row_sumexp[row];  // softmax_j * g = exp(x_j - m) * scale
+  int64_t tl = target[row] - vocab_start;
+  if (tl < 0 || tl >= V) tl = -1;
+  // position of the target inside the vector body, in elements (or out of reach)
+  const int64_t tv = (tl >= head) ? (tl - head) : -1;
+
+  int64_t i = tid;
+  for (; i + (UNROLL - 1) * CE_THREADS < nvec; i += UNROLL * CE_THREADS) {
+    u32x4_t v[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) v[u] = __builtin_nontemporal_load(vp + i + u * CE_THREADS);
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+      float f[EPV];
+      Elem<T>::unpack(v[u], f);
+#pragma unroll
+      for (int e = 0; e < EPV; e++) f[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc)) * scale;
+      const int64_t base = (i + u * CE_THREADS) * EPV;
+      if ((uint64_t)(tv - base) < (uint64_t)EPV) {
+        const int e = (int)(tv - base);
+#pragma unroll
+        for (int q = 0; q < EPV; q++)
+          if (q == e) f[q] -= g;
+      }
+      __builtin_nontemporal_store(Elem<T>::pack(f), vp + i + u * CE_THREADS);
+    }
+  }
+  for (; i < nvec; i += CE_THREADS) {
+    u32x4_t v = __builtin_nontemporal_load(vp + i);
+    float f[EPV];
+    Elem<T>::unpack(v, f);
+#pragma unroll
+    for (int e = 0; e < EPV; e++) f[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc)) * scale;
+    const int64_t base = i * EPV;
+    if ((uint64_t)(tv - base) < (uint64_t)EPV) {
+      const int e = (int)(tv - base);
+#pragma unroll
+      for (int q = 0; q < EPV; q++)
+        if (q == e) f[q] -= g;
+    }
+    __builtin_nontemporal_store(Elem<T>::pack(f), vp + i);
+  }
+  {
+    const int64_t tail0 = head + nvec * EPV;
+    const int n_edge = head + (int)(V - tail0);
+    if (tid < n_edge) {
+      int64_t j = tid < head ? tid : tail0 + (tid - head);
+      float f = Elem<T>::ld(rp + j);
+      f = __builtin_amdgcn_exp2f(__builtin_fmaf(f, LOG2E, -mc)) * scale;
+      if (j == tl) f -= g;
+      Elem<T>::st(rp + j, f);
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int mtp_vocab_ce_fwd(const void* logits, const int64_t* target, float* loss, float* row_max,
+                                float* row_sumexp, float* pred, int64_t n_rows, int64_t vocab,
+                                int64_t vocab_start, int dtype, void* stream) {
+  MTP_REQUIRE(n_rows >= 0 && vocab >= 1, MTP_EINVAL, "vocab_ce_fwd: n_rows=%lld vocab=%lld", (long long)n_rows,
+              (long long)vocab);
+  MTP_REQUIRE(n_rows < (1ll << 31), MTP_EUNSUPPORTED, "vocab_ce_fwd: n_rows=%lld exceeds 2^31-1", (long long)n_rows);
+  if (n_rows == 0) return MTP_OK;
+  MTP_REQUIRE(logits && target && loss && row_max && row_sumexp && pred, MTP_EINVAL, "vocab_ce_fwd: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((unsigned)n_rows), block(CE_THREADS);
+  if (dtype == MTP_F32) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 3) == 0, MTP_EINVAL, "vocab_ce_fwd: fp32 logits not 4-byte aligned");
+    hipLaunchKernelGGL(vocab_ce_fwd_kernel<float>, grid, block, 0, s, (const float*)logits, target, loss, row_max,
+                       row_sumexp, pred, vocab, vocab_start);
+  } else if (dtype == MTP_BF16) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL, "vocab_ce_fwd: bf16 logits not 2-byte aligned");
+    hipLaunchKernelGGL(vocab_ce_fwd_kernel<uint16_t>, grid, block, 0, s, (const uint16_t*)logits, target, loss,
+                       row_max, row_sumexp, pred, vocab, vocab_start);
+  } else {
+    MTP_REQUIRE(false, MTP_EINVAL, "vocab_ce_fwd: unknown dtype %d", dtype);
+  }
+  MTP_CHECK_LAUNCH("vocab_ce_fwd");
+  return MTP_OK;
+}
+
+extern "C" int mtp_vocab_ce_bwd(void* logits, const int64_t* target, const float* row_max, const float* row_sumexp,
+                                const float* grad_out, int64_t n_rows, int64_t vocab, int64_t vocab_start, int dtype,
+                                void* stream) {
+  MTP_REQUIRE(n_rows >= 0 && vocab >= 1, MTP_EINVAL, "vocab_ce_bwd: n_rows=%lld vocab=%lld", (long long)n_rows,
+              (long long)vocab);
+  MTP_REQUIRE(n_rows < (1ll << 31), MTP_EUNSUPPORTED, "vocab_ce_bwd: n_rows=%lld exceeds 2^31-1", (long long)n_rows);
+  if (n_rows == 0) return MTP_OK;
+  MTP_REQUIRE(logits && target && row_max && row_sumexp, MTP_EINVAL, "vocab_ce_bwd: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((unsigned)n_rows), block(CE_THREADS);
+  if (dtype == MTP_F32) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 3) == 0, MTP_EINVAL, "vocab_ce_bwd: fp32 logits not 4-byte aligned");
+    hipLaunchKernelGGL(vocab_ce_bwd_kernel<float>, grid, block, 0, s, (float*)logits, target, row_max, row_sumexp,
+                       grad_out, vocab, vocab_start);
+  } else if (dtype == MTP_BF16) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL, "vocab_ce_bwd: bf16 logits not 2-byte aligned");
+    hipLaunchKernelGGL(vocab_ce_bwd_kernel<uint16_t>, grid, block, 0, s, (uint16_t*)logits, target, row_max,
+                       row_sumexp, grad_out, vocab, vocab_start);
+  } else {
+    MTP_REQUIRE(false, MTP_EINVAL, "vocab_ce_bwd: unknown dtype %d", dtype);
+  }
+  MTP_CHECK_LAUNCH("vocab_ce_bwd");
+  return MTP_OK;
+}

@@ -1,0 +1,245 @@
+"""Tensor-level wrappers over the C ABI: shape/dtype/device checks, output
+allocation through PyTorch's caching allocator, and the current HIP stream.
+
+PyTorch is plumbing here (device memory and streams); every FLOP and every
+byte moved happens inside ``libmerak_tp_gfx950.so``.  CPU tensors are rejected:
+there is no fallback path.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import (EPI_BIAS, EPI_BIAS_GELU, EPI_GELU, EPI_NONE, EPI_SWIGLU,
+                   MTP_BF16, MTP_F32)
+
+_DTYPES = {torch.float32: MTP_F32, torch.bfloat16: MTP_BF16}
+_arch_ok = {}
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError(f"merak_amd kernels take float32 or bfloat16 tensors, got {t.dtype}") from None
+
+
+def _require_gpu(*ts: torch.Tensor) -> torch.device:
+    dev = None
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(
+                "merak_amd kernels run on an MI355X (gfx950) device only; got a tensor on "
+                f"{t.device}. There is no CPU fallback.")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    if idx not in _arch_ok:
+        with torch.cuda.device(idx):
+            arch = _lib.device_arch()
+        if arch != "gfx950":
+            raise RuntimeError(f"merak_amd kernels are built for gfx950 only; device {idx} is {arch}")
+        _arch_ok[idx] = True
+    return dev
+
+
+def _stream(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _contig(t: torch.Tensor) -> torch.Tensor:
+    return t if t.is_contiguous() else t.contiguous()
+
+
+# --------------------------------------------------------------------------- linear
+def linear_fwd(x2d: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], epilogue: int = EPI_NONE,
+               want_pre: bool = True) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """(y, act) = epilogue(x2d @ w.T + bias).  x2d [M,K], w [N,K] contiguous, same dtype."""
+    dev = _require_gpu(x2d, w, bias)
+    M, K = x2d.shape
+    N, K2 = w.shape
+    if K != K2:
+        raise ValueError(f"linear_fwd: x is [*, {K}] but weight is [{N}, {K2}]")
+    if w.dtype != x2d.dtype or (bias is not None and bias.dtype != x2d.dtype):
+        raise TypeError("linear_fwd: x, weight and bias must share one dtype")
+    x2d, w = _contig(x2d), _contig(w)
+    has_act = epilogue in (EPI_BIAS_GELU, EPI_SWIGLU, EPI_GELU)
+    y = torch.empty((M, N), dtype=x2d.dtype, device=dev) if (want_pre or not has_act) else None
+    act = None
+    if has_act:
+        act = torch.empty((M, N // 2 if epilogue == EPI_SWIGLU else N), dtype=x2d.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_linear_fwd(_p(x2d), _p(w), _p(bias), _p(y), _p(act), M, N, K, _dt(x2d), epilogue,
+                                             _stream(dev)), "mtp_linear_fwd")
+    return y, act
+
+
+def linear_dgrad(dy2d: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    dev = _require_gpu(dy2d, w)
+    M, N = dy2d.shape
+    N2, K = w.shape
+    if N != N2 or dy2d.dtype != w.dtype:
+        raise ValueError("linear_dgrad: dy/weight mismatch")
+    dy2d, w = _contig(dy2d), _contig(w)
+    dx = torch.empty((M, K), dtype=dy2d.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_linear_dgrad(_p(dy2d), _p(w), _p(dx), M, N, K, _dt(dy2d), _stream(dev)),
+                   "mtp_linear_dgrad")
+    return dx
+
+
+def linear_wgrad(dy2d: torch.Tensor, x2d: torch.Tensor, want_db: bool, out_dtype: Optional[torch.dtype] = None,
+                 dw: Optional[torch.Tensor] = None, db: Optional[torch.Tensor] = None,
+                 accumulate: bool = False) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    dev = _require_gpu(dy2d, x2d, dw, db)
+    M, N = dy2d.shape
+    M2, K = x2d.shape
+    if M != M2 or dy2d.dtype != x2d.dtype:
+        raise ValueError("linear_wgrad: dy/x mismatch")
+    dy2d, x2d = _contig(dy2d), _contig(x2d)
+    out_dtype = out_dtype or (dw.dtype if dw is not None else dy2d.dtype)
+    if dw is None:
+        if accumulate:
+            raise ValueError("linear_wgrad: accumulate needs an existing dw")
+        dw = torch.empty((N, K), dtype=out_dtype, device=dev)
+    if want_db and db is None:
+        if accumulate:
+            raise ValueError("linear_wgrad: accumulate needs an existing db")
+        db = torch.empty((N,), dtype=out_dtype, device=dev)
+    if dw.shape != (N, K) or not dw.is_contiguous() or dw.dtype != out_dtype:
+        raise ValueError("linear_wgrad: dw must be a contiguous [N,K] tensor of the output dtype")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_linear_wgrad(_p(dy2d), _p(x2d), _p(dw), _p(db) if want_db else None, M, N, K,
+                                               _dt(dy2d), _DTYPES[out_dtype], int(accumulate), _stream(dev)),
+                   "mtp_linear_wgrad")
+    return dw, (db if want_db else None)
+
+
+def activation_bwd(dact: torch.Tensor, y: torch.Tensor, epilogue: int) -> torch.Tensor:
+    dev = _require_gpu(dact, y)
+    M, N = y.shape
+    dact, y = _contig(dact), _contig(y)
+    dy = torch.empty_like(y)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_activation_bwd(_p(dact), _p(y), _p(dy), M, N, _dt(y), epilogue, _stream(dev)),
+                   "mtp_activation_bwd")
+    return dy
+
+
+# --------------------------------------------------------------------------- embedding
+def embedding_gather(ids: torch.Tensor, table: torch.Tensor, vocab_start: int, vocab_end: int,
+                     oob_count: Optional[torch.Tensor] = None) -> torch.Tensor:
+    dev = _require_gpu(ids, table, oob_count)
+    if ids.dtype != torch.int64:
+        raise TypeError(f"embedding ids must be int64, got {ids.dtype}")
+    if table.dim() != 2 or not table.is_contiguous():
+        raise ValueError("embedding table must be a contiguous [rows, dim] tensor")
+    if table.shape[0] != vocab_end - vocab_start:
+        raise ValueError("embedding table rows do not match the vocab range")
+    flat = _contig(ids).view(-1)
+    out = torch.empty((flat.numel(), table.shape[1]), dtype=table.dtype, device=dev)
+    row_bytes = table.shape[1] * table.element_size()
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_embedding_gather(_p(flat), _p(table), _p(out), flat.numel(), row_bytes, vocab_start,
+                                                   vocab_end, _p(oob_count), _stream(dev)), "mtp_embedding_gather")
+    return out.view(*ids.shape, table.shape[1])
+
+
+def embedding_bwd(ids: torch.Tensor, dout: torch.Tensor, rows: int, vocab_start: int, vocab_end: int) -> torch.Tensor:
+    """Dense fp32 gradient [rows, dim] of the lookup."""
+    dev = _require_gpu(ids, dout)
+    flat = _contig(ids).view(-1)
+    dim = dout.shape[-1]
+    d2 = _contig(dout).view(-1, dim)
+    dtable = torch.zeros((rows, dim), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_embedding_bwd(_p(flat), _p(d2), _p(dtable), flat.numel(), dim, _dt(d2), vocab_start,
+                                                vocab_end, _stream(dev)), "mtp_embedding_bwd")
+    return dtable
+
+
+# --------------------------------------------------------------------------- cross entropy
+def vocab_ce_fwd(logits2d: torch.Tensor, target1d: torch.Tensor, vocab_start: int):
+    """-> (loss, row_max, row_sumexp, pred), all fp32 [n_rows]."""
+    dev = _require_gpu(logits2d, target1d)
+    if target1d.dtype != torch.int64:
+        raise TypeError(f"cross-entropy targets must be int64, got {target1d.dtype}")
+    if not logits2d.is_contiguous():
+        raise ValueError("vocab_parallel_cross_entropy needs contiguous logits")
+    n, v = logits2d.shape
+    if target1d.numel() != n:
+        raise ValueError(f"target has {target1d.numel()} entries for {n} logits rows")
+    target1d = _contig(target1d)
+    out = torch.empty((4, n), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_vocab_ce_fwd(_p(logits2d), _p(target1d), _p(out[0]), _p(out[1]), _p(out[2]),
+                                               _p(out[3]), n, v, vocab_start, _dt(logits2d), _stream(dev)),
+                   "mtp_vocab_ce_fwd")
+    return out[0], out[1], out[2], out[3]
+
+
+def vocab_ce_bwd_(logits2d: torch.Tensor, target1d: torch.Tensor, row_max: torch.Tensor, row_sumexp: torch.Tensor,
+                  grad_out: Optional[torch.Tensor], vocab_start: int) -> torch.Tensor:
+    """In place: logits2d <- (softmax - onehot) * grad_out.  Returns logits2d."""
+    dev = _require_gpu(logits2d, target1d, row_max, row_sumexp, grad_out)
+    n, v = logits2d.shape
+    if grad_out is not None:
+        grad_out = _contig(grad_out.to(torch.float32))
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_vocab_ce_bwd(_p(logits2d), _p(_contig(target1d)), _p(row_max), _p(row_sumexp),
+                                               _p(grad_out), n, v, vocab_start, _dt(logits2d), _stream(dev)),
+                   "mtp_vocab_ce_bwd")
+    return logits2d
+
+
+# --------------------------------------------------------------------------- decode
+def gemv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE) -> torch.Tensor:
+    dev = _require_gpu(x, w, bias)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise TypeError("gemv is bf16 only")
+    B, K = x.shape
+    N = w.shape[0]
+    x, w = _contig(x), _contig(w)
+    y = torch.empty((B, N // 2 if epilogue == EPI_SWIGLU else N), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_gemv(_p(x), _p(w), _p(bias), _p(y), B, N, K, epilogue, _stream(dev)), "mtp_gemv")
+    return y
+
+
+def gemv_argmax(x: torch.Tensor, w: torch.Tensor, workspace: Optional[torch.Tensor] = None):
+    """-> (idx int64 [B], maxval fp32 [B]) without materialising the logits."""
+    dev = _require_gpu(x, w, workspace)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise TypeError("gemv_argmax is bf16 only")
+    B, K = x.shape
+    N = w.shape[0]
+    x, w = _contig(x), _contig(w)
+    need = _lib.lib().mtp_gemv_argmax_workspace_bytes(B, N, K)
+    if workspace is None:
+        workspace = torch.empty((need,), dtype=torch.uint8, device=dev)
+    idx = torch.empty((B,), dtype=torch.int64, device=dev)
+    val = torch.empty((B,), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_gemv_argmax(_p(x), _p(w), _p(idx), _p(val), _p(workspace), workspace.numel(), B, N, K,
+                                              _stream(dev)), "mtp_gemv_argmax")
+    return idx, val
+
+
+def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
+    dev = _require_gpu(logits)
+    l2 = _contig(logits).view(-1, logits.shape[-1])
+    idx = torch.empty((l2.shape[0],), dtype=torch.int64, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_argmax_rows(_p(l2), _p(idx), l2.shape[0], l2.shape[1], _dt(l2), _stream(dev)),
+                   "mtp_argmax_rows")
+    return idx.view(logits.shape[:-1])

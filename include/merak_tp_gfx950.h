@@ -149,7 +149,9 @@ int mtp_vocab_ce_fwd(const void* logits, const int64_t* target,
  * (cross_entropy.py:86-106).  row_max / row_sumexp are the (globally
  * combined) values from the forward.  grad_out may be NULL (= 1 for every
  * row), which together with out-of-range targets yields the softmax the
- * reference leaves in the caller's logits after forward (:80). */
+ * reference leaves in the caller's logits after forward (:80).
+ * row_max == row_sumexp == NULL means the buffer already holds that softmax
+ * (the reference's backward, :92-104): logits[i,j] <- (logits[i,j] - onehot) * grad_out[i]. */
 int mtp_vocab_ce_bwd(void* logits, const int64_t* target,
                      const float* row_max, const float* row_sumexp,
                      const float* grad_out,

@@ -288,9 +288,14 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
     }
     return n0 + wn * WN + j * 32;
   };
-  const int col_limit_main = p.N;
+  // first column past the valid range of block j: SwiGLU gate blocks end at `half` (the columns after it
+  // are the up matrix, owned by other blocks)
+  auto lim_of_block = [&](int j) -> int {
+    if (EPI == MTP_EPI_SWIGLU) return j < TJ / 2 ? p.half : p.N;
+    return p.N;
+  };
 
-  auto flush = [&](int i, void* out, int64_t ld, int nblk, auto colfn, int col_limit, bool f32out, bool accumulate) {
+  auto flush = [&](int i, void* out, int64_t ld, int nblk, auto colfn, auto limfn, bool f32out, bool accumulate) {
     // 16-byte chunks of the staged 32 x (nblk*32) block
     const int esz = f32out ? 4 : 2;
     const int chunks_per_row = nblk * 32 * esz / 16;
@@ -302,6 +307,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
       const int e0 = cc * epc;           // element offset inside the staged row
       const int j = e0 >> 5;
       const int col = colfn(j) + (e0 & 31);
+      const int col_limit = limfn(j);
       const int row = mrow0 + r;
       if (row < p.M && col < col_limit) {
         u32x4_t v = *reinterpret_cast<const u32x4_t*>(stage + r * PITCH + cc * 16);
@@ -357,7 +363,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
               const int col = cb + 8 * g + 4 * lh + e;
-              b4[e] = col < col_limit_main ? bf16_bits_to_f32(p.bias[col]) : 0.f;
+              b4[e] = col < lim_of_block(j) ? bf16_bits_to_f32(p.bias[col]) : 0.f;
             }
           }
         }
@@ -375,7 +381,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
             *reinterpret_cast<f32x4_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 4) = v;
           }
         wave_lds_sync();
-        flush(i, p.C, p.ldc, TJ, col_of_block, col_limit_main, true, p.accumulate != 0);
+        flush(i, p.C, p.ldc, TJ, col_of_block, lim_of_block, true, p.accumulate != 0);
         wave_lds_sync();
       }
     } else {
@@ -393,7 +399,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
             *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
           }
         wave_lds_sync();
-        flush(i, p.C, p.ldc, TJ, col_of_block, col_limit_main, false, p.accumulate != 0);
+        flush(i, p.C, p.ldc, TJ, col_of_block, lim_of_block, false, p.accumulate != 0);
         wave_lds_sync();
       }
       if (EPI == MTP_EPI_BIAS_GELU || EPI == MTP_EPI_GELU) {
@@ -406,7 +412,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
             *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
           }
         wave_lds_sync();
-        flush(i, p.C2, p.ldc2, TJ, col_of_block, col_limit_main, false, false);
+        flush(i, p.C2, p.ldc2, TJ, col_of_block, lim_of_block, false, false);
         wave_lds_sync();
       }
       if (EPI == MTP_EPI_SWIGLU) {
@@ -423,7 +429,8 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
           }
         wave_lds_sync();
         auto act_col = [&](int j) -> int { return n0 + wn * (BN / 4) + j * 32; };
-        flush(i, p.C2, p.ldc2, HJ, act_col, p.half, false, false);
+        auto act_lim = [&](int) -> int { return p.half; };
+        flush(i, p.C2, p.ldc2, HJ, act_col, act_lim, false, false);
         wave_lds_sync();
       }
     }

@@ -43,13 +43,13 @@ extern "C" int mtp_linear_fwd(const void* x, const void* w, const void* bias, vo
   MTP_REQUIRE(epilogue >= MTP_EPI_NONE && epilogue <= MTP_EPI_GELU, MTP_EINVAL, "linear_fwd: unknown epilogue %d",
               epilogue);
   const bool has_act = epilogue == MTP_EPI_BIAS_GELU || epilogue == MTP_EPI_SWIGLU || epilogue == MTP_EPI_GELU;
+  if (M == 0) return MTP_OK;
   MTP_REQUIRE(has_act ? act != nullptr : act == nullptr, MTP_EINVAL,
               "linear_fwd: act must be given exactly for the activation epilogues");
   MTP_REQUIRE(has_act || y, MTP_EINVAL, "linear_fwd: null output");
   MTP_REQUIRE((epilogue != MTP_EPI_BIAS && epilogue != MTP_EPI_BIAS_GELU) || bias, MTP_EINVAL,
               "linear_fwd: bias epilogue without bias");
   MTP_REQUIRE(epilogue != MTP_EPI_SWIGLU || N % 2 == 0, MTP_EINVAL, "linear_fwd: SwiGLU needs an even N");
-  if (M == 0) return MTP_OK;
   MTP_REQUIRE(x && w, MTP_EINVAL, "linear_fwd: null input");
   hipStream_t s = (hipStream_t)stream;
   const void* use_bias = (epilogue == MTP_EPI_NONE || epilogue == MTP_EPI_GELU) ? nullptr : bias;
@@ -59,11 +59,14 @@ extern "C" int mtp_linear_fwd(const void* x, const void* w, const void* bias, vo
     if (epilogue == MTP_EPI_SWIGLU && !use_bias) use_bias = nullptr;
     return mtp_gemm_bf16_nt(x, w, use_bias, y, act, M, N, K, epi, s);
   }
-  // general path: GEMM (+bias) into y, then the activation as a second pass
-  MTP_REQUIRE(y, MTP_EUNSUPPORTED, "linear_fwd: this shape needs the pre-activation buffer y");
-  rc = mtp_gemm_generic(x, K, 1, w, K, 1, use_bias, y, N, M, N, K, dtype, dtype, 0, s);
+  // general path: GEMM (+bias) into y, then the activation as a second pass.  Without y the GELU forms
+  // run in place in act; SwiGLU's act is half as wide as the pre-activation, so it needs y.
+  void* pre = y;
+  if (!pre && epilogue != MTP_EPI_SWIGLU) pre = act;
+  MTP_REQUIRE(pre, MTP_EUNSUPPORTED, "linear_fwd: this shape needs the pre-activation buffer y");
+  rc = mtp_gemm_generic(x, K, 1, w, K, 1, use_bias, pre, N, M, N, K, dtype, dtype, 0, s);
   if (rc) return rc;
-  if (has_act) return mtp_act_fwd(y, act, M, N, dtype, epilogue == MTP_EPI_SWIGLU, s);
+  if (has_act) return mtp_act_fwd(pre, act, M, N, dtype, epilogue == MTP_EPI_SWIGLU, s);
   return MTP_OK;
 }
 

@@ -19,7 +19,7 @@ namespace {
 constexpr int CE_THREADS = 256;
 constexpr int CE_WAVES = CE_THREADS / MTP_WAVE;
 constexpr float LOG2E = 1.4426950408889634f;
-constexpr float NEG_BIG = -3.0e38f;  // finite stand-in for -inf: keeps (-inf) - m well defined
+constexpr float NEG_BIG = -1.0e30f;  // finite stand-in for -inf: NEG_BIG * log2(e) stays finite, exp2 of it is 0
 
 template <typename T> struct Elem;
 template <> struct Elem<float> {
@@ -65,15 +65,38 @@ __device__ __forceinline__ void row_split(const T* p, int64_t V, int& head, int6
   nvec = (V - h) / EPV;
 }
 
+// Products and differences that must be rounded on their own (the default -ffp-contract=fast would fuse
+// a*b - c into an fma, whose result differs from fl(a*b) - c by the rounding residual of a*b; for the
+// -1e30 "no data yet" sentinel that residual is astronomically large).
+__device__ __forceinline__ float mul_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a * b;
+}
+__device__ __forceinline__ float sub_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a - b;
+}
+
+// Running (max, sum-exp) pair.  Exponentials are taken as exp2(fma(x, c, -fl(m*c))) with c = log2(e): one
+// VALU op per element for the argument.  The rounding of m*c is the same for every term that shares
+// an m, so s always means sum_j exp2(x_j*c - fl(m*c)) consistently; the residual fl(m*c) - m*c is
+// exact in an fma and is folded back in once per row (ms_exact_sum).
 struct MaxSum {
   float m, s;
 };
 __device__ __forceinline__ MaxSum ms_combine(MaxSum a, MaxSum b) {
   float m = fmaxf(a.m, b.m);
+  const float mc = mul_rn(m, LOG2E);  // explicitly rounded products: no fma contraction here
   MaxSum r;
   r.m = m;
-  r.s = a.s * __builtin_amdgcn_exp2f((a.m - m) * LOG2E) + b.s * __builtin_amdgcn_exp2f((b.m - m) * LOG2E);
+  r.s = a.s * __builtin_amdgcn_exp2f(sub_rn(mul_rn(a.m, LOG2E), mc)) +
+        b.s * __builtin_amdgcn_exp2f(sub_rn(mul_rn(b.m, LOG2E), mc));
   return r;
+}
+// exp2(fl(m*c) - m*c): turns the consistent-but-shifted sum into sum_j exp((x_j - m))
+__device__ __forceinline__ float ms_residual_scale(float m) {
+  const float mc = mul_rn(m, LOG2E);
+  return __builtin_amdgcn_exp2f(-__builtin_fmaf(m, LOG2E, -mc));
 }
 
 template <int N>
@@ -82,8 +105,8 @@ __device__ __forceinline__ void ms_accumulate(MaxSum& acc, const float* f) {
 #pragma unroll
   for (int i = 1; i < N; i++) lm = fmaxf(lm, f[i]);
   float m = fmaxf(acc.m, lm);
-  float mc = m * LOG2E;
-  float s = acc.s * __builtin_amdgcn_exp2f(acc.m * LOG2E - mc);
+  float mc = mul_rn(m, LOG2E);
+  float s = acc.s * __builtin_amdgcn_exp2f(sub_rn(mul_rn(acc.m, LOG2E), mc));
 #pragma unroll
   for (int i = 0; i < N; i++) s += __builtin_amdgcn_exp2f(__builtin_fmaf(f[i], LOG2E, -mc));
   acc.m = m;
@@ -155,6 +178,7 @@ __global__ __launch_bounds__(CE_THREADS) void vocab_ce_fwd_kernel(
     MaxSum t{sm[0], ss[0]};
 #pragma unroll
     for (int w = 1; w < CE_WAVES; w++) t = ms_combine(t, MaxSum{sm[w], ss[w]});
+    t.s *= ms_residual_scale(t.m);
     const int64_t tl = target[row] - vocab_start;
     const bool in_range = tl >= 0 && tl < V;
     const float x_t = in_range ? Elem<T>::ld(rp + tl) : 0.0f;
@@ -181,8 +205,11 @@ __global__ __launch_bounds__(CE_THREADS) void vocab_ce_bwd_kernel(
   u32x4_t* vp = reinterpret_cast<u32x4_t*>(rp + head);
 
   const float g = grad_out ? grad_out[row] : 1.0f;
-  const float mc = row_max[row] * LOG2E;
-  const float scale = g / row_sumexp[row];  // softmax_j * g = exp(x_j - m) * scale
+  // row_max == nullptr: the buffer already holds the softmax, so the "exponential" is the value itself
+  const bool from_softmax = row_max == nullptr;
+  const float mc = from_softmax ? 0.0f : mul_rn(row_max[row], LOG2E);
+  // softmax_j * g = exp2(x_j*c - fl(m*c)) * scale, the rounding residual of m*c folded into scale
+  const float scale = from_softmax ? g : g * ms_residual_scale(row_max[row]) / row_sumexp[row];
   int64_t tl = target[row] - vocab_start;
   if (tl < 0 || tl >= V) tl = -1;
   // position of the target inside the vector body, in elements (or out of reach)
@@ -198,7 +225,7 @@ __global__ __launch_bounds__(CE_THREADS) void vocab_ce_bwd_kernel(
       float f[EPV];
       Elem<T>::unpack(v[u], f);
 #pragma unroll
-      for (int e = 0; e < EPV; e++) f[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc)) * scale;
+      for (int e = 0; e < EPV; e++) f[e] = (from_softmax ? f[e] : __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc))) * scale;
       const int64_t base = (i + u * CE_THREADS) * EPV;
       if ((uint64_t)(tv - base) < (uint64_t)EPV) {
         const int e = (int)(tv - base);
@@ -214,7 +241,7 @@ __global__ __launch_bounds__(CE_THREADS) void vocab_ce_bwd_kernel(
     float f[EPV];
     Elem<T>::unpack(v, f);
 #pragma unroll
-    for (int e = 0; e < EPV; e++) f[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc)) * scale;
+    for (int e = 0; e < EPV; e++) f[e] = (from_softmax ? f[e] : __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc))) * scale;
     const int64_t base = i * EPV;
     if ((uint64_t)(tv - base) < (uint64_t)EPV) {
       const int e = (int)(tv - base);
@@ -230,7 +257,7 @@ __global__ __launch_bounds__(CE_THREADS) void vocab_ce_bwd_kernel(
     if (tid < n_edge) {
       int64_t j = tid < head ? tid : tail0 + (tid - head);
       float f = Elem<T>::ld(rp + j);
-      f = __builtin_amdgcn_exp2f(__builtin_fmaf(f, LOG2E, -mc)) * scale;
+      f = (from_softmax ? f : __builtin_amdgcn_exp2f(__builtin_fmaf(f, LOG2E, -mc))) * scale;
       if (j == tl) f -= g;
       Elem<T>::st(rp + j, f);
     }
@@ -271,7 +298,9 @@ extern "C" int mtp_vocab_ce_bwd(void* logits, const int64_t* target, const float
               (long long)vocab);
   MTP_REQUIRE(n_rows < (1ll << 31), MTP_EUNSUPPORTED, "vocab_ce_bwd: n_rows=%lld exceeds 2^31-1", (long long)n_rows);
   if (n_rows == 0) return MTP_OK;
-  MTP_REQUIRE(logits && target && row_max && row_sumexp, MTP_EINVAL, "vocab_ce_bwd: null pointer");
+  MTP_REQUIRE(logits && target, MTP_EINVAL, "vocab_ce_bwd: null pointer");
+  MTP_REQUIRE((row_max == nullptr) == (row_sumexp == nullptr), MTP_EINVAL,
+              "vocab_ce_bwd: row_max and row_sumexp must both be given or both be null");
   hipStream_t s = (hipStream_t)stream;
   dim3 grid((unsigned)n_rows), block(CE_THREADS);
   if (dtype == MTP_F32) {

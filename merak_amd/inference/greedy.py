@@ -1,0 +1,50 @@
+"""Greedy decode tail on the gfx950 kernels.
+
+The reference's generation loop slices one position out of the logits and
+takes ``torch.argmax(logits, dim=-1).view(-1)``
+(Merak/inference/text_generation_inference.py:223,226-227).  Here the LM-head
+product and the argmax are one kernel pass over the weight matrix: the [B, V]
+logits are never written.  ``DecodeStep`` strings the single-token linears of
+a Llama-shaped block in front of it (QKV, gate/up with SwiGLU, down), each a
+GEMV that streams its weight once.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import ops
+
+
+def greedy_from_logits(logits: torch.Tensor) -> torch.Tensor:
+    """``torch.argmax(logits, dim=-1).view(-1)`` for materialised logits (first index on ties, NaN wins)."""
+    return ops.argmax_rows(logits).view(-1)
+
+
+def greedy_next_token(hidden: torch.Tensor, lm_head_weight: torch.Tensor,
+                      workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """argmax_n hidden[b] . lm_head_weight[n] for B <= 32 single-token rows, bf16."""
+    idx, _ = ops.gemv_argmax(hidden, lm_head_weight, workspace)
+    return idx
+
+
+class DecodeStep:
+    """Single-token pass through QKV, gate/up (+SwiGLU), down and the LM head with fused argmax.
+
+    Only the linears of the step live here (attention itself is outside the
+    tensor-parallel layers); weights are the layers' own [out, in] bf16 tensors.
+    """
+
+    def __init__(self, w_qkv, w_gate_up, w_down, w_lm_head, max_batch: int = 32):
+        self.w_qkv, self.w_gate_up, self.w_down, self.w_lm_head = w_qkv, w_gate_up, w_down, w_lm_head
+        from .. import _lib
+        need = _lib.lib().mtp_gemv_argmax_workspace_bytes(max_batch, w_lm_head.shape[0], w_lm_head.shape[1])
+        self.workspace = torch.empty((need,), dtype=torch.uint8, device=w_lm_head.device)
+
+    def __call__(self, x: torch.Tensor):
+        qkv = ops.gemv(x, self.w_qkv)
+        h = ops.gemv(x, self.w_gate_up, None, ops.EPI_SWIGLU)
+        out = ops.gemv(h, self.w_down)
+        token = greedy_next_token(out, self.w_lm_head, self.workspace)
+        return qkv, out, token

@@ -1,0 +1,107 @@
+"""Vocab-parallel cross entropy on the gfx950 kernels.
+
+Same call as Merak/core/mpu/cross_entropy.py:109-118: per-position loss of the
+shape of ``target`` from this rank's slice of the logits; targets outside the
+slice (``-100`` included) contribute no one-hot term, exactly like the
+reference's mask (:48-62).  Differences in *how*, not in *what*:
+
+* one pass computes max and sum-exp together in fp32 (the reference makes
+  about eight passes over the logits in the logits' own dtype);
+* the forward leaves the logits untouched; the backward overwrites them with
+  the gradient and returns that same storage, so — like the reference, which
+  reuses the buffer for the softmax (:37,70,80,92) — no second
+  [tokens, vocab] tensor is ever allocated;
+* for bf16 logits the loss is returned in fp32 unless
+  ``loss_in_logits_dtype=True``.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .initialize import get_model_parallel_rank, get_model_parallel_world_size
+from .utils import VocabUtility
+
+
+def _vocab_range(partition_vocab_size):
+    get_vocab_range = VocabUtility.vocab_range_from_per_partition_vocab_size
+    rank = get_model_parallel_rank()
+    world_size = get_model_parallel_world_size()
+    return get_vocab_range(partition_vocab_size, rank, world_size)
+
+
+class _VocabParallelCrossEntropy(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, vocab_parallel_logits, target, loss_in_logits_dtype, materialize_softmax):
+        if get_model_parallel_world_size() != 1:
+            raise RuntimeError(
+                "vocab_parallel_cross_entropy at tensor-parallel size > 1 needs the MAX/SUM/SUM exchange of "
+                "cross_entropy.py:33,64,72; on one rank use vocab_parallel_cross_entropy_partials() and "
+                "vocab_parallel_cross_entropy_backward_() around your own reduction")
+        partition_vocab_size = vocab_parallel_logits.size()[-1]
+        vocab_start_index, _ = _vocab_range(partition_vocab_size)
+        # [*, partition-vocab-size] view; like the reference (:55) this requires contiguous logits
+        logits_2d = vocab_parallel_logits.view(-1, partition_vocab_size)
+        target_1d = target.reshape(-1)
+        loss, row_max, row_sumexp, _ = ops.vocab_ce_fwd(logits_2d, target_1d, vocab_start_index)
+        ctx.vocab_start = vocab_start_index
+        ctx.materialized = bool(materialize_softmax)
+        if materialize_softmax:
+            # reproduce the reference's side effect: the caller's logits now hold the softmax (:80)
+            ops.vocab_ce_bwd_(logits_2d, torch.full_like(target_1d, -1), row_max, row_sumexp, None,
+                              vocab_start_index)
+        ctx.save_for_backward(vocab_parallel_logits, target_1d, row_max, row_sumexp)
+        loss = loss.view_as(target)
+        if loss_in_logits_dtype:
+            loss = loss.to(vocab_parallel_logits.dtype)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        logits, target_1d, row_max, row_sumexp = ctx.saved_tensors
+        partition_vocab_size = logits.size()[-1]
+        grad_2d = logits.view(-1, partition_vocab_size)
+        g = grad_output.reshape(-1)
+        if ctx.materialized:
+            # the buffer already holds the softmax (cross_entropy.py:92-104)
+            row_max = row_sumexp = None
+        ops.vocab_ce_bwd_(grad_2d, target_1d, row_max, row_sumexp, g, ctx.vocab_start)
+        return logits, None, None, None
+
+
+def vocab_parallel_cross_entropy(vocab_parallel_logits, target, loss_in_logits_dtype=False,
+                                 materialize_softmax=False):
+    """Cross entropy loss when logits are split across tensor parallel ranks.
+
+    Args:
+        vocab_parallel_logits: logits split across tensor parallel ranks,
+            [sequence_length, batch_size, vocab_size / num_parallel_ranks], contiguous
+        target: correct vocab ids of dimension [sequence_length, micro_batch_size]
+    """
+    return _VocabParallelCrossEntropy.apply(vocab_parallel_logits, target, loss_in_logits_dtype,
+                                            materialize_softmax)
+
+
+def vocab_parallel_cross_entropy_partials(vocab_parallel_logits, target):
+    """This rank's (row_max, row_sumexp, predicted_logit) over its vocab slice, fp32, each shaped like ``target``.
+
+    They are what the reference all-reduces with MAX, SUM and SUM (cross_entropy.py:33,64,72), except
+    that row_sumexp is relative to the *local* row_max (rescale by exp(local_max - global_max) before
+    summing) and predicted_logit is the raw logit (0 where the target is outside this slice)."""
+    partition_vocab_size = vocab_parallel_logits.size()[-1]
+    vocab_start_index, _ = _vocab_range(partition_vocab_size)
+    logits_2d = vocab_parallel_logits.view(-1, partition_vocab_size)
+    _, row_max, row_sumexp, pred = ops.vocab_ce_fwd(logits_2d, target.reshape(-1), vocab_start_index)
+    return row_max.view_as(target), row_sumexp.view_as(target), pred.view_as(target)
+
+
+def vocab_parallel_cross_entropy_backward_(vocab_parallel_logits, target, global_row_max, global_row_sumexp,
+                                           grad_output):
+    """In place gradient of this rank's logits slice given the globally combined max / sum-exp."""
+    partition_vocab_size = vocab_parallel_logits.size()[-1]
+    vocab_start_index, _ = _vocab_range(partition_vocab_size)
+    logits_2d = vocab_parallel_logits.view(-1, partition_vocab_size)
+    ops.vocab_ce_bwd_(logits_2d, target.reshape(-1), global_row_max.reshape(-1).contiguous(),
+                      global_row_sumexp.reshape(-1).contiguous(), grad_output.reshape(-1), vocab_start_index)
+    return vocab_parallel_logits

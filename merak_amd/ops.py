@@ -79,8 +79,15 @@ def linear_fwd(x2d: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
     if has_act:
         act = torch.empty((M, N // 2 if epilogue == EPI_SWIGLU else N), dtype=x2d.dtype, device=dev)
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().mtp_linear_fwd(_p(x2d), _p(w), _p(bias), _p(y), _p(act), M, N, K, _dt(x2d), epilogue,
-                                             _stream(dev)), "mtp_linear_fwd")
+        rc = _lib.lib().mtp_linear_fwd(_p(x2d), _p(w), _p(bias), _p(y), _p(act), M, N, K, _dt(x2d), epilogue,
+                                       _stream(dev))
+        if rc == -2 and y is None:
+            # shapes served by the general kernel need the pre-activation buffer for SwiGLU
+            y = torch.empty((M, N), dtype=x2d.dtype, device=dev)
+            rc = _lib.lib().mtp_linear_fwd(_p(x2d), _p(w), _p(bias), _p(y), _p(act), M, N, K, _dt(x2d), epilogue,
+                                           _stream(dev))
+            y = None
+        _lib.check(rc, "mtp_linear_fwd")
     return y, act
 
 
@@ -188,9 +195,11 @@ def vocab_ce_fwd(logits2d: torch.Tensor, target1d: torch.Tensor, vocab_start: in
     return out[0], out[1], out[2], out[3]
 
 
-def vocab_ce_bwd_(logits2d: torch.Tensor, target1d: torch.Tensor, row_max: torch.Tensor, row_sumexp: torch.Tensor,
-                  grad_out: Optional[torch.Tensor], vocab_start: int) -> torch.Tensor:
-    """In place: logits2d <- (softmax - onehot) * grad_out.  Returns logits2d."""
+def vocab_ce_bwd_(logits2d: torch.Tensor, target1d: torch.Tensor, row_max: Optional[torch.Tensor],
+                  row_sumexp: Optional[torch.Tensor], grad_out: Optional[torch.Tensor], vocab_start: int) -> torch.Tensor:
+    """In place: logits2d <- (softmax - onehot) * grad_out.  Returns logits2d.
+
+    row_max = row_sumexp = None: logits2d already holds the softmax."""
     dev = _require_gpu(logits2d, target1d, row_max, row_sumexp, grad_out)
     n, v = logits2d.shape
     if grad_out is not None:

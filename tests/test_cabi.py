@@ -1,0 +1,58 @@
+"""The C-ABI library loads on a machine without a GPU and exports exactly what the header declares.
+No compute entry point is called here."""
+import ctypes
+import os
+import re
+
+from merak_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "merak_tp_gfx950.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mtp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    names = _declared()
+    assert len(names) >= 15
+    handle = ctypes.CDLL(str(_lib.LIB_PATH))
+    for n in names:
+        assert hasattr(handle, n), f"{n} declared in the header but not exported"
+    assert sorted(_lib.SIGNATURES) == names, "ctypes signatures and header disagree"
+
+
+def test_loader_and_versions():
+    lib = _lib.lib()
+    assert lib.mtp_abi_version() == _lib.ABI_VERSION == 1
+    hdr = open(os.path.join(ROOT, "include", "merak_tp_gfx950.h")).read()
+    assert f"#define MTP_ABI_VERSION {_lib.ABI_VERSION}" in hdr
+    for name, val in (("MTP_F32", _lib.MTP_F32), ("MTP_BF16", _lib.MTP_BF16), ("MTP_EPI_NONE", _lib.EPI_NONE),
+                      ("MTP_EPI_BIAS", _lib.EPI_BIAS), ("MTP_EPI_BIAS_GELU", _lib.EPI_BIAS_GELU),
+                      ("MTP_EPI_SWIGLU", _lib.EPI_SWIGLU), ("MTP_EPI_GELU", _lib.EPI_GELU)):
+        assert re.search(rf"#define {name}\s+{val}\b", hdr), name
+
+
+def test_argument_errors_are_reported_without_a_device():
+    lib = _lib.lib()
+    # validation happens before any launch: these return error codes on a GPU-less host
+    assert lib.mtp_gemv_argmax_workspace_bytes(32, 128256, 4096) == ((128256 + 15) // 16) * 32 * 8
+    assert lib.mtp_vocab_ce_fwd(None, None, None, None, None, None, 4, 0, 0, 0, None) == -1
+    assert b"vocab" in lib.mtp_last_error()
+    assert lib.mtp_linear_fwd(None, None, None, None, None, 4, 4, 4, 7, 0, None) == -1
+    assert lib.mtp_gemv(None, None, None, None, 33, 8, 8, 0, None) == -2
+    assert b"B=33" in lib.mtp_last_error()
+    assert lib.mtp_stream_copy(None, None, 24, None) == -1
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setenv("MERAK_AMD_LIB", str(tmp_path / "nope.so"))
+    monkeypatch.setattr(_lib, "_lib", None)
+    try:
+        _lib.lib()
+    except _lib.KernelLibraryMissing as e:
+        assert "no CPU/eager fallback" in str(e)
+    else:
+        raise AssertionError("a missing kernel library must raise")

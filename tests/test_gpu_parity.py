@@ -1,0 +1,400 @@
+"""Parity of the HIP path with the CPU oracle, through the C ABI (ctypes) on an MI355X.
+
+Tolerances (relative error = ||got - ref|| / ||ref|| unless stated):
+  embedding gather, argmax indices ........ bit-exact
+  fp32 paths .............................. 1e-4
+  bf16 GEMM outputs and gradients ......... 1e-2 against the fp32 oracle
+  cross-entropy loss ...................... 1e-5 (bf16 logits are upcast; the oracle runs the reference
+                                            algorithm in fp32 on the same bf16 values)
+"""
+import json
+import os
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from merak_amd import mpu, ops, set_args
+from merak_amd.inference import DecodeStep, greedy_from_logits, greedy_next_token
+from oracle import tp_reference as R
+
+pytestmark = pytest.mark.gpu
+G = os.path.join(os.path.dirname(__file__), "golden")
+
+TOL_F32, TOL_BF16, TOL_LOSS = 1e-4, 1e-2, 1e-5
+
+
+def rel(got, ref):
+    got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
+    return ((got - ref).norm() / ref.norm().clamp_min(1e-300)).item()
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(1234 + seed)
+
+
+# =============================================================================== cross entropy
+@pytest.mark.parametrize("case", json.load(open(os.path.join(G, "ce_small.json"))),
+                         ids=lambda c: f"start{c['vocab_start']}_t{c['target']}")
+@pytest.mark.parametrize("dtype", [torch.float32])
+def test_ce_golden_vectors(gpu, case, dtype):
+    x = torch.tensor(case["logits"], dtype=dtype, device=gpu)
+    t = torch.tensor(case["target"], device=gpu)
+    loss, m, s, pred = ops.vocab_ce_fwd(x, t, case["vocab_start"])
+    assert rel(loss, torch.tensor(case["loss"])) < TOL_LOSS
+    g = torch.tensor(case["grad_output"], dtype=torch.float32, device=gpu)
+    ops.vocab_ce_bwd_(x, t, m, s, g, case["vocab_start"])
+    assert rel(x, torch.tensor(case["grad"])) < TOL_F32
+
+
+@pytest.mark.parametrize("dtype,n,v", [
+    (torch.float32, 64, 50257),     # GPT-2 vocab: rows are not 16-byte aligned
+    (torch.bfloat16, 64, 128256),   # Llama-3 vocab
+    (torch.float32, 7, 1), (torch.float32, 3, 5), (torch.bfloat16, 5, 9), (torch.bfloat16, 4, 1031),
+    (torch.float32, 2, 2048 + 3), (torch.bfloat16, 1, 40000),
+])
+def test_ce_forward_backward_vs_oracle(gpu, dtype, n, v):
+    x = torch.randn(n, v, generator=gen(1)).to(dtype)
+    t = torch.randint(0, v, (n,), generator=gen(2))
+    t[torch.randperm(n, generator=gen(3))[: max(1, n // 20)]] = -100      # 5% "ignore" labels
+    g = torch.full((n,), 1.0 / n)
+    ref_loss, ref_grad = R.cross_entropy_fp32(x, t, 0, g)
+    xg = x.to(gpu)
+    loss, m, s, pred = ops.vocab_ce_fwd(xg, t.to(gpu), 0)
+    assert torch.equal(xg.cpu(), x), "forward must not modify the logits"
+    # 1e-5 relative; a vocabulary of one gives an exactly zero loss, so an absolute floor of 1e-6 is allowed
+    assert (loss.cpu() - ref_loss).abs().max() <= TOL_LOSS * max(ref_loss.abs().max().item(), 0.1)
+    assert rel(loss, ref_loss) < TOL_LOSS or v == 1
+    assert torch.equal(m.cpu(), x.float().max(-1).values)
+    out = ops.vocab_ce_bwd_(xg, t.to(gpu), m, s, g.to(gpu), 0)
+    assert out.data_ptr() == xg.data_ptr(), "gradient must reuse the logits storage"
+    assert rel(xg, ref_grad) < (TOL_F32 if dtype == torch.float32 else TOL_BF16)
+
+
+def test_ce_autograd_function_matches_reference_semantics(gpu):
+    n, v = 48, 50257
+    x = torch.randn(4, 12, v, generator=gen(4))
+    t = torch.randint(0, v, (4, 12), generator=gen(5))
+    t[0, 0] = -100
+    ref_loss, ref_grad = R.cross_entropy_fp32(x.view(n, v), t.view(n), 0, torch.full((n,), 1.0 / n))
+    xg = x.to(gpu).requires_grad_(True)
+    logits = xg * 1.0                                   # a non-leaf, as the LM head's output would be
+    loss = mpu.vocab_parallel_cross_entropy(logits, t.to(gpu))
+    assert loss.shape == t.shape and loss.dtype == torch.float32
+    torch.mean(loss.view(-1)).backward()                # merak_trainer.py:323-325
+    assert rel(loss.view(-1), ref_loss) < TOL_LOSS
+    assert rel(xg.grad.view(n, v), ref_grad) < TOL_F32
+    # opt-in: reproduce the reference's side effect (caller's logits end up holding the softmax)
+    y = x.to(gpu).clone()
+    l2 = mpu.vocab_parallel_cross_entropy(y, t.to(gpu), materialize_softmax=True)
+    assert rel(y.view(n, v), torch.softmax(x.view(n, v), -1)) < TOL_F32 and rel(l2.view(-1), ref_loss) < TOL_LOSS
+
+
+def test_ce_bf16_loss_dtype_flag_and_materialized_backward(gpu):
+    n, v = 16, 4096
+    x = torch.randn(n, v, generator=gen(6)).bfloat16()
+    t = torch.randint(0, v, (n,), generator=gen(7))
+    g = torch.rand(n, generator=gen(8))
+    ref_loss, ref_grad = R.cross_entropy_fp32(x, t, 0, g)
+    xg = x.to(gpu).requires_grad_(True)
+    lg = xg * 1
+    loss = mpu.vocab_parallel_cross_entropy(lg, t.to(gpu), loss_in_logits_dtype=True, materialize_softmax=True)
+    assert loss.dtype == torch.bfloat16                 # cross_entropy.py:77 returns the logits dtype
+    (loss.float() * g.to(gpu)).sum().backward()
+    assert rel(xg.grad, ref_grad) < 2 * TOL_BF16        # softmax was rounded to bf16 once more on the way
+
+
+def test_ce_one_rank_share_combines_to_full(gpu):
+    """8 vocab slices, each through the kernel with its [start, end); MAX/SUM/SUM on the host."""
+    n, v, p = 32, 8 * 1002, 8
+    x = torch.randn(n, v, generator=gen(9)).bfloat16()
+    t = torch.randint(0, v, (n,), generator=gen(10))
+    t[3] = -100
+    full_loss, full_grad = R.cross_entropy_fp32(x, t, 0, torch.ones(n))
+    mpu.set_model_parallel_world_size(p)
+    parts, slices = [], []
+    for r in range(p):
+        mpu.set_model_parallel_rank(r)
+        sl = x[:, r * 1002:(r + 1) * 1002].contiguous().to(gpu)
+        m, s, pr = mpu.vocab_parallel_cross_entropy_partials(sl, t.to(gpu))
+        om, os_, opr, inr = R.cross_entropy_partials(x[:, r * 1002:(r + 1) * 1002], t, r * 1002)
+        assert torch.equal(m.cpu(), om) and rel(s, os_) < TOL_LOSS and torch.equal(pr.cpu(), opr)
+        parts.append((m.cpu(), s.cpu(), pr.cpu(), inr))
+        slices.append(sl)
+    loss, gm, gs = R.combine_partials(*zip(*parts))
+    assert rel(loss, full_loss) < TOL_LOSS
+    for r in range(p):
+        mpu.set_model_parallel_rank(r)
+        mpu.vocab_parallel_cross_entropy_backward_(slices[r], t.to(gpu), gm.to(gpu), gs.to(gpu), torch.ones(n, device=gpu))
+        assert rel(slices[r], full_grad[:, r * 1002:(r + 1) * 1002]) < TOL_BF16
+
+
+def test_ce_empty_and_errors(gpu):
+    loss, *_ = ops.vocab_ce_fwd(torch.empty(0, 17, device=gpu), torch.empty(0, dtype=torch.int64, device=gpu), 0)
+    assert loss.numel() == 0
+    with pytest.raises(TypeError):
+        ops.vocab_ce_fwd(torch.randn(2, 4, device=gpu), torch.zeros(2, dtype=torch.int32, device=gpu), 0)
+    with pytest.raises(ValueError, match="contiguous"):
+        ops.vocab_ce_fwd(torch.randn(4, 8, device=gpu)[:, ::2], torch.zeros(4, dtype=torch.int64, device=gpu), 0)
+    with pytest.raises(TypeError):
+        ops.vocab_ce_fwd(torch.randn(2, 4, device=gpu).half(), torch.zeros(2, dtype=torch.int64, device=gpu), 0)
+
+
+def test_ce_full_size_llama_vocab(gpu):
+    """[8192, 128256] bf16 with 5% -100 labels: oracle on a sample of rows; whole-tensor properties."""
+    n, v = 8192, 128256
+    x = torch.empty(n, v, dtype=torch.bfloat16, device=gpu).normal_(generator=torch.Generator(device=gpu).manual_seed(1238))
+    t = torch.randint(0, v, (n,), generator=gen(11))
+    t[torch.randperm(n, generator=gen(12))[: n // 20]] = -100
+    tg = t.to(gpu)
+    loss, m, s, pred = ops.vocab_ce_fwd(x, tg, 0)
+    rows = torch.randperm(n, generator=gen(13))[:48]
+    rows[0] = (t == -100).nonzero()[0, 0]
+    xs = x[rows.to(gpu)].cpu()
+    g = torch.full((n,), 1.0 / n)
+    ref_loss, ref_grad = R.cross_entropy_fp32(xs, t[rows], 0, g[rows])
+    assert rel(loss.cpu()[rows], ref_loss) < TOL_LOSS
+    assert bool(torch.isfinite(loss).all()) and float(loss.min()) > 0
+    ops.vocab_ce_bwd_(x, tg, m, s, g.to(gpu), 0)
+    assert rel(x[rows.to(gpu)], ref_grad) < TOL_BF16
+    # each gradient row sums to g_i * (1 - [target in range])  (softmax sums to one, minus the one-hot)
+    rowsum = x.float().sum(-1).cpu() * n
+    expect = (t == -100).float()
+    assert (rowsum - expect).abs().max() < 0.05
+
+
+# =============================================================================== embedding
+@pytest.mark.parametrize("dtype,v,h", [(torch.bfloat16, 1000, 4096), (torch.float32, 777, 33), (torch.bfloat16, 50, 7),
+                                        (torch.float32, 64, 1)])
+def test_embedding_exact(gpu, dtype, v, h):
+    table = torch.randn(v, h, generator=gen(20)).to(dtype)
+    ids = torch.randint(0, v, (3, 11), generator=gen(21))
+    out = ops.embedding_gather(ids.to(gpu), table.to(gpu), 0, v)
+    assert out.shape == (3, 11, h) and torch.equal(out.cpu(), R.vocab_parallel_embedding_forward(ids, table, 0, v, 1))
+    lo, hi = v // 4, v // 2                                   # one rank's slice: outside ids give exact zeros
+    shard = table[lo:hi].contiguous()
+    out = ops.embedding_gather(ids.to(gpu), shard.to(gpu), lo, hi)
+    assert torch.equal(out.cpu(), R.vocab_parallel_embedding_forward(ids, shard, lo, hi, 4))
+
+
+def test_embedding_module_forward_backward(gpu):
+    set_args(use_cpu_initialization=True, params_dtype=torch.bfloat16)
+    torch.manual_seed(0)
+    emb = mpu.VocabParallelEmbedding(512, 64, init_method=torch.nn.init.normal_).to(gpu)
+    ids = torch.randint(0, 512, (4, 33), generator=gen(22))
+    ids[0, :5] = 7                                            # repeated ids accumulate
+    out = emb(ids.to(gpu))
+    assert torch.equal(out.cpu(), emb.weight.detach().cpu()[ids])
+    dout = torch.randn(4, 33, 64, generator=gen(23)).bfloat16()
+    out.backward(dout.to(gpu))
+    ref = R.embedding_backward(ids, dout, 512, 0, 512)
+    assert emb.weight.grad.dtype == torch.bfloat16 and rel(emb.weight.grad, ref) < TOL_BF16
+    dt = ops.embedding_bwd(ids.to(gpu), dout.to(gpu), 512, 0, 512)
+    assert rel(dt, ref) < TOL_F32
+    empty = ops.embedding_gather(torch.empty(0, dtype=torch.int64, device=gpu), emb.weight.detach(), 0, 512)
+    assert empty.shape == (0, 64)
+    oob = torch.zeros(1, dtype=torch.int32, device=gpu)
+    ops.embedding_gather(torch.tensor([1, 600, -3], device=gpu), emb.weight.detach(), 0, 512, oob)
+    assert oob.item() == 2
+
+
+def test_embedding_full_size_llama_table(gpu):
+    v, h, n = 128256, 4096, 8192
+    table = torch.empty(v, h, dtype=torch.bfloat16, device=gpu).normal_(0, 0.02, generator=torch.Generator(device=gpu).manual_seed(1239))
+    ids = torch.randint(0, v, (n,), generator=gen(24))
+    out = ops.embedding_gather(ids.to(gpu), table, 0, v)
+    pick = torch.randperm(n, generator=gen(25))[:256]
+    host_rows = table[ids[pick].to(gpu)].cpu()                # plain copies of the source rows to the host
+    assert torch.equal(out.cpu()[pick], R.vocab_parallel_embedding_forward(torch.arange(256), host_rows, 0, 256, 1))
+    # checksum of checksums: a pure gather preserves every row's bit pattern
+    src = table.view(torch.int16).to(torch.int64).sum(-1)[ids.to(gpu)]
+    assert torch.equal(out.view(torch.int16).to(torch.int64).sum(-1), src)
+
+
+# =============================================================================== linear layers
+def _lin_inputs(m, n, k, dtype, seed, bias=True):
+    x = torch.randn(m, k, generator=gen(seed)).to(dtype)
+    w = (torch.randn(n, k, generator=gen(seed + 1)) * 0.02).to(dtype)
+    b = (torch.randn(n, generator=gen(seed + 2)) * 0.02).to(dtype) if bias else None
+    dy = torch.randn(m, n, generator=gen(seed + 3)).to(dtype)
+    return x, w, b, dy
+
+
+@pytest.mark.parametrize("dtype,m,n,k", [
+    (torch.float32, 1024, 3072, 768),       # GPT-2-small column layer, fewer tokens
+    (torch.float32, 1024, 768, 3072),       # GPT-2-small row layer
+    (torch.bfloat16, 512, 6144, 4096),      # Llama-3-8B QKV
+    (torch.bfloat16, 256, 4096, 14336),     # Llama-3-8B down
+    (torch.bfloat16, 512, 1280, 8192),      # Llama-70B tp=8 QKV shard
+    (torch.bfloat16, 512, 8192, 1024),      # Llama-70B tp=8 o-proj shard
+    (torch.bfloat16, 300, 520, 136), (torch.bfloat16, 64, 50, 27), (torch.bfloat16, 1, 8, 8),
+    (torch.float32, 100, 77, 33), (torch.float32, 1, 1, 1), (torch.bfloat16, 257, 255, 72),
+])
+def test_linear_fwd_bwd_vs_oracle(gpu, dtype, m, n, k):
+    tol = TOL_F32 if dtype == torch.float32 else TOL_BF16
+    x, w, b, dy = _lin_inputs(m, n, k, dtype, 30)
+    xf, wf, bf, dyf = x.float(), w.float(), b.float(), dy.float()
+    ref, _ = R.column_parallel_linear_forward(xf, wf, bf)
+    y, _ = ops.linear_fwd(x.to(gpu), w.to(gpu), b.to(gpu), ops.EPI_BIAS)
+    assert rel(y, ref) < tol
+    y0, _ = ops.linear_fwd(x.to(gpu), w.to(gpu), None, ops.EPI_NONE)
+    assert rel(y0, R.row_parallel_linear_forward(xf, wf, None)[0]) < tol
+    rdx, rdw, rdb = R.linear_backward(xf, wf, dyf, True)
+    assert rel(ops.linear_dgrad(dy.to(gpu), w.to(gpu)), rdx) < tol
+    dw, db = ops.linear_wgrad(dy.to(gpu), x.to(gpu), True)
+    assert dw.dtype == dtype and rel(dw, rdw) < tol and rel(db, rdb) < tol
+    if dtype == torch.bfloat16:                       # fp32 main-gradient accumulation
+        acc = torch.ones(n, k, device=gpu)
+        accb = torch.ones(n, device=gpu)
+        ops.linear_wgrad(dy.to(gpu), x.to(gpu), True, dw=acc, db=accb, accumulate=True)
+        assert rel(acc - 1, rdw) < TOL_F32 * 10 and rel(accb - 1, rdb) < TOL_F32 * 10
+
+
+@pytest.mark.parametrize("dtype,m,n,k", [(torch.float32, 512, 3072, 768), (torch.bfloat16, 512, 3072, 768),
+                                          (torch.bfloat16, 200, 136, 72), (torch.float32, 33, 20, 10)])
+def test_bias_gelu_epilogue(gpu, dtype, m, n, k):
+    tol = TOL_F32 if dtype == torch.float32 else TOL_BF16
+    x, w, b, dy = _lin_inputs(m, n, k, dtype, 40)
+    pre = R.column_parallel_linear_forward(x.float(), w.float(), b.float())[0]
+    y, act = ops.linear_fwd(x.to(gpu), w.to(gpu), b.to(gpu), ops.EPI_BIAS_GELU)
+    assert rel(y, pre) < tol and rel(act, R.gelu_new(pre)) < tol
+    _, act_only = ops.linear_fwd(x.to(gpu), w.to(gpu), b.to(gpu), ops.EPI_BIAS_GELU, want_pre=False)
+    assert torch.equal(act_only, act)
+    d = ops.activation_bwd(dy.to(gpu), y, ops.EPI_BIAS_GELU)
+    assert rel(d, dy.float() * R.gelu_new_grad(y.float().cpu())) < tol
+
+
+@pytest.mark.parametrize("dtype,m,n,k", [(torch.bfloat16, 512, 2 * 14336, 4096), (torch.bfloat16, 512, 2 * 3584, 8192),
+                                          (torch.bfloat16, 130, 2 * 100, 72), (torch.float32, 65, 2 * 24, 40),
+                                          (torch.bfloat16, 40, 2 * 13, 16)])
+def test_swiglu_epilogue(gpu, dtype, m, n, k):
+    tol = TOL_F32 if dtype == torch.float32 else TOL_BF16
+    x, w, _, _ = _lin_inputs(m, n, k, dtype, 50, bias=False)
+    pre = F.linear(x.float(), w.float())
+    y, act = ops.linear_fwd(x.to(gpu), w.to(gpu), None, ops.EPI_SWIGLU)
+    assert act.shape == (m, n // 2) and rel(y, pre) < tol
+    assert rel(act, R.swiglu(y.float().cpu())) < tol     # activation of the stored (rounded) pre-activation
+    dact = torch.randn(m, n // 2, generator=gen(54)).to(dtype)
+    d = ops.activation_bwd(dact.to(gpu), y, ops.EPI_SWIGLU)
+    assert rel(d, R.swiglu_backward(dact.float(), y.float().cpu())) < tol
+
+
+def test_gpt2_small_fp32_full_size(gpu):
+    """Config 1 in full: Column 768->3072 bias+GeLU, Row 3072->768 bias, 8x1024 tokens, fp32, via the modules."""
+    set_args(use_cpu_initialization=True, params_dtype=torch.float32)
+    torch.manual_seed(1)
+    init = lambda t: torch.nn.init.normal_(t, 0.0, 0.02)
+    col = mpu.ColumnParallelLinear(768, 3072, gather_output=False, init_method=init, activation="gelu_new")
+    row = mpu.RowParallelLinear(3072, 768, input_is_parallel=True, init_method=init)
+    with torch.no_grad():
+        col.bias.normal_(0, 0.02); row.bias.normal_(0, 0.02)
+    x = torch.randn(8, 1024, 768, generator=gen(60))
+    dy = torch.randn(8, 1024, 768, generator=gen(61))
+    # oracle chain on the host (reference op order), autograd for the backward
+    xr = x.clone().requires_grad_(True)
+    wc, bc, wr, br = (p.detach().clone().requires_grad_(True) for p in (col.weight, col.bias, row.weight, row.bias))
+    h = R.gelu_new(R.column_parallel_linear_forward(xr, wc, bc)[0])
+    out_ref, none = R.row_parallel_linear_forward(h, wr, br)
+    out_ref.backward(dy)
+    col.to(gpu); row.to(gpu)
+    xg = x.to(gpu).requires_grad_(True)
+    hg, b1 = col(xg)
+    out, b2 = row(hg)
+    assert b1 is None and b2 is None and out.shape == (8, 1024, 768)
+    out.backward(dy.to(gpu))
+    assert rel(out, out_ref) < TOL_F32 and rel(xg.grad, xr.grad) < TOL_F32
+    for p, r in ((col.weight, wc), (col.bias, bc), (row.weight, wr), (row.bias, br)):
+        assert rel(p.grad, r.grad) < TOL_F32
+
+
+@pytest.mark.parametrize("name,m,k,n", [("llama8b_qkv", 4096, 4096, 6144), ("llama8b_down", 4096, 14336, 4096),
+                                         ("llama70b_tp8_qkv", 8192, 8192, 1280), ("llama70b_tp8_oproj", 8192, 1024, 8192)])
+def test_linear_full_size_sampled(gpu, name, m, k, n):
+    """Full BASELINE shapes: oracle on sampled rows of Y, dX and dW; linearity in X over the whole output."""
+    g = torch.Generator(device=gpu).manual_seed(1240)
+    x = torch.empty(m, k, device=gpu).normal_(generator=g).bfloat16()
+    w = torch.empty(n, k, device=gpu).normal_(0, 0.02, generator=g).bfloat16()
+    dy = torch.empty(m, n, device=gpu).normal_(generator=g).bfloat16()
+    y, _ = ops.linear_fwd(x, w, None, ops.EPI_NONE)
+    dx = ops.linear_dgrad(dy, w)
+    dw, _ = ops.linear_wgrad(dy, x, False)
+    rm = torch.randperm(m, generator=gen(70))[:32].to(gpu)
+    rn = torch.randperm(n, generator=gen(71))[:32].to(gpu)
+    xs, ws, dys = x[rm].cpu().float(), w.cpu().float(), dy[rm].cpu().float()
+    assert rel(y[rm], R.row_parallel_linear_forward(xs, ws, None)[0]) < TOL_BF16
+    assert rel(dx[rm], R.linear_backward(xs, ws, dys, False)[0]) < TOL_BF16
+    ref_dw = R.linear_backward(x.cpu().float(), ws[rn.cpu()], dy[:, rn].cpu().float(), False)[1]
+    assert rel(dw[rn], ref_dw) < TOL_BF16
+    y2, _ = ops.linear_fwd((x.float() * 2).bfloat16(), w, None, ops.EPI_NONE)     # exact in bf16: scaling by 2
+    assert torch.equal(y2.float(), y.float() * 2)
+
+
+def test_module_surface_on_gpu(gpu):
+    set_args(use_cpu_initialization=True, params_dtype=torch.bfloat16)
+    torch.manual_seed(2)
+    col = mpu.ColumnParallelLinear(256, 512, skip_bias_add=True, gather_output=False).to(gpu)
+    x = torch.randn(2, 5, 256, generator=gen(80)).bfloat16()
+    out, ob = col(x.to(gpu).transpose(0, 1))                    # non-contiguous (seq, batch, hidden) view
+    assert ob is col.bias and out.shape == (5, 2, 512)
+    ref = R.column_parallel_linear_forward(x.float().transpose(0, 1), col.weight.detach().cpu().float(),
+                                           col.bias.detach().cpu().float(), True)[0]
+    assert rel(out, ref) < TOL_BF16
+    row = mpu.RowParallelLinear(512, 256, bias=True, input_is_parallel=True, skip_bias_add=True).to(gpu)
+    o2, b2 = row(out)
+    assert b2 is row.bias and o2.shape == (5, 2, 256)
+    set_args(use_cpu_initialization=False, params_dtype=torch.float32)
+    dev_layer = mpu.ColumnParallelLinear(64, 64, init_method=lambda t: torch.nn.init.normal_(t, 0, 0.02))
+    assert dev_layer.weight.is_cuda and dev_layer.bias.is_cuda
+    empty, _ = dev_layer(torch.empty(0, 64, device=gpu))
+    assert empty.shape == (0, 64)
+
+
+# =============================================================================== decode
+@pytest.mark.parametrize("b,n,k", [(1, 64, 256), (8, 1000, 512), (32, 4096, 1024), (5, 130, 4104), (17, 77, 40),
+                                    (32, 6144, 4096), (8, 4096, 14336)])
+def test_gemv_and_fused_argmax(gpu, b, n, k):
+    x = torch.randn(b, k, generator=gen(90)).bfloat16()
+    w = (torch.randn(n, k, generator=gen(91)) * 0.02).bfloat16()
+    ref = F.linear(x.float(), w.float())
+    y = ops.gemv(x.to(gpu), w.to(gpu))
+    assert rel(y, ref) < TOL_BF16
+    idx, val = ops.gemv_argmax(x.to(gpu), w.to(gpu))
+    assert idx.dtype == torch.int64 and torch.equal(idx.cpu(), R.greedy_argmax(ref))
+    assert rel(val, ref.max(-1).values) < TOL_F32
+    assert torch.equal(greedy_from_logits(ref.to(gpu)).cpu(), R.greedy_argmax(ref))
+
+
+def test_argmax_ties_and_nan(gpu):
+    k, n = 256, 999
+    x = torch.randn(4, k, generator=gen(92)).bfloat16()
+    w = (torch.randn(n, k, generator=gen(93)) * 0.02).bfloat16()
+    ref = F.linear(x.float(), w.float())
+    best = ref.argmax(-1)
+    for b in range(4):                      # duplicate each winner's weight row at a lower and a higher index
+        w[5 + b] = w[best[b]]
+        w[900 + b] = w[best[b]]
+    ref = F.linear(x.float(), w.float())
+    idx, _ = ops.gemv_argmax(x.to(gpu), w.to(gpu))
+    assert torch.equal(idx.cpu(), R.greedy_argmax(ref))     # exact ties: the first index wins
+    assert all(int(i) <= 5 + 3 or int(i) == int(best[b]) for b, i in enumerate(idx.cpu()))
+    logits = ref.clone()
+    logits[1, 700] = float("nan"); logits[1, 800] = float("nan"); logits[2, 3] = float("inf")
+    assert torch.equal(greedy_from_logits(logits.to(gpu)).cpu(), R.greedy_argmax(logits))
+    assert torch.equal(greedy_from_logits(logits.bfloat16().to(gpu)).cpu(), R.greedy_argmax(logits.bfloat16()))
+
+
+@pytest.mark.parametrize("b", [1, 8, 32])
+def test_decode_step_llama8b_full_size(gpu, b):
+    """Config 5: QKV 4096->6144, gate/up 4096->2x14336 (+SwiGLU), down 14336->4096, LM head 4096->128256."""
+    g = torch.Generator(device=gpu).manual_seed(1241)
+    mk = lambda n, k: torch.empty(n, k, device=gpu).normal_(0, 0.02, generator=g).bfloat16()
+    wq, wg, wd, wl = mk(6144, 4096), mk(2 * 14336, 4096), mk(4096, 14336), mk(128256, 4096)
+    x = torch.randn(b, 4096, generator=gen(94)).bfloat16()
+    step = DecodeStep(wq, wg, wd, wl)
+    qkv, out, tok = step(x.to(gpu))
+    rq, ro, rlogits, rtok = R.decode_step(x, wq.cpu(), wg.cpu(), wd.cpu(), wl.cpu())
+    assert rel(qkv, rq.float()) < TOL_BF16 and rel(out, ro.float()) < TOL_BF16
+    # the greedy pick is compared on identical inputs to the LM head: feed the kernel's own `out`
+    ref_tok = R.greedy_argmax(F.linear(out.cpu().float(), wl.cpu().float()))
+    assert torch.equal(tok.cpu(), ref_tok)
+    assert torch.equal(greedy_next_token(out, wl).cpu(), ref_tok)

@@ -1,0 +1,159 @@
+"""Host-side behaviour of the drop-in layers: constructor contract, attributes, parameter tags,
+state-dict names, weight sharding, the plug-in boundary (build_layers), and the refusal to run
+anywhere but on the GPU kernels.  No GPU needed."""
+import json
+import os
+
+import pytest
+import torch
+import torch.nn as nn
+from hypothesis import given, settings, strategies as st
+
+from merak_amd import mpu, set_args, get_args
+from merak_amd.tensor_parallel import (ColPara, RowPara, build_layers, init_method_normal,
+                                       scaled_init_method_normal)
+from oracle import tp_reference as R
+
+G = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def test_column_parallel_contract():
+    l = mpu.ColumnParallelLinear(12, 20)
+    assert l.weight.shape == (20, 12) and l.bias.shape == (20,)
+    assert l.gather_output is True and l.skip_bias_add is False  # class defaults, layers.py:193-196
+    assert l.input_size == 12 and l.output_size == 20 and l.output_size_per_partition == 20
+    assert l.weight.model_parallel and l.weight.partition_dim == 0 and l.weight.partition_stride == 1
+    assert l.bias.model_parallel and l.bias.partition_dim == 0 and l.bias.stride == 1
+    assert torch.count_nonzero(l.bias) == 0
+    assert l.master_weight is None
+    assert repr(l) == "ColumnParallelLinear(in_features=12, out_features=20, bias=True)"
+    nb = mpu.ColumnParallelLinear(12, 20, bias=False)
+    assert nb.bias is None and [n for n, _ in nb.named_parameters()] == ["weight"]
+    pos = mpu.ColumnParallelLinear(12, 20, True, False, nn.init.xavier_normal_)  # model_parallel.py:143-156
+    assert pos.gather_output is False
+
+
+def test_row_parallel_contract():
+    l = mpu.RowParallelLinear(12, 20, input_is_parallel=True)
+    assert l.weight.shape == (20, 12) and l.bias.shape == (20,)
+    assert l.weight.partition_dim == 1 and not hasattr(l.bias, "model_parallel")  # row bias is not sharded
+    assert l.input_size_per_partition == 12
+    assert repr(l) == "RowParallelLinear(in_features=12, out_features=20, bias=True)"
+
+
+def test_shard_shapes_at_tp8_match_llama70b_rank():
+    mpu.set_model_parallel_world_size(8)
+    mpu.set_model_parallel_rank(3)
+    set_args(use_cpu_initialization=True, params_dtype=torch.bfloat16)
+    col = mpu.ColumnParallelLinear(64, 8 * 1280, bias=False, gather_output=False)
+    row = mpu.RowParallelLinear(8 * 3584, 64, bias=False, input_is_parallel=True)
+    emb = mpu.VocabParallelEmbedding(128256, 8)
+    assert col.weight.shape == (1280, 64) and col.weight.dtype == torch.bfloat16
+    assert row.weight.shape == (64, 3584)
+    assert (emb.vocab_start_index, emb.vocab_end_index) == (3 * 16032, 4 * 16032)
+    assert emb.weight.shape == (16032, 8)
+    with pytest.raises(AssertionError, match="50257 is not divisible by 8"):
+        mpu.VocabParallelEmbedding(50257, 8)
+
+
+def test_cpu_init_shards_like_the_reference():
+    s = json.load(open(os.path.join(G, "shard_table.json")))
+
+    def arange_init(t):
+        with torch.no_grad():
+            t.copy_(torch.tensor([[10.0 * r + c for c in range(t.shape[1])] for r in range(t.shape[0])]))
+        return t
+
+    mpu.set_model_parallel_world_size(s["world"])
+    for rank in range(s["world"]):
+        mpu.set_model_parallel_rank(rank)
+        for stride, key in ((1, "column_stride1"), (2, "column_stride2")):
+            l = mpu.ColumnParallelLinear(s["in"], s["out"], bias=False, init_method=arange_init, stride=stride,
+                                         keep_master_weight_for_test=True)
+            assert l.master_weight.shape == (s["out"], s["in"])
+            assert torch.equal(l.weight.data, l.master_weight[s[key][str(rank)]])
+            assert l.weight.partition_stride == stride
+    mpu.set_model_parallel_world_size(s["row_world"])
+    for rank in range(s["row_world"]):
+        mpu.set_model_parallel_rank(rank)
+        l = mpu.RowParallelLinear(s["row_in"], 4, bias=False, init_method=arange_init,
+                                  keep_master_weight_for_test=True)
+        assert torch.equal(l.weight.data, l.master_weight[:, s["row_stride1"][str(rank)]])
+
+
+def test_params_dtype_and_init_methods():
+    set_args(use_cpu_initialization=True, params_dtype=torch.bfloat16)
+    torch.manual_seed(0)
+    l = mpu.ColumnParallelLinear(256, 512, init_method=init_method_normal(0.02))
+    assert l.weight.dtype == torch.bfloat16 and l.bias.dtype == torch.bfloat16
+    assert abs(l.weight.float().std().item() - 0.02) < 2e-3
+    r = mpu.RowParallelLinear(256, 512, init_method=scaled_init_method_normal(0.02, 8))
+    assert abs(r.weight.float().std().item() - 0.02 / 4.0) < 1e-3
+    assert abs(scaled_init_method_normal(0.02, {"a": 4, "b": 4})(torch.empty(512, 512)).std().item() - 0.005) < 1e-3
+
+
+def test_state_dict_names_and_boundary():
+    lin = nn.Linear(16, 8)          # as set_mp_attr leaves it at mp=2: out_features already divided
+    lin.mp_attr = "col"
+    mpu.set_model_parallel_world_size(2)
+    mpu.set_model_parallel_rank(1)
+    col = build_layers("q_proj", lin, 2, init_method_normal(0.02), scaled_init_method_normal(0.02, 2))
+    assert isinstance(col, ColPara) and col.col_linear.output_size == 16 and col.weight.shape == (8, 16)
+    assert sorted(col.state_dict()) == ["col_linear.bias", "col_linear.weight"]
+    assert col.col_linear.gather_output is False and col.need_permute is False
+    lin2 = nn.Linear(8, 16, bias=False)
+    lin2.mp_attr = "row_mlp"
+    row = build_layers("down_proj", lin2, 2, init_method_normal(0.02), scaled_init_method_normal(0.02, 2))
+    assert isinstance(row, RowPara) and row.row_linear.input_size == 16 and row.weight.shape == (16, 8)
+    assert sorted(row.state_dict()) == ["row_linear.weight"] and row.bias is None
+    assert row.row_linear.input_is_parallel is True
+    plain = nn.Linear(4, 4)
+    assert build_layers("x", plain, 2, None, None) is plain        # untagged: returned unchanged
+    assert build_layers("ln", nn.LayerNorm(4), 2, None, None) is None
+    set_args(use_cpu_initialization=True, tp_overlapping_level=2)
+    with pytest.raises(NotImplementedError):
+        ColPara(4, 4, init_method_normal(0.02))
+
+
+def test_forward_refuses_cpu_tensors_and_other_dtypes():
+    l = mpu.ColumnParallelLinear(8, 8)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        l(torch.randn(2, 8))
+    e = mpu.VocabParallelEmbedding(16, 4)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        e(torch.tensor([1, 2]))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        mpu.vocab_parallel_cross_entropy(torch.randn(2, 8), torch.tensor([1, 2]))
+
+
+def test_mappings_and_groups_at_size_one_and_above():
+    x = torch.randn(2, 6)
+    for f in (mpu.copy_to_model_parallel_region, mpu.reduce_from_model_parallel_region,
+              mpu.scatter_to_model_parallel_region, mpu.gather_from_model_parallel_region):
+        assert f(x) is x                       # every collective is bypassed at world size 1 (mappings.py:36,53,89)
+    assert mpu.get_model_parallel_world_size() == 1 and mpu.get_model_parallel_rank() == 0
+    mpu.set_model_parallel_world_size(3)
+    mpu.set_model_parallel_rank(2)
+    assert torch.equal(mpu.scatter_to_model_parallel_region(x), x[:, 4:6])
+    with pytest.raises(RuntimeError, match="other tensor-parallel ranks"):
+        mpu.gather_from_model_parallel_region(x)
+    with pytest.raises(RuntimeError, match="MAX/SUM/SUM"):
+        mpu.vocab_parallel_cross_entropy(torch.randn(2, 8), torch.tensor([1, 2]))
+
+
+def test_split_tensor_along_last_dim():
+    x = torch.arange(24.).view(2, 12)
+    parts = mpu.split_tensor_along_last_dim(x, 3)
+    assert [p.shape for p in parts] == [(2, 4)] * 3 and not parts[1].is_contiguous()
+    assert all(p.is_contiguous() for p in mpu.split_tensor_along_last_dim(x, 3, True))
+    with pytest.raises(AssertionError, match="12 is not divisible by 5"):
+        mpu.split_tensor_along_last_dim(x, 5)
+
+
+@settings(max_examples=200, deadline=None)
+@given(per=st.integers(1, 10 ** 6), world=st.integers(1, 64), data=st.data())
+def test_vocab_utility_matches_oracle(per, world, data):
+    rank = data.draw(st.integers(0, world - 1))
+    got = mpu.VocabUtility.vocab_range_from_global_vocab_size(per * world, rank, world)
+    assert got == R.vocab_range_from_global_vocab_size(per * world, rank, world) == (rank * per, rank * per + per)
+    assert mpu.divide(per * world, world) == per

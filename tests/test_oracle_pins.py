@@ -1,0 +1,221 @@
+"""Pins the CPU oracle (oracle/tp_reference.py) against things it was not written from:
+hand-computed golden vectors, library routines, closed forms, autograd in fp64, brute force.
+A dropped term, a wrong sign, a transposed operand or an off-by-one index fails at least one test."""
+import json
+import math
+import os
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import tp_reference as R
+
+G = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _load(name):
+    with open(os.path.join(G, name)) as f:
+        return json.load(f)
+
+
+# ------------------------------------------------------------------ cross entropy
+@pytest.mark.parametrize("case", _load("ce_small.json"), ids=lambda c: f"start{c['vocab_start']}_t{c['target']}")
+def test_ce_golden(case):
+    x = torch.tensor(case["logits"], dtype=torch.float64)
+    t = torch.tensor(case["target"], dtype=torch.int64)
+    v = x.shape[1]
+    loss, sm, mask, mt = R.vocab_parallel_cross_entropy_forward(x.clone(), t, case["vocab_start"],
+                                                                case["vocab_start"] + v)
+    assert torch.allclose(loss, torch.tensor(case["loss"], dtype=torch.float64), rtol=1e-12, atol=1e-12)
+    g = R.vocab_parallel_cross_entropy_backward(sm, mask, mt, torch.tensor(case["grad_output"], dtype=torch.float64))
+    assert torch.allclose(g, torch.tensor(case["grad"], dtype=torch.float64), rtol=1e-10, atol=1e-12)
+
+
+def test_ce_matches_library_in_range():
+    torch.manual_seed(1)
+    x = torch.randn(64, 1000, dtype=torch.float64) * 3
+    t = torch.randint(0, 1000, (64,))
+    loss, *_ = R.vocab_parallel_cross_entropy_forward(x.clone(), t, 0, 1000)
+    assert torch.allclose(loss, F.cross_entropy(x, t, reduction="none"), rtol=1e-12, atol=1e-12)
+
+
+def test_ce_out_of_range_is_lse_minus_max():
+    torch.manual_seed(2)
+    x = torch.randn(16, 333, dtype=torch.float64)
+    t = torch.tensor([-100, 333, 400, -1] * 4)
+    loss, sm, *_ = R.vocab_parallel_cross_entropy_forward(x.clone(), t, 0, 333)
+    assert torch.allclose(loss, torch.logsumexp(x, -1) - x.max(-1).values, rtol=1e-12)
+    assert torch.allclose(sm, torch.softmax(x, -1), rtol=1e-12)  # and the input now holds the softmax
+
+
+def test_ce_is_in_place_and_shaped_like_target():
+    x = torch.randn(3, 5, 11)
+    t = torch.randint(0, 11, (3, 5))
+    buf = x.clone()
+    loss, sm, *_ = R.vocab_parallel_cross_entropy_forward(buf, t, 0, 11)
+    assert loss.shape == t.shape and sm.data_ptr() == buf.data_ptr()
+    assert torch.allclose(buf, torch.softmax(x, -1), atol=1e-6)
+
+
+def test_ce_backward_is_autograd_of_closed_form():
+    torch.manual_seed(3)
+    x = torch.randn(12, 50, dtype=torch.float64, requires_grad=True)
+    t = torch.randint(0, 50, (12,))
+    t[::4] = -100
+    g = torch.rand(12, dtype=torch.float64)
+    inr = (t >= 0) & (t < 50)
+    closed = torch.where(inr, torch.logsumexp(x, -1) - x.gather(1, t.clamp(0, 49)[:, None])[:, 0],
+                         torch.logsumexp(x, -1) - x.max(-1).values.detach())
+    (ref,) = torch.autograd.grad((closed * g).sum(), x)
+    loss, grad = R.cross_entropy_fp32(x.detach(), t, 0, g)
+    assert torch.allclose(loss.double(), closed.detach(), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(grad.double(), ref, rtol=1e-4, atol=1e-7)
+
+
+def test_ce_partials_over_8_slices_combine_to_full():
+    torch.manual_seed(4)
+    n, v, p = 10, 64, 8
+    x = torch.randn(n, v) * 2
+    t = torch.randint(0, v, (n,))
+    t[0] = -100
+    full, _ = R.cross_entropy_fp32(x, t, 0)
+    parts = [R.cross_entropy_partials(x[:, r * 8:(r + 1) * 8], t, r * 8) for r in range(p)]
+    loss, gm, gs = R.combine_partials(*zip(*parts))
+    assert torch.allclose(loss, full, rtol=1e-6, atol=1e-6)
+    assert torch.equal(gm, x.max(-1).values)
+
+
+# ------------------------------------------------------------------ activations
+def test_activation_golden():
+    a = _load("activations.json")
+    x = torch.tensor(a["x"], dtype=torch.float64)
+    assert torch.allclose(R.gelu_new(x), torch.tensor(a["gelu_new"], dtype=torch.float64), rtol=1e-12, atol=1e-15)
+    y = torch.cat([x, torch.ones_like(x)])
+    assert torch.allclose(R.swiglu(y), torch.tensor(a["silu"], dtype=torch.float64), rtol=1e-12, atol=1e-15)
+
+
+def test_activation_derivatives_are_autograd():
+    x = torch.linspace(-5, 5, 101, dtype=torch.float64, requires_grad=True)
+    (g,) = torch.autograd.grad(R.gelu_new(x).sum(), x)
+    assert torch.allclose(R.gelu_new_grad(x.detach()), g, rtol=1e-10, atol=1e-12)
+    y = torch.randn(7, 10, dtype=torch.float64, requires_grad=True)
+    d = torch.randn(7, 5, dtype=torch.float64)
+    (gy,) = torch.autograd.grad((R.swiglu(y) * d).sum(), y)
+    assert torch.allclose(R.swiglu_backward(d, y.detach()), gy, rtol=1e-10, atol=1e-12)
+    # the library's tanh-approximate GELU is the same function
+    assert torch.allclose(R.gelu_new(x.detach()), F.gelu(x.detach(), approximate="tanh"), rtol=1e-10, atol=1e-12)
+
+
+# ------------------------------------------------------------------ linear
+def test_linear_forward_brute_force_and_tuple_contract():
+    torch.manual_seed(5)
+    x = torch.randn(2, 3, 4, dtype=torch.float64)
+    w = torch.randn(5, 4, dtype=torch.float64)
+    b = torch.randn(5, dtype=torch.float64)
+    brute = torch.zeros(2, 3, 5, dtype=torch.float64)
+    for i in range(2):
+        for j in range(3):
+            for n in range(5):
+                brute[i, j, n] = sum(x[i, j, k] * w[n, k] for k in range(4)) + b[n]
+    out, ob = R.column_parallel_linear_forward(x, w, b)
+    assert ob is None and torch.allclose(out, brute, rtol=1e-12)
+    out, ob = R.column_parallel_linear_forward(x, w, b, skip_bias_add=True)
+    assert ob is b and torch.allclose(out, brute - b, rtol=1e-12)
+    out, ob = R.row_parallel_linear_forward(x, w, b)
+    assert ob is None and torch.allclose(out, brute, rtol=1e-12)
+    out, ob = R.row_parallel_linear_forward(x, w, b, skip_bias_add=True)
+    assert ob is b and torch.allclose(out, brute - b, rtol=1e-12)
+    out, ob = R.row_parallel_linear_forward(x, w, None)
+    assert ob is None and torch.allclose(out, brute - b, rtol=1e-12)
+
+
+def test_linear_backward_is_autograd():
+    torch.manual_seed(6)
+    x = torch.randn(4, 3, 6, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(5, 6, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(5, dtype=torch.float64, requires_grad=True)
+    dy = torch.randn(4, 3, 5, dtype=torch.float64)
+    gx, gw, gb = torch.autograd.grad((F.linear(x, w, b) * dy).sum(), (x, w, b))
+    dx, dw, db = R.linear_backward(x.detach(), w.detach(), dy, True)
+    assert torch.allclose(dx, gx) and torch.allclose(dw, gw) and torch.allclose(db, gb)
+    assert dw.shape == w.shape and dx.shape == x.shape  # a transposed operand would change these
+
+
+# ------------------------------------------------------------------ embedding
+def test_embedding_forward_exact_and_shard_zero_rows():
+    torch.manual_seed(7)
+    table = torch.randn(32, 6)
+    ids = torch.randint(0, 32, (3, 7))
+    assert torch.equal(R.vocab_parallel_embedding_forward(ids, table, 0, 32, 1), table[ids])
+    full = torch.zeros(3, 7, 6)
+    for r in range(4):  # 4 ranks of 8 rows: sum of the masked partial outputs is the full lookup
+        part = R.vocab_parallel_embedding_forward(ids, table[8 * r:8 * r + 8], 8 * r, 8 * r + 8, 4)
+        outside = (ids < 8 * r) | (ids >= 8 * r + 8)
+        assert torch.equal(part[outside], torch.zeros_like(part[outside]))
+        full += part
+    assert torch.equal(full, table[ids])
+
+
+def test_embedding_backward_is_autograd_and_brute_force():
+    torch.manual_seed(8)
+    table = torch.randn(16, 4, requires_grad=True)
+    ids = torch.tensor([[1, 1, 5], [15, 0, 1]])
+    dout = torch.randn(2, 3, 4)
+    (g,) = torch.autograd.grad((F.embedding(ids, table) * dout).sum(), table)
+    assert torch.allclose(R.embedding_backward(ids, dout, 16, 0, 16), g, atol=1e-6)
+    shard = R.embedding_backward(ids, dout, 8, 0, 8)  # rank 0 of 2: id 15 is not ours
+    brute = torch.zeros(8, 4)
+    for i in range(2):
+        for j in range(3):
+            if ids[i, j] < 8:
+                brute[ids[i, j]] += dout[i, j]
+    assert torch.allclose(shard, brute, atol=1e-6)
+
+
+# ------------------------------------------------------------------ sharding, integers, argmax
+def test_shard_master_weight_golden_table():
+    s = _load("shard_table.json")
+    master = torch.tensor([[10.0 * r + c for c in range(s["in"])] for r in range(s["out"])])
+    for rank in range(s["world"]):
+        for stride, key in ((1, "column_stride1"), (2, "column_stride2")):
+            got = R.shard_master_weight(master, s["out"] // s["world"], 0, stride, rank, s["world"])
+            assert torch.equal(got, master[s[key][str(rank)]])
+    master = torch.tensor([[10.0 * r + c for c in range(s["row_in"])] for r in range(4)])
+    for rank in range(s["row_world"]):
+        got = R.shard_master_weight(master, s["row_in"] // s["row_world"], 1, 1, rank, s["row_world"])
+        assert torch.equal(got, master[:, s["row_stride1"][str(rank)]])
+
+
+def test_vocab_ranges_and_divide():
+    assert R.vocab_range_from_global_vocab_size(128256, 3, 8) == (3 * 16032, 4 * 16032)
+    assert R.vocab_range_from_per_partition_vocab_size(10, 2, 99) == (20, 30)
+    with pytest.raises(AssertionError, match="50257 is not divisible by 8"):
+        R.vocab_range_from_global_vocab_size(50257, 0, 8)
+    covered = []
+    for r in range(4):
+        a, b = R.vocab_range_from_global_vocab_size(1000, r, 4)
+        covered += list(range(a, b))
+    assert covered == list(range(1000))
+
+
+def test_greedy_argmax_first_index_on_ties():
+    x = torch.tensor([[1.0, 5.0, 5.0, 2.0], [7.0, 7.0, 7.0, 7.0], [-1.0, -3.0, -0.5, -0.5]])
+    assert R.greedy_argmax(x).tolist() == [1, 0, 2]
+    torch.manual_seed(9)
+    y = torch.randn(5, 1000)
+    brute = [max(range(1000), key=lambda j: (y[i, j].item(), -j)) for i in range(5)]
+    assert R.greedy_argmax(y).tolist() == brute
+    assert R.greedy_argmax(y).dtype == torch.int64
+
+
+def test_decode_step_reduces_to_plain_linears():
+    torch.manual_seed(10)
+    x = torch.randn(3, 16).bfloat16()
+    wq, wg, wd, wl = (torch.randn(*s).bfloat16() * 0.1 for s in ((24, 16), (64, 16), (16, 32), (100, 16)))
+    qkv, out, logits, tok = R.decode_step(x, wq, wg, wd, wl)
+    assert torch.equal(qkv, F.linear(x.float(), wq.float()).bfloat16())
+    y = F.linear(x.float(), wg.float()).bfloat16().float()
+    h = (F.silu(y[:, :32]) * y[:, 32:]).bfloat16()
+    assert torch.equal(out, F.linear(h.float(), wd.float()).bfloat16())
+    assert torch.equal(tok, F.linear(out.float(), wl.float()).argmax(-1))

@@ -1,0 +1,345 @@
+#!/usr/bin/env python3
+"""Benchmark of the tensor-parallel hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+
+Headline (``value``): TFLOP/s of one rank's Llama-3-8B-shaped linears, forward +
+backward, bf16 with fp32 accumulate, on 4096 tokens:
+    QKV 4096->6144, gate/up 4096->2x14336 with fused SwiGLU, down 14336->4096.
+A step is: 3 forwards (Y = X W^T, SwiGLU fused into the gate/up epilogue), the
+SwiGLU backward, 3 input gradients (dX = dY W) and 3 weight gradients
+(dW = dY^T X).  FLOPs counted: 6*M*K*N per layer (4947.8 GFLOP per step); the
+activation work is executed inside the timed region but not counted.
+
+Inputs are resident in HBM before the timed region.  Timing: W warm-up steps,
+then K steps between two ``torch.cuda.synchronize()`` calls.  The per-kernel
+figures under ``roofline`` / ``kernels`` come from HIP events recorded on the
+launch stream around each launch, inside this same process.
+
+``secondary`` carries the other pieces of the path (cross entropy, embedding
+gather, decode GEMV + argmax, the Llama-70B tp=8 shard shapes and the fp32
+GPT-2 shapes) — one number each, same event timing.  ``cpu_baseline`` is the
+CPU oracle (the reference's op sequence in torch fp32) on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_F32_TFLOPS = 157.3     # MI355X fp32 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+LLAMA8B = [  # (name, K, N, epilogue)
+    ("qkv", 4096, 6144, "none"),
+    ("gate_up", 4096, 2 * 14336, "swiglu"),
+    ("down", 14336, 4096, "none"),
+]
+LLAMA70B_TP8 = [
+    ("qkv", 8192, 1280, "none"),
+    ("gate_up", 8192, 2 * 3584, "swiglu"),
+    ("down", 3584, 8192, "none"),
+    ("o_proj", 1024, 8192, "none"),
+]
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(1234 + seed)
+
+
+class Timer:
+    """HIP events on the current stream (the stream every kernel here is launched on)."""
+
+    def __init__(self):
+        self.t = {}
+
+    def run(self, name, fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        evs = []
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        ms = [a.elapsed_time(b) for a, b in evs]
+        self.t[name] = statistics.mean(ms)
+        return self.t[name]
+
+
+def build_linear_workload(dev, layers, M, seed):
+    from merak_amd import ops
+    out = []
+    for i, (name, K, N, epi) in enumerate(layers):
+        x = torch.randn(M, K, generator=gen(seed + 10 * i)).bfloat16().to(dev)
+        w = (torch.randn(N, K, generator=gen(seed + 10 * i + 1)) * 0.02).bfloat16().to(dev)
+        n_out = N // 2 if epi == "swiglu" else N
+        dy = torch.randn(M, n_out, generator=gen(seed + 10 * i + 2)).bfloat16().to(dev)
+        out.append(dict(name=name, K=K, N=N, M=M, epi=ops.EPI_SWIGLU if epi == "swiglu" else ops.EPI_NONE,
+                        x=x, w=w, dy=dy, flops=6.0 * M * K * N))
+    return out
+
+
+def linear_step(work):
+    """fwd + bwd of every layer; returns nothing (outputs are dropped, as a trainer's would be consumed)."""
+    from merak_amd import ops
+    for L in work:
+        y, act = ops.linear_fwd(L["x"], L["w"], None, L["epi"], want_pre=True)
+        g = L["dy"]
+        if L["epi"] == ops.EPI_SWIGLU:
+            g = ops.activation_bwd(g, y, ops.EPI_SWIGLU)
+        ops.linear_dgrad(g, L["w"])
+        ops.linear_wgrad(g, L["x"], False)
+
+
+def per_kernel(work, timer, reps):
+    """Average launch duration of each GEMM launch of the step, by HIP events."""
+    from merak_amd import ops
+    rows = []
+    for L in work:
+        M, K, N = L["M"], L["K"], L["N"]
+        y, act = ops.linear_fwd(L["x"], L["w"], None, L["epi"], want_pre=True)
+        g = L["dy"] if L["epi"] != ops.EPI_SWIGLU else ops.activation_bwd(L["dy"], y, ops.EPI_SWIGLU)
+        for kind, fn in (("fwd", lambda: ops.linear_fwd(L["x"], L["w"], None, L["epi"], want_pre=True)),
+                         ("dgrad", lambda: ops.linear_dgrad(g, L["w"])),
+                         ("wgrad", lambda: ops.linear_wgrad(g, L["x"], False))):
+            ms = timer.run(f"{L['name']}.{kind}", fn, reps)
+            rows.append(dict(kernel=f"{L['name']}.{kind}", M=M, N=N, K=K, ms=round(ms, 4),
+                             tflops=round(2.0 * M * N * K / ms / 1e9, 1)))
+        if L["epi"] == ops.EPI_SWIGLU:
+            ms = timer.run(f"{L['name']}.swiglu_bwd", lambda: ops.activation_bwd(L["dy"], y, ops.EPI_SWIGLU), reps)
+            rows.append(dict(kernel=f"{L['name']}.swiglu_bwd", ms=round(ms, 4),
+                             gbs=round((M * N // 2 * 2 + 2 * M * N * 2) / ms / 1e6, 1)))
+    return rows
+
+
+def cpu_baseline(sample_tokens):
+    """The oracle (reference op order, torch fp32) on `sample_tokens` tokens of the Llama-3-8B workload."""
+    from oracle import tp_reference as R
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    M = sample_tokens
+    flops = 0.0
+    layers = []
+    for i, (name, K, N, epi) in enumerate(LLAMA8B):
+        x = torch.randn(M, K, generator=gen(20 + 10 * i))
+        w = torch.randn(N, K, generator=gen(21 + 10 * i)) * 0.02
+        dy = torch.randn(M, N // 2 if epi == "swiglu" else N, generator=gen(22 + 10 * i))
+        layers.append((x, w, dy, epi))
+        flops += 6.0 * M * K * N
+
+    def step():
+        for x, w, dy, epi in layers:
+            y, _ = R.column_parallel_linear_forward(x, w, None)
+            g = dy
+            if epi == "swiglu":
+                R.swiglu(y)
+                g = R.swiglu_backward(dy, y)
+            R.linear_backward(x, w, g, False)
+
+    step()
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        step()
+        ts.append(time.perf_counter() - t0)
+    sec = statistics.median(ts)
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"value": round(flops / sec / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"llama3-8b QKV+gate/up(SwiGLU)+down fwd+bwd on {M} of 4096 tokens, fp32 torch CPU ops in the "
+                      f"reference's order, median of 3 ({sec:.2f} s/step); cpu: {model}"}
+
+
+def secondary(dev, timer, reps, with_cpu):
+    from merak_amd import ops, _lib
+    from oracle import tp_reference as R
+    out = {}
+    # --- vocab cross entropy, Llama-3 vocabulary, 8192 tokens, bf16, 5% labels = -100
+    n, v = 8192, 128256
+    g = torch.Generator(device=dev).manual_seed(1238)
+    logits = torch.empty(n, v, dtype=torch.bfloat16, device=dev).normal_(generator=g)
+    tgt = torch.randint(0, v, (n,), generator=gen(4))
+    tgt[torch.randperm(n, generator=gen(5))[: n // 20]] = -100
+    tgt = tgt.to(dev)
+    go = torch.full((n,), 1.0 / n, device=dev)
+    f_ms = timer.run("ce.fwd", lambda: ops.vocab_ce_fwd(logits, tgt, 0), reps)
+    loss, m, s, _ = ops.vocab_ce_fwd(logits, tgt, 0)
+    work = logits.clone()
+    b_ms = timer.run("ce.bwd", lambda: ops.vocab_ce_bwd_(work, tgt, m, s, go, 0), reps)
+    nbytes = n * v * 2
+    out["vocab_ce_c4"] = {
+        "shape": [n, v], "dtype": "bf16", "fwd_us": round(f_ms * 1e3, 1), "bwd_us": round(b_ms * 1e3, 1),
+        "fwd_GBs": round(nbytes / f_ms / 1e6, 1), "bwd_GBs": round(2 * nbytes / b_ms / 1e6, 1),
+        "fwd_bwd_GBs": round(3 * nbytes / (f_ms + b_ms) / 1e6, 1),
+        "frac_hbm_peak": round(3 * nbytes / (f_ms + b_ms) / 1e6 / PEAK_HBM_GBS, 4)}
+    if with_cpu:
+        rows = 64
+        xs = logits[:rows].cpu()
+        torch.set_num_threads(os.cpu_count() or 1)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            R.cross_entropy_fp32(xs, tgt[:rows].cpu(), 0, go[:rows].cpu())
+        sec = (time.perf_counter() - t0) / 3
+        out["vocab_ce_c4"]["cpu_port_GBs"] = round(3 * rows * v * 2 / sec / 1e9, 2)
+        out["vocab_ce_c4"]["cpu_sample"] = f"{rows} of {n} rows, fp32 multi-pass oracle"
+    del work
+    # --- GPT-2 vocabulary fp32 (config 1)
+    n1, v1 = 8192, 50257
+    lg1 = torch.empty(n1, v1, device=dev).normal_(generator=g)
+    t1 = torch.randint(0, v1, (n1,), generator=gen(6)).to(dev)
+    f1 = timer.run("ce1.fwd", lambda: ops.vocab_ce_fwd(lg1, t1, 0), reps)
+    _, m1, s1, _ = ops.vocab_ce_fwd(lg1, t1, 0)
+    b1 = timer.run("ce1.bwd", lambda: ops.vocab_ce_bwd_(lg1, t1, m1, s1, go, 0), reps)
+    out["vocab_ce_c1"] = {"shape": [n1, v1], "dtype": "f32", "fwd_us": round(f1 * 1e3, 1), "bwd_us": round(b1 * 1e3, 1),
+                          "fwd_bwd_GBs": round(3 * n1 * v1 * 4 / (f1 + b1) / 1e6, 1)}
+    del lg1
+    # --- embedding gather
+    h = 4096
+    table = torch.empty(v, h, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=g)
+    ids = torch.randint(0, v, (n,), generator=gen(7)).to(dev)
+    e_ms = timer.run("emb", lambda: ops.embedding_gather(ids, table, 0, v), reps)
+    out["embedding_c4"] = {"rows": n, "dim": h, "us": round(e_ms * 1e3, 1),
+                           "GBs": round((2 * n * h * 2 + n * 8) / e_ms / 1e6, 1)}
+    # --- decode step: QKV, gate/up+SwiGLU, down, LM head + argmax (the table doubles as the LM head)
+    mk = lambda nn, kk: torch.empty(nn, kk, device=dev).normal_(0, 0.02, generator=g).bfloat16()
+    wq, wg, wd = mk(6144, 4096), mk(2 * 14336, 4096), mk(4096, 14336)
+    wbytes = (wq.numel() + wg.numel() + wd.numel() + table.numel()) * 2
+    from merak_amd.inference import DecodeStep
+    step = DecodeStep(wq, wg, wd, table)
+    dec = {}
+    for b in (1, 8, 32):
+        x = torch.randn(b, 4096, generator=gen(8)).bfloat16().to(dev)
+        ms = timer.run(f"decode.b{b}", lambda: step(x), reps)
+        lm = timer.run(f"lmhead.b{b}", lambda: ops.gemv_argmax(x, table, step.workspace), reps)
+        dec[f"B{b}"] = {"us_per_step": round(ms * 1e3, 1), "tokens_per_s": round(b / ms * 1e3, 1),
+                        "GBs": round(wbytes / ms / 1e6, 1), "frac_hbm_peak": round(wbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                        "lm_head_argmax_us": round(lm * 1e3, 1), "lm_head_GBs": round(table.numel() * 2 / lm / 1e6, 1)}
+    out["decode_c5"] = dec
+    del table, wq, wg, wd, step
+    # --- Llama-70B tp=8 shard shapes
+    w3 = build_linear_workload(dev, LLAMA70B_TP8, 8192, 100)
+    ms3 = timer.run("c3.step", lambda: linear_step(w3), max(3, reps // 2))
+    fl3 = sum(L["flops"] for L in w3)
+    out["linear_c3_llama70b_tp8"] = {"ms_per_step": round(ms3, 4), "tflops": round(fl3 / ms3 / 1e9, 1),
+                                     "frac_bf16_peak": round(fl3 / ms3 / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    del w3
+    # --- GPT-2-small fp32 (config 1): Column 768->3072 bias+GeLU, Row 3072->768 bias
+    M1 = 8192
+    x1 = torch.randn(M1, 768, generator=gen(9)).to(dev)
+    wc = (torch.randn(3072, 768, generator=gen(10)) * 0.02).to(dev)
+    wr = (torch.randn(768, 3072, generator=gen(11)) * 0.02).to(dev)
+    bc, br = torch.zeros(3072, device=dev), torch.zeros(768, device=dev)
+    dy1 = torch.randn(M1, 768, generator=gen(12)).to(dev)
+
+    def c1_step():
+        y, a = ops.linear_fwd(x1, wc, bc, ops.EPI_BIAS_GELU)
+        o, _ = ops.linear_fwd(a, wr, br, ops.EPI_BIAS)
+        da = ops.linear_dgrad(dy1, wr)
+        ops.linear_wgrad(dy1, a, True)
+        dpre = ops.activation_bwd(da, y, ops.EPI_BIAS_GELU)
+        ops.linear_dgrad(dpre, wc)
+        ops.linear_wgrad(dpre, x1, True)
+
+    ms1 = timer.run("c1.step", c1_step, max(3, reps // 2))
+    fl1 = 2 * 6.0 * M1 * 768 * 3072
+    out["linear_c1_gpt2_fp32"] = {"ms_per_step": round(ms1, 4), "tflops": round(fl1 / ms1 / 1e9, 1),
+                                  "frac_f32_peak": round(fl1 / ms1 / 1e9 / PEAK_F32_TFLOPS, 4)}
+    # --- what this GPU does on a plain copy and on a register-resident MFMA loop
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    st = torch.cuda.current_stream().cuda_stream
+    c_ms = timer.run("copy", lambda: _lib.check(_lib.lib().mtp_stream_copy(src.data_ptr(), dst.data_ptr(), src.numel(), st), "copy"), reps)
+    sink = torch.empty(64 * 4096, device=dev)
+    iters = 8192
+    p_ms = timer.run("mfma", lambda: _lib.check(_lib.lib().mtp_mfma_peak(sink.data_ptr(), 4096, iters, st), "peak"), 3)
+    out["device_reference"] = {"copy_1GiB_GBs_read_plus_write": round(2 * src.numel() / c_ms / 1e6, 1),
+                               "mfma_loop_bf16_tflops": round(4096 * iters * 32 * 32 * 16 * 2 / p_ms / 1e9, 1)}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="headline only (no secondary figures)")
+    ap.add_argument("--cpu-tokens", type=int, default=1024)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (no collectives, one rank's share "
+              "of the tensor-parallel layers per process). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X (gfx950) device", file=sys.stderr)
+        sys.exit(2)
+    from merak_amd import _lib
+    _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    M = 4096
+    work = build_linear_workload(dev, LLAMA8B, M, 20)
+    flops = sum(L["flops"] for L in work)
+    for _ in range(args.warmup):
+        linear_step(work)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        linear_step(work)
+    torch.cuda.synchronize()
+    sec = time.perf_counter() - t0
+    ms_per_step = sec / args.steps * 1e3
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+
+    timer = Timer()
+    reps = max(5, min(20, args.steps))
+    kernels = per_kernel(work, timer, reps)
+    gemms = [k for k in kernels if "tflops" in k]
+    dom = max(gemms, key=lambda k: k["ms"])
+    roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "launch_ms": dom["ms"], "flops_per_launch": 2.0 * dom["M"] * dom["N"] * dom["K"]}
+    del work
+    result = {
+        "metric": "TP-shard linear fwd+bwd TFLOP/s (% bf16 peak); vocab-CE HBM GB/s",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "llama3-8b single-rank (tp=1) QKV 4096->6144 + gate/up 4096->2x14336 (fused SwiGLU) + "
+                               "down 14336->4096, fwd+bwd on 4096 tokens, bf16 / fp32 accumulate",
+                   "tokens": M, "flops_per_step": flops},
+        "frac_bf16_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not args.no_extras:
+        result["secondary"] = secondary(dev, timer, reps, not args.no_cpu)
+        ce = result["secondary"]["vocab_ce_c4"]
+        result["vocab_ce_GBs"] = ce["fwd_bwd_GBs"]
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(args.cpu_tokens)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

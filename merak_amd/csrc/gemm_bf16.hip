@@ -25,6 +25,7 @@
 //     L2) walk neighbouring tiles.
 #include "mtp_common.h"
 #include <type_traits>
+#include <utility>
 
 namespace {
 
@@ -46,6 +47,22 @@ struct GemmArgs {
 
 enum : int { OUT_BF16 = 0, OUT_F32 = 1 };
 
+// compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{})
+template <int... Is, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+// one scheduling group of N instructions of the class MASK (N may be 0: nothing emitted)
+template <int MASK, int N>
+__device__ __forceinline__ void sched_group() {
+  if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
+}
+constexpr int SG_MFMA = 0x008, SG_VMEM_RD = 0x020, SG_DS_RD = 0x100;
+
 // LDS hand-over between lanes of one wave: DS operations of a wave complete in order, the fence and
 // the scheduling barrier keep the compiler from moving accesses across the hand-over point.
 __device__ __forceinline__ void wave_lds_sync() {
@@ -54,11 +71,28 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_wave_barrier();
 }
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int64_t bytes) {
+// Raw buffer resource (stride 0): base address, num_records in bytes, gfx9 dword3 for untyped 32-bit data.
+typedef __attribute__((ext_vector_type(4))) int rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, int64_t bytes) {
   if (bytes < 0) bytes = 0;
   // offsets are tile relative and below 2^31; 0x80000000 is the "read as zero" marker
   const uint32_t n = bytes > 0x80000000ll ? 0x80000000u : (uint32_t)bytes;
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
+  const uint64_t b = reinterpret_cast<uint64_t>(base);
+  return rsrc_t{(int)(uint32_t)b, (int)((b >> 32) & 0xffffu), (int)n, 0x00020000};
+}
+
+// One DMA instruction: 64 lanes x 16 bytes from the buffer (VGPR offset voff, range checked; scalar offset
+// soff, not checked) to LDS bytes [lds_addr, lds_addr + 1024) in lane order.  Written as inline assembly on
+// purpose: the compiler then does not model the LDS write, and so does not put an s_waitcnt vmcnt(0) in
+// front of every later ds_read_b64_tr_b16 (which it cannot prove independent of an in-flight DMA).  The
+// kernel orders DMA against LDS reads itself: s_waitcnt vmcnt(0) + s_barrier once per k-tile.
+__device__ __forceinline__ void dma16(rsrc_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff));
+}
+__device__ __forceinline__ uint32_t lds_addr_of(const void* p) {
+  return (uint32_t)(uintptr_t)(const void __attribute__((address_space(3)))*)p;
 }
 
 // XCD-aware, grouped mapping of the linear workgroup id to a tile.
@@ -82,31 +116,147 @@ __device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& 
   tn = r / gsz;
 }
 
+// t-th block of a TI x TJ grid walked in growing squares: (0,0); (1,0) (1,1) (0,1); (2,0) (2,1) (2,2) (0,2) (1,2); ...
+struct BlockIJ {
+  int i, j;
+};
+constexpr BlockIJ shell_pair(int t, int TI, int TJ) {
+  int n = 0;
+  for (int d = 0; d < (TI > TJ ? TI : TJ); d++) {
+    for (int j = 0; j <= d; j++)
+      if (d < TI && j < TJ) {
+        if (n == t) return BlockIJ{d, j};
+        n++;
+      }
+    for (int i = 0; i < d; i++)
+      if (i < TI && d < TJ) {
+        if (n == t) return BlockIJ{i, d};
+        n++;
+      }
+  }
+  return BlockIJ{0, 0};
+}
+
 // ---------------------------------------------------------------------------
-// LDS tile of a "row" operand: ROWS x 64 bf16, 128 bytes per row, the 16-byte
-// chunk c of row r is stored at chunk position c ^ ((r >> 1) & 7).
-// One DMA instruction fills 8 rows (1 KiB, lane l -> row l/8, position l%8).
+// Operands.  Each describes one side of the product for one workgroup: how its
+// 64-deep k-tile is fetched into LDS by DMA and how a wave reads its MFMA
+// fragments back.  "rows" below are the operand's M (or N) indices.
+//
+// RowOperand: memory is [rows, K] with K contiguous.  LDS tile = ROWS x 64 bf16,
+//   128 bytes per row; the 16-byte chunk c of row r sits at chunk position
+//   c ^ ((r >> 1) & 7).  One DMA instruction fills 8 rows (lane l -> row l/8,
+//   position l%8).  Fragment = one ds_read_b128 (8 consecutive k of one row).
+//
+// ColOperand: memory is [K, rows] with rows contiguous (a transposed operand).
+//   LDS tile = 64 x ROWS bf16 in the same orientation, 2*ROWS bytes per k-row;
+//   chunk c of k-row k sits at position c ^ ((k & 3) << 2).  One DMA
+//   instruction fills 1 KiB of consecutive k-rows.  Fragment = two
+//   ds_read_b64_tr_b16: inside each group of 16 lanes, lane i supplies the address
+//   of 4 consecutive rows-elements of k-row (i/4) and receives, transposed, the
+//   4 consecutive k of row i — exactly the MFMA operand layout.
 // ---------------------------------------------------------------------------
 template <int ROWS>
-struct RowTile {
+struct RowOperand {
   static constexpr int BYTES = ROWS * 128;
-  static constexpr int INSTR_PER_WAVE = ROWS / 32;  // 4 waves, 8 rows per instruction
+  static constexpr int NINSTR = ROWS / 32;  // DMA instructions per wave per k-tile
+  static constexpr int NREADS = 1;          // LDS reads per fragment
+  rsrc_t rsrc;
+  uint32_t voff[NINSTR];
+  uint32_t fo[4];
+  int chunk, K;
 
-  // LDS byte address of fragment rows (row = row0 + lane%32), k16 step kk: 8 elements at k = 16kk + 8(lane/32)
-  __device__ static __forceinline__ uint32_t frag_offset(int row, int kk, int h) {
-    return (uint32_t)(row * 128 + ((((2 * kk + h) ^ (row >> 1)) & 7) << 4));
+  // rowmap(r): global row (relative to row0) of tile row r, or a negative value for "no such row"
+  template <typename RowMap>
+  __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int row0, int nrows, int K_, int lane,
+                                       int wave, int wave_row0, RowMap rowmap) {
+    K = K_;
+    // VGPR offsets are range checked against num_records: rows past the edge read as zero.  The k-tile
+    // advance goes into the scalar offset (not checked; the ragged last k-tile is masked by hand).
+    rsrc = make_rsrc(base + (int64_t)row0 * ld, (int64_t)(nrows - row0) * ld * 2);
+    chunk = (lane & 7) ^ ((4 * wave + (lane >> 4)) & 7);
+    const int lrow = lane >> 3;
+#pragma unroll
+    for (int j = 0; j < NINSTR; j++) {
+      const int r = (wave + 4 * j) * 8 + lrow;
+      const int64_t gr = rowmap(r);
+      voff[j] = (gr < 0 || gr >= nrows - row0) ? 0x80000000u : (uint32_t)((gr * ld + chunk * 8) * 2);
+    }
+    const int row = wave_row0 + (lane & 31), h = lane >> 5;
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) fo[kk] = (uint32_t)(row * 128 + ((((2 * kk + h) ^ (row >> 1)) & 7) << 4));
+  }
+  // j-th DMA instruction of this wave for k-tile kt; tile = LDS byte address of the operand's stage
+  __device__ __forceinline__ void issue(int kt, uint32_t tile, int wave, int j) const {
+    const bool dead = kt * BK + chunk * 8 >= K;  // only ever true in a ragged last k-tile (or past the end)
+    dma16(rsrc, tile + (wave + 4 * j) * 1024, dead ? 0x80000000u : voff[j], (uint32_t)(kt * BK * 2));
+  }
+  __device__ __forceinline__ bf16x8_t frag(const char* tile, int kk, int blk) const {
+    return *reinterpret_cast<const bf16x8_t*>(tile + fo[kk] + blk * 4096);
   }
 };
+
+template <int ROWS>
+struct ColOperand {
+  static_assert(ROWS == 256, "transposed operands are built for 256-wide tiles");
+  static constexpr int BYTES = 64 * ROWS * 2;
+  static constexpr int NINSTR = BYTES / 1024 / 4;
+  static constexpr int NREADS = 2;
+  const char* base;    // &mem[0][row0]
+  int64_t total;       // bytes from base to the end of the matrix
+  int64_t ktile_bytes; // 64 * ld * 2
+  uint32_t voff[NINSTR];
+  uint32_t lane_base;
+  uint32_t moff[4];
+
+  __device__ __forceinline__ void init(const uint16_t* mem, int64_t ld, int row0, int K_, int lane, int wave,
+                                       int wave_row0) {
+    base = reinterpret_cast<const char*>(mem + row0);
+    total = ((int64_t)K_ * ld - row0) * 2;
+    ktile_bytes = (int64_t)BK * ld * 2;
+    // DMA: instruction q = wave + 4j covers k-rows 2q, 2q+1 (512 bytes each); lane l -> k-row 2q + l/32,
+    // LDS position l%32, which holds chunk position ^ ((k & 3) << 2)
+    const int ksub = lane >> 5;
+    const int c = (lane & 31) ^ (((2 * wave + ksub) & 3) << 2);
+#pragma unroll
+    for (int j = 0; j < NINSTR; j++) {
+      const int krow = 2 * (wave + 4 * j) + ksub;
+      voff[j] = (uint32_t)(((int64_t)krow * ld + c * 8) * 2);
+    }
+    // fragment reads
+    const int G = lane >> 4, i = lane & 15, kq = i >> 2;
+    const int cw = wave_row0 >> 3;  // first chunk of the wave's rows (a multiple of 16)
+    lane_base = (uint32_t)((8 * (G >> 1) + kq) * (ROWS * 2) + (cw + 2 * (G & 1) + ((i & 3) >> 1)) * 16 + 8 * (i & 1));
+#pragma unroll
+    for (int blk = 0; blk < 4; blk++) moff[blk] = (uint32_t)(64 * (blk ^ kq));
+  }
+  __device__ __forceinline__ void issue(int kt, uint32_t tile, int wave, int j) const {
+    // the whole address, k-tile advance included, goes through the range check: k-rows past K and the
+    // tail of the last row read as zero
+    const rsrc_t r = make_rsrc(base + kt * ktile_bytes, total - kt * ktile_bytes);
+    dma16(r, tile + (wave + 4 * j) * 1024, voff[j], 0);
+  }
+  __device__ __forceinline__ bf16x8_t frag(const char* tile, int kk, int blk) const {
+    const char* a = tile + lane_base + moff[blk] + kk * (16 * ROWS * 2);
+    const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+        (bf16x4_t __attribute__((address_space(3)))*)(a));
+    const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+        (bf16x4_t __attribute__((address_space(3)))*)(a + 4 * ROWS * 2));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  }
+};
+
+template <int LAY, int ROWS> struct OperandOf { using type = RowOperand<ROWS>; };
+template <int ROWS> struct OperandOf<LAY_COL, ROWS> { using type = ColOperand<ROWS>; };
 
 // The body lives in a __device__ function: it uses device-only types (__amdgpu_buffer_rsrc_t) that the
 // host pass over a __global__ function cannot digest.
 template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT>
 __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
-  static_assert(ALAY == LAY_ROW && BLAY == LAY_ROW, "layout not built yet");
+  static_assert(EPI != MTP_EPI_SWIGLU || BLAY == LAY_ROW, "the SwiGLU row interleave is a forward (row B) feature");
   constexpr int TI = BM / 64, TJ = BN / 64;  // 32x32 blocks per wave in m and n
-  using ATile = RowTile<BM>;
-  using BTile = RowTile<BN>;
-  constexpr int STAGE_BYTES = ATile::BYTES + BTile::BYTES;
+  using AOp = typename OperandOf<ALAY, BM>::type;
+  using BOp = typename OperandOf<BLAY, BN>::type;
+  constexpr int STAGE_BYTES = AOp::BYTES + BOp::BYTES;
   __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE_BYTES];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -123,64 +273,40 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   const int m0 = tm * BM;
   const int n0 = tn * BN_SPAN;
 
-  // ---- DMA addressing -------------------------------------------------------
-  // Every DMA instruction moves 8 tile rows; instruction q = wave + 4j.  The per-lane byte offset
-  // (row * ld + chunk * 8) * 2 goes into the VGPR offset, which the buffer range check covers: rows
-  // past the matrix edge land beyond num_records and read as zero.  The k-tile advance goes into the
-  // scalar offset (not range checked, always inside the row; the ragged last k-tile is masked by hand).
-  // A: rows m0.. of [M,K]
-  const __amdgpu_buffer_rsrc_t rsrcA = make_rsrc(p.A + (int64_t)m0 * p.lda, (int64_t)(p.M - m0) * p.lda * 2);
-  // B: LDS row r of the tile maps to a global row of [N,K].  Plain: n0 + r.  SwiGLU: the wave-column wn
-  // owns LDS rows [wn*BN/2, (wn+1)*BN/2): first half gate rows, second half the matching up rows.
-  const __amdgpu_buffer_rsrc_t rsrcB = make_rsrc(p.B + (int64_t)n0 * p.ldb, (int64_t)(p.N - n0) * p.ldb * 2);
-  const int chunk = (lane & 7) ^ ((4 * wave + (lane >> 4)) & 7);  // k chunk (8 elements) this lane fetches
-  const int lrow = lane >> 3;
-  uint32_t voffA[ATile::INSTR_PER_WAVE], voffB[BTile::INSTR_PER_WAVE];
-#pragma unroll
-  for (int j = 0; j < ATile::INSTR_PER_WAVE; j++) {
-    const int r = (wave + 4 * j) * 8 + lrow;
-    voffA[j] = (uint32_t)(((int64_t)r * p.lda + chunk * 8) * 2);
+  AOp opA;
+  BOp opB;
+  if constexpr (ALAY == LAY_ROW)
+    opA.init(p.A, p.lda, m0, p.M, p.K, lane, wave, wm * (BM / 2), [](int r) -> int64_t { return r; });
+  else
+    opA.init(p.A, p.lda, m0, p.K, lane, wave, wm * (BM / 2));
+  if constexpr (BLAY == LAY_ROW) {
+    // LDS row r of the B tile maps to a global row of [N,K].  Plain: n0 + r.  SwiGLU: the wave-column wn
+    // owns LDS rows [wn*BN/2, (wn+1)*BN/2): first half gate rows, second half the matching up rows.
+    opB.init(p.B, p.ldb, n0, p.N, p.K, lane, wave, wn * (BN / 2), [&](int r) -> int64_t {
+      if (EPI == MTP_EPI_SWIGLU) {
+        const int seg = r / (BN / 4), in = r % (BN / 4);
+        const int64_t gr = ((seg & 1) ? p.half : 0) + (seg >> 1) * (BN / 4) + in;
+        // gate rows at or past `half` belong to the up matrix: no such row
+        return (!(seg & 1) && n0 + gr >= p.half) ? -1 : gr;
+      }
+      return r;
+    });
+  } else {
+    opB.init(p.B, p.ldb, n0, p.K, lane, wave, wn * (BN / 2));
   }
-#pragma unroll
-  for (int j = 0; j < BTile::INSTR_PER_WAVE; j++) {
-    const int r = (wave + 4 * j) * 8 + lrow;
-    int64_t gr = r;  // relative to n0
-    if (EPI == MTP_EPI_SWIGLU) {
-      const int seg = r / (BN / 4), in = r % (BN / 4);
-      gr = ((seg & 1) ? p.half : 0) + (seg >> 1) * (BN / 4) + in;
-      // gate rows at or past `half` belong to the up matrix: treat as out of range
-      if (!(seg & 1) && n0 + gr >= p.half) gr = (int64_t)p.N;
-    }
-    voffB[j] = (uint32_t)((gr * p.ldb + chunk * 8) * 2);
-    if (gr >= p.N - n0) voffB[j] = 0x80000000u;
-  }
-
-  auto issue_loads = [&](int kt, int buf) {
-    char* la = lds + buf * STAGE_BYTES;
-    char* lb = la + ATile::BYTES;
-    const bool dead = kt * BK + chunk * 8 >= p.K;  // only ever true in a ragged last k-tile
-    const uint32_t soff = (uint32_t)(kt * BK * 2);
-#pragma unroll
-    for (int j = 0; j < ATile::INSTR_PER_WAVE; j++) {
-      const int q = wave + 4 * j;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, LDS_PTR(la + q * 1024), 16, dead ? 0x80000000u : voffA[j], soff,
-                                               0, 0);
-    }
-#pragma unroll
-    for (int j = 0; j < BTile::INSTR_PER_WAVE; j++) {
-      const int q = wave + 4 * j;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, LDS_PTR(lb + q * 1024), 16, dead ? 0x80000000u : voffB[j], soff,
-                                               0, 0);
-    }
+  constexpr int NDMA = AOp::NINSTR + BOp::NINSTR;  // DMA instructions per wave per k-tile
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr_of(lds));
+  auto issue_one = [&](int kt, int buf, int d) {  // d-th DMA instruction of the k-tile
+    const uint32_t la = lds0 + buf * STAGE_BYTES;
+    if (d < AOp::NINSTR)
+      opA.issue(kt, la, wave, d);
+    else
+      opB.issue(kt, la + AOp::BYTES, wave, d - AOp::NINSTR);
   };
-
-  // ---- fragment addressing ---------------------------------------------------
-  uint32_t fa[4], fb[4];  // per k16 step, block 0; further blocks are +32 rows = +4096 bytes
+  auto issue_loads = [&](int kt, int buf) {
 #pragma unroll
-  for (int kk = 0; kk < 4; kk++) {
-    fa[kk] = ATile::frag_offset(wm * (BM / 2) + l32, kk, lh);
-    fb[kk] = BTile::frag_offset(wn * (BN / 2) + l32, kk, lh);
-  }
+    for (int d = 0; d < NDMA; d++) issue_one(kt, buf, d);
+  };
 
   f32x16_t acc[TI][TJ];
 #pragma unroll
@@ -196,37 +322,42 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   // in registers: the ds_reads of k16-step s+1 are in flight while the MFMAs of step s issue.
   const int KT = (p.K + BK - 1) / BK;
   bf16x8_t af[2][TI], bfr[2][TJ];
-  // Reads are issued A0 B0 A1 B1 ... and the MFMAs walk the block grid in growing squares
+  // Fragments are read in the order A0 B0 A1 B1 ... and the MFMAs walk the block grid in growing squares
   // ((0,0); (1,0) (1,1) (0,1); ...), so the first MFMAs of a step depend only on the oldest reads.
-  auto read_frags = [&](int buf, int kk, int slot) {
+  constexpr int TMAX = TI > TJ ? TI : TJ;
+  constexpr int NFR = TI + TJ;   // fragments per k16 step
+  constexpr int NMF = TI * TJ;   // MFMAs per k16 step
+  auto read_one = [&](int buf, int kk, int slot, auto u_tag) {  // u-th fragment in A0 B0 A1 B1 ... order
+    constexpr int u = decltype(u_tag)::value;
     const char* la = lds + buf * STAGE_BYTES;
-    const char* lb = la + ATile::BYTES;
-#pragma unroll
-    for (int d = 0; d < (TI > TJ ? TI : TJ); d++) {
-      if (d < TI) af[slot][d] = *reinterpret_cast<const bf16x8_t*>(la + fa[kk] + d * 4096);
-      if (d < TJ) bfr[slot][d] = *reinterpret_cast<const bf16x8_t*>(lb + fb[kk] + d * 4096);
-    }
+    // with TI == TJ the order alternates; otherwise the longer side's leftovers come last
+    constexpr int d = u < 2 * (TI < TJ ? TI : TJ) ? u / 2 : u - (TI < TJ ? TI : TJ);
+    constexpr bool is_a = u < 2 * (TI < TJ ? TI : TJ) ? (u % 2 == 0) : (TI > TJ);
+    if constexpr (is_a)
+      af[slot][d] = opA.frag(la, kk, d);
+    else
+      bfr[slot][d] = opB.frag(la + AOp::BYTES, kk, d);
+  };
+  auto read_frags = [&](int buf, int kk, int slot) {
+    static_for<NFR>([&](auto u) { read_one(buf, kk, slot, u); });
+  };
+  auto mfma_one = [&](int slot, auto t_tag) {  // t-th MFMA of a step in shell order
+    constexpr int t = decltype(t_tag)::value;
+    constexpr int i = shell_pair(t, TI, TJ).i, j = shell_pair(t, TI, TJ).j;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[slot][j], af[slot][i], acc[i][j], 0, 0, 0);
   };
   auto mfmas = [&](int slot) {
-#pragma unroll
-    for (int d = 0; d < (TI > TJ ? TI : TJ); d++) {
-#pragma unroll
-      for (int j = 0; j <= d; j++)  // row d of the shell
-        if (d < TI && j < TJ)
-          acc[d][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[slot][j], af[slot][d], acc[d][j], 0, 0, 0);
-#pragma unroll
-      for (int i = 0; i < d; i++)  // column d of the shell
-        if (i < TI && d < TJ)
-          acc[i][d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[slot][d], af[slot][i], acc[i][d], 0, 0, 0);
-    }
+    static_for<NMF>([&](auto t) { mfma_one(slot, t); });
   };
 
   // One k-tile.  FULL: tiles kt+1 and kt+2 exist, so the prefetches are unconditional and the body is a
-  // single basic block whose instruction mix is pinned by the sched_group_barrier sequence:
-  //   steps 0-2 : 8 x (2 MFMA, 1 LDS read)
-  //   step 3    : 8 x (1 MFMA, 1 DMA, 1 LDS read, 1 MFMA, 1 DMA)   [16 DMA instructions per wave at 256x256]
+  // single basic block whose instruction order is pinned:
+  //   steps 0-2 : sched_group_barrier sequence, per LDS read its share of the step's MFMAs
+  //   step 3    : written out by hand (MFMA, DMA, fragment read of the next tile, ...) with scheduling
+  //               barriers in between, because the DMA is inline assembly the group barriers cannot see
   auto ktile = [&](int kt, auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
+    constexpr int NDS = TI * AOp::NREADS + TJ * BOp::NREADS;           // LDS reads per k16 step
     const int buf = kt & 1;
     read_frags(buf, 1, 1);
     mfmas(0);
@@ -234,29 +365,34 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
     mfmas(1);
     read_frags(buf, 3, 1);
     mfmas(0);
-    if (FULL) {
-#pragma unroll
-      for (int t = 0; t < 3 * (TI + TJ); t++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, (TI * TJ) / (TI + TJ), 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                      // DS read
-      }
+    if constexpr (FULL) {
+      static_for<3 * NDS>([&](auto t) {
+        // spread NMF MFMAs over NDS reads: read u gets floor((u+1)*NMF/NDS) - floor(u*NMF/NDS) of them
+        constexpr int u = decltype(t)::value % NDS;
+        sched_group<SG_MFMA, (u + 1) * NMF / NDS - u * NMF / NDS>();
+        sched_group<SG_DS_RD, 1>();
+      });
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): tile kt+1 has landed in the other stage
     __syncthreads();                     // ... for every wave, and everyone is done reading this stage
-    if (FULL || kt + 2 < KT) issue_loads(kt + 2, buf);
-    if (FULL || kt + 1 < KT) read_frags(buf ^ 1, 0, 0);
-    mfmas(1);
-    if (FULL) {
-      constexpr int NDMA = ATile::INSTR_PER_WAVE + BTile::INSTR_PER_WAVE;
-      constexpr int NMF = TI * TJ, NDS = TI + TJ;
-      static_assert(NMF % NDS == 0 && NDMA % NDS == 0, "schedule assumes these ratios");
-#pragma unroll
-      for (int t = 0; t < NDS; t++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x020, NDMA / NDS, 0);        // VMEM read (DMA)
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 // DS read
-        __builtin_amdgcn_sched_group_barrier(0x008, NMF / NDS - 1, 0);     // MFMA
-      }
+    if constexpr (FULL) {
+      __builtin_amdgcn_sched_barrier(0);
+      static_for<NMF>([&](auto t_tag) {
+        constexpr int t = decltype(t_tag)::value;
+        mfma_one(1, t_tag);
+        // DMA instructions and next-tile fragment reads spread evenly over the step's MFMAs
+        static_for<(t + 1) * NDMA / NMF - t * NDMA / NMF>([&](auto e) {
+          issue_one(kt + 2, buf, t * NDMA / NMF + decltype(e)::value);
+        });
+        static_for<(t + 1) * NFR / NMF - t * NFR / NMF>([&](auto e) {
+          read_one(buf ^ 1, 0, 0, std::integral_constant<int, t * NFR / NMF + decltype(e)::value>{});
+        });
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    } else {
+      if (kt + 2 < KT) issue_loads(kt + 2, buf);
+      if (kt + 1 < KT) read_frags(buf ^ 1, 0, 0);
+      mfmas(1);
     }
   };
 
@@ -485,10 +621,36 @@ int mtp_gemm_bf16_nt(const void* A, const void* B, const void* bias, void* C, vo
   return MTP_EINVAL;
 }
 
-// dgrad / wgrad on the bf16 MFMA kernel: not built yet, the caller falls back to the general kernel.
-int mtp_gemm_bf16_dgrad(const void*, const void*, void*, int64_t, int64_t, int64_t, hipStream_t) {
-  return MTP_EUNSUPPORTED;
+// dX[M,K] = dY[M,N] W[N,K]: GEMM (M, K, reduce N) with A = dY (row) and B = W read as [reduce, cols] (col).
+int mtp_gemm_bf16_dgrad(const void* dy, const void* w, void* dx, int64_t M, int64_t N, int64_t K, hipStream_t s) {
+  GemmArgs a{};
+  a.A = (const uint16_t*)dy;
+  a.B = (const uint16_t*)w;
+  a.C = dx;
+  a.M = (int)M;
+  a.N = (int)K;
+  a.K = (int)N;
+  a.lda = N;
+  a.ldb = K;
+  a.ldc = K;
+  return launch<256, 256, LAY_ROW, LAY_COL, MTP_EPI_NONE, OUT_BF16>(a, s);
 }
-int mtp_gemm_bf16_wgrad(const void*, const void*, void*, void*, int64_t, int64_t, int64_t, int, int, hipStream_t) {
-  return MTP_EUNSUPPORTED;
+
+// dW[N,K] (+)= dY[M,N]^T X[M,K]: GEMM (N, K, reduce M) with both operands transposed (col).
+int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
+                        int dw_dtype, int accumulate, hipStream_t s) {
+  if (db) return MTP_EUNSUPPORTED;  // bias gradient: served by the general path for now
+  GemmArgs a{};
+  a.A = (const uint16_t*)dy;
+  a.B = (const uint16_t*)x;
+  a.C = dw;
+  a.M = (int)N;
+  a.N = (int)K;
+  a.K = (int)M;
+  a.lda = N;
+  a.ldb = K;
+  a.ldc = K;
+  a.accumulate = accumulate;
+  if (dw_dtype == MTP_F32) return launch<256, 256, LAY_COL, LAY_COL, MTP_EPI_NONE, OUT_F32>(a, s);
+  return launch<256, 256, LAY_COL, LAY_COL, MTP_EPI_NONE, OUT_BF16>(a, s);
 }

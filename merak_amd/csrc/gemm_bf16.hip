@@ -9,10 +9,13 @@
 //   dgrad    dX = dY W   : A = dY row, B = W col            (M=tokens, N=in,  K=out)
 //   wgrad    dW = dY^T X : A = dY col, B = X col            (M=out,    N=in,  K=tokens)
 //
-// Structure (one workgroup = 4 waves = one BMxBN tile, BK = 64):
+// Structure (one workgroup = 4 or 8 waves = one BMxBN tile, BK = 32):
 //   * global -> LDS with buffer_load_dwordx4 ... lds (no VGPR staging; rows and
 //     columns past the matrix edge read as zero through the buffer range check),
-//     double buffered, one s_barrier per k-tile;
+//     a ring of 4 stages of 32-deep k-tiles: tile kt+3 is requested while tile
+//     kt is multiplied, its DMA instructions spread evenly between the MFMAs
+//     (a burst of them right after a barrier backs up the address path and
+//     stalls MFMA issue), one s_barrier per k-tile;
 //   * LDS tiles are XOR-swizzled at 16-byte granularity so both the 1 KiB
 //     linear DMA writes and the ds_read_b128 / ds_read_b64_tr_b16 fragment
 //     reads are bank-conflict free;
@@ -24,12 +27,15 @@
 //   * workgroup ids are remapped so that the 32 CUs of one XCD (which share an
 //     L2) walk neighbouring tiles.
 #include "mtp_common.h"
+#include <stdlib.h>
 #include <type_traits>
 #include <utility>
 
 namespace {
 
-constexpr int BK = 64;
+constexpr int BK = 32;      // k-tile depth
+constexpr int NSTAGE = 4;   // LDS ring: 4 x (16 KiB A + 16 KiB B) at 256x256
+constexpr int KSTEPS = BK / 16;  // MFMA k16 steps per k-tile
 constexpr int LAY_ROW = 0;  // reduction dimension contiguous
 constexpr int LAY_COL = 1;  // M (or N) contiguous
 
@@ -43,6 +49,8 @@ struct GemmArgs {
   int64_t lda, ldb, ldc, ldc2;
   int accumulate;      // C += result
   int half;            // SwiGLU: number of gate columns (N/2)
+  int debug;           // measurement only (MTP_GEMM_DEBUG): 1 = every tile loads tile (0,0), 2 = no epilogue
+                       // stores, 4 = every DMA reads out of range (no memory traffic).  Results are wrong with any bit set.
 };
 
 enum : int { OUT_BF16 = 0, OUT_F32 = 1 };
@@ -70,6 +78,10 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
   __builtin_amdgcn_wave_barrier();
 }
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
+// expcnt 6:4 and lgkmcnt 11:8 left at their maxima)
+constexpr int vmcnt_imm(int n) { return (n & 0xf) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
 // Raw buffer resource (stride 0): base address, num_records in bytes, gfx9 dword3 for untyped 32-bit data.
 typedef __attribute__((ext_vector_type(4))) int rsrc_t;
@@ -139,30 +151,31 @@ constexpr BlockIJ shell_pair(int t, int TI, int TJ) {
 
 // ---------------------------------------------------------------------------
 // Operands.  Each describes one side of the product for one workgroup: how its
-// 64-deep k-tile is fetched into LDS by DMA and how a wave reads its MFMA
+// 32-deep k-tile is fetched into LDS by DMA and how a wave reads its MFMA
 // fragments back.  "rows" below are the operand's M (or N) indices.
 //
-// RowOperand: memory is [rows, K] with K contiguous.  LDS tile = ROWS x 64 bf16,
-//   128 bytes per row; the 16-byte chunk c of row r sits at chunk position
-//   c ^ ((r >> 1) & 7).  One DMA instruction fills 8 rows (lane l -> row l/8,
-//   position l%8).  Fragment = one ds_read_b128 (8 consecutive k of one row).
+// RowOperand: memory is [rows, K] with K contiguous.  LDS tile = ROWS x 32 bf16,
+//   64 bytes per row; the 16-byte chunk c of row r sits at chunk position
+//   c ^ ((r >> 2) & 3), which spreads any 16 consecutive rows read at one k over
+//   all 64 banks.  One DMA instruction fills 16 rows (lane l -> row l/4,
+//   position l%4).  Fragment = one ds_read_b128 (8 consecutive k of one row).
 //
 // ColOperand: memory is [K, rows] with rows contiguous (a transposed operand).
-//   LDS tile = 64 x ROWS bf16 in the same orientation, 2*ROWS bytes per k-row;
+//   LDS tile = 32 x ROWS bf16 in the same orientation, 2*ROWS bytes per k-row;
 //   chunk c of k-row k sits at position c ^ ((k & 3) << 2).  One DMA
 //   instruction fills 1 KiB of consecutive k-rows.  Fragment = two
 //   ds_read_b64_tr_b16: inside each group of 16 lanes, lane i supplies the address
 //   of 4 consecutive rows-elements of k-row (i/4) and receives, transposed, the
 //   4 consecutive k of row i — exactly the MFMA operand layout.
 // ---------------------------------------------------------------------------
-template <int ROWS>
+template <int ROWS, int NW>
 struct RowOperand {
-  static constexpr int BYTES = ROWS * 128;
-  static constexpr int NINSTR = ROWS / 32;  // DMA instructions per wave per k-tile
-  static constexpr int NREADS = 1;          // LDS reads per fragment
+  static constexpr int BYTES = ROWS * BK * 2;
+  static constexpr int NINSTR = ROWS / 16 / NW;  // DMA instructions per wave per k-tile (16 rows each)
+  static constexpr int NREADS = 1;               // LDS reads per fragment
   rsrc_t rsrc;
   uint32_t voff[NINSTR];
-  uint32_t fo[4];
+  uint32_t fo[KSTEPS];
   int chunk, K;
 
   // rowmap(r): global row (relative to row0) of tile row r, or a negative value for "no such row"
@@ -173,37 +186,47 @@ struct RowOperand {
     // VGPR offsets are range checked against num_records: rows past the edge read as zero.  The k-tile
     // advance goes into the scalar offset (not checked; the ragged last k-tile is masked by hand).
     rsrc = make_rsrc(base + (int64_t)row0 * ld, (int64_t)(nrows - row0) * ld * 2);
-    chunk = (lane & 7) ^ ((4 * wave + (lane >> 4)) & 7);
-    const int lrow = lane >> 3;
+    // lane l of instruction q fills row 16q + l/4, position l%4; (row >> 2) & 3 = (l >> 4) & 3
+    chunk = (lane & 3) ^ ((lane >> 4) & 3);
+    const int lrow = lane >> 2;
 #pragma unroll
     for (int j = 0; j < NINSTR; j++) {
-      const int r = (wave + 4 * j) * 8 + lrow;
+      const int r = (wave + NW * j) * 16 + lrow;
       const int64_t gr = rowmap(r);
       voff[j] = (gr < 0 || gr >= nrows - row0) ? 0x80000000u : (uint32_t)((gr * ld + chunk * 8) * 2);
     }
     const int row = wave_row0 + (lane & 31), h = lane >> 5;
 #pragma unroll
-    for (int kk = 0; kk < 4; kk++) fo[kk] = (uint32_t)(row * 128 + ((((2 * kk + h) ^ (row >> 1)) & 7) << 4));
+    for (int kk = 0; kk < KSTEPS; kk++) fo[kk] = (uint32_t)(row * 64 + ((((2 * kk + h) ^ (row >> 2)) & 3) << 4));
   }
-  // j-th DMA instruction of this wave for k-tile kt; tile = LDS byte address of the operand's stage
-  __device__ __forceinline__ void issue(int kt, uint32_t tile, int wave, int j) const {
-    const bool dead = kt * BK + chunk * 8 >= K;  // only ever true in a ragged last k-tile (or past the end)
-    dma16(rsrc, tile + (wave + 4 * j) * 1024, dead ? 0x80000000u : voff[j], (uint32_t)(kt * BK * 2));
+  // Per k-tile state of the DMA.  INSIDE: the caller knows the k-tile lies completely below K (no tail
+  // masking needed).
+  struct Prep {
+    uint32_t soff;
+    bool dead;
+  };
+  template <bool INSIDE>
+  __device__ __forceinline__ Prep prep(int kt) const {
+    return Prep{(uint32_t)(kt * BK * 2), !INSIDE && kt * BK + chunk * 8 >= K};  // ragged last k-tile / past the end
+  }
+  // j-th DMA instruction of this wave; tile = LDS byte address of the operand's stage
+  __device__ __forceinline__ void issue(const Prep& pp, uint32_t tile, int wave, int j) const {
+    dma16(rsrc, tile + (wave + NW * j) * 1024, pp.dead ? 0x80000000u : voff[j], pp.soff);
   }
   __device__ __forceinline__ bf16x8_t frag(const char* tile, int kk, int blk) const {
-    return *reinterpret_cast<const bf16x8_t*>(tile + fo[kk] + blk * 4096);
+    return *reinterpret_cast<const bf16x8_t*>(tile + fo[kk] + blk * (32 * BK * 2));
   }
 };
 
-template <int ROWS>
+template <int ROWS, int NW>
 struct ColOperand {
   static_assert(ROWS == 256, "transposed operands are built for 256-wide tiles");
-  static constexpr int BYTES = 64 * ROWS * 2;
-  static constexpr int NINSTR = BYTES / 1024 / 4;
+  static constexpr int BYTES = BK * ROWS * 2;
+  static constexpr int NINSTR = BYTES / 1024 / NW;
   static constexpr int NREADS = 2;
   const char* base;    // &mem[0][row0]
   int64_t total;       // bytes from base to the end of the matrix
-  int64_t ktile_bytes; // 64 * ld * 2
+  int64_t ktile_bytes; // BK * ld * 2
   uint32_t voff[NINSTR];
   uint32_t lane_base;
   uint32_t moff[4];
@@ -213,27 +236,37 @@ struct ColOperand {
     base = reinterpret_cast<const char*>(mem + row0);
     total = ((int64_t)K_ * ld - row0) * 2;
     ktile_bytes = (int64_t)BK * ld * 2;
-    // DMA: instruction q = wave + 4j covers k-rows 2q, 2q+1 (512 bytes each); lane l -> k-row 2q + l/32,
+    // DMA: instruction q = wave + NW*j covers k-rows 2q, 2q+1 (512 bytes each); lane l -> k-row 2q + l/32,
     // LDS position l%32, which holds chunk position ^ ((k & 3) << 2)
     const int ksub = lane >> 5;
     const int c = (lane & 31) ^ (((2 * wave + ksub) & 3) << 2);
 #pragma unroll
     for (int j = 0; j < NINSTR; j++) {
-      const int krow = 2 * (wave + 4 * j) + ksub;
+      const int krow = 2 * (wave + NW * j) + ksub;
       voff[j] = (uint32_t)(((int64_t)krow * ld + c * 8) * 2);
     }
-    // fragment reads
+    // fragment reads: lane (group G = l/16, i = l%16) addresses k-row 8*(G/2) + i/4 (+16kk, +4 for the
+    // second read) and rows 16*(G%2) + 4*(i%4) .. +3 of the block; the chunk swizzle is applied per block
     const int G = lane >> 4, i = lane & 15, kq = i >> 2;
-    const int cw = wave_row0 >> 3;  // first chunk of the wave's rows (a multiple of 16)
-    lane_base = (uint32_t)((8 * (G >> 1) + kq) * (ROWS * 2) + (cw + 2 * (G & 1) + ((i & 3) >> 1)) * 16 + 8 * (i & 1));
+    const int cw = wave_row0 >> 3;  // first chunk of the wave's rows
+    lane_base = (uint32_t)((8 * (G >> 1) + kq) * (ROWS * 2) + 8 * (i & 1));
 #pragma unroll
-    for (int blk = 0; blk < 4; blk++) moff[blk] = (uint32_t)(64 * (blk ^ kq));
+    for (int blk = 0; blk < 4; blk++) {
+      const int c2 = cw + 4 * blk + 2 * (G & 1) + ((i & 3) >> 1);
+      moff[blk] = (uint32_t)((c2 ^ (kq << 2)) * 16);
+    }
   }
-  __device__ __forceinline__ void issue(int kt, uint32_t tile, int wave, int j) const {
+  struct Prep {
+    rsrc_t r;
+  };
+  template <bool INSIDE>
+  __device__ __forceinline__ Prep prep(int kt) const {
     // the whole address, k-tile advance included, goes through the range check: k-rows past K and the
     // tail of the last row read as zero
-    const rsrc_t r = make_rsrc(base + kt * ktile_bytes, total - kt * ktile_bytes);
-    dma16(r, tile + (wave + 4 * j) * 1024, voff[j], 0);
+    return Prep{make_rsrc(base + kt * ktile_bytes, total - kt * ktile_bytes)};
+  }
+  __device__ __forceinline__ void issue(const Prep& pp, uint32_t tile, int wave, int j) const {
+    dma16(pp.r, tile + (wave + NW * j) * 1024, voff[j], 0);
   }
   __device__ __forceinline__ bf16x8_t frag(const char* tile, int kk, int blk) const {
     const char* a = tile + lane_base + moff[blk] + kk * (16 * ROWS * 2);
@@ -245,23 +278,27 @@ struct ColOperand {
   }
 };
 
-template <int LAY, int ROWS> struct OperandOf { using type = RowOperand<ROWS>; };
-template <int ROWS> struct OperandOf<LAY_COL, ROWS> { using type = ColOperand<ROWS>; };
+template <int LAY, int ROWS, int NW> struct OperandOf { using type = RowOperand<ROWS, NW>; };
+template <int ROWS, int NW> struct OperandOf<LAY_COL, ROWS, NW> { using type = ColOperand<ROWS, NW>; };
 
-// The body lives in a __device__ function: it uses device-only types (__amdgpu_buffer_rsrc_t) that the
-// host pass over a __global__ function cannot digest.
-template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT>
+// The body lives in a __device__ function: it uses inline assembly operands that the host pass over a
+// __global__ function would trip on.
+template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT, int NW>
 __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   static_assert(EPI != MTP_EPI_SWIGLU || BLAY == LAY_ROW, "the SwiGLU row interleave is a forward (row B) feature");
-  constexpr int TI = BM / 64, TJ = BN / 64;  // 32x32 blocks per wave in m and n
-  using AOp = typename OperandOf<ALAY, BM>::type;
-  using BOp = typename OperandOf<BLAY, BN>::type;
+  static_assert(NW == 4 || NW == 8, "4 waves (2x2) or 8 waves (2x4) per workgroup");
+  constexpr int WGM = 2, WGN = NW / 2;                         // wave grid over the tile
+  constexpr int TI = BM / (32 * WGM), TJ = BN / (32 * WGN);    // 32x32 blocks per wave in m and n
+  static_assert(EPI != MTP_EPI_SWIGLU || TJ % 2 == 0, "SwiGLU pairs gate and up blocks inside a wave");
+  using AOp = typename OperandOf<ALAY, BM, NW>::type;
+  using BOp = typename OperandOf<BLAY, BN, NW>::type;
   constexpr int STAGE_BYTES = AOp::BYTES + BOp::BYTES;
-  __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE_BYTES];
+  static_assert(NSTAGE * STAGE_BYTES <= 128 * 1024, "LDS ring too large");
+  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE_BYTES];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   const int lh = lane >> 5, l32 = lane & 31;
 
   const int tiles_m = (p.M + BM - 1) / BM;
@@ -272,40 +309,55 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM;
   const int n0 = tn * BN_SPAN;
+  // load origins (debug 1: all tiles load tile (0,0); debug 8: two A tiles, one B tile: a cache-resident set)
+  const int lm0 = (p.debug & 1) ? 0 : (p.debug & 8) ? (tm & 1) * BM : m0;
+  const int ln0 = (p.debug & 9) ? 0 : n0;
 
   AOp opA;
   BOp opB;
   if constexpr (ALAY == LAY_ROW)
-    opA.init(p.A, p.lda, m0, p.M, p.K, lane, wave, wm * (BM / 2), [](int r) -> int64_t { return r; });
+    opA.init(p.A, p.lda, lm0, p.M, p.K, lane, wave, wm * (BM / WGM), [](int r) -> int64_t { return r; });
   else
-    opA.init(p.A, p.lda, m0, p.K, lane, wave, wm * (BM / 2));
+    opA.init(p.A, p.lda, lm0, p.K, lane, wave, wm * (BM / WGM));
   if constexpr (BLAY == LAY_ROW) {
     // LDS row r of the B tile maps to a global row of [N,K].  Plain: n0 + r.  SwiGLU: the wave-column wn
-    // owns LDS rows [wn*BN/2, (wn+1)*BN/2): first half gate rows, second half the matching up rows.
-    opB.init(p.B, p.ldb, n0, p.N, p.K, lane, wave, wn * (BN / 2), [&](int r) -> int64_t {
+    // owns LDS rows [wn*BN/WGN, (wn+1)*BN/WGN): first half gate rows, second half the matching up rows.
+    opB.init(p.B, p.ldb, ln0, p.N, p.K, lane, wave, wn * (BN / WGN), [&](int r) -> int64_t {
       if (EPI == MTP_EPI_SWIGLU) {
-        const int seg = r / (BN / 4), in = r % (BN / 4);
-        const int64_t gr = ((seg & 1) ? p.half : 0) + (seg >> 1) * (BN / 4) + in;
+        constexpr int SEG = BN / (2 * WGN);
+        const int seg = r / SEG, in = r % SEG;
+        const int64_t gr = ((seg & 1) ? p.half : 0) + (seg >> 1) * SEG + in;
         // gate rows at or past `half` belong to the up matrix: no such row
-        return (!(seg & 1) && n0 + gr >= p.half) ? -1 : gr;
+        return (!(seg & 1) && ln0 + gr >= p.half) ? -1 : gr;
       }
       return r;
     });
   } else {
-    opB.init(p.B, p.ldb, n0, p.K, lane, wave, wn * (BN / 2));
+    opB.init(p.B, p.ldb, ln0, p.K, lane, wave, wn * (BN / WGN));
   }
+  if (p.debug & 4) {  // measurement: every DMA reads out of range (zero fill, no memory traffic)
+#pragma unroll
+    for (int j = 0; j < AOp::NINSTR; j++) opA.voff[j] = 0x80000000u;
+#pragma unroll
+    for (int j = 0; j < BOp::NINSTR; j++) opB.voff[j] = 0x80000000u;
+  }
+
   constexpr int NDMA = AOp::NINSTR + BOp::NINSTR;  // DMA instructions per wave per k-tile
   const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr_of(lds));
-  auto issue_one = [&](int kt, int buf, int d) {  // d-th DMA instruction of the k-tile
-    const uint32_t la = lds0 + buf * STAGE_BYTES;
-    if (d < AOp::NINSTR)
-      opA.issue(kt, la, wave, d);
+  // d-th DMA instruction of a k-tile whose per-tile state (pa, pb) has been prepared; A and B alternate
+  auto issue_one = [&](const typename AOp::Prep& pa, const typename BOp::Prep& pb, int stage, int d) {
+    const uint32_t la = lds0 + stage * STAGE_BYTES;
+    static_assert(AOp::NINSTR == BOp::NINSTR, "the DMA order alternates A and B");
+    if ((d & 1) == 0)
+      opA.issue(pa, la, wave, d >> 1);
     else
-      opB.issue(kt, la + AOp::BYTES, wave, d - AOp::NINSTR);
+      opB.issue(pb, la + AOp::BYTES, wave, d >> 1);
   };
-  auto issue_loads = [&](int kt, int buf) {
+  auto issue_loads = [&](int kt) {  // all of k-tile kt, tail masking on
+    const auto pa = opA.template prep<false>(kt);
+    const auto pb = opB.template prep<false>(kt);
 #pragma unroll
-    for (int d = 0; d < NDMA; d++) issue_one(kt, buf, d);
+    for (int d = 0; d < NDMA; d++) issue_one(pa, pb, kt % NSTAGE, d);
   };
 
   f32x16_t acc[TI][TJ];
@@ -317,19 +369,15 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
   // ---- main loop ---------------------------------------------------------------
-  // Two LDS stages.  Tile kt+1 is requested as soon as the barrier at the end of tile kt-1 has freed its
-  // stage, i.e. a full k-tile (64 MFMAs per wave) ahead of its first use.  Fragments are double buffered
-  // in registers: the ds_reads of k16-step s+1 are in flight while the MFMAs of step s issue.
   const int KT = (p.K + BK - 1) / BK;
   bf16x8_t af[2][TI], bfr[2][TJ];
   // Fragments are read in the order A0 B0 A1 B1 ... and the MFMAs walk the block grid in growing squares
   // ((0,0); (1,0) (1,1) (0,1); ...), so the first MFMAs of a step depend only on the oldest reads.
-  constexpr int TMAX = TI > TJ ? TI : TJ;
   constexpr int NFR = TI + TJ;   // fragments per k16 step
   constexpr int NMF = TI * TJ;   // MFMAs per k16 step
-  auto read_one = [&](int buf, int kk, int slot, auto u_tag) {  // u-th fragment in A0 B0 A1 B1 ... order
+  auto read_one = [&](int stage, int kk, int slot, auto u_tag) {  // u-th fragment in A0 B0 A1 B1 ... order
     constexpr int u = decltype(u_tag)::value;
-    const char* la = lds + buf * STAGE_BYTES;
+    const char* la = lds + stage * STAGE_BYTES;
     // with TI == TJ the order alternates; otherwise the longer side's leftovers come last
     constexpr int d = u < 2 * (TI < TJ ? TI : TJ) ? u / 2 : u - (TI < TJ ? TI : TJ);
     constexpr bool is_a = u < 2 * (TI < TJ ? TI : TJ) ? (u % 2 == 0) : (TI > TJ);
@@ -338,8 +386,8 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
     else
       bfr[slot][d] = opB.frag(la + AOp::BYTES, kk, d);
   };
-  auto read_frags = [&](int buf, int kk, int slot) {
-    static_for<NFR>([&](auto u) { read_one(buf, kk, slot, u); });
+  auto read_frags = [&](int stage, int kk, int slot) {
+    static_for<NFR>([&](auto u) { read_one(stage, kk, slot, u); });
   };
   auto mfma_one = [&](int slot, auto t_tag) {  // t-th MFMA of a step in shell order
     constexpr int t = decltype(t_tag)::value;
@@ -350,77 +398,114 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
     static_for<NMF>([&](auto t) { mfma_one(slot, t); });
   };
 
-  // One k-tile.  FULL: tiles kt+1 and kt+2 exist, so the prefetches are unconditional and the body is a
-  // single basic block whose instruction order is pinned:
-  //   steps 0-2 : sched_group_barrier sequence, per LDS read its share of the step's MFMAs
-  //   step 3    : written out by hand (MFMA, DMA, fragment read of the next tile, ...) with scheduling
-  //               barriers in between, because the DMA is inline assembly the group barriers cannot see
+  // One k-tile = KSTEPS k16 steps.  Step s multiplies the fragments in register slot s%2 while the
+  // fragments of the following step (the first step of tile kt+1 for the last one) are read into the
+  // other slot, and while the DMA instructions of tile kt+NSTAGE-1 — whose stage was released by the
+  // barrier that ended tile kt-1 — are issued one every few MFMAs.
+  //
+  // In the last step the first PRE MFMAs are issued before the barrier: they use the step's oldest
+  // fragments and give its youngest LDS reads time to land, so the lgkmcnt(0) the barrier needs is free.
+  // The s_waitcnt vmcnt in front of the barrier only asks for tile kt+1; the tiles requested after it
+  // may still be in flight.
+  //
+  // FULL: tiles up to kt+NSTAGE-1 lie completely below K.  The instruction order of the whole tile is
+  // pinned with scheduling barriers (the DMA is inline assembly, which sched_group_barrier cannot place).
+  constexpr int TILE_MF = KSTEPS * NMF;       // MFMAs per k-tile
+  constexpr int PRE = NMF * 3 / 8, REST = NMF - PRE;
+  // MFMA index (0 .. TILE_MF-1) after which the d-th DMA instruction is issued
+  auto dma_slot = [](int d) constexpr { return d * TILE_MF / NDMA + 1; };
   auto ktile = [&](int kt, auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
-    constexpr int NDS = TI * AOp::NREADS + TJ * BOp::NREADS;           // LDS reads per k16 step
-    const int buf = kt & 1;
-    read_frags(buf, 1, 1);
-    mfmas(0);
-    read_frags(buf, 2, 0);
-    mfmas(1);
-    read_frags(buf, 3, 1);
-    mfmas(0);
+    const int stage = kt % NSTAGE, nxt = (kt + 1) % NSTAGE;
     if constexpr (FULL) {
-      static_for<3 * NDS>([&](auto t) {
-        // spread NMF MFMAs over NDS reads: read u gets floor((u+1)*NMF/NDS) - floor(u*NMF/NDS) of them
-        constexpr int u = decltype(t)::value % NDS;
-        sched_group<SG_MFMA, (u + 1) * NMF / NDS - u * NMF / NDS>();
-        sched_group<SG_DS_RD, 1>();
-      });
-    }
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): tile kt+1 has landed in the other stage
-    __syncthreads();                     // ... for every wave, and everyone is done reading this stage
-    if constexpr (FULL) {
+      const auto pa = opA.template prep<true>(kt + NSTAGE - 1);
+      const auto pb = opB.template prep<true>(kt + NSTAGE - 1);
+      const int dst = (kt + NSTAGE - 1) % NSTAGE;
+      constexpr int dma_before_barrier = [&]() constexpr {
+        int n = 0;
+        for (int d = 0; d < NDMA; d++) n += (d * TILE_MF / NDMA + 1) < (KSTEPS - 1) * NMF + PRE ? 1 : 0;
+        return n;
+      }();
       __builtin_amdgcn_sched_barrier(0);
-      static_for<NMF>([&](auto t_tag) {
-        constexpr int t = decltype(t_tag)::value;
-        mfma_one(1, t_tag);
-        // DMA instructions and next-tile fragment reads spread evenly over the step's MFMAs
-        static_for<(t + 1) * NDMA / NMF - t * NDMA / NMF>([&](auto e) {
-          issue_one(kt + 2, buf, t * NDMA / NMF + decltype(e)::value);
+      static_for<KSTEPS>([&](auto s_tag) {
+        constexpr int s = decltype(s_tag)::value;
+        constexpr bool last = s == KSTEPS - 1;
+        static_for<NMF>([&](auto t_tag) {
+          constexpr int t = decltype(t_tag)::value;
+          constexpr int g = s * NMF + t;  // MFMA index inside the tile
+          if constexpr (last && t == PRE) {
+            // tile kt+1 has landed (later tiles may still be in flight) ...
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3) * NDMA + dma_before_barrier));
+            __syncthreads();  // ... for every wave, and everyone is done reading this stage
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          mfma_one(s & 1, t_tag);
+          static_for<NDMA>([&](auto d_tag) {
+            constexpr int d = decltype(d_tag)::value;
+            if constexpr (d * TILE_MF / NDMA + 1 == g + 1) issue_one(pa, pb, dst, d);
+          });
+          if constexpr (!last) {
+            // fragments of step s+1, spread over this step's MFMAs
+            static_for<(t + 1) * NFR / NMF - t * NFR / NMF>([&](auto e) {
+              read_one(stage, s + 1, (s + 1) & 1, std::integral_constant<int, t * NFR / NMF + decltype(e)::value>{});
+            });
+          } else if constexpr (t >= PRE) {
+            // fragments of the first step of tile kt+1, spread over the MFMAs after the barrier
+            constexpr int r = t - PRE;
+            static_for<(r + 1) * NFR / REST - r * NFR / REST>([&](auto e) {
+              read_one(nxt, 0, (s + 1) & 1, std::integral_constant<int, r * NFR / REST + decltype(e)::value>{});
+            });
+          }
+          __builtin_amdgcn_sched_barrier(0);
         });
-        static_for<(t + 1) * NFR / NMF - t * NFR / NMF>([&](auto e) {
-          read_one(buf ^ 1, 0, 0, std::integral_constant<int, t * NFR / NMF + decltype(e)::value>{});
-        });
-        __builtin_amdgcn_sched_barrier(0);
       });
     } else {
-      if (kt + 2 < KT) issue_loads(kt + 2, buf);
-      if (kt + 1 < KT) read_frags(buf ^ 1, 0, 0);
-      mfmas(1);
+      if (kt + NSTAGE - 1 < KT) issue_loads(kt + NSTAGE - 1);
+      static_for<KSTEPS - 1>([&](auto s_tag) {
+        constexpr int s = decltype(s_tag)::value;
+        read_frags(stage, s + 1, (s + 1) & 1);
+        mfmas(s & 1);
+      });
+      // wait for everything but (at most) the tile just requested
+      if (kt + NSTAGE - 1 < KT)
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(NSTAGE >= 3 ? NDMA : 0));
+      else
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+      __syncthreads();
+      if (kt + 1 < KT) read_frags(nxt, 0, KSTEPS & 1);
+      mfmas((KSTEPS - 1) & 1);
     }
   };
+  static_assert(KSTEPS % 2 == 0, "slot parity assumes an even number of k16 steps per tile");
 
-  issue_loads(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+#pragma unroll
+  for (int t = 0; t < NSTAGE - 1; t++)
+    if (t < KT) issue_loads(t);
+  __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
   __syncthreads();
-  if (KT > 1) issue_loads(1, 1);
   read_frags(0, 0, 0);
   int kt = 0;
-  for (; kt + 2 < KT; kt++) ktile(kt, std::true_type{});
+  const int KT_inside = p.K / BK;  // k-tiles that lie completely below K
+  for (; kt + NSTAGE - 1 < KT_inside; kt++) ktile(kt, std::true_type{});
   for (; kt < KT; kt++) ktile(kt, std::false_type{});
-  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
   __syncthreads();  // the epilogue reuses the tile buffers
+  if (p.debug & 2) return;
 
   // ---- epilogue ----------------------------------------------------------------
   // acc[i][j][r]: row m = m0 + wm*BM/2 + 32i + l32, column block j, n_local = 8*(r/4) + 4*lh + r%4.
   // Stage 32 rows x (BN/2) columns per wave through LDS, then 16-byte row-contiguous stores.
-  constexpr int WN = BN / 2;                       // columns per wave
+  constexpr int WN = BN / WGN;                     // columns per wave
   constexpr int ESZ = (OUT == OUT_F32) ? 4 : 2;
   constexpr int PITCH = WN * ESZ + 16;             // bytes per staged row (+16: spread rows over banks)
-  static_assert(4 * 32 * PITCH <= 2 * STAGE_BYTES, "epilogue staging exceeds the tile buffers");
+  static_assert(NW * 32 * PITCH <= NSTAGE * STAGE_BYTES, "epilogue staging exceeds the tile buffers");
   char* stage = lds + wave * (32 * PITCH);
 
   // global column of the first element of block j for this wave (main output C)
   auto col_of_block = [&](int j) -> int {
     if (EPI == MTP_EPI_SWIGLU) {
       const int hj = TJ / 2;
-      return (j < hj ? 0 : p.half) + n0 + wn * (BN / 4) + (j % hj) * 32;
+      return (j < hj ? 0 : p.half) + n0 + wn * (WN / 2) + (j % hj) * 32;
     }
     return n0 + wn * WN + j * 32;
   };
@@ -431,13 +516,54 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
     return p.N;
   };
 
-  auto flush = [&](int i, void* out, int64_t ld, int nblk, auto colfn, auto limfn, bool f32out, bool accumulate) {
+  // The whole tile lies inside the matrix: the epilogue needs no bounds checks.
+  const bool tile_inside = m0 + BM <= p.M && (EPI == MTP_EPI_SWIGLU ? n0 + BN / 2 <= p.half : n0 + BN <= p.N);
+
+  auto flush = [&](int i, void* out, int64_t ld, auto nblk_tag, auto colfn, auto limfn, auto f32_tag, bool accumulate) {
+    constexpr int nblk = decltype(nblk_tag)::value;
+    constexpr bool f32out = decltype(f32_tag)::value;
+    {
+      // Fast path: 16-byte aligned rows of a tile that is completely inside: lane l owns chunk l % CPR of
+      // rows l / CPR, l / CPR + 64 / CPR, ...; one address computation, then constant strides.
+      constexpr int esz_c = f32out ? 4 : 2;
+      constexpr int CPR = nblk * 32 * esz_c / 16, RPI = 64 / CPR, ITERS = 32 / RPI;
+      const int r0 = lane / CPR, cc = lane % CPR;
+      const int e0 = cc * (16 / esz_c);
+      const int col = colfn(e0 >> 5) + (e0 & 31);
+      char* gp = (char*)out + ((int64_t)(m0 + wm * (BM / WGM) + 32 * i + r0) * ld + col) * esz_c;
+      const bool aligned = ((reinterpret_cast<uintptr_t>(out) | (uintptr_t)(ld * esz_c)) & 15) == 0;
+      if (tile_inside && aligned) {
+        const char* sp = stage + r0 * PITCH + cc * 16;
+        const int64_t gstride = (int64_t)RPI * ld * esz_c;
+#pragma unroll
+        for (int it = 0; it < ITERS; it++) {
+          u32x4_t v = *reinterpret_cast<const u32x4_t*>(sp + it * RPI * PITCH);
+          u32x4_t* q = reinterpret_cast<u32x4_t*>(gp + it * gstride);
+          if (accumulate) {
+            const u32x4_t o = *q;
+            if (f32out) {
+              v.x = __float_as_uint(__uint_as_float(v.x) + __uint_as_float(o.x));
+              v.y = __float_as_uint(__uint_as_float(v.y) + __uint_as_float(o.y));
+              v.z = __float_as_uint(__uint_as_float(v.z) + __uint_as_float(o.z));
+              v.w = __float_as_uint(__uint_as_float(v.w) + __uint_as_float(o.w));
+            } else {
+              v.x = pack_bf16x2(bf16_lo(v.x) + bf16_lo(o.x), bf16_hi(v.x) + bf16_hi(o.x));
+              v.y = pack_bf16x2(bf16_lo(v.y) + bf16_lo(o.y), bf16_hi(v.y) + bf16_hi(o.y));
+              v.z = pack_bf16x2(bf16_lo(v.z) + bf16_lo(o.z), bf16_hi(v.z) + bf16_hi(o.z));
+              v.w = pack_bf16x2(bf16_lo(v.w) + bf16_lo(o.w), bf16_hi(v.w) + bf16_hi(o.w));
+            }
+          }
+          __builtin_nontemporal_store(v, q);  // written once, read by a later kernel: keep it out of the way of A/B in L2
+        }
+        return;
+      }
+    }
     // 16-byte chunks of the staged 32 x (nblk*32) block
     const int esz = f32out ? 4 : 2;
     const int chunks_per_row = nblk * 32 * esz / 16;
     const int epc = 16 / esz;  // elements per chunk
     const int total = 32 * chunks_per_row;
-    const int mrow0 = m0 + wm * (BM / 2) + 32 * i;
+    const int mrow0 = m0 + wm * (BM / WGM) + 32 * i;
     for (int c = lane; c < total; c += 64) {
       const int r = c / chunks_per_row, cc = c - r * chunks_per_row;
       const int e0 = cc * epc;           // element offset inside the staged row
@@ -517,26 +643,37 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
             *reinterpret_cast<f32x4_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 4) = v;
           }
         wave_lds_sync();
-        flush(i, p.C, p.ldc, TJ, col_of_block, lim_of_block, true, p.accumulate != 0);
+        flush(i, p.C, p.ldc, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::true_type{}, p.accumulate != 0);
         wave_lds_sync();
       }
     } else {
-      // round to bf16 once; the activation sees the rounded value, as the unfused layers would
+      // round to bf16 once (one v_cvt_pk_bf16_f32 per pair); an activation sees the rounded value, as
+      // the unfused layers would
+      uint32_t pk[TJ][8];
 #pragma unroll
       for (int j = 0; j < TJ; j++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) pre[j][r] = bf16_bits_to_f32(f32_to_bf16_bits(pre[j][r]));
+        for (int q = 0; q < 8; q++) pk[j][q] = pack_bf16x2(pre[j][2 * q], pre[j][2 * q + 1]);
       if (p.C) {
 #pragma unroll
         for (int j = 0; j < TJ; j++)
 #pragma unroll
           for (int g = 0; g < 4; g++) {
-            u32x2_t v = {pack_bf16x2(pre[j][4 * g], pre[j][4 * g + 1]), pack_bf16x2(pre[j][4 * g + 2], pre[j][4 * g + 3])};
+            u32x2_t v = {pk[j][2 * g], pk[j][2 * g + 1]};
             *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
           }
         wave_lds_sync();
-        flush(i, p.C, p.ldc, TJ, col_of_block, lim_of_block, false, p.accumulate != 0);
+        flush(i, p.C, p.ldc, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::false_type{}, p.accumulate != 0);
         wave_lds_sync();
+      }
+      if (EPI != MTP_EPI_NONE && EPI != MTP_EPI_BIAS) {
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+#pragma unroll
+          for (int q = 0; q < 8; q++) {
+            pre[j][2 * q] = bf16_lo(pk[j][q]);
+            pre[j][2 * q + 1] = bf16_hi(pk[j][q]);
+          }
       }
       if (EPI == MTP_EPI_BIAS_GELU || EPI == MTP_EPI_GELU) {
 #pragma unroll
@@ -548,7 +685,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
             *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
           }
         wave_lds_sync();
-        flush(i, p.C2, p.ldc2, TJ, col_of_block, lim_of_block, false, false);
+        flush(i, p.C2, p.ldc2, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::false_type{}, false);
         wave_lds_sync();
       }
       if (EPI == MTP_EPI_SWIGLU) {
@@ -564,28 +701,35 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
             *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
           }
         wave_lds_sync();
-        auto act_col = [&](int j) -> int { return n0 + wn * (BN / 4) + j * 32; };
+        auto act_col = [&](int j) -> int { return n0 + wn * (WN / 2) + j * 32; };
         auto act_lim = [&](int) -> int { return p.half; };
-        flush(i, p.C2, p.ldc2, HJ, act_col, act_lim, false, false);
+        flush(i, p.C2, p.ldc2, std::integral_constant<int, HJ>{}, act_col, act_lim, std::false_type{}, false);
         wave_lds_sync();
       }
     }
   }
 }
 
-template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT>
-__global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs p) {
-  gemm_bf16_body<BM, BN, ALAY, BLAY, EPI, OUT>(p);
+template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs p) {
+  gemm_bf16_body<BM, BN, ALAY, BLAY, EPI, OUT, NW>(p);
 }
 
 template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT>
-int launch(const GemmArgs& a, hipStream_t s) {
+int launch(GemmArgs a, hipStream_t s) {
+  if (const char* e = getenv("MTP_GEMM_DEBUG")) a.debug = atoi(e);
+  int nw = 4;
+  if (const char* e = getenv("MTP_GEMM_WAVES")) nw = atoi(e);
   const int tiles_m = (a.M + BM - 1) / BM;
   const int span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
   const int bn_span = (EPI == MTP_EPI_SWIGLU) ? BN / 2 : BN;
   const int tiles_n = (span + bn_span - 1) / bn_span;
-  hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256),
-                     0, s, a);
+  if (nw == 8)
+    hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, 8>), dim3((unsigned)(tiles_m * tiles_n)),
+                       dim3(512), 0, s, a);
+  else
+    hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, 4>), dim3((unsigned)(tiles_m * tiles_n)),
+                       dim3(256), 0, s, a);
   MTP_CHECK_LAUNCH("gemm_bf16");
   return MTP_OK;
 }

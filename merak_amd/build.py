@@ -27,7 +27,9 @@ SOURCES = [
     "embedding.hip",
     "gemv.hip",
     "elementwise.hip",
-    "gemm_bf16.hip",
+    "gemm_bf16_fwd.hip",
+    "gemm_bf16_dgrad.hip",
+    "gemm_bf16_wgrad.hip",
     "gemm_generic.hip",
     "linear.hip",
 ]

@@ -26,6 +26,7 @@
 //     and writes 16 bytes per lane, 256 contiguous bytes per row;
 //   * workgroup ids are remapped so that the 32 CUs of one XCD (which share an
 //     L2) walk neighbouring tiles.
+#pragma once
 #include "mtp_common.h"
 #include <stdlib.h>
 #include <type_traits>
@@ -168,10 +169,14 @@ constexpr BlockIJ shell_pair(int t, int TI, int TJ) {
 //   of 4 consecutive rows-elements of k-row (i/4) and receives, transposed, the
 //   4 consecutive k of row i — exactly the MFMA operand layout.
 // ---------------------------------------------------------------------------
+constexpr int LROWS = 256;  // rows of the LDS tile layout; narrower tiles (192, 128) use its first rows
+
 template <int ROWS, int NW>
 struct RowOperand {
-  static constexpr int BYTES = ROWS * BK * 2;
-  static constexpr int NINSTR = ROWS / 16 / NW;  // DMA instructions per wave per k-tile (16 rows each)
+  static_assert(ROWS <= LROWS && ROWS % 64 == 0, "tile rows: 64, 128, 192 or 256");
+  static constexpr int BYTES = LROWS * BK * 2;
+  // DMA instructions per wave per k-tile (16 rows each); instructions whose rows all lie past ROWS are skipped
+  static constexpr int NINSTR = (ROWS / 16 + NW - 1) / NW;
   static constexpr int NREADS = 1;               // LDS reads per fragment
   rsrc_t rsrc;
   uint32_t voff[NINSTR];
@@ -192,7 +197,7 @@ struct RowOperand {
 #pragma unroll
     for (int j = 0; j < NINSTR; j++) {
       const int r = (wave + NW * j) * 16 + lrow;
-      const int64_t gr = rowmap(r);
+      const int64_t gr = r < ROWS ? rowmap(r) : -1;
       voff[j] = (gr < 0 || gr >= nrows - row0) ? 0x80000000u : (uint32_t)((gr * ld + chunk * 8) * 2);
     }
     const int row = wave_row0 + (lane & 31), h = lane >> 5;
@@ -220,8 +225,8 @@ struct RowOperand {
 
 template <int ROWS, int NW>
 struct ColOperand {
-  static_assert(ROWS == 256, "transposed operands are built for 256-wide tiles");
-  static constexpr int BYTES = BK * ROWS * 2;
+  static_assert(ROWS <= LROWS && ROWS % 64 == 0, "tile rows: 64, 128, 192 or 256");
+  static constexpr int BYTES = BK * LROWS * 2;
   static constexpr int NINSTR = BYTES / 1024 / NW;
   static constexpr int NREADS = 2;
   const char* base;    // &mem[0][row0]
@@ -243,13 +248,14 @@ struct ColOperand {
 #pragma unroll
     for (int j = 0; j < NINSTR; j++) {
       const int krow = 2 * (wave + NW * j) + ksub;
-      voff[j] = (uint32_t)(((int64_t)krow * ld + c * 8) * 2);
+      // chunks past the tile's ROWS are not fetched (narrow tiles)
+      voff[j] = c * 8 < ROWS ? (uint32_t)(((int64_t)krow * ld + c * 8) * 2) : 0x80000000u;
     }
     // fragment reads: lane (group G = l/16, i = l%16) addresses k-row 8*(G/2) + i/4 (+16kk, +4 for the
     // second read) and rows 16*(G%2) + 4*(i%4) .. +3 of the block; the chunk swizzle is applied per block
     const int G = lane >> 4, i = lane & 15, kq = i >> 2;
     const int cw = wave_row0 >> 3;  // first chunk of the wave's rows
-    lane_base = (uint32_t)((8 * (G >> 1) + kq) * (ROWS * 2) + 8 * (i & 1));
+    lane_base = (uint32_t)((8 * (G >> 1) + kq) * (LROWS * 2) + 8 * (i & 1));
 #pragma unroll
     for (int blk = 0; blk < 4; blk++) {
       const int c2 = cw + 4 * blk + 2 * (G & 1) + ((i & 3) >> 1);
@@ -269,11 +275,11 @@ struct ColOperand {
     dma16(pp.r, tile + (wave + NW * j) * 1024, voff[j], 0);
   }
   __device__ __forceinline__ bf16x8_t frag(const char* tile, int kk, int blk) const {
-    const char* a = tile + lane_base + moff[blk] + kk * (16 * ROWS * 2);
+    const char* a = tile + lane_base + moff[blk] + kk * (16 * LROWS * 2);
     const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
         (bf16x4_t __attribute__((address_space(3)))*)(a));
     const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-        (bf16x4_t __attribute__((address_space(3)))*)(a + 4 * ROWS * 2));
+        (bf16x4_t __attribute__((address_space(3)))*)(a + 4 * LROWS * 2));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   }
 };
@@ -347,11 +353,18 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   // d-th DMA instruction of a k-tile whose per-tile state (pa, pb) has been prepared; A and B alternate
   auto issue_one = [&](const typename AOp::Prep& pa, const typename BOp::Prep& pb, int stage, int d) {
     const uint32_t la = lds0 + stage * STAGE_BYTES;
-    static_assert(AOp::NINSTR == BOp::NINSTR, "the DMA order alternates A and B");
-    if ((d & 1) == 0)
-      opA.issue(pa, la, wave, d >> 1);
-    else
-      opB.issue(pb, la + AOp::BYTES, wave, d >> 1);
+    // A and B alternate while both have instructions left
+    constexpr int NMIN = AOp::NINSTR < BOp::NINSTR ? AOp::NINSTR : BOp::NINSTR;
+    if (d < 2 * NMIN) {
+      if ((d & 1) == 0)
+        opA.issue(pa, la, wave, d >> 1);
+      else
+        opB.issue(pb, la + AOp::BYTES, wave, d >> 1);
+    } else if (AOp::NINSTR > BOp::NINSTR) {
+      opA.issue(pa, la, wave, d - NMIN);
+    } else {
+      opB.issue(pb, la + AOp::BYTES, wave, d - NMIN);
+    }
   };
   auto issue_loads = [&](int kt) {  // all of k-tile kt, tail masking on
     const auto pa = opA.template prep<false>(kt);
@@ -526,13 +539,16 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
       // Fast path: 16-byte aligned rows of a tile that is completely inside: lane l owns chunk l % CPR of
       // rows l / CPR, l / CPR + 64 / CPR, ...; one address computation, then constant strides.
       constexpr int esz_c = f32out ? 4 : 2;
-      constexpr int CPR = nblk * 32 * esz_c / 16, RPI = 64 / CPR, ITERS = 32 / RPI;
-      const int r0 = lane / CPR, cc = lane % CPR;
+      constexpr int CPR = nblk * 32 * esz_c / 16;                            // 16-byte chunks per staged row
+      constexpr int CPRP = CPR <= 4 ? 4 : CPR <= 8 ? 8 : CPR <= 16 ? 16 : 32;  // lanes per row (power of two)
+      constexpr int RPI = 64 / CPRP, ITERS = 32 / RPI;
+      const int r0 = lane / CPRP, cc = lane % CPRP;
       const int e0 = cc * (16 / esz_c);
       const int col = colfn(e0 >> 5) + (e0 & 31);
       char* gp = (char*)out + ((int64_t)(m0 + wm * (BM / WGM) + 32 * i + r0) * ld + col) * esz_c;
       const bool aligned = ((reinterpret_cast<uintptr_t>(out) | (uintptr_t)(ld * esz_c)) & 15) == 0;
       if (tile_inside && aligned) {
+        if (CPRP != CPR && cc >= CPR) return;
         const char* sp = stage + r0 * PITCH + cc * 16;
         const int64_t gstride = (int64_t)RPI * ld * esz_c;
 #pragma unroll
@@ -675,7 +691,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
             pre[j][2 * q + 1] = bf16_hi(pk[j][q]);
           }
       }
-      if (EPI == MTP_EPI_BIAS_GELU || EPI == MTP_EPI_GELU) {
+      if constexpr (EPI == MTP_EPI_BIAS_GELU || EPI == MTP_EPI_GELU) {
 #pragma unroll
         for (int j = 0; j < TJ; j++)
 #pragma unroll
@@ -688,7 +704,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
         flush(i, p.C2, p.ldc2, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::false_type{}, false);
         wave_lds_sync();
       }
-      if (EPI == MTP_EPI_SWIGLU) {
+      if constexpr (EPI == MTP_EPI_SWIGLU) {
         constexpr int HJ = TJ / 2;
 #pragma unroll
         for (int j = 0; j < HJ; j++)
@@ -715,86 +731,91 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs p) {
   gemm_bf16_body<BM, BN, ALAY, BLAY, EPI, OUT, NW>(p);
 }
 
-template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT>
-int launch(GemmArgs a, hipStream_t s) {
-  if (const char* e = getenv("MTP_GEMM_DEBUG")) a.debug = atoi(e);
-  int nw = 4;
-  if (const char* e = getenv("MTP_GEMM_WAVES")) nw = atoi(e);
-  const int tiles_m = (a.M + BM - 1) / BM;
-  const int span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
-  const int bn_span = (EPI == MTP_EPI_SWIGLU) ? BN / 2 : BN;
-  const int tiles_n = (span + bn_span - 1) / bn_span;
-  if (nw == 8)
-    hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, 8>), dim3((unsigned)(tiles_m * tiles_n)),
-                       dim3(512), 0, s, a);
-  else
-    hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, 4>), dim3((unsigned)(tiles_m * tiles_n)),
-                       dim3(256), 0, s, a);
-  MTP_CHECK_LAUNCH("gemm_bf16");
-  return MTP_OK;
+// ---------------------------------------------------------------------------
+// Tile configurations and their choice.
+//
+// All 256 CUs work on one tile each, so a launch takes ceil(tiles / 256) rounds of one tile time.  A
+// 256x256 tile has the best arithmetic intensity, but problems whose tile count is a little over a
+// multiple of 256 (or well below 256) finish sooner with a narrower tile.  pick_config() estimates
+// rounds x tile cost for each configuration that the kernel at hand was built with.
+// ---------------------------------------------------------------------------
+struct TileCfg {
+  int bm, bn, nw;
+  float eff;  // relative speed of one tile's inner loop per flop (256x256 = 1), from measurement
+};
+// 256x256 runs with 8 waves (2 per SIMD: one wave's barrier and LDS waits are covered by the other's
+// MFMAs, and the epilogue's VALU work is spread over twice the waves); the narrow tiles were measured
+// best as listed.
+constexpr TileCfg kCfgs[] = {
+    {256, 256, 8, 1.00f}, {256, 192, 4, 0.92f}, {192, 256, 4, 0.92f}, {256, 128, 4, 0.85f}, {128, 256, 8, 0.85f},
+};
+constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
+
+template <int EPI>
+constexpr bool cfg_valid(int c) {
+  const TileCfg t = kCfgs[c];
+  const int wgn = t.nw / 2;
+  if (t.bn % (32 * wgn) != 0) return false;
+  const int tj = t.bn / (32 * wgn);
+  if (EPI == MTP_EPI_SWIGLU && tj % 2 != 0) return false;
+  return true;
 }
 
-}  // namespace
-
-// Entry used by the C API layer (linear.hip).
-int mtp_gemm_bf16_nt(const void* A, const void* B, const void* bias, void* C, void* C2, int64_t M, int64_t N,
-                     int64_t K, int epilogue, hipStream_t s) {
-  GemmArgs a{};
-  a.A = (const uint16_t*)A;
-  a.B = (const uint16_t*)B;
-  a.bias = (const uint16_t*)bias;
-  a.C = C;
-  a.C2 = C2;
-  a.M = (int)M;
-  a.N = (int)N;
-  a.K = (int)K;
-  a.lda = K;
-  a.ldb = K;
-  a.ldc = N;
-  a.accumulate = 0;
-  a.half = (int)(N / 2);
-  a.ldc2 = (epilogue == MTP_EPI_SWIGLU) ? N / 2 : N;
-  switch (epilogue) {
-    case MTP_EPI_NONE: return launch<256, 256, LAY_ROW, LAY_ROW, MTP_EPI_NONE, OUT_BF16>(a, s);
-    case MTP_EPI_BIAS: return launch<256, 256, LAY_ROW, LAY_ROW, MTP_EPI_BIAS, OUT_BF16>(a, s);
-    case MTP_EPI_BIAS_GELU: return launch<256, 256, LAY_ROW, LAY_ROW, MTP_EPI_BIAS_GELU, OUT_BF16>(a, s);
-    case MTP_EPI_GELU: return launch<256, 256, LAY_ROW, LAY_ROW, MTP_EPI_GELU, OUT_BF16>(a, s);
-    case MTP_EPI_SWIGLU: return launch<256, 256, LAY_ROW, LAY_ROW, MTP_EPI_SWIGLU, OUT_BF16>(a, s);
+template <int EPI>
+int pick_config(const GemmArgs& a) {
+  if (const char* e = getenv("MTP_GEMM_CFG")) {
+    const int c = atoi(e);
+    if (c >= 0 && c < kNumCfgs) return c;
   }
-  mtp_set_error("gemm_bf16: unknown epilogue %d", epilogue);
+  const int64_t span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
+  int best = 0;
+  double best_t = 1e300;
+  for (int c = 0; c < kNumCfgs; c++) {
+    const TileCfg t = kCfgs[c];
+    const int bn_span = (EPI == MTP_EPI_SWIGLU) ? t.bn / 2 : t.bn;
+    const int64_t tiles = ((a.M + t.bm - 1) / t.bm) * ((span + bn_span - 1) / bn_span);
+    const int64_t rounds = (tiles + 255) / 256;
+    if (!cfg_valid<EPI>(c)) continue;
+    const double cost = (double)rounds * t.bm * t.bn / t.eff;
+    if (cost < best_t * 0.999) {
+      best_t = cost;
+      best = c;
+    }
+  }
+  return best;
+}
+
+template <int C, int ALAY, int BLAY, int EPI, int OUT>
+int launch_cfg(const GemmArgs& a, hipStream_t s) {
+  if constexpr (!cfg_valid<EPI>(C)) {
+    mtp_set_error("gemm_bf16: tile configuration %d cannot serve this epilogue", C);
+    return MTP_EINVAL;
+  } else {
+    constexpr int BM = kCfgs[C].bm, BN = kCfgs[C].bn, NW = kCfgs[C].nw;
+    const int tiles_m = (a.M + BM - 1) / BM;
+    const int span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
+    const int bn_span = (EPI == MTP_EPI_SWIGLU) ? BN / 2 : BN;
+    const int tiles_n = (span + bn_span - 1) / bn_span;
+    hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, NW>), dim3((unsigned)(tiles_m * tiles_n)),
+                       dim3(NW * 64), 0, s, a);
+    MTP_CHECK_LAUNCH("gemm_bf16");
+    return MTP_OK;
+  }
+}
+
+template <int ALAY, int BLAY, int EPI, int OUT>
+int launch(GemmArgs a, hipStream_t s) {
+  if (const char* e = getenv("MTP_GEMM_DEBUG")) a.debug = atoi(e);
+  int c = pick_config<EPI>(a);
+  if (!cfg_valid<EPI>(c)) c = 0;
+  switch (c) {
+    case 0: return launch_cfg<0, ALAY, BLAY, EPI, OUT>(a, s);
+    case 1: return launch_cfg<1, ALAY, BLAY, EPI, OUT>(a, s);
+    case 2: return launch_cfg<2, ALAY, BLAY, EPI, OUT>(a, s);
+    case 3: return launch_cfg<3, ALAY, BLAY, EPI, OUT>(a, s);
+    case 4: return launch_cfg<4, ALAY, BLAY, EPI, OUT>(a, s);
+  }
   return MTP_EINVAL;
 }
 
-// dX[M,K] = dY[M,N] W[N,K]: GEMM (M, K, reduce N) with A = dY (row) and B = W read as [reduce, cols] (col).
-int mtp_gemm_bf16_dgrad(const void* dy, const void* w, void* dx, int64_t M, int64_t N, int64_t K, hipStream_t s) {
-  GemmArgs a{};
-  a.A = (const uint16_t*)dy;
-  a.B = (const uint16_t*)w;
-  a.C = dx;
-  a.M = (int)M;
-  a.N = (int)K;
-  a.K = (int)N;
-  a.lda = N;
-  a.ldb = K;
-  a.ldc = K;
-  return launch<256, 256, LAY_ROW, LAY_COL, MTP_EPI_NONE, OUT_BF16>(a, s);
-}
-
-// dW[N,K] (+)= dY[M,N]^T X[M,K]: GEMM (N, K, reduce M) with both operands transposed (col).
-int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
-                        int dw_dtype, int accumulate, hipStream_t s) {
-  if (db) return MTP_EUNSUPPORTED;  // bias gradient: served by the general path for now
-  GemmArgs a{};
-  a.A = (const uint16_t*)dy;
-  a.B = (const uint16_t*)x;
-  a.C = dw;
-  a.M = (int)N;
-  a.N = (int)K;
-  a.K = (int)M;
-  a.lda = N;
-  a.ldb = K;
-  a.ldc = K;
-  a.accumulate = accumulate;
-  if (dw_dtype == MTP_F32) return launch<256, 256, LAY_COL, LAY_COL, MTP_EPI_NONE, OUT_F32>(a, s);
-  return launch<256, 256, LAY_COL, LAY_COL, MTP_EPI_NONE, OUT_BF16>(a, s);
-}
+}  // namespace

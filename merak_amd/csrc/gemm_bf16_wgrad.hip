@@ -1,0 +1,20 @@
+// dW[N,K] (+)= dY[M,N]^T X[M,K]: GEMM (N, K, reduce M) with both operands transposed (col).
+#include "gemm_bf16_kernel.h"
+
+int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
+                        int dw_dtype, int accumulate, hipStream_t s) {
+  if (db) return MTP_EUNSUPPORTED;  // bias gradient: served by the general path
+  GemmArgs a{};
+  a.A = (const uint16_t*)dy;
+  a.B = (const uint16_t*)x;
+  a.C = dw;
+  a.M = (int)N;
+  a.N = (int)K;
+  a.K = (int)M;
+  a.lda = N;
+  a.ldb = K;
+  a.ldc = K;
+  a.accumulate = accumulate;
+  if (dw_dtype == MTP_F32) return launch<LAY_COL, LAY_COL, MTP_EPI_NONE, OUT_F32>(a, s);
+  return launch<LAY_COL, LAY_COL, MTP_EPI_NONE, OUT_BF16>(a, s);
+}

@@ -11,9 +11,10 @@
 // X is tiny and stays in L2/L1.  The result tile D[i][b] needs no cross-lane
 // reduction.
 //
-// A workgroup of 8 waves owns 16*R weight rows; wave w owns the w-th eighth of
-// K (split-K inside the workgroup), the 8 partial tiles are summed through
-// LDS in a fixed order, so results are bit-reproducible run to run.
+// A workgroup of 8 waves owns 16*R weight rows; the 128-byte k-pairs of those
+// rows are dealt round-robin to the waves (split-K inside the workgroup), the 8
+// partial tiles are summed through LDS in a fixed order, so results are
+// bit-reproducible run to run.
 #include "mtp_common.h"
 #include <stdlib.h>
 
@@ -35,14 +36,22 @@ __device__ __forceinline__ bool arg_better(float va, int64_t ia, float vb, int64
   return va > vb || (va == vb && ia < ib);
 }
 
+// `ok` is a compile-time true on the unguarded path, which then has no branches at all
 __device__ __forceinline__ bf16x8_t load_frag(const uint16_t* p, bool ok) {
   u32x4_t v = {0u, 0u, 0u, 0u};
   if (ok) v = *reinterpret_cast<const u32x4_t*>(p);
   return __builtin_bit_cast(bf16x8_t, v);
 }
 
+// weights are read exactly once: streaming (non-temporal) loads keep them from displacing X in the caches
+__device__ __forceinline__ bf16x8_t load_frag_nt(const uint16_t* p, bool ok) {
+  u32x4_t v = {0u, 0u, 0u, 0u};
+  if (ok) v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+  return __builtin_bit_cast(bf16x8_t, v);
+}
+
 // MODE 0: store Y (+bias); MODE 1: SwiGLU store; MODE 2: argmax partials
-template <int R, int NB, int MODE>
+template <int R, int NB, int MODE, bool GUARD>
 __global__ __launch_bounds__(GV_THREADS) void gemv_kernel(const uint16_t* __restrict__ x,
                                                           const uint16_t* __restrict__ w,
                                                           const uint16_t* __restrict__ bias,
@@ -82,12 +91,16 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_kernel(const uint16_t* __rest
     xp[nb] = x + (int64_t)b * K + 8 * lg;
   }
 
-  // this wave's k-steps (32 elements each)
-  const int64_t steps = (K + 31) >> 5;
-  const int64_t per = (steps + GV_WAVES - 1) / GV_WAVES;
-  const int64_t s0 = wave * per;
-  int64_t s1 = s0 + per;
-  if (s1 > steps) s1 = steps;
+  // This wave's k range, in pairs of 32-element steps: a pair covers 64 elements = one 128-byte line of
+  // every weight row, and the two 64-byte halves of a line are requested by adjacent instructions, so the
+  // second request merges with the first one's miss instead of finding the line evicted again (with 16
+  // rows x 8 groups x 8 waves in flight the L1 holds nothing for long).
+  // Pairs are dealt round-robin to the 8 waves (wave w takes pairs w, w+8, ...): the waves advance in
+  // step, so at any moment the workgroup reads 1 KiB contiguous from each of its rows, which keeps
+  // DRAM pages open much longer than eight far-apart 128-byte streams per row would.
+  const int64_t pairs = (K + 63) >> 6;
+  const int64_t p0 = wave;
+  const int64_t p1 = pairs;
 
   f32x4_t acc[R][NB];
 #pragma unroll
@@ -95,34 +108,46 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_kernel(const uint16_t* __rest
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) acc[r][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  if (s0 < s1) {
-    bf16x8_t a_cur[R], b_cur[NB];
-    {
-      const int64_t k = s0 * 32;
-      const bool ok = k + 8 * lg < K;
-#pragma unroll
-      for (int r = 0; r < R; r++) a_cur[r] = load_frag(wp[r] + k, ok);
-#pragma unroll
-      for (int nb = 0; nb < NB; nb++) b_cur[nb] = load_frag(xp[nb] + k, ok);
-    }
-    for (int64_t s = s0; s < s1; s++) {
-      bf16x8_t a_nxt[R], b_nxt[NB];
-      const int64_t kn = (s + 1) * 32;
-      const bool okn = (s + 1 < s1) && (kn + 8 * lg < K);
-#pragma unroll
-      for (int r = 0; r < R; r++) a_nxt[r] = load_frag(wp[r] + kn, okn);
-#pragma unroll
-      for (int nb = 0; nb < NB; nb++) b_nxt[nb] = load_frag(xp[nb] + kn, okn);
+  if (p0 < p1) {
+    bf16x8_t a_cur[R][2], b_cur[NB][2];
+    // GUARD: K is not a multiple of 64, the last pair is partly (or half) past the end of the rows
+    auto load_pair = [&](int64_t pr, bf16x8_t (&a)[R][2], bf16x8_t (&b)[NB][2]) {
+      const int64_t k = pr * 64;
 #pragma unroll
       for (int r = 0; r < R; r++)
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-          acc[r][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[r], b_cur[nb], acc[r][nb], 0, 0, 0);
+        for (int hf = 0; hf < 2; hf++) a[r][hf] = load_frag_nt(wp[r] + k + 32 * hf, !GUARD || (k + 32 * hf + 8 * lg < K));
 #pragma unroll
-      for (int r = 0; r < R; r++) a_cur[r] = a_nxt[r];
+      for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++) b_cur[nb] = b_nxt[nb];
+        for (int hf = 0; hf < 2; hf++) b[nb][hf] = load_frag(xp[nb] + k + 32 * hf, !GUARD || (k + 32 * hf + 8 * lg < K));
+    };
+    auto multiply = [&]() {
+#pragma unroll
+      for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+          for (int nb = 0; nb < NB; nb++)
+            acc[r][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[r][hf], b_cur[nb][hf], acc[r][nb], 0, 0, 0);
+    };
+    load_pair(p0, a_cur, b_cur);
+    // all but the last pair: fetch the next pair (unconditionally: it exists), multiply the current one
+    int64_t pr = p0;
+    for (; pr + GV_WAVES < p1; pr += GV_WAVES) {
+      bf16x8_t a_nxt[R][2], b_nxt[NB][2];
+      load_pair(pr + GV_WAVES, a_nxt, b_nxt);
+      multiply();
+#pragma unroll
+      for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) a_cur[r][hf] = a_nxt[r][hf];
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) b_cur[nb][hf] = b_nxt[nb][hf];
     }
+    multiply();
   }
 
   // ---- sum the 8 k-slices through LDS, one row group at a time -------------
@@ -302,10 +327,11 @@ int pick_rows_per_wg(int64_t B, int64_t N, int64_t K, int mode) {
   // Aim for at least ~2 workgroups per CU (256 CUs); more rows per workgroup
   // means fewer re-reads of X from L2.
   const int64_t groups = (N + 15) / 16;
-  int r = 8;
+  // Measured on the 128256 x 4096 LM head: 4 groups for B <= 16 (2 workgroups per CU), 8 for larger
+  // batches (fewer re-reads of X); small matrices want at least ~2 workgroups per CU.
+  int r = B > 16 ? 8 : 4;
   while (r > 1 && groups / r < 512) r >>= 1;
   if (mode == 1 && r < 2) r = 2;
-  (void)B;
   (void)K;
   return r;
 }
@@ -318,9 +344,17 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   const unsigned n_wg = (unsigned)((span + rows_per_wg - 1) / rows_per_wg);
   if (n_wg_out) *n_wg_out = n_wg;
   const int NB = B > 16 ? 2 : 1;
-#define GV_LAUNCH(RR, NNB)                                                                                     \
-  hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE>), dim3(n_wg), dim3(GV_THREADS), 0, s, (const uint16_t*)x,      \
-                     (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part, (int)B, N, K)
+#define GV_LAUNCH(RR, NNB)                                                                                      \
+  do {                                                                                                          \
+    if (K % 64 == 0)                                                                                            \
+      hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, false>), dim3(n_wg), dim3(GV_THREADS), 0, s,               \
+                         (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part,     \
+                         (int)B, N, K);                                                                         \
+    else                                                                                                        \
+      hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, true>), dim3(n_wg), dim3(GV_THREADS), 0, s,                \
+                         (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part,     \
+                         (int)B, N, K);                                                                         \
+  } while (0)
   if (NB == 1) {
     if (R == 8) GV_LAUNCH(8, 1);
     else if (R == 4) GV_LAUNCH(4, 1);

@@ -39,6 +39,10 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3     # MI355X fp32 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# HBM bytes per launch of the gate/up GEMMs, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file
+# scaled by a 1 GiB copy kernel (x2.000 / x1.000): profiles/hbm_traffic_fetch_write_size.txt
+HBM_TRAFFIC_BYTES = {"gate_up.fwd": 1.860e9, "gate_up.wgrad": 1.644e9, "gate_up.dgrad": 0.889e9}
+
 LLAMA8B = [  # (name, K, N, epilogue)
     ("qkv", 4096, 6144, "none"),
     ("gate_up", 4096, 2 * 14336, "swiglu"),
@@ -317,7 +321,8 @@ def main():
     gemms = [k for k in kernels if "tflops" in k]
     dom = max(gemms, key=lambda k: k["ms"])
     roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "unit": "TFLOP/s", "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4),
+                "traffic": HBM_TRAFFIC_BYTES.get(dom["kernel"]),
                 "launch_ms": dom["ms"], "flops_per_launch": 2.0 * dom["M"] * dom["N"] * dom["K"]}
     del work
     result = {

@@ -195,6 +195,13 @@ def secondary(dev, timer, reps, with_cpu):
         "fwd_GBs": round(nbytes / f_ms / 1e6, 1), "bwd_GBs": round(2 * nbytes / b_ms / 1e6, 1),
         "fwd_bwd_GBs": round(3 * nbytes / (f_ms + b_ms) / 1e6, 1),
         "frac_hbm_peak": round(3 * nbytes / (f_ms + b_ms) / 1e6 / PEAK_HBM_GBS, 4)}
+    # forward+backward in one launch (what mpu.vocab_loss_fn runs): same algorithmic bytes, one read + one write moved
+    o_ms = timer.run("ce.fwd_bwd", lambda: ops.vocab_ce_fwd_bwd_(work, tgt, 0, None, 1.0 / n), reps)
+    out["vocab_ce_c4"].update({
+        "two_launch_fwd_bwd_GBs": out["vocab_ce_c4"]["fwd_bwd_GBs"],
+        "one_launch_us": round(o_ms * 1e3, 1), "one_launch_hbm_GBs": round(2 * nbytes / o_ms / 1e6, 1),
+        "fwd_bwd_GBs": round(3 * nbytes / o_ms / 1e6, 1),
+        "frac_hbm_peak": round(3 * nbytes / o_ms / 1e6 / PEAK_HBM_GBS, 4)})
     if with_cpu:
         rows = 64
         xs = logits[:rows].cpu()
@@ -213,8 +220,10 @@ def secondary(dev, timer, reps, with_cpu):
     f1 = timer.run("ce1.fwd", lambda: ops.vocab_ce_fwd(lg1, t1, 0), reps)
     _, m1, s1, _ = ops.vocab_ce_fwd(lg1, t1, 0)
     b1 = timer.run("ce1.bwd", lambda: ops.vocab_ce_bwd_(lg1, t1, m1, s1, go, 0), reps)
+    o1 = timer.run("ce1.fwd_bwd", lambda: ops.vocab_ce_fwd_bwd_(lg1, t1, 0, None, 1.0 / n1), reps)
     out["vocab_ce_c1"] = {"shape": [n1, v1], "dtype": "f32", "fwd_us": round(f1 * 1e3, 1), "bwd_us": round(b1 * 1e3, 1),
-                          "fwd_bwd_GBs": round(3 * n1 * v1 * 4 / (f1 + b1) / 1e6, 1)}
+                          "two_launch_fwd_bwd_GBs": round(3 * n1 * v1 * 4 / (f1 + b1) / 1e6, 1),
+                          "one_launch_us": round(o1 * 1e3, 1), "fwd_bwd_GBs": round(3 * n1 * v1 * 4 / o1 / 1e6, 1)}
     del lg1
     # --- embedding gather
     h = 4096

@@ -158,6 +158,30 @@ int mtp_vocab_ce_bwd(void* logits, const int64_t* target,
                      int64_t n_rows, int64_t vocab, int64_t vocab_start,
                      int dtype, void* stream);
 
+/* Forward and backward in one launch, for callers that know the upstream
+ * gradient of the per-row losses before the forward runs (the trainer's
+ * loss = mean(losses), Merak/merak_trainer.py:313-326, makes it 1/n_rows
+ * times the loss scale).  Outputs as mtp_vocab_ce_fwd (cross_entropy.py:29-84),
+ * and logits[i,j] <- (softmax[i,j] - onehot) * g_i as mtp_vocab_ce_bwd
+ * (:92-104), with g_i = (grad_rows ? grad_rows[i] : 1) * grad_scale.  Each row
+ * stays in registers between the two, so memory sees one read and one write
+ * of the logits.  Rows longer than mtp_vocab_ce_fwd_bwd_max_vocab(dtype)
+ * return MTP_EUNSUPPORTED (use the two calls above). */
+int mtp_vocab_ce_fwd_bwd(void* logits, const int64_t* target,
+                         const float* grad_rows, float grad_scale,
+                         float* loss, float* row_max, float* row_sumexp, float* pred,
+                         int64_t n_rows, int64_t vocab, int64_t vocab_start,
+                         int dtype, void* stream);
+int64_t mtp_vocab_ce_fwd_bwd_max_vocab(int dtype);
+
+/* grad[i,:] *= grad_rows[i] / assumed for the rows where grad_rows[i] !=
+ * assumed; rows where they are equal are not touched (no memory traffic).
+ * Turns the gradient mtp_vocab_ce_fwd_bwd wrote for an assumed upstream
+ * gradient into the one for the upstream gradient autograd delivers
+ * (cross_entropy.py:103, grad_input.mul_(grad_output.unsqueeze(-1))). */
+int mtp_vocab_ce_rescale(void* grad, const float* grad_rows, float assumed,
+                         int64_t n_rows, int64_t vocab, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------
  * Decode step (Merak/inference/text_generation_inference.py:223,226-227):
  * a handful of single-token activation rows through a linear layer, and the

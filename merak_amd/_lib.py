@@ -36,6 +36,9 @@ SIGNATURES = {
     "mtp_embedding_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _i64, _i64, _vp]),
     "mtp_vocab_ce_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "mtp_vocab_ce_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "mtp_vocab_ce_fwd_bwd": (_int, [_vp, _vp, _vp, C.c_float, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "mtp_vocab_ce_fwd_bwd_max_vocab": (_i64, [_int]),
+    "mtp_vocab_ce_rescale": (_int, [_vp, _vp, C.c_float, _i64, _i64, _int, _vp]),
     "mtp_gemv": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "mtp_gemv_argmax_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "mtp_gemv_argmax": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),

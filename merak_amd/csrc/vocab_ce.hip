@@ -264,6 +264,191 @@ __global__ __launch_bounds__(CE_THREADS) void vocab_ce_bwd_kernel(
   }
 }
 
+// ---- forward and backward in one pass ---------------------------------------
+// One 1024-lane workgroup per row keeps the whole row in registers (NV 16-byte
+// vectors per lane): loaded once, reduced to (max, sum-exp), then rewritten in
+// place as (softmax - onehot) * g.  HBM sees one read and one write of the row
+// instead of two reads and a write.
+constexpr int FU_THREADS = 1024;
+constexpr int FU_WAVES = FU_THREADS / MTP_WAVE;
+
+template <typename T, int NV>
+__global__ __launch_bounds__(FU_THREADS) void vocab_ce_fused_kernel(
+    T* __restrict__ logits, const int64_t* __restrict__ target, const float* __restrict__ grad_rows,
+    float grad_scale, float* __restrict__ loss, float* __restrict__ row_max, float* __restrict__ row_sumexp,
+    float* __restrict__ pred, int64_t V, int64_t vocab_start) {
+  constexpr int EPV = Elem<T>::EPV;
+  const int64_t row = blockIdx.x;
+  T* rp = logits + row * V;
+  const int tid = threadIdx.x;
+
+  int head;
+  int64_t nvec64;
+  row_split(rp, V, head, nvec64);
+  const int nvec = (int)nvec64;  // the host checked nvec <= NV * FU_THREADS
+  u32x4_t* vp = reinterpret_cast<u32x4_t*>(rp + head);
+  const int tail0 = head + nvec * EPV;
+  const int n_edge = head + (int)(V - tail0);
+  const int edge_j = tid < head ? tid : tail0 + (tid - head);
+  const bool has_edge = tid < n_edge;
+
+  u32x4_t v[NV] = {};
+#pragma unroll
+  for (int u = 0; u < NV; u++)
+    if (tid + u * FU_THREADS < nvec) v[u] = __builtin_nontemporal_load(vp + tid + u * FU_THREADS);
+  float fe = NEG_BIG;
+  if (has_edge) fe = Elem<T>::ld(rp + edge_j);
+
+  int64_t tl = target[row] - vocab_start;
+  if (tl < 0 || tl >= V) tl = -1;
+  float x_t = 0.0f;
+  if (tid == 0 && tl >= 0) x_t = Elem<T>::ld(rp + tl);  // read before any lane of this row stores
+  const float g = (grad_rows ? grad_rows[row] : 1.0f) * grad_scale;
+
+  __shared__ float red_m[FU_WAVES], red_s[FU_WAVES];
+
+  // row maximum
+  float lm = fe;
+#pragma unroll
+  for (int u = 0; u < NV; u++)
+    if (tid + u * FU_THREADS < nvec) {
+      float f[EPV];
+      Elem<T>::unpack(v[u], f);
+#pragma unroll
+      for (int e = 0; e < EPV; e++) lm = fmaxf(lm, f[e]);
+    }
+  // keep the row as loaded: without this the compiler carries the unpacked floats of one phase into the
+  // next, which doubles the registers a bf16 row needs
+#pragma unroll
+  for (int u = 0; u < NV; u++) asm volatile("" : "+v"(v[u]));
+  lm = wave_max(lm);
+  if ((tid & 63) == 0) red_m[tid >> 6] = lm;
+  __syncthreads();
+  float m = red_m[0];
+#pragma unroll
+  for (int w = 1; w < FU_WAVES; w++) m = fmaxf(m, red_m[w]);
+  const float mc = mul_rn(m, LOG2E);
+
+  // sum of exponentials, same term as the two-kernel path: exp2(fma(x, c, -fl(m*c)))
+  float ls = has_edge ? __builtin_amdgcn_exp2f(__builtin_fmaf(fe, LOG2E, -mc)) : 0.0f;
+#pragma unroll
+  for (int u = 0; u < NV; u++)
+    if (tid + u * FU_THREADS < nvec) {
+      float f[EPV];
+      Elem<T>::unpack(v[u], f);
+#pragma unroll
+      for (int e = 0; e < EPV; e++) ls += __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc));
+    }
+#pragma unroll
+  for (int u = 0; u < NV; u++) asm volatile("" : "+v"(v[u]));
+  ls = wave_sum(ls);
+  if ((tid & 63) == 0) red_s[tid >> 6] = ls;
+  __syncthreads();
+  float s_raw = red_s[0];
+#pragma unroll
+  for (int w = 1; w < FU_WAVES; w++) s_raw += red_s[w];
+  const float resid = ms_residual_scale(m);
+
+  if (tid == 0) {
+    const float s = s_raw * resid;
+    row_max[row] = m;
+    row_sumexp[row] = s;
+    pred[row] = x_t;
+    loss[row] = logf(s) - (tl >= 0 ? (x_t - m) : 0.0f);
+  }
+
+  // gradient, in place
+  const float scale = g / s_raw;  // exp2(x*c - fl(m*c)) / s_raw = softmax: the residual cancels
+  const int tv = (tl >= head) ? (int)(tl - head) : -1;
+#pragma unroll
+  for (int u = 0; u < NV; u++)
+    if (tid + u * FU_THREADS < nvec) {
+      float f[EPV];
+      Elem<T>::unpack(v[u], f);
+#pragma unroll
+      for (int e = 0; e < EPV; e++) f[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc)) * scale;
+      const int base = (tid + u * FU_THREADS) * EPV;
+      if ((unsigned)(tv - base) < (unsigned)EPV) {
+        const int e = tv - base;
+#pragma unroll
+        for (int q = 0; q < EPV; q++)
+          if (q == e) f[q] -= g;
+      }
+      __builtin_nontemporal_store(Elem<T>::pack(f), vp + tid + u * FU_THREADS);
+    }
+  if (has_edge) {
+    float f = __builtin_amdgcn_exp2f(__builtin_fmaf(fe, LOG2E, -mc)) * scale;
+    if (edge_j == tl) f -= g;
+    Elem<T>::st(rp + edge_j, f);
+  }
+}
+
+// grad[i,:] *= grad_rows[i] / assumed, skipped for rows where the two are equal
+template <typename T>
+__global__ __launch_bounds__(CE_THREADS) void vocab_ce_rescale_kernel(T* __restrict__ grad,
+                                                                     const float* __restrict__ grad_rows,
+                                                                     float assumed, int64_t V) {
+  constexpr int EPV = Elem<T>::EPV;
+  const int64_t row = blockIdx.x;
+  const float gr = grad_rows[row];
+  if (gr == assumed) return;
+  const float ratio = gr / assumed;
+  T* rp = grad + row * V;
+  const int tid = threadIdx.x;
+  int head;
+  int64_t nvec;
+  row_split(rp, V, head, nvec);
+  u32x4_t* vp = reinterpret_cast<u32x4_t*>(rp + head);
+  for (int64_t i = tid; i < nvec; i += CE_THREADS) {
+    u32x4_t v = __builtin_nontemporal_load(vp + i);
+    float f[EPV];
+    Elem<T>::unpack(v, f);
+#pragma unroll
+    for (int e = 0; e < EPV; e++) f[e] *= ratio;
+    __builtin_nontemporal_store(Elem<T>::pack(f), vp + i);
+  }
+  const int64_t tail0 = head + nvec * EPV;
+  const int n_edge = head + (int)(V - tail0);
+  if (tid < n_edge) {
+    int64_t j = tid < head ? tid : tail0 + (tid - head);
+    Elem<T>::st(rp + j, Elem<T>::ld(rp + j) * ratio);
+  }
+}
+
+template <typename T, int NV>
+void launch_fused(void* logits, const int64_t* target, const float* grad_rows, float grad_scale, float* loss,
+                  float* row_max, float* row_sumexp, float* pred, int64_t n_rows, int64_t vocab,
+                  int64_t vocab_start, hipStream_t s) {
+  hipLaunchKernelGGL((vocab_ce_fused_kernel<T, NV>), dim3((unsigned)n_rows), dim3(FU_THREADS), 0, s, (T*)logits,
+                     target, grad_rows, grad_scale, loss, row_max, row_sumexp, pred, vocab, vocab_start);
+}
+
+template <typename T>
+int dispatch_fused(void* logits, const int64_t* target, const float* grad_rows, float grad_scale, float* loss,
+                   float* row_max, float* row_sumexp, float* pred, int64_t n_rows, int64_t vocab,
+                   int64_t vocab_start, hipStream_t s) {
+  // the row's aligned body has at most vocab / EPV vectors whatever its start address
+  const int64_t nvec_max = vocab / Elem<T>::EPV;
+  const int64_t need = (nvec_max + FU_THREADS - 1) / FU_THREADS;
+#define MTP_FUSED_CASE(NV)                                                                                      \
+  if (need <= NV) {                                                                                             \
+    launch_fused<T, NV>(logits, target, grad_rows, grad_scale, loss, row_max, row_sumexp, pred, n_rows, vocab,  \
+                        vocab_start, s);                                                                        \
+    return MTP_OK;                                                                                              \
+  }
+  if (vocab <= 20ll * FU_THREADS * Elem<T>::EPV) {
+    MTP_FUSED_CASE(4)
+    MTP_FUSED_CASE(8)
+    MTP_FUSED_CASE(12)
+    MTP_FUSED_CASE(16)
+    MTP_FUSED_CASE(20)
+  }
+#undef MTP_FUSED_CASE
+  mtp_set_error("vocab_ce_fwd_bwd: a row of %lld elements does not fit the register-resident kernel (limit %lld)",
+                (long long)vocab, (long long)(20ll * FU_THREADS * Elem<T>::EPV));
+  return MTP_EUNSUPPORTED;
+}
+
 }  // namespace
 
 extern "C" int mtp_vocab_ce_fwd(const void* logits, const int64_t* target, float* loss, float* row_max,
@@ -315,5 +500,64 @@ extern "C" int mtp_vocab_ce_bwd(void* logits, const int64_t* target, const float
     MTP_REQUIRE(false, MTP_EINVAL, "vocab_ce_bwd: unknown dtype %d", dtype);
   }
   MTP_CHECK_LAUNCH("vocab_ce_bwd");
+  return MTP_OK;
+}
+
+extern "C" int64_t mtp_vocab_ce_fwd_bwd_max_vocab(int dtype) {
+  if (dtype == MTP_F32) return 20ll * FU_THREADS * Elem<float>::EPV;
+  if (dtype == MTP_BF16) return 20ll * FU_THREADS * Elem<uint16_t>::EPV;
+  return 0;
+}
+
+extern "C" int mtp_vocab_ce_fwd_bwd(void* logits, const int64_t* target, const float* grad_rows, float grad_scale,
+                                    float* loss, float* row_max, float* row_sumexp, float* pred, int64_t n_rows,
+                                    int64_t vocab, int64_t vocab_start, int dtype, void* stream) {
+  MTP_REQUIRE(n_rows >= 0 && vocab >= 1, MTP_EINVAL, "vocab_ce_fwd_bwd: n_rows=%lld vocab=%lld", (long long)n_rows,
+              (long long)vocab);
+  MTP_REQUIRE(n_rows < (1ll << 31), MTP_EUNSUPPORTED, "vocab_ce_fwd_bwd: n_rows=%lld exceeds 2^31-1",
+              (long long)n_rows);
+  if (n_rows == 0) return MTP_OK;
+  MTP_REQUIRE(logits && target && loss && row_max && row_sumexp && pred, MTP_EINVAL, "vocab_ce_fwd_bwd: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  int rc;
+  if (dtype == MTP_F32) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 3) == 0, MTP_EINVAL,
+                "vocab_ce_fwd_bwd: fp32 logits not 4-byte aligned");
+    rc = dispatch_fused<float>(logits, target, grad_rows, grad_scale, loss, row_max, row_sumexp, pred, n_rows, vocab,
+                               vocab_start, s);
+  } else if (dtype == MTP_BF16) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL,
+                "vocab_ce_fwd_bwd: bf16 logits not 2-byte aligned");
+    rc = dispatch_fused<uint16_t>(logits, target, grad_rows, grad_scale, loss, row_max, row_sumexp, pred, n_rows,
+                                  vocab, vocab_start, s);
+  } else {
+    MTP_REQUIRE(false, MTP_EINVAL, "vocab_ce_fwd_bwd: unknown dtype %d", dtype);
+  }
+  if (rc != MTP_OK) return rc;
+  MTP_CHECK_LAUNCH("vocab_ce_fwd_bwd");
+  return MTP_OK;
+}
+
+extern "C" int mtp_vocab_ce_rescale(void* grad, const float* grad_rows, float assumed, int64_t n_rows, int64_t vocab,
+                                    int dtype, void* stream) {
+  MTP_REQUIRE(n_rows >= 0 && vocab >= 1, MTP_EINVAL, "vocab_ce_rescale: n_rows=%lld vocab=%lld", (long long)n_rows,
+              (long long)vocab);
+  MTP_REQUIRE(n_rows < (1ll << 31), MTP_EUNSUPPORTED, "vocab_ce_rescale: n_rows=%lld exceeds 2^31-1",
+              (long long)n_rows);
+  MTP_REQUIRE(assumed != 0.0f && assumed == assumed, MTP_EINVAL, "vocab_ce_rescale: assumed scale must be non-zero");
+  if (n_rows == 0) return MTP_OK;
+  MTP_REQUIRE(grad && grad_rows, MTP_EINVAL, "vocab_ce_rescale: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((unsigned)n_rows), block(CE_THREADS);
+  if (dtype == MTP_F32) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(grad) & 3) == 0, MTP_EINVAL, "vocab_ce_rescale: fp32 buffer not 4-byte aligned");
+    hipLaunchKernelGGL(vocab_ce_rescale_kernel<float>, grid, block, 0, s, (float*)grad, grad_rows, assumed, vocab);
+  } else if (dtype == MTP_BF16) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(grad) & 1) == 0, MTP_EINVAL, "vocab_ce_rescale: bf16 buffer not 2-byte aligned");
+    hipLaunchKernelGGL(vocab_ce_rescale_kernel<uint16_t>, grid, block, 0, s, (uint16_t*)grad, grad_rows, assumed, vocab);
+  } else {
+    MTP_REQUIRE(false, MTP_EINVAL, "vocab_ce_rescale: unknown dtype %d", dtype);
+  }
+  MTP_CHECK_LAUNCH("vocab_ce_rescale");
   return MTP_OK;
 }

@@ -12,7 +12,14 @@ reference's mask (:48-62).  Differences in *how*, not in *what*:
   reuses the buffer for the softmax (:37,70,80,92) — no second
   [tokens, vocab] tensor is ever allocated;
 * for bf16 logits the loss is returned in fp32 unless
-  ``loss_in_logits_dtype=True``.
+  ``loss_in_logits_dtype=True``;
+* ``fused_backward_scale=g`` (an extension) runs forward and backward in one
+  launch for the case where the upstream gradient of every per-position loss
+  is known to be ``g`` before the forward — ``vocab_loss_fn`` below, the
+  trainer's ``mean`` (Merak/merak_trainer.py:313-326), passes ``1/n``.  Like
+  the reference, this forward overwrites the caller's logits (there with the
+  softmax, here with the finished gradient); ``backward`` checks the real
+  upstream gradient on the device and rescales only the rows where it differs.
 """
 from __future__ import annotations
 
@@ -70,8 +77,33 @@ class _VocabParallelCrossEntropy(torch.autograd.Function):
         return logits, None, None, None
 
 
+class _VocabParallelCrossEntropyFused(torch.autograd.Function):
+    """Forward that already writes the gradient for an assumed uniform upstream gradient."""
+
+    @staticmethod
+    def forward(ctx, vocab_parallel_logits, target, loss_in_logits_dtype, assumed_grad):
+        partition_vocab_size = vocab_parallel_logits.size()[-1]
+        vocab_start_index, _ = _vocab_range(partition_vocab_size)
+        logits_2d = vocab_parallel_logits.view(-1, partition_vocab_size)
+        target_1d = target.reshape(-1)
+        loss, _, _, _ = ops.vocab_ce_fwd_bwd_(logits_2d, target_1d, vocab_start_index, None, assumed_grad)
+        ctx.assumed_grad = float(assumed_grad)
+        ctx.save_for_backward(vocab_parallel_logits)
+        loss = loss.view_as(target)
+        if loss_in_logits_dtype:
+            loss = loss.to(vocab_parallel_logits.dtype)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (grad,) = ctx.saved_tensors
+        grad_2d = grad.view(-1, grad.size()[-1])
+        ops.vocab_ce_rescale_(grad_2d, grad_output.reshape(-1), ctx.assumed_grad)
+        return grad, None, None, None
+
+
 def vocab_parallel_cross_entropy(vocab_parallel_logits, target, loss_in_logits_dtype=False,
-                                 materialize_softmax=False):
+                                 materialize_softmax=False, fused_backward_scale=None):
     """Cross entropy loss when logits are split across tensor parallel ranks.
 
     Args:
@@ -79,8 +111,31 @@ def vocab_parallel_cross_entropy(vocab_parallel_logits, target, loss_in_logits_d
             [sequence_length, batch_size, vocab_size / num_parallel_ranks], contiguous
         target: correct vocab ids of dimension [sequence_length, micro_batch_size]
     """
+    if fused_backward_scale is not None and not materialize_softmax:
+        g = float(fused_backward_scale)
+        if g == 0.0 or g != g:
+            raise ValueError("fused_backward_scale must be a non-zero number")
+        fits = vocab_parallel_logits.size()[-1] <= ops.vocab_ce_fused_max_vocab(vocab_parallel_logits.dtype)
+        if fits and get_model_parallel_world_size() == 1:
+            return _VocabParallelCrossEntropyFused.apply(vocab_parallel_logits, target, loss_in_logits_dtype, g)
     return _VocabParallelCrossEntropy.apply(vocab_parallel_logits, target, loss_in_logits_dtype,
                                             materialize_softmax)
+
+
+def vocab_loss_fn(outputs, labels, loss_scale=1.0):
+    """The trainer's loss over vocab-parallel logits, Merak/merak_trainer.py:313-326:
+    ``mean`` of the per-position losses.  The mean makes every position's upstream gradient
+    ``loss_scale / n``, which is handed to the one-launch forward+backward kernel; multiply the
+    returned loss by ``loss_scale`` (or anything else) as usual — a different factor only costs the
+    rescale pass in backward."""
+    if isinstance(outputs, tuple):
+        outputs = outputs[0]
+    if isinstance(labels, tuple):
+        labels = labels[0]
+    n = labels.numel()
+    losses = vocab_parallel_cross_entropy(outputs, labels,
+                                          fused_backward_scale=(float(loss_scale) / n) if n else None)
+    return torch.mean(losses.view(-1))
 
 
 def vocab_parallel_cross_entropy_partials(vocab_parallel_logits, target):

@@ -211,6 +211,50 @@ def vocab_ce_bwd_(logits2d: torch.Tensor, target1d: torch.Tensor, row_max: Optio
     return logits2d
 
 
+def vocab_ce_fused_max_vocab(dtype: torch.dtype) -> int:
+    """Longest row the one-launch forward+backward kernel keeps in registers."""
+    return int(_lib.lib().mtp_vocab_ce_fwd_bwd_max_vocab(_DTYPES[dtype]))
+
+
+def vocab_ce_fwd_bwd_(logits2d: torch.Tensor, target1d: torch.Tensor, vocab_start: int,
+                      grad_rows: Optional[torch.Tensor] = None, grad_scale: float = 1.0):
+    """One launch: -> (loss, row_max, row_sumexp, pred) and, in place,
+    logits2d <- (softmax - onehot) * grad_rows[i] * grad_scale."""
+    dev = _require_gpu(logits2d, target1d, grad_rows)
+    if target1d.dtype != torch.int64:
+        raise TypeError(f"cross-entropy targets must be int64, got {target1d.dtype}")
+    if not logits2d.is_contiguous():
+        raise ValueError("vocab_parallel_cross_entropy needs contiguous logits")
+    n, v = logits2d.shape
+    if target1d.numel() != n:
+        raise ValueError(f"target has {target1d.numel()} entries for {n} logits rows")
+    if grad_rows is not None:
+        grad_rows = _contig(grad_rows.to(torch.float32))
+        if grad_rows.numel() != n:
+            raise ValueError(f"grad_rows has {grad_rows.numel()} entries for {n} logits rows")
+    target1d = _contig(target1d)
+    out = torch.empty((4, n), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_vocab_ce_fwd_bwd(_p(logits2d), _p(target1d), _p(grad_rows), float(grad_scale),
+                                                   _p(out[0]), _p(out[1]), _p(out[2]), _p(out[3]), n, v,
+                                                   vocab_start, _dt(logits2d), _stream(dev)),
+                   "mtp_vocab_ce_fwd_bwd")
+    return out[0], out[1], out[2], out[3]
+
+
+def vocab_ce_rescale_(grad2d: torch.Tensor, grad_rows: torch.Tensor, assumed: float) -> torch.Tensor:
+    """In place: rows of grad2d whose grad_rows[i] differs from ``assumed`` are scaled by grad_rows[i]/assumed."""
+    dev = _require_gpu(grad2d, grad_rows)
+    n, v = grad2d.shape
+    grad_rows = _contig(grad_rows.to(torch.float32))
+    if grad_rows.numel() != n:
+        raise ValueError(f"grad_rows has {grad_rows.numel()} entries for {n} rows")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_vocab_ce_rescale(_p(grad2d), _p(grad_rows), float(assumed), n, v, _dt(grad2d),
+                                                   _stream(dev)), "mtp_vocab_ce_rescale")
+    return grad2d
+
+
 # --------------------------------------------------------------------------- decode
 def gemv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE) -> torch.Tensor:
     dev = _require_gpu(x, w, bias)

@@ -163,6 +163,109 @@ def test_ce_full_size_llama_vocab(gpu):
     assert (rowsum - expect).abs().max() < 0.05
 
 
+@pytest.mark.parametrize("dtype,n,v", [
+    (torch.float32, 64, 50257), (torch.bfloat16, 64, 128256), (torch.float32, 7, 1), (torch.float32, 3, 5),
+    (torch.bfloat16, 5, 9), (torch.bfloat16, 4, 1031), (torch.float32, 2, 2048 + 3), (torch.bfloat16, 3, 40000),
+    (torch.float32, 2, 81920), (torch.bfloat16, 2, 163840),     # the longest rows that stay in registers
+    (torch.bfloat16, 3, 8192 * 4 + 5), (torch.float32, 5, 4096 * 4 + 1), (torch.bfloat16, 6, 8192 * 12 - 3),
+])
+def test_ce_one_launch_forward_backward(gpu, dtype, n, v):
+    """mtp_vocab_ce_fwd_bwd against the oracle and against the two-launch path on the same inputs."""
+    x = torch.randn(n, v, generator=gen(14)).to(dtype)
+    t = torch.randint(0, v, (n,), generator=gen(15))
+    t[torch.randperm(n, generator=gen(16))[: max(1, n // 20)]] = -100
+    gr = torch.rand(n, generator=gen(17)) + 0.5
+    scale = 0.25
+    ref_loss, ref_grad = R.cross_entropy_fp32(x, t, 0, gr * scale)
+    tol_g = TOL_F32 if dtype == torch.float32 else TOL_BF16
+    a, b = x.to(gpu), x.to(gpu)
+    loss, m, s, pred = ops.vocab_ce_fwd_bwd_(a, t.to(gpu), 0, gr.to(gpu), scale)
+    loss2, m2, s2, pred2 = ops.vocab_ce_fwd(b, t.to(gpu), 0)
+    ops.vocab_ce_bwd_(b, t.to(gpu), m2, s2, (gr * scale).to(gpu), 0)
+    assert (loss.cpu() - ref_loss).abs().max() <= TOL_LOSS * max(ref_loss.abs().max().item(), 0.1)
+    assert torch.equal(m, m2) and torch.equal(pred, pred2) and rel(s, s2) < TOL_LOSS
+    assert rel(a, ref_grad) < tol_g and rel(a, b) < tol_g
+    # no per-row gradient: g = grad_scale for every row
+    c = x.to(gpu)
+    ops.vocab_ce_fwd_bwd_(c, t.to(gpu), 0, None, 1.0 / n)
+    assert rel(c, R.cross_entropy_fp32(x, t, 0, torch.full((n,), 1.0 / n))[1]) < tol_g
+
+
+def test_ce_one_launch_vocab_slice_and_limits(gpu):
+    n, v, start = 8, 1002, 3006
+    x = torch.randn(n, v, generator=gen(18)).bfloat16()
+    t = torch.randint(0, 8 * v, (n,), generator=gen(19))
+    t[0], t[1] = start, start + v - 1                    # first and last id of this slice
+    om, os_, opr, inr = R.cross_entropy_partials(x, t, start)
+    xg = x.to(gpu)
+    _, m, s, pr = ops.vocab_ce_fwd_bwd_(xg, t.to(gpu), start, None, 1.0)
+    assert torch.equal(m.cpu(), om) and rel(s, os_) < TOL_LOSS and torch.equal(pr.cpu(), opr)
+    sm = torch.softmax(x.float(), -1)
+    onehot = torch.zeros(n, v)
+    onehot[inr, (t - start)[inr]] = 1.0
+    assert rel(xg, sm - onehot) < TOL_BF16
+    # rows too long for the registers: the C entry point says so, the module falls back to two launches
+    for dtype in (torch.float32, torch.bfloat16):
+        lim = ops.vocab_ce_fused_max_vocab(dtype)
+        assert lim == {torch.float32: 81920, torch.bfloat16: 163840}[dtype]
+        big = torch.zeros(1, lim + 1, dtype=dtype, device=gpu)
+        with pytest.raises(RuntimeError, match="does not fit"):
+            ops.vocab_ce_fwd_bwd_(big, torch.zeros(1, dtype=torch.int64, device=gpu), 0)
+    big = torch.randn(2, 81920 + 7, generator=gen(20))
+    bt = torch.tensor([5, 81920])
+    bg = big.to(gpu).requires_grad_(True)
+    mpu.vocab_loss_fn(bg * 1.0, bt.to(gpu)).backward()
+    assert rel(bg.grad, R.cross_entropy_fp32(big, bt, 0, torch.full((2,), 0.5))[1]) < TOL_F32
+    empty = ops.vocab_ce_fwd_bwd_(torch.empty(0, 17, device=gpu), torch.empty(0, dtype=torch.int64, device=gpu), 0)
+    assert empty[0].numel() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ce_vocab_loss_fn_autograd(gpu, dtype):
+    """The trainer's mean loss (merak_trainer.py:313-326) through the one-launch kernel: the assumed upstream
+    gradient 1/n is what autograd delivers; a different one (loss scaling, per-position masks) is corrected."""
+    n, v = 48, 50257
+    x = torch.randn(4, 12, v, generator=gen(21)).to(dtype)
+    t = torch.randint(0, v, (4, 12), generator=gen(22))
+    t[0, 0] = -100
+    tol_g = TOL_F32 if dtype == torch.float32 else TOL_BF16
+    ref_loss, ref_grad = R.cross_entropy_fp32(x.view(n, v), t.view(n), 0, torch.full((n,), 1.0 / n))
+    xg = x.to(gpu).requires_grad_(True)
+    loss = mpu.vocab_loss_fn((xg * 1.0,), (t.to(gpu),))
+    assert loss.dim() == 0 and abs(loss.item() - ref_loss.mean().item()) < TOL_LOSS * ref_loss.mean().item() * 10
+    loss.backward()
+    assert rel(xg.grad.view(n, v), ref_grad) < tol_g
+    # upstream gradient differs from the assumption: scaled loss and a per-position mask
+    mask = (torch.rand(4, 12, generator=gen(23)) > 0.3).float()
+    xg2 = x.to(gpu).requires_grad_(True)
+    losses = mpu.vocab_parallel_cross_entropy(xg2 * 1.0, t.to(gpu), fused_backward_scale=1.0 / n)
+    assert rel(losses.view(-1), ref_loss) < TOL_LOSS
+    (1024.0 * (losses * mask.to(gpu)).sum() / mask.sum()).backward()
+    ref2 = R.cross_entropy_fp32(x.view(n, v), t.view(n), 0, 1024.0 * mask.view(n) / mask.sum())[1]
+    assert rel(xg2.grad.view(n, v), ref2) < 2 * tol_g       # bf16: rounded once more by the rescale
+    assert bool((xg2.grad.view(n, v)[mask.view(n) == 0] == 0).all())
+
+
+def test_ce_one_launch_full_size_llama_vocab(gpu):
+    n, v = 8192, 128256
+    x = torch.empty(n, v, dtype=torch.bfloat16, device=gpu).normal_(generator=torch.Generator(device=gpu).manual_seed(1239))
+    t = torch.randint(0, v, (n,), generator=gen(24))
+    t[torch.randperm(n, generator=gen(25))[: n // 20]] = -100
+    rows = torch.randperm(n, generator=gen(26))[:48]
+    rows[0] = (t == -100).nonzero()[0, 0]
+    xs = x[rows.to(gpu)].cpu()
+    ref_loss, ref_grad = R.cross_entropy_fp32(xs, t[rows], 0, torch.full((48,), 1.0 / n))
+    loss, m, s, pred = ops.vocab_ce_fwd_bwd_(x, t.to(gpu), 0, None, 1.0 / n)
+    assert rel(loss.cpu()[rows], ref_loss) < TOL_LOSS
+    assert bool(torch.isfinite(loss).all()) and float(loss.min()) > 0
+    assert rel(x[rows.to(gpu)], ref_grad) < TOL_BF16
+    rowsum = x.float().sum(-1).cpu() * n
+    assert (rowsum - (t == -100).float()).abs().max() < 0.05
+    before = x[:64].clone()
+    ops.vocab_ce_rescale_(x, torch.full((n,), 1.0 / n, device=gpu), 1.0 / n)      # equal: must not touch anything
+    assert torch.equal(x[:64], before)
+
+
 # =============================================================================== embedding
 @pytest.mark.parametrize("dtype,v,h", [(torch.bfloat16, 1000, 4096), (torch.float32, 777, 33), (torch.bfloat16, 50, 7),
                                         (torch.float32, 64, 1)])

@@ -3,13 +3,20 @@
 // reduces the LM-head row straight to (max, argmax) without ever writing the
 // logits (Merak/inference/text_generation_inference.py:223,226-227).
 //
-// The weight matrix is streamed from HBM exactly once.  It feeds the A operand
-// of v_mfma_f32_16x16x32_bf16 directly from global memory: lane (i = l%16,
-// g = l/16) loads the 16 bytes W[row0+i][k0+8g .. k0+8g+7], so four lanes
-// cover 64 contiguous bytes of a weight row and consecutive k-steps walk
-// along it.  The B operand is X^T (lane (b = l%16, g) loads X[b][k0+8g..]);
-// X is tiny and stays in L2/L1.  The result tile D[i][b] needs no cross-lane
-// reduction.
+// The weight matrix is streamed from HBM exactly once, straight into the A
+// operand of v_mfma_f32_16x16x32_bf16 (lane (i = l%16, g = l/16) supplies row
+// i, k-group g).  What one load instruction touches decides the bandwidth: 16
+// rows x 64 bytes (the natural operand layout) uses half of every 128-byte
+// line per instruction and stalls near 5.7 TB/s; 8 rows x 128 bytes reaches
+// 6.9 TB/s.  So the two loads of a 64-element k-pair are arranged as
+//   load A: lane (i,g) <- row i%8,     bytes 64*(i/8)     + 16 g of the pair
+//   load B: lane (i,g) <- row 8 + i%8, bytes 64*(1 - i/8) + 16 g
+// and the two MFMA operands are picked per lane: first half of the pair =
+// (i < 8 ? A : B), which holds row i at position i; second half = (i < 8 ? B : A),
+// which holds row i^8 at position i and is rotated 8 lanes inside its group of
+// 16 (one DPP move per register) to put row i at position i as well.
+// The B operand is X^T (lane (b = l%16, g) loads X[b][k0+8g..]); X is tiny
+// and stays in L2/L1.  The result tile D[i][b] needs no cross-lane reduction.
 //
 // A workgroup of 8 waves owns 16*R weight rows; the 128-byte k-pairs of those
 // rows are dealt round-robin to the waves (split-K inside the workgroup), the 8
@@ -36,6 +43,22 @@ __device__ __forceinline__ bool arg_better(float va, int64_t ia, float vb, int64
   return va > vb || (va == vb && ia < ib);
 }
 
+// The same order as one unsigned 64-bit key (row indices are below 2^31): larger key = better candidate,
+// 0 = no candidate.  High word: the float mapped monotonically to unsigned, every NaN to the top; low word:
+// the complement of the index, so that equal values prefer the lower index.
+__device__ __forceinline__ uint64_t arg_key(float v, int64_t n) {
+  const uint32_t u = v == 0.0f ? 0u : __float_as_uint(v);  // -0 and +0 compare equal
+  uint32_t o = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+  if (v != v) o = 0xffffffffu;
+  return ((uint64_t)o << 32) | (uint32_t)(0xffffffffu - (uint32_t)n);
+}
+__device__ __forceinline__ float arg_key_value(uint64_t key) {
+  const uint32_t o = (uint32_t)(key >> 32);
+  if (o == 0xffffffffu) return __uint_as_float(0x7fc00000u);
+  return __uint_as_float((o & 0x80000000u) ? (o ^ 0x80000000u) : ~o);
+}
+__device__ __forceinline__ int32_t arg_key_index(uint64_t key) { return (int32_t)(0xffffffffu - (uint32_t)key); }
+
 // `ok` is a compile-time true on the unguarded path, which then has no branches at all
 __device__ __forceinline__ bf16x8_t load_frag(const uint16_t* p, bool ok) {
   u32x4_t v = {0u, 0u, 0u, 0u};
@@ -50,13 +73,18 @@ __device__ __forceinline__ bf16x8_t load_frag_nt(const uint16_t* p, bool ok) {
   return __builtin_bit_cast(bf16x8_t, v);
 }
 
+// value of the lane 8 places around inside each group of 16 lanes (DPP row_ror:8), i.e. of lane ^ 8
+__device__ __forceinline__ uint32_t rot8_in_row(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xf, 0xf, false);
+}
+
 // MODE 0: store Y (+bias); MODE 1: SwiGLU store; MODE 2: argmax partials
-template <int R, int NB, int MODE, bool GUARD>
+template <int R, int NB, int MODE, bool GUARD, int D>
 __global__ __launch_bounds__(GV_THREADS) void gemv_kernel(const uint16_t* __restrict__ x,
                                                           const uint16_t* __restrict__ w,
                                                           const uint16_t* __restrict__ bias,
                                                           uint16_t* __restrict__ y, ArgPart* __restrict__ part,
-                                                          int B, int64_t N, int64_t K) {
+                                                          int B, int64_t N, int64_t K, int rot_mul) {
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
@@ -65,24 +93,35 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_kernel(const uint16_t* __rest
 
   // rows of the R groups owned by this workgroup
   const int64_t half = N >> 1;  // SwiGLU: W = [gate rows | up rows]
-  int64_t grow[R];
+  // Per row group: a wave-uniform base (first row of the group) and 32-bit per-lane element offsets for
+  // the two loads.  GUARD (K not a multiple of 64) keeps the plain layout: load A = first 64 bytes of the
+  // pair at row li, load B = the next 64.  Rows past the end are clamped to the last row (never stored).
+  const uint16_t* wbase[R];
+  uint32_t offa[R], offb[R];
 #pragma unroll
   for (int r = 0; r < R; r++) {
-    int64_t row;
+    int64_t row0, lim;
     if (MODE == 1) {
       const int64_t j0 = (int64_t)blockIdx.x * (8 * R);
-      row = (r < R / 2) ? j0 + 16 * r + li : half + j0 + 16 * (r - R / 2) + li;
-      const int64_t lim = (r < R / 2) ? half : N;
-      if (row >= lim) row = lim - 1;
+      row0 = (r < R / 2) ? j0 + 16 * r : half + j0 + 16 * (r - R / 2);
+      lim = (r < R / 2) ? half : N;
     } else {
-      row = (int64_t)blockIdx.x * (16 * R) + 16 * r + li;
-      if (row >= N) row = N - 1;
+      row0 = (int64_t)blockIdx.x * (16 * R) + 16 * r;
+      lim = N;
     }
-    grow[r] = row;
+    if (row0 >= lim) row0 = lim - 1;                 // a group entirely past the end reads the last row
+    const int last = (int)(lim - 1 - row0);          // >= 0: largest valid row offset inside this group
+    wbase[r] = w + row0 * K;
+    if (GUARD) {
+      const int ra = li < last ? li : last;
+      offa[r] = (uint32_t)(ra * K + 8 * lg);
+      offb[r] = offa[r] + 32;
+    } else {
+      const int ra = (li & 7) < last ? (li & 7) : last, rb = 8 + (li & 7) < last ? 8 + (li & 7) : last;
+      offa[r] = (uint32_t)(ra * K + 32 * (li >> 3) + 8 * lg);
+      offb[r] = (uint32_t)(rb * K + 32 * (1 - (li >> 3)) + 8 * lg);
+    }
   }
-  const uint16_t* wp[R];
-#pragma unroll
-  for (int r = 0; r < R; r++) wp[r] = w + grow[r] * K + 8 * lg;
   const uint16_t* xp[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
@@ -100,52 +139,100 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_kernel(const uint16_t* __rest
   // DRAM pages open much longer than eight far-apart 128-byte streams per row would.
   const int64_t pairs = (K + 63) >> 6;
   const int64_t p0 = wave;
-  const int64_t p1 = pairs;
+  // Every workgroup starts its walk along k at a different pair and wraps around: if all of them began at
+  // k = 0 the whole chip would, at any moment, ask for the same few hundred bytes of every row, which
+  // (rows being a power-of-two apart) live in the same few memory channels.
+  const int64_t rot = GUARD || (pairs % GV_WAVES) ? 0 : ((int64_t)blockIdx.x * rot_mul) % pairs;
 
   f32x4_t acc[R][NB];
 #pragma unroll
   for (int r = 0; r < R; r++)
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) acc[r][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const bool low = li < 8;
 
-  if (p0 < p1) {
-    bf16x8_t a_cur[R][2], b_cur[NB][2];
+  // D pairs (8 apart) per step: with few rows per workgroup this is what keeps enough bytes in flight.
+  // The host only picks D > 1 when every wave's share of the pairs is a multiple of D.
+  const int64_t n_it = ((pairs - p0 + GV_WAVES - 1) / GV_WAVES) / D;
+  if (n_it > 0) {
+    // SwiGLU: the "up" rows sit exactly N/2 rows below the "gate" rows of the same workgroup, for the usual
+    // shapes a large power of two apart, i.e. in the same memory channel and bank but another DRAM page.
+    // Walking both at the same k makes the two streams evict each other's open page, so the up rows walk
+    // half a row ahead (XS = 2 sets of X fragments, one per k position).
+    constexpr int XS = (MODE == 1 && !GUARD && NB == 1) ? 2 : 1;
+    const int64_t up_shift = (XS == 2 && pairs % GV_WAVES == 0) ? ((pairs / 2) & ~(int64_t)(GV_WAVES - 1)) : 0;
+    bf16x8_t a_cur[D][R][2], b_cur[D][XS][NB][2];
     // GUARD: K is not a multiple of 64, the last pair is partly (or half) past the end of the rows
-    auto load_pair = [&](int64_t pr, bf16x8_t (&a)[R][2], bf16x8_t (&b)[NB][2]) {
-      const int64_t k = pr * 64;
+    auto load_set = [&](int64_t pq0, bf16x8_t (&a)[D][R][2], bf16x8_t (&b)[D][XS][NB][2]) {
 #pragma unroll
-      for (int r = 0; r < R; r++)
+      for (int d = 0; d < D; d++) {
+        int64_t pr = pq0 + d * GV_WAVES;
+        if (pr >= pairs) pr -= pairs;
+        int64_t pu = pr + up_shift;
+        if (pu >= pairs) pu -= pairs;
+        const int64_t ks[2] = {pr * 64, pu * 64};
 #pragma unroll
-        for (int hf = 0; hf < 2; hf++) a[r][hf] = load_frag_nt(wp[r] + k + 32 * hf, !GUARD || (k + 32 * hf + 8 * lg < K));
+        for (int r = 0; r < R; r++) {
+          const int64_t k = ks[(XS == 2 && r >= R / 2) ? 1 : 0];
+          a[d][r][0] = load_frag_nt(wbase[r] + k + offa[r], !GUARD || (k + 8 * lg < K));
+          a[d][r][1] = load_frag_nt(wbase[r] + k + offb[r], !GUARD || (k + 32 + 8 * lg < K));
+        }
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++)
+        for (int xs = 0; xs < XS; xs++)
 #pragma unroll
-        for (int hf = 0; hf < 2; hf++) b[nb][hf] = load_frag(xp[nb] + k + 32 * hf, !GUARD || (k + 32 * hf + 8 * lg < K));
+          for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++)
+              b[d][xs][nb][hf] = load_frag(xp[nb] + ks[xs] + 32 * hf, !GUARD || (ks[xs] + 32 * hf + 8 * lg < K));
+      }
     };
     auto multiply = [&]() {
 #pragma unroll
-      for (int hf = 0; hf < 2; hf++)
+      for (int d = 0; d < D; d++)
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          // GUARD: a[0] / a[1] are the halves themselves.  Otherwise pick them per lane out of loads A and
+          // B; the second half then sits 8 lanes away inside its group of 16 (row i^8 at position i): one
+          // DPP rotation per register puts it in place.
+          bf16x8_t h0 = a_cur[d][r][0], h1 = a_cur[d][r][1];
+          if (!GUARD) {
+            h0 = low ? a_cur[d][r][0] : a_cur[d][r][1];
+            const u32x4_t t = __builtin_bit_cast(u32x4_t, low ? a_cur[d][r][1] : a_cur[d][r][0]);
+            u32x4_t rt;
+            rt.x = rot8_in_row(t.x); rt.y = rot8_in_row(t.y); rt.z = rot8_in_row(t.z); rt.w = rot8_in_row(t.w);
+            h1 = __builtin_bit_cast(bf16x8_t, rt);
+          }
+          const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
+#pragma unroll
+          for (int nb = 0; nb < NB; nb++) {
+            acc[r][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(h0, b_cur[d][xs][nb][0], acc[r][nb], 0, 0, 0);
+            acc[r][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(h1, b_cur[d][xs][nb][1], acc[r][nb], 0, 0, 0);
+          }
+        }
+    };
+    int64_t pq = p0 + rot;  // first pair of the step in flight; pairs % 8 == 0 whenever rot != 0, so wrapping keeps the wave's residue
+    if (pq >= pairs) pq -= pairs;
+    load_set(pq, a_cur, b_cur);
+    // all but the last step: fetch the next one (unconditionally: it exists), multiply the current one
+    for (int64_t it = 1; it < n_it; it++) {
+      bf16x8_t a_nxt[D][R][2], b_nxt[D][XS][NB][2];
+      pq += GV_WAVES * D;
+      if (pq >= pairs) pq -= pairs;
+      load_set(pq, a_nxt, b_nxt);
+      multiply();
+#pragma unroll
+      for (int d = 0; d < D; d++) {
 #pragma unroll
         for (int r = 0; r < R; r++)
 #pragma unroll
+          for (int hf = 0; hf < 2; hf++) a_cur[d][r][hf] = a_nxt[d][r][hf];
+#pragma unroll
+        for (int xs = 0; xs < XS; xs++)
+#pragma unroll
           for (int nb = 0; nb < NB; nb++)
-            acc[r][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[r][hf], b_cur[nb][hf], acc[r][nb], 0, 0, 0);
-    };
-    load_pair(p0, a_cur, b_cur);
-    // all but the last pair: fetch the next pair (unconditionally: it exists), multiply the current one
-    int64_t pr = p0;
-    for (; pr + GV_WAVES < p1; pr += GV_WAVES) {
-      bf16x8_t a_nxt[R][2], b_nxt[NB][2];
-      load_pair(pr + GV_WAVES, a_nxt, b_nxt);
-      multiply();
 #pragma unroll
-      for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) a_cur[r][hf] = a_nxt[r][hf];
-#pragma unroll
-      for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) b_cur[nb][hf] = b_nxt[nb][hf];
+            for (int hf = 0; hf < 2; hf++) b_cur[d][xs][nb][hf] = b_nxt[d][xs][nb][hf];
+      }
     }
     multiply();
   }
@@ -201,68 +288,74 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_kernel(const uint16_t* __rest
       }
     }
   } else {
+    // 512 / (16 NB) lanes per batch row: each folds its share of the 16 R rows, then a butterfly inside the
+    // lane group.  (value, index) travel as one 64-bit key whose unsigned maximum is torch.argmax's choice.
     const int64_t n0 = (int64_t)blockIdx.x * (16 * R);
-    for (int b = wave; b < B; b += GV_WAVES) {
-      float bv = 0.f;
-      int64_t bi = INT64_MAX;
-      bool have = false;
-      for (int rl = lane; rl < 16 * R; rl += 64) {
+    constexpr int TPB = GV_THREADS / (16 * NB);
+    const int b = tid / TPB, sub = tid % TPB;
+    uint64_t key = 0;
+    if (b < B)
+      for (int rl = sub; rl < 16 * R; rl += TPB) {
         const int64_t n = n0 + rl;
         if (n < N) {
-          const float v = fin[b][rl];
-          if (!have || arg_better(v, n, bv, bi)) {
-            bv = v;
-            bi = n;
-            have = true;
-          }
+          const uint64_t kk = arg_key(fin[b][rl], n);
+          key = kk > key ? kk : key;
         }
       }
 #pragma unroll
-      for (int o = 32; o > 0; o >>= 1) {
-        const float ov = __shfl_xor(bv, o, 64);
-        const int64_t oi = __shfl_xor(bi, o, 64);
-        const int oh = __shfl_xor((int)have, o, 64);
-        if (oh && (!have || arg_better(ov, oi, bv, bi))) {
-          bv = ov;
-          bi = oi;
-          have = true;
-        }
-      }
-      if (lane == 0) part[(int64_t)blockIdx.x * B + b] = ArgPart{bv, (int32_t)bi};
+    for (int o = TPB / 2; o > 0; o >>= 1) {
+      const uint64_t ok = (uint64_t)__shfl_xor((long long)key, o, 64);
+      key = ok > key ? ok : key;
     }
+    if (sub == 0 && b < B) part[(int64_t)blockIdx.x * B + b] = ArgPart{arg_key_value(key), arg_key_index(key)};
   }
 }
 
+// One workgroup per batch row folds that row's per-workgroup partials.
 __global__ __launch_bounds__(256) void argmax_finish_kernel(const ArgPart* __restrict__ part, int n_part, int B,
                                                             int64_t* __restrict__ idx, float* __restrict__ maxval) {
+  const int b = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  for (int b = wave; b < B; b += 4) {
-    float bv = 0.f;
-    int64_t bi = INT64_MAX;
-    bool have = false;
-    for (int p = lane; p < n_part; p += 64) {
-      const ArgPart a = part[(int64_t)p * B + b];
-      if (!have || arg_better(a.v, a.i, bv, bi)) {
-        bv = a.v;
-        bi = a.i;
-        have = true;
-      }
+  float bv = 0.f;
+  int64_t bi = INT64_MAX;
+  bool have = false;
+  for (int p = threadIdx.x; p < n_part; p += 256) {
+    const ArgPart a = part[(int64_t)p * B + b];
+    if (!have || arg_better(a.v, a.i, bv, bi)) {
+      bv = a.v;
+      bi = a.i;
+      have = true;
     }
+  }
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(bv, o, 64);
-      const int64_t oi = __shfl_xor(bi, o, 64);
-      const int oh = __shfl_xor((int)have, o, 64);
-      if (oh && (!have || arg_better(ov, oi, bv, bi))) {
-        bv = ov;
-        bi = oi;
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, 64);
+    const int64_t oi = __shfl_xor(bi, o, 64);
+    const int oh = __shfl_xor((int)have, o, 64);
+    if (oh && (!have || arg_better(ov, oi, bv, bi))) {
+      bv = ov;
+      bi = oi;
+      have = true;
+    }
+  }
+  __shared__ float sv[4];
+  __shared__ int64_t si[4];
+  __shared__ int sh[4];
+  if (lane == 0) {
+    sv[wave] = bv;
+    si[wave] = bi;
+    sh[wave] = have;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int wv = 1; wv < 4; wv++)
+      if (sh[wv] && (!have || arg_better(sv[wv], si[wv], bv, bi))) {
+        bv = sv[wv];
+        bi = si[wv];
         have = true;
       }
-    }
-    if (lane == 0) {
-      idx[b] = bi;
-      if (maxval) maxval[b] = bv;
-    }
+    idx[b] = bi;
+    if (maxval) maxval[b] = bv;
   }
 }
 
@@ -318,54 +411,71 @@ __global__ __launch_bounds__(256) void argmax_rows_kernel(const T* __restrict__ 
   }
 }
 
-int pick_rows_per_wg(int64_t B, int64_t N, int64_t K, int mode) {
-  const char* e = getenv("MTP_GEMV_R");
-  if (e) {
+struct GemvCfg {
+  int R;  // 16-row groups per workgroup
+  int D;  // k-pairs in flight per wave and step
+};
+
+bool depth_ok(int64_t K, int d) { return d == 1 || (K % 64 == 0 && ((K / 64) % (GV_WAVES * d)) == 0); }
+
+GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode) {
+  const int64_t groups = ((mode == 1 ? N / 2 : N) + 15) / 16 * (mode == 1 ? 2 : 1);
+  // Bytes in flight are what a bandwidth-bound kernel lives on: R*D k-pairs (2 KiB each) per wave.  Large
+  // matrices take them as rows (X is re-read from L2 once per 16*R rows, which is what batches above 16
+  // care about); matrices with few row groups keep every CU busy by going deeper along k instead.
+  // Measured on 128256x4096, 28672x4096, 6144x4096, 4096x14336, 8192x3584 and 1280x8192 at B = 1, 8, 32.
+  GemvCfg c{B > 16 ? 8 : 4, 1};
+  while (c.R > 1 && groups / c.R < 190) c.R >>= 1;
+  if (mode == 1 && c.R < 2) c.R = 2;
+  c.D = (B > 16 || c.R >= 4) ? 1 : 2;
+  while (!depth_ok(K, c.D)) c.D >>= 1;
+  if (const char* e = getenv("MTP_GEMV_R")) {
     const int r = atoi(e);
-    if (r == 1 || r == 2 || r == 4 || r == 8) return (mode == 1 && r == 1) ? 2 : r;
+    if (r == 1 || r == 2 || r == 4 || r == 8) c.R = (mode == 1 && r == 1) ? 2 : r;
+    if (c.R * c.D > 4) c.D = c.R >= 4 ? 1 : 4 / c.R;
   }
-  // Aim for at least ~2 workgroups per CU (256 CUs); more rows per workgroup
-  // means fewer re-reads of X from L2.
-  const int64_t groups = (N + 15) / 16;
-  // Measured on the 128256 x 4096 LM head: 4 groups for B <= 16 (2 workgroups per CU), 8 for larger
-  // batches (fewer re-reads of X); small matrices want at least ~2 workgroups per CU.
-  int r = B > 16 ? 8 : 4;
-  while (r > 1 && groups / r < 512) r >>= 1;
-  if (mode == 1 && r < 2) r = 2;
-  (void)K;
-  return r;
+  if (const char* e = getenv("MTP_GEMV_D")) {
+    const int d = atoi(e);
+    if ((d == 1 || d == 2 || d == 4) && c.R * d <= 4 && depth_ok(K, d)) c.D = d;
+  }
+  if (c.R >= 4) c.D = 1;
+  return c;
 }
 
 template <int MODE>
 int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart* part, int64_t B, int64_t N,
-                int64_t K, int R, hipStream_t s, unsigned* n_wg_out) {
+                int64_t K, GemvCfg cfg, hipStream_t s, unsigned* n_wg_out) {
+  const int R = cfg.R;
   const int64_t rows_per_wg = (MODE == 1) ? 8 * R : 16 * R;
   const int64_t span = (MODE == 1) ? N / 2 : N;
   const unsigned n_wg = (unsigned)((span + rows_per_wg - 1) / rows_per_wg);
   if (n_wg_out) *n_wg_out = n_wg;
   const int NB = B > 16 ? 2 : 1;
-#define GV_LAUNCH(RR, NNB)                                                                                      \
-  do {                                                                                                          \
-    if (K % 64 == 0)                                                                                            \
-      hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, false>), dim3(n_wg), dim3(GV_THREADS), 0, s,               \
-                         (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part,     \
-                         (int)B, N, K);                                                                         \
-    else                                                                                                        \
-      hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, true>), dim3(n_wg), dim3(GV_THREADS), 0, s,                \
-                         (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part,     \
-                         (int)B, N, K);                                                                         \
+  int rot_mul = 1;
+  if (const char* e = getenv("MTP_GEMV_ROT")) rot_mul = atoi(e);
+#define GV_LAUNCH(RR, NNB, GG, DD)                                                                              \
+  hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD>), dim3(n_wg), dim3(GV_THREADS), 0, s,                  \
+                     (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part, (int)B, \
+                     N, K, rot_mul)
+#define GV_BY_DEPTH(RR, NNB)                                                   \
+  do {                                                                         \
+    if (K % 64 != 0) GV_LAUNCH(RR, NNB, true, 1);                              \
+    else if (RR * 4 <= 4 && cfg.D == 4) GV_LAUNCH(RR, NNB, false, (RR * 4 <= 4 ? 4 : 1)); \
+    else if (RR * 2 <= 4 && cfg.D == 2) GV_LAUNCH(RR, NNB, false, (RR * 2 <= 4 ? 2 : 1)); \
+    else GV_LAUNCH(RR, NNB, false, 1);                                         \
   } while (0)
   if (NB == 1) {
-    if (R == 8) GV_LAUNCH(8, 1);
-    else if (R == 4) GV_LAUNCH(4, 1);
-    else if (R == 2) GV_LAUNCH(2, 1);
-    else if constexpr (MODE != 1) GV_LAUNCH(1, 1);
+    if (R == 8) GV_BY_DEPTH(8, 1);
+    else if (R == 4) GV_BY_DEPTH(4, 1);
+    else if (R == 2) GV_BY_DEPTH(2, 1);
+    else if constexpr (MODE != 1) GV_BY_DEPTH(1, 1);
   } else {
-    if (R == 8) GV_LAUNCH(8, 2);
-    else if (R == 4) GV_LAUNCH(4, 2);
-    else if (R == 2) GV_LAUNCH(2, 2);
-    else if constexpr (MODE != 1) GV_LAUNCH(1, 2);
+    if (R == 8) GV_BY_DEPTH(8, 2);
+    else if (R == 4) GV_BY_DEPTH(4, 2);
+    else if (R == 2) GV_BY_DEPTH(2, 2);
+    else if constexpr (MODE != 1) GV_BY_DEPTH(1, 2);
   }
+#undef GV_BY_DEPTH
 #undef GV_LAUNCH
   MTP_CHECK_LAUNCH("gemv");
   return MTP_OK;
@@ -395,11 +505,10 @@ extern "C" int mtp_gemv(const void* x, const void* w, const void* bias, void* y,
   hipStream_t s = (hipStream_t)stream;
   if (epilogue == MTP_EPI_SWIGLU) {
     MTP_REQUIRE(N % 2 == 0, MTP_EINVAL, "gemv: SwiGLU needs an even N, got %lld", (long long)N);
-    const int R = pick_rows_per_wg(B, N, K, 1);
-    return launch_gemv<1>(x, w, bias, y, nullptr, B, N, K, R, s, nullptr);
+    return launch_gemv<1>(x, w, bias, y, nullptr, B, N, K, pick_gemv_cfg(B, N, K, 1), s, nullptr);
   }
-  const int R = pick_rows_per_wg(B, N, K, 0);
-  return launch_gemv<0>(x, w, epilogue == MTP_EPI_NONE ? nullptr : bias, y, nullptr, B, N, K, R, s, nullptr);
+  return launch_gemv<0>(x, w, epilogue == MTP_EPI_NONE ? nullptr : bias, y, nullptr, B, N, K,
+                        pick_gemv_cfg(B, N, K, 0), s, nullptr);
 }
 
 extern "C" int64_t mtp_gemv_argmax_workspace_bytes(int64_t B, int64_t N, int64_t K) {
@@ -419,11 +528,10 @@ extern "C" int mtp_gemv_argmax(const void* x, const void* w, int64_t* idx, float
               (long long)mtp_gemv_argmax_workspace_bytes(B, N, K));
   MTP_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7) == 0, MTP_EINVAL, "gemv_argmax: workspace not 8-byte aligned");
   hipStream_t s = (hipStream_t)stream;
-  const int R = pick_rows_per_wg(B, N, K, 2);
   unsigned n_wg = 0;
-  rc = launch_gemv<2>(x, w, nullptr, nullptr, (ArgPart*)workspace, B, N, K, R, s, &n_wg);
+  rc = launch_gemv<2>(x, w, nullptr, nullptr, (ArgPart*)workspace, B, N, K, pick_gemv_cfg(B, N, K, 2), s, &n_wg);
   if (rc) return rc;
-  hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(256), 0, s, (const ArgPart*)workspace, (int)n_wg, (int)B,
+  hipLaunchKernelGGL(argmax_finish_kernel, dim3((unsigned)B), dim3(256), 0, s, (const ArgPart*)workspace, (int)n_wg, (int)B,
                      idx, maxval);
   MTP_CHECK_LAUNCH("argmax_finish");
   return MTP_OK;

@@ -480,6 +480,14 @@ def test_argmax_ties_and_nan(gpu):
     idx, _ = ops.gemv_argmax(x.to(gpu), w.to(gpu))
     assert torch.equal(idx.cpu(), R.greedy_argmax(ref))     # exact ties: the first index wins
     assert all(int(i) <= 5 + 3 or int(i) == int(best[b]) for b, i in enumerate(idx.cpu()))
+    # an all-zero activation row makes every logit equal: index 0, for every batch size class and k layout
+    for bb, kk in ((1, 256), (20, 256), (3, 264)):
+        wz = (torch.randn(n, kk, generator=gen(95)) * 0.02).bfloat16()
+        xz = torch.randn(bb, kk, generator=gen(96)).bfloat16()
+        xz[bb // 2] = 0
+        iz, vz = ops.gemv_argmax(xz.to(gpu), wz.to(gpu))
+        assert torch.equal(iz.cpu(), R.greedy_argmax(F.linear(xz.float(), wz.float()))) and int(iz[bb // 2]) == 0
+        assert float(vz[bb // 2]) == 0.0
     logits = ref.clone()
     logits[1, 700] = float("nan"); logits[1, 800] = float("nan"); logits[2, 3] = float("inf")
     assert torch.equal(greedy_from_logits(logits.to(gpu)).cpu(), R.greedy_argmax(logits))

@@ -232,6 +232,13 @@ def secondary(dev, timer, reps, with_cpu):
     e_ms = timer.run("emb", lambda: ops.embedding_gather(ids, table, 0, v), reps)
     out["embedding_c4"] = {"rows": n, "dim": h, "us": round(e_ms * 1e3, 1),
                            "GBs": round((2 * n * h * 2 + n * 8) / e_ms / 1e6, 1)}
+    # dense gradient: the scatter itself (into an existing table) and with the zero fill of the [V, H] table
+    dout = torch.empty(n, h, dtype=torch.bfloat16, device=dev).normal_(generator=g)
+    dtab = torch.zeros(v, h, dtype=torch.bfloat16, device=dev)
+    eb_ms = timer.run("emb.bwd", lambda: ops.embedding_bwd(ids, dout, v, 0, v, out=dtab), reps)
+    ebz_ms = timer.run("emb.bwd0", lambda: ops.embedding_bwd(ids, dout, v, 0, v), max(3, reps // 4))
+    out["embedding_c4"].update({"bwd_scatter_us": round(eb_ms * 1e3, 1), "bwd_with_zero_fill_us": round(ebz_ms * 1e3, 1)})
+    del dout, dtab
     # --- decode step: QKV, gate/up+SwiGLU, down, LM head + argmax (the table doubles as the LM head)
     mk = lambda nn, kk: torch.empty(nn, kk, device=dev).normal_(0, 0.02, generator=g).bfloat16()
     wq, wg, wd = mk(6144, 4096), mk(2 * 14336, 4096), mk(4096, 14336)

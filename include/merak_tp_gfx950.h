@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTP_ABI_VERSION 1
+#define MTP_ABI_VERSION 2
 
 /* element types */
 #define MTP_F32  0
@@ -115,11 +115,18 @@ int mtp_embedding_gather(const int64_t* ids, const void* table, void* out,
                          int32_t* oob_count, void* stream);
 
 /* Dense gradient of the lookup: dtable[ids[i]-vocab_start,:] += dout[i,:]
- * for in-range ids, accumulated in fp32 (dtable is fp32 [rows,dim]).  This is
- * the embedding_dense_backward ATen runs behind F.embedding (layers.py:156).
- * The caller zeroes dtable first unless it wants accumulation. */
-int mtp_embedding_bwd(const int64_t* ids, const void* dout, float* dtable,
-                      int64_t n_ids, int64_t dim, int dtype,
+ * for in-range ids; dtable is [rows,dim] of dtable_dtype (fp32, or bf16 for
+ * bf16 dout).  This is the embedding_dense_backward ATen runs behind
+ * F.embedding (layers.py:156).  Tokens that share an id are summed in
+ * ascending token order in fp32 and added to the table row once, so the
+ * result is reproducible bit for bit.  The caller zeroes dtable first unless
+ * it wants accumulation, e.g. onto the LM-head weight gradient when the two
+ * are tied (Merak/core/pipeline/module.py:646-662).  workspace: device scratch
+ * of mtp_embedding_bwd_workspace_bytes(n_ids) bytes, 8-byte aligned. */
+int64_t mtp_embedding_bwd_workspace_bytes(int64_t n_ids);
+int mtp_embedding_bwd(const int64_t* ids, const void* dout, void* dtable,
+                      void* workspace, int64_t workspace_bytes,
+                      int64_t n_ids, int64_t dim, int dtype, int dtable_dtype,
                       int64_t vocab_start, int64_t vocab_end, void* stream);
 
 /* ------------------------------------------------------------------------

@@ -30,25 +30,70 @@ __global__ __launch_bounds__(256) void embedding_gather_kernel(const int64_t* __
   }
 }
 
-// dtable[id - start, :] += dout[i, :]  (fp32 atomics; one thread per element pair)
-template <typename T>
+// ---- dense gradient of the lookup ---------------------------------------------
+// dtable[id - start, :] += sum of dout[i, :] over the tokens i with ids[i] == id, added in ascending i with
+// fp32 accumulation: the result does not depend on scheduling (no atomics on the gradient).
+//
+// Pass 1 (one workgroup per token) chains the tokens of equal id: leader[i] = no earlier token has this id,
+// next[i] = the next later token with it (or -1).  Pass 2 (one workgroup per token and 1024-column chunk)
+// lets each leader walk its chain and write its table row once.  Pass 1 compares every pair of tokens
+// (n^2 / 2 id loads from L2), which is a few tens of microseconds at 8192 tokens.
+struct TokenLink {
+  int32_t next;    // next token with the same id, -1 at the end of the chain
+  int32_t leader;  // 1: first token of its id (and the id is in range)
+};
+
+__global__ __launch_bounds__(256) void embedding_link_kernel(const int64_t* __restrict__ ids,
+                                                             TokenLink* __restrict__ link, int n_ids,
+                                                             int64_t vocab_start, int64_t vocab_end) {
+  const int i = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int64_t id = ids[i];
+  if (id < vocab_start || id >= vocab_end) {
+    if (tid == 0) link[i] = TokenLink{-1, 0};
+    return;
+  }
+  int dup = 0;
+  for (int j = tid; j < i; j += 256) dup |= ids[j] == id;
+  dup = __syncthreads_or(dup);
+  __shared__ int first_after;
+  if (tid == 0) first_after = INT32_MAX;
+  __syncthreads();
+  for (int base = i + 1; base < n_ids; base += 256) {
+    const int j = base + tid;
+    const int hit = j < n_ids && ids[j] == id;
+    if (hit) atomicMin(&first_after, j);
+    if (__syncthreads_or(hit)) break;
+  }
+  if (tid == 0) link[i] = TokenLink{first_after == INT32_MAX ? -1 : first_after, dup ? 0 : 1};
+}
+
+template <typename T, typename TO>
 __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t* __restrict__ ids,
-                                                            const T* __restrict__ dout, float* __restrict__ dtable,
-                                                            int64_t n_ids, int64_t dim, int64_t vocab_start,
-                                                            int64_t vocab_end) {
-  const int64_t total = n_ids * dim;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int64_t r = i / dim;
-    const int64_t c = i - r * dim;
-    const int64_t id = ids[r];
-    if (id < vocab_start || id >= vocab_end) continue;
-    float g;
-    if constexpr (sizeof(T) == 2)
-      g = bf16_bits_to_f32(dout[i]);
+                                                            const T* __restrict__ dout, TO* __restrict__ dtable,
+                                                            const TokenLink* __restrict__ link, int64_t dim,
+                                                            int64_t vocab_start) {
+  const int i = blockIdx.x;
+  if (!link[i].leader) return;
+  const int64_t c0 = ((int64_t)blockIdx.y * 256 + threadIdx.x) * 4;
+  if (c0 >= dim) return;
+  const int nc = dim - c0 < 4 ? (int)(dim - c0) : 4;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int j = i; j >= 0; j = link[j].next) {
+    const T* src = dout + (int64_t)j * dim + c0;
+    for (int e = 0; e < nc; e++) {
+      if constexpr (sizeof(T) == 2)
+        acc[e] += bf16_bits_to_f32(src[e]);
+      else
+        acc[e] += src[e];
+    }
+  }
+  TO* dst = dtable + (ids[i] - vocab_start) * dim + c0;
+  for (int e = 0; e < nc; e++) {
+    if constexpr (sizeof(TO) == 2)
+      dst[e] = f32_to_bf16_bits(bf16_bits_to_f32(dst[e]) + acc[e]);
     else
-      g = dout[i];
-    unsafeAtomicAdd(dtable + (id - vocab_start) * dim + c, g);
+      dst[e] += acc[e];
   }
 }
 
@@ -85,23 +130,44 @@ extern "C" int mtp_embedding_gather(const int64_t* ids, const void* table, void*
   return launch_gather<uint8_t>(ids, table, out, n_ids, row_bytes, vocab_start, vocab_end, oob_count, s);
 }
 
-extern "C" int mtp_embedding_bwd(const int64_t* ids, const void* dout, float* dtable, int64_t n_ids, int64_t dim,
-                                 int dtype, int64_t vocab_start, int64_t vocab_end, void* stream) {
+extern "C" int64_t mtp_embedding_bwd_workspace_bytes(int64_t n_ids) {
+  return n_ids > 0 ? n_ids * (int64_t)sizeof(TokenLink) : 0;
+}
+
+extern "C" int mtp_embedding_bwd(const int64_t* ids, const void* dout, void* dtable, void* workspace,
+                                 int64_t workspace_bytes, int64_t n_ids, int64_t dim, int dtype, int dtable_dtype,
+                                 int64_t vocab_start, int64_t vocab_end, void* stream) {
   MTP_REQUIRE(n_ids >= 0 && dim >= 1, MTP_EINVAL, "embedding_bwd: n_ids=%lld dim=%lld", (long long)n_ids,
               (long long)dim);
+  MTP_REQUIRE(n_ids < (1ll << 31), MTP_EUNSUPPORTED, "embedding_bwd: n_ids=%lld exceeds 2^31-1", (long long)n_ids);
   MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16, MTP_EINVAL, "embedding_bwd: unknown dtype %d", dtype);
+  MTP_REQUIRE(dtable_dtype == MTP_F32 || dtable_dtype == MTP_BF16, MTP_EINVAL,
+              "embedding_bwd: unknown dtable_dtype %d", dtable_dtype);
   if (n_ids == 0) return MTP_OK;
-  MTP_REQUIRE(ids && dout && dtable, MTP_EINVAL, "embedding_bwd: null pointer");
+  MTP_REQUIRE(ids && dout && dtable && workspace, MTP_EINVAL, "embedding_bwd: null pointer");
+  MTP_REQUIRE(workspace_bytes >= mtp_embedding_bwd_workspace_bytes(n_ids), MTP_EWORKSPACE,
+              "embedding_bwd: workspace %lld < %lld bytes", (long long)workspace_bytes,
+              (long long)mtp_embedding_bwd_workspace_bytes(n_ids));
+  MTP_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7) == 0, MTP_EINVAL, "embedding_bwd: workspace not 8-byte aligned");
+  const int64_t chunks = (dim + 1023) / 1024;
+  MTP_REQUIRE(chunks <= 65535, MTP_EUNSUPPORTED, "embedding_bwd: dim=%lld too large", (long long)dim);
   hipStream_t s = (hipStream_t)stream;
-  const int64_t total = n_ids * dim;
-  int64_t blocks = (total + 255) / 256;
-  if (blocks > 256 * 64) blocks = 256 * 64;
-  if (dtype == MTP_F32)
-    hipLaunchKernelGGL(embedding_bwd_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, s, ids, (const float*)dout,
-                       dtable, n_ids, dim, vocab_start, vocab_end);
+  TokenLink* link = (TokenLink*)workspace;
+  hipLaunchKernelGGL(embedding_link_kernel, dim3((unsigned)n_ids), dim3(256), 0, s, ids, link, (int)n_ids,
+                     vocab_start, vocab_end);
+  MTP_CHECK_LAUNCH("embedding_link");
+  const dim3 grid((unsigned)n_ids, (unsigned)chunks), block(256);
+  if (dtype == MTP_F32 && dtable_dtype == MTP_F32)
+    hipLaunchKernelGGL((embedding_bwd_kernel<float, float>), grid, block, 0, s, ids, (const float*)dout,
+                       (float*)dtable, link, dim, vocab_start);
+  else if (dtype == MTP_BF16 && dtable_dtype == MTP_F32)
+    hipLaunchKernelGGL((embedding_bwd_kernel<uint16_t, float>), grid, block, 0, s, ids, (const uint16_t*)dout,
+                       (float*)dtable, link, dim, vocab_start);
+  else if (dtype == MTP_BF16 && dtable_dtype == MTP_BF16)
+    hipLaunchKernelGGL((embedding_bwd_kernel<uint16_t, uint16_t>), grid, block, 0, s, ids, (const uint16_t*)dout,
+                       (uint16_t*)dtable, link, dim, vocab_start);
   else
-    hipLaunchKernelGGL(embedding_bwd_kernel<uint16_t>, dim3((unsigned)blocks), dim3(256), 0, s, ids,
-                       (const uint16_t*)dout, dtable, n_ids, dim, vocab_start, vocab_end);
+    MTP_REQUIRE(false, MTP_EUNSUPPORTED, "embedding_bwd: fp32 gradients into a bf16 table are not supported");
   MTP_CHECK_LAUNCH("embedding_bwd");
   return MTP_OK;
 }

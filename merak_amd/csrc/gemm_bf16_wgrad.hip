@@ -1,9 +1,8 @@
 // dW[N,K] (+)= dY[M,N]^T X[M,K]: GEMM (N, K, reduce M) with both operands transposed (col).
 #include "gemm_bf16_kernel.h"
 
-int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
-                        int dw_dtype, int accumulate, hipStream_t s) {
-  if (db) return MTP_EUNSUPPORTED;  // bias gradient: served by the general path
+int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, int64_t M, int64_t N, int64_t K, int dw_dtype,
+                        int accumulate, hipStream_t s) {
   GemmArgs a{};
   a.A = (const uint16_t*)dy;
   a.B = (const uint16_t*)x;

@@ -125,8 +125,9 @@ class _EmbeddingFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         (ids,) = ctx.saved_tensors
-        dtable = ops.embedding_bwd(ids, grad_out, ctx.wshape[0], *ctx.range)
-        return None, dtable.to(ctx.wdtype), None, None
+        grad_out = grad_out if grad_out.dtype == ctx.wdtype else grad_out.to(ctx.wdtype)
+        dtable = ops.embedding_bwd(ids, grad_out, ctx.wshape[0], *ctx.range, dtype=ctx.wdtype)
+        return None, dtable, None, None
 
 
 # --------------------------------------------------------------------------- modules

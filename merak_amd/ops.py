@@ -162,17 +162,28 @@ def embedding_gather(ids: torch.Tensor, table: torch.Tensor, vocab_start: int, v
     return out.view(*ids.shape, table.shape[1])
 
 
-def embedding_bwd(ids: torch.Tensor, dout: torch.Tensor, rows: int, vocab_start: int, vocab_end: int) -> torch.Tensor:
-    """Dense fp32 gradient [rows, dim] of the lookup."""
-    dev = _require_gpu(ids, dout)
+def embedding_bwd(ids: torch.Tensor, dout: torch.Tensor, rows: int, vocab_start: int, vocab_end: int,
+                  out: Optional[torch.Tensor] = None, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Dense gradient [rows, dim] of the lookup, reproducible bit for bit.
+
+    ``out`` given: the gradient is added onto it (e.g. the tied LM head's weight gradient);
+    otherwise a zero-filled table of ``dtype`` (default: dout's) is created."""
+    dev = _require_gpu(ids, dout, out)
     flat = _contig(ids).view(-1)
     dim = dout.shape[-1]
     d2 = _contig(dout).view(-1, dim)
-    dtable = torch.zeros((rows, dim), dtype=torch.float32, device=dev)
+    if flat.dtype != torch.int64:
+        raise TypeError(f"embedding ids must be int64, got {flat.dtype}")
+    if out is None:
+        out = torch.zeros((rows, dim), dtype=dtype or d2.dtype, device=dev)
+    elif tuple(out.shape) != (rows, dim) or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous [{rows}, {dim}] tensor")
+    lib = _lib.lib()
+    ws = torch.empty((max(int(lib.mtp_embedding_bwd_workspace_bytes(flat.numel())), 8),), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().mtp_embedding_bwd(_p(flat), _p(d2), _p(dtable), flat.numel(), dim, _dt(d2), vocab_start,
-                                                vocab_end, _stream(dev)), "mtp_embedding_bwd")
-    return dtable
+        _lib.check(lib.mtp_embedding_bwd(_p(flat), _p(d2), _p(out), _p(ws), ws.numel(), flat.numel(), dim, _dt(d2),
+                                         _dt(out), vocab_start, vocab_end, _stream(dev)), "mtp_embedding_bwd")
+    return out
 
 
 # --------------------------------------------------------------------------- cross entropy

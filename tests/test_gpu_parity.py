@@ -292,13 +292,44 @@ def test_embedding_module_forward_backward(gpu):
     out.backward(dout.to(gpu))
     ref = R.embedding_backward(ids, dout, 512, 0, 512)
     assert emb.weight.grad.dtype == torch.bfloat16 and rel(emb.weight.grad, ref) < TOL_BF16
-    dt = ops.embedding_bwd(ids.to(gpu), dout.to(gpu), 512, 0, 512)
-    assert rel(dt, ref) < TOL_F32
+    dt = ops.embedding_bwd(ids.to(gpu), dout.to(gpu), 512, 0, 512, dtype=torch.float32)
+    assert dt.dtype == torch.float32 and rel(dt, ref) < TOL_F32
     empty = ops.embedding_gather(torch.empty(0, dtype=torch.int64, device=gpu), emb.weight.detach(), 0, 512)
     assert empty.shape == (0, 64)
     oob = torch.zeros(1, dtype=torch.int32, device=gpu)
     ops.embedding_gather(torch.tensor([1, 600, -3], device=gpu), emb.weight.detach(), 0, 512, oob)
     assert oob.item() == 2
+
+
+@pytest.mark.parametrize("dtype,n,v,h,lo,hi", [
+    (torch.bfloat16, 4096, 1000, 4096, 0, 1000),      # many repeats per id
+    (torch.float32, 513, 64, 77, 0, 64),              # row length not a multiple of 4
+    (torch.bfloat16, 700, 4000, 1030, 1000, 2000),    # one rank's vocabulary slice: ids outside it contribute nothing
+    (torch.bfloat16, 300, 16, 8, 0, 16),
+])
+def test_embedding_backward_reproducible(gpu, dtype, n, v, h, lo, hi):
+    ids = torch.randint(0, v, (n,), generator=gen(27))
+    ids[: n // 3] = lo + 1                                     # one id carried by a third of the tokens
+    dout = torch.randn(n, h, generator=gen(28)).to(dtype)
+    ref = R.embedding_backward(ids, dout, hi - lo, lo, hi)
+    a = ops.embedding_bwd(ids.to(gpu), dout.to(gpu), hi - lo, lo, hi, dtype=torch.float32)
+    b = ops.embedding_bwd(ids.to(gpu), dout.to(gpu), hi - lo, lo, hi, dtype=torch.float32)
+    assert rel(a, ref) < TOL_F32 and torch.equal(a, b), "same inputs, same bits"
+    # the documented order: ascending token index, fp32 running sum
+    seq = torch.zeros(h)
+    for i in range(n // 3):
+        seq += dout[i].float()
+    extra = (ids[n // 3:] == lo + 1).nonzero().flatten() + n // 3
+    for i in extra.tolist():
+        seq += dout[i].float()
+    assert torch.equal(a[1].cpu(), seq)
+    # accumulation onto an existing gradient (tied LM head), in the table's own dtype
+    base = torch.randn(hi - lo, h, generator=gen(29)).to(dtype)
+    tied = ops.embedding_bwd(ids.to(gpu), dout.to(gpu), hi - lo, lo, hi, out=base.to(gpu))
+    assert tied.dtype == dtype and rel(tied, ref + base.float()) < (TOL_F32 if dtype == torch.float32 else TOL_BF16)
+    untouched = torch.ones(hi - lo, dtype=torch.bool)
+    untouched[ids[(ids >= lo) & (ids < hi)] - lo] = False
+    assert torch.equal(tied.cpu()[untouched], base[untouched])
 
 
 def test_embedding_full_size_llama_table(gpu):

@@ -41,7 +41,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM bytes per launch of the gate/up GEMMs, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file
 # scaled by a 1 GiB copy kernel (x2.000 / x1.000): profiles/hbm_traffic_fetch_write_size.txt
-HBM_TRAFFIC_BYTES = {"gate_up.fwd": 1.860e9, "gate_up.wgrad": 1.644e9, "gate_up.dgrad": 0.889e9}
+HBM_TRAFFIC_BYTES = {"gate_up.fwd": 1.805e9, "gate_up.wgrad": 1.645e9, "gate_up.dgrad": 0.889e9}
 
 LLAMA8B = [  # (name, K, N, epilogue)
     ("qkv", 4096, 6144, "none"),
@@ -290,9 +290,13 @@ def secondary(dev, timer, reps, with_cpu):
     c_ms = timer.run("copy", lambda: _lib.check(_lib.lib().mtp_stream_copy(src.data_ptr(), dst.data_ptr(), src.numel(), st), "copy"), reps)
     sink = torch.empty(64 * 4096, device=dev)
     iters = 8192
-    p_ms = timer.run("mfma", lambda: _lib.check(_lib.lib().mtp_mfma_peak(sink.data_ptr(), 4096, iters, st), "peak"), 3)
+    # register-resident MFMA loop, no memory traffic at all: what the matrix cores sustain under the power
+    # limit with smooth operands and with operands of random sign and mantissa (what N(0,1) data looks like)
+    p_ms = timer.run("mfma", lambda: _lib.check(_lib.lib().mtp_mfma_peak(sink.data_ptr(), 4096, iters, 0, st), "peak"), 3)
+    r_ms = timer.run("mfma_r", lambda: _lib.check(_lib.lib().mtp_mfma_peak(sink.data_ptr(), 4096, iters, 1, st), "peak"), 3)
     out["device_reference"] = {"copy_1GiB_GBs_read_plus_write": round(2 * src.numel() / c_ms / 1e6, 1),
-                               "mfma_loop_bf16_tflops": round(4096 * iters * 32 * 32 * 16 * 2 / p_ms / 1e9, 1)}
+                               "mfma_loop_bf16_tflops_smooth_operands": round(4096 * iters * 32 * 32 * 16 * 2 / p_ms / 1e9, 1),
+                               "mfma_loop_bf16_tflops_random_operands": round(4096 * iters * 32 * 32 * 16 * 2 / r_ms / 1e9, 1)}
     return out
 
 
@@ -340,7 +344,14 @@ def main():
                 "unit": "TFLOP/s", "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4),
                 "traffic": HBM_TRAFFIC_BYTES.get(dom["kernel"]),
                 "launch_ms": dom["ms"], "flops_per_launch": 2.0 * dom["M"] * dom["N"] * dom["K"]}
-    del work
+    # what the matrix cores sustain on this board with no memory traffic at all (register-resident MFMA loop on
+    # operands of random sign and mantissa): the chip runs against its power limit well below the published peak
+    sink = torch.empty(64 * 4096, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    r_ms = timer.run("mfma_r", lambda: _lib.check(_lib.lib().mtp_mfma_peak(sink.data_ptr(), 4096, 8192, 1, st), "peak"), 3)
+    roofline["mfma_loop_random_operands"] = round(4096 * 8192 * 32 * 32 * 16 * 2 / r_ms / 1e9, 1)
+    roofline["frac_of_mfma_loop"] = round(dom["tflops"] / roofline["mfma_loop_random_operands"], 4)
+    del work, sink
     result = {
         "metric": "TP-shard linear fwd+bwd TFLOP/s (% bf16 peak); vocab-CE HBM GB/s",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

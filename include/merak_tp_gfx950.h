@@ -223,9 +223,12 @@ int mtp_argmax_rows(const void* logits, int64_t* idx,
 /* dst[0:bytes] = src[0:bytes] with 16-byte accesses; bytes % 16 == 0. */
 int mtp_stream_copy(const void* src, void* dst, int64_t bytes, void* stream);
 /* Register-resident bf16 MFMA loop: iters x 32x32x16 MFMAs per wave on
- * `waves_per_cu * cu_count` waves; writes one float per lane to sink
- * (>= 64*waves floats).  Reports nothing itself: time it with events. */
-int mtp_mfma_peak(float* sink, int64_t n_waves, int64_t iters, void* stream);
+ * n_waves waves (iters a multiple of 16); writes one float per lane to sink
+ * (>= 64*n_waves floats).  random_data != 0 feeds operands with random
+ * signs and mantissas, 0 feeds smooth small values: the sustained rate differs
+ * because the chip runs against its power limit.  Reports nothing itself:
+ * time it with events. */
+int mtp_mfma_peak(float* sink, int64_t n_waves, int64_t iters, int random_data, void* stream);
 
 #ifdef __cplusplus
 }

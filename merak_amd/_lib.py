@@ -45,7 +45,7 @@ SIGNATURES = {
     "mtp_gemv_argmax": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "mtp_argmax_rows": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "mtp_stream_copy": (_int, [_vp, _vp, _i64, _vp]),
-    "mtp_mfma_peak": (_int, [_vp, _i64, _i64, _vp]),
+    "mtp_mfma_peak": (_int, [_vp, _i64, _i64, _int, _vp]),
 }
 
 _lock = threading.Lock()

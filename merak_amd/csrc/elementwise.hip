@@ -113,20 +113,44 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(const u32x4_t* __restr
   for (; i < nvec; i += stride) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
-__global__ __launch_bounds__(256) void mfma_peak_kernel(float* __restrict__ sink, int64_t iters) {
+// Register-resident MFMA loop.  What the matrix cores sustain depends on the operand bits, because the chip
+// runs against a power limit: `random_data` fills the four A and four B fragments with pseudo-random
+// mantissas and signs (exponents around 1.0, like N(0,1) activations); otherwise they hold small smooth
+// values that toggle few wires.  Fragments rotate so that consecutive MFMAs see different operands.
+__global__ __launch_bounds__(256) void mfma_peak_kernel(float* __restrict__ sink, int64_t iters, int random_data) {
   const int lane = threadIdx.x & 63;
-  bf16x8_t a, b;
+  bf16x8_t a[4], b[4];
+  uint32_t rng = 0x9e3779b9u * (uint32_t)(blockIdx.x * 256 + threadIdx.x + 1);
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
-    a[i] = (__bf16)(0.001f * (lane + i));
-    b[i] = (__bf16)(0.002f * (lane - i));
+  for (int f = 0; f < 4; f++) {
+    u32x4_t ra, rb;
+    uint32_t* pa = reinterpret_cast<uint32_t*>(&ra);
+    uint32_t* pb = reinterpret_cast<uint32_t*>(&rb);
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      if (random_data) {
+        // two bf16 per word: sign and 7 mantissa bits random, exponent 0x7e..0x7f (values in +-[0.5, 2))
+        rng ^= rng << 13; rng ^= rng >> 17; rng ^= rng << 5;
+        pa[q] = (rng & 0x80ff80ffu) | 0x3f003f00u;
+        rng ^= rng << 13; rng ^= rng >> 17; rng ^= rng << 5;
+        pb[q] = (rng & 0x80ff80ffu) | 0x3f003f00u;
+      } else {
+        pa[q] = pack_bf16x2(0.001f * (lane + 2 * q + f), 0.001f * (lane + 2 * q + 1 + f));
+        pb[q] = pack_bf16x2(0.002f * (lane - 2 * q - f), 0.002f * (lane - 2 * q - 1 - f));
+      }
+    }
+    a[f] = __builtin_bit_cast(bf16x8_t, ra);
+    b[f] = __builtin_bit_cast(bf16x8_t, rb);
   }
   f32x16_t c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
-  for (int64_t it = 0; it < iters; it += 4) {
-    c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c0, 0, 0, 0);
-    c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c1, 0, 0, 0);
-    c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c2, 0, 0, 0);
-    c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c3, 0, 0, 0);
+  for (int64_t it = 0; it < iters; it += 16) {
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[f], b[f], c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[f], b[(f + 1) & 3], c1, 0, 0, 0);
+      c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[f], b[(f + 2) & 3], c2, 0, 0, 0);
+      c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[f], b[(f + 3) & 3], c3, 0, 0, 0);
+    }
   }
   float s = 0.f;
 #pragma unroll
@@ -203,10 +227,11 @@ extern "C" int mtp_stream_copy(const void* src, void* dst, int64_t bytes, void* 
   return MTP_OK;
 }
 
-extern "C" int mtp_mfma_peak(float* sink, int64_t n_waves, int64_t iters, void* stream) {
-  MTP_REQUIRE(sink && n_waves >= 4 && n_waves % 4 == 0 && iters >= 4 && iters % 4 == 0, MTP_EINVAL,
-              "mfma_peak: n_waves and iters must be positive multiples of 4");
-  hipLaunchKernelGGL(mfma_peak_kernel, dim3((unsigned)(n_waves / 4)), dim3(256), 0, (hipStream_t)stream, sink, iters);
+extern "C" int mtp_mfma_peak(float* sink, int64_t n_waves, int64_t iters, int random_data, void* stream) {
+  MTP_REQUIRE(sink && n_waves >= 4 && n_waves % 4 == 0 && iters >= 16 && iters % 16 == 0, MTP_EINVAL,
+              "mfma_peak: n_waves must be a positive multiple of 4 and iters of 16");
+  hipLaunchKernelGGL(mfma_peak_kernel, dim3((unsigned)(n_waves / 4)), dim3(256), 0, (hipStream_t)stream, sink, iters,
+                     random_data);
   MTP_CHECK_LAUNCH("mfma_peak");
   return MTP_OK;
 }

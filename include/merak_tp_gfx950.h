@@ -217,6 +217,23 @@ int mtp_gemv_argmax(const void* x, const void* w,
 int mtp_argmax_rows(const void* logits, int64_t* idx,
                     int64_t B, int64_t V, int dtype, void* stream);
 
+/* Sampling tail of the generation loop
+ * (Merak/inference/text_generation_inference.py:229-235 with top_k_logits,
+ * :35-69): z = float(logits)/temperature; top_k > 0 drops z below the k-th
+ * largest; top_p > 0 drops, in descending order, every token whose
+ * predecessors already hold more than top_p of the remaining softmax mass
+ * (the first token always stays); then one token per row is drawn with
+ * probability softmax(z kept).  The draw replaces torch.multinomial's private
+ * random stream by the caller's uniforms[b] in [0,1): token = first index
+ * whose cumulative kept probability, in index order, exceeds uniforms[b].
+ * logits: [B,V] f32 or bf16, untouched.  tokens (int64 [B]) and filtered
+ * (f32 [B,V]: z where kept, -inf where dropped, what top_k_logits returns) may
+ * each be NULL.  Same inputs give the same outputs bit for bit. */
+int mtp_sample_top_k_top_p(const void* logits, int dtype, int64_t B, int64_t V,
+                           float temperature, int top_k, float top_p,
+                           const float* uniforms, int64_t* tokens, float* filtered,
+                           void* stream);
+
 /* ------------------------------------------------------------------------
  * Measurement helpers (used by bench.py to state what this GPU can do).
  * ------------------------------------------------------------------------ */

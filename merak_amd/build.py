@@ -26,7 +26,7 @@ SOURCES = [
     "vocab_ce.hip",
     "embedding.hip",
     "gemv.hip",
-    "elementwise.hip",
+    "elementwise.hip", "sampling.hip",
     "gemm_bf16_fwd.hip",
     "gemm_bf16_dgrad.hip",
     "gemm_bf16_wgrad.hip",

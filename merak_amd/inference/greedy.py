@@ -29,6 +29,22 @@ def greedy_next_token(hidden: torch.Tensor, lm_head_weight: torch.Tensor,
     return idx
 
 
+def top_k_logits(logits: torch.Tensor, top_k: int = 0, top_p: float = 0.0) -> torch.Tensor:
+    """The reference's filter (text_generation_inference.py:35-69) on fp32 [B, V] logits: a new tensor with
+    ``-inf`` where the reference writes its ``filter_value`` (the reference edits its argument in place)."""
+    return ops.sample_top_k_top_p(logits, 1.0, top_k, top_p, None, want_filtered=True)[1]
+
+
+def sample_next_token(logits: torch.Tensor, temperature: float = 1.0, top_k: int = 0, top_p: float = 0.0,
+                      uniforms: Optional[torch.Tensor] = None, generator: Optional[torch.Generator] = None):
+    """The live branch of the reference's loop (:229-235): ``logits.float() / temperature``, ``top_k_logits``,
+    softmax, one multinomial draw per row.  The draw uses ``uniforms`` (fp32 [B] in [0, 1); drawn from
+    ``generator`` or the default CUDA generator when omitted) instead of ``torch.multinomial``'s own stream."""
+    if uniforms is None:
+        uniforms = torch.rand((logits.shape[0],), device=logits.device, generator=generator)
+    return ops.sample_top_k_top_p(logits, temperature, top_k, top_p, uniforms)[0]
+
+
 class DecodeStep:
     """Single-token pass through QKV, gate/up (+SwiGLU), down and the LM head with fused argmax.
 

@@ -307,3 +307,30 @@ def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
         _lib.check(_lib.lib().mtp_argmax_rows(_p(l2), _p(idx), l2.shape[0], l2.shape[1], _dt(l2), _stream(dev)),
                    "mtp_argmax_rows")
     return idx.view(logits.shape[:-1])
+
+
+def sample_top_k_top_p(logits: torch.Tensor, temperature: float = 1.0, top_k: int = 0, top_p: float = 0.0,
+                       uniforms: Optional[torch.Tensor] = None, want_filtered: bool = False):
+    """-> (tokens int64 [B] or None, filtered fp32 [B, V] or None).
+
+    tokens are drawn when ``uniforms`` (fp32 [B], values in [0, 1)) is given."""
+    dev = _require_gpu(logits, uniforms)
+    if logits.dim() != 2:
+        raise ValueError("sample_top_k_top_p takes [B, V] logits")
+    logits = _contig(logits)
+    B, V = logits.shape
+    tokens = filtered = None
+    if uniforms is not None:
+        uniforms = _contig(uniforms.to(torch.float32)).view(-1)
+        if uniforms.numel() != B:
+            raise ValueError(f"uniforms has {uniforms.numel()} entries for {B} rows")
+        tokens = torch.empty((B,), dtype=torch.int64, device=dev)
+    if want_filtered:
+        filtered = torch.empty((B, V), dtype=torch.float32, device=dev)
+    if tokens is None and filtered is None:
+        raise ValueError("nothing to compute: give uniforms and/or want_filtered=True")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_sample_top_k_top_p(_p(logits), _dt(logits), B, V, float(temperature), int(top_k),
+                                                     float(top_p), _p(uniforms), _p(tokens), _p(filtered),
+                                                     _stream(dev)), "mtp_sample_top_k_top_p")
+    return tokens, filtered

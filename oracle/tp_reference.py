@@ -257,3 +257,34 @@ def decode_step(x, w_qkv, w_gate_up, w_down, w_lm_head):
     out = lin(h, w_down).to(x.dtype)
     logits = lin(out, w_lm_head)
     return qkv, out, logits, greedy_argmax(logits)
+
+
+def top_k_logits(logits, top_k=0, top_p=0.0, filter_value=-float("inf")):
+    """top_k_logits of Merak/inference/text_generation_inference.py:35-69, op for op, IN PLACE on ``logits``
+    ([B, V] fp32) like the reference."""
+    if top_k > 0:
+        kth = torch.topk(logits, top_k)[0][..., -1, None]                       # :50
+        logits[logits < kth] = filter_value                                      # :50-51
+    if top_p > 0.0:
+        sorted_logits, sorted_indices = torch.sort(logits, descending=True, dim=-1)   # :55-56
+        cumulative_probs = torch.cumsum(F.softmax(sorted_logits, dim=-1), dim=-1)     # :57-58
+        remove = cumulative_probs > top_p                                        # :61
+        remove[..., 1:] = remove[..., :-1].clone()                               # :64
+        remove[..., 0] = 0                                                       # :65
+        for i in range(sorted_indices.size(0)):                                  # :66-68
+            logits[i][sorted_indices[i][remove[i]]] = filter_value
+    return logits
+
+
+def sample_tail(logits, temperature, top_k, top_p, uniforms):
+    """The sampling branch of the generation loop (:229-235): float(), /= temperature, top_k_logits, softmax,
+    one draw per row.  torch.multinomial's random stream cannot be reproduced outside torch, so the draw is
+    the inverse CDF over the same probabilities in index order (fp64) at the supplied uniforms [B]:
+    token = first j with cumsum(p)[j] > u * sum(p).  Returns (tokens int64 [B], probs fp64 [B, V])."""
+    z = logits.float() / temperature                                             # :230-231
+    z = top_k_logits(z, top_k=top_k, top_p=top_p)                                # :232-233
+    probs = F.softmax(z.double(), dim=-1)                                        # :234
+    cdf = torch.cumsum(probs, dim=-1)
+    target = uniforms.double().view(-1, 1) * cdf[:, -1:]
+    tokens = (cdf <= target).sum(-1).clamp_max(logits.shape[-1] - 1)             # :235 (see above)
+    return tokens, probs

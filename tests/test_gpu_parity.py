@@ -540,3 +540,66 @@ def test_decode_step_llama8b_full_size(gpu, b):
     ref_tok = R.greedy_argmax(F.linear(out.cpu().float(), wl.cpu().float()))
     assert torch.equal(tok.cpu(), ref_tok)
     assert torch.equal(greedy_next_token(out, wl).cpu(), ref_tok)
+
+
+# =============================================================================== sampling tail
+@pytest.mark.parametrize("dtype,b,v,temp,top_k,top_p", [
+    (torch.float32, 4, 1000, 1.0, 0, 0.0), (torch.float32, 4, 1000, 0.7, 10, 0.0), (torch.float32, 4, 1000, 1.3, 0, 0.9),
+    (torch.float32, 8, 50257, 0.9, 50, 0.95), (torch.bfloat16, 8, 128256, 0.8, 40, 0.9),
+    (torch.bfloat16, 3, 128256, 1.0, 0, 0.5), (torch.float32, 2, 7, 1.0, 3, 0.6), (torch.float32, 5, 1, 1.0, 1, 0.9),
+    (torch.float32, 3, 300, 1.0, 300, 0.9999), (torch.bfloat16, 32, 32000, 0.6, 1, 0.0),
+])
+def test_sampling_filter_and_draw_vs_oracle(gpu, dtype, b, v, temp, top_k, top_p):
+    """mtp_sample_top_k_top_p against the restated top_k_logits + softmax + inverse CDF: the filtered logits bit
+    for bit (bf16 logits give many exactly equal values: a tie that straddles the top-p boundary is kept whole
+    here, in part by the reference, so only such ties may differ), the drawn token for the same uniforms."""
+    x = (torch.randn(b, v, generator=gen(100)) * 2.5).to(dtype)
+    u = torch.rand(b, generator=gen(101))
+    ref_tok, ref_probs = R.sample_tail(x.clone(), temp, top_k, top_p, u)
+    ref_f = R.top_k_logits(x.float() / temp, top_k=top_k, top_p=top_p)
+    tok, filt = ops.sample_top_k_top_p(x.to(gpu), temp, top_k, top_p, u.to(gpu), want_filtered=True)
+    filt, tok = filt.cpu(), tok.cpu()
+    kept, ref_kept = filt > -float("inf"), ref_f > -float("inf")
+    assert torch.equal(filt[kept], (x.float() / temp)[kept]), "kept logits are float(x) / temperature, untouched"
+    for r in range(b):
+        diff = kept[r] != ref_kept[r]
+        if diff.any():      # only members of the tie at the boundary value, and only kept in addition
+            vals = (x.float() / temp)[r][diff]
+            assert top_p > 0 and bool((vals == vals[0]).all()) and bool(kept[r][diff].all())
+            assert float(vals[0]) == float(filt[r][kept[r]].min())
+        else:
+            assert int(tok[r]) == int(ref_tok[r]) or _near_cdf_step(ref_probs[r], float(u[r]))
+        assert kept[r][tok[r]], "the drawn token is one that was kept"
+    tok2, filt2 = ops.sample_top_k_top_p(x.to(gpu), temp, top_k, top_p, u.to(gpu), want_filtered=True)
+    assert torch.equal(tok2.cpu(), tok) and torch.equal(filt2.cpu(), filt), "same inputs, same bits"
+
+
+def _near_cdf_step(probs, u, eps=1e-5):
+    cdf = torch.cumsum(probs, -1)
+    return bool(((cdf - u * cdf[-1]).abs() < eps).any())
+
+
+def test_sampling_follows_the_distribution_and_api(gpu):
+    from merak_amd.inference import sample_next_token, top_k_logits
+    x = torch.randn(1, 40, generator=gen(102))
+    n = 32768
+    xs = x.expand(n, 40).contiguous().to(gpu)
+    us = torch.rand(n, generator=gen(103)).to(gpu)
+    toks = sample_next_token(xs, temperature=0.9, top_k=12, top_p=0.0, uniforms=us)
+    probs = R.sample_tail(x.clone(), 0.9, 12, 0.0, torch.zeros(1))[1][0]
+    freq = torch.bincount(toks.cpu(), minlength=40).double() / n
+    assert (freq - probs).abs().max() < 0.012 and bool((freq[probs == 0] == 0).all())
+    # u = 0 draws the first kept token, u just below 1 the last one
+    kept = (probs > 0).nonzero().flatten()
+    ends = sample_next_token(xs[:2], 0.9, 12, 0.0, torch.tensor([0.0, 0.99999994], device=gpu)).cpu()
+    assert int(ends[0]) == int(kept[0]) and int(ends[1]) == int(kept[-1])
+    f = top_k_logits(xs[:3], top_k=5)
+    assert torch.equal(f.cpu(), R.top_k_logits(x.expand(3, 40).clone(), top_k=5))
+    assert sample_next_token(xs[:4], generator=torch.Generator(device=gpu).manual_seed(1)).shape == (4,)
+    with pytest.raises(RuntimeError, match="temperature"):
+        ops.sample_top_k_top_p(xs[:1], 0.0, 0, 0.0, us[:1])
+    with pytest.raises(RuntimeError, match="out of range"):        # torch.topk's complaint in the reference
+        ops.sample_top_k_top_p(xs[:1], 1.0, 41, 0.0, us[:1])
+    with pytest.raises(ValueError):
+        ops.sample_top_k_top_p(xs[:1])
+    assert ops.sample_top_k_top_p(torch.empty(0, 9, device=gpu), 1.0, 0, 0.0, torch.empty(0, device=gpu))[0].numel() == 0

@@ -219,3 +219,59 @@ def test_decode_step_reduces_to_plain_linears():
     h = (F.silu(y[:, :32]) * y[:, 32:]).bfloat16()
     assert torch.equal(out, F.linear(h.float(), wd.float()).bfloat16())
     assert torch.equal(tok, F.linear(out.float(), wl.float()).argmax(-1))
+
+
+# ------------------------------------------------------------------------------- sampling tail
+def test_top_k_top_p_filter_hand_cases():
+    """Worked by hand from text_generation_inference.py:48-68.  probs 0.5/0.3/0.15/0.05 (logits = log p)."""
+    lp = torch.tensor([[0.3, 0.05, 0.5, 0.15]]).log()
+    inf = float("inf")
+    # top_k = 2: the 2nd largest is log 0.3; everything below it goes
+    assert torch.equal(R.top_k_logits(lp.clone(), top_k=2) == -inf, torch.tensor([[False, True, False, True]]))
+    # top_p = 0.7: sorted cumulative 0.5, 0.8, 0.95, 1.0 -> "> 0.7" from the 2nd on, shifted right by one: the
+    # token that crosses the threshold stays, the rest goes
+    assert torch.equal(R.top_k_logits(lp.clone(), top_p=0.7) == -inf, torch.tensor([[False, True, False, True]]))
+    # top_p = 0.4: even the first token is above the threshold, and is kept regardless (:65)
+    assert torch.equal(R.top_k_logits(lp.clone(), top_p=0.4) == -inf, torch.tensor([[True, True, False, True]]))
+    # top_p = 0.85: cumulative 0.5, 0.8 <= 0.85 < 0.95: three tokens stay
+    assert torch.equal(R.top_k_logits(lp.clone(), top_p=0.85) == -inf, torch.tensor([[False, True, False, False]]))
+    # ties with the k-th value stay (strict "<" at :50)
+    t = torch.tensor([[1.0, 3.0, 2.0, 2.0, 0.0]])
+    assert torch.equal(R.top_k_logits(t.clone(), top_k=2) == -inf, torch.tensor([[True, False, False, False, True]]))
+    # kept values are untouched; the function edits its argument
+    x = lp.clone()
+    y = R.top_k_logits(x, top_k=3)
+    assert y is x and torch.equal(x[0, [0, 2, 3]], lp[0, [0, 2, 3]])
+
+
+def test_top_k_top_p_filter_matches_library_warpers():
+    """Same rule as transformers' TopK/TopP warpers away from exact threshold equality."""
+    from transformers.generation.logits_process import TopKLogitsWarper, TopPLogitsWarper
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(6, 997, generator=g) * 3
+    for k in (1, 5, 50):
+        assert torch.equal(R.top_k_logits(x.clone(), top_k=k), TopKLogitsWarper(top_k=k)(None, x.clone()))
+    for p in (0.1, 0.5, 0.9, 0.999):
+        assert torch.equal(R.top_k_logits(x.clone(), top_p=p), TopPLogitsWarper(top_p=p)(None, x.clone()))
+    both = TopPLogitsWarper(top_p=0.8)(None, TopKLogitsWarper(top_k=40)(None, x.clone()))
+    assert torch.equal(R.top_k_logits(x.clone(), top_k=40, top_p=0.8), both)
+
+
+def test_sample_tail_is_inverse_cdf_and_follows_the_distribution():
+    import numpy as np
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(4, 50, generator=g) * 2
+    u = torch.rand(4, generator=g)
+    tok, probs = R.sample_tail(x, 0.7, 10, 0.9, u)
+    ref_probs = F.softmax(R.top_k_logits(x.float() / 0.7, 10, 0.9).double(), -1)
+    assert torch.allclose(probs, ref_probs)
+    for b in range(4):        # numpy's searchsorted on the cumulative distribution
+        cdf = np.cumsum(probs[b].numpy())
+        assert int(tok[b]) == int(np.searchsorted(cdf, float(u[b].double()) * cdf[-1], side="right"))
+        assert probs[b, tok[b]] > 0
+    # frequencies over many uniforms approach the probabilities (8 kept tokens, 40000 draws)
+    one = torch.randn(1, 30, generator=g)
+    us = torch.rand(40000, generator=g)
+    toks, pr = R.sample_tail(one.expand(40000, 30).clone(), 1.0, 8, 0.0, us)
+    freq = torch.bincount(toks, minlength=30).double() / 40000
+    assert (freq - pr[0]).abs().max() < 0.01 and int((pr[0] > 0).sum()) == 8

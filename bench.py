@@ -253,6 +253,17 @@ def secondary(dev, timer, reps, with_cpu):
         dec[f"B{b}"] = {"us_per_step": round(ms * 1e3, 1), "tokens_per_s": round(b / ms * 1e3, 1),
                         "GBs": round(wbytes / ms / 1e6, 1), "frac_hbm_peak": round(wbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
                         "lm_head_argmax_us": round(lm * 1e3, 1), "lm_head_GBs": round(table.numel() * 2 / lm / 1e6, 1)}
+    # sampling tail on materialised LM-head logits (temperature 0.8, top-k 50, top-p 0.95), kernel only
+    smp = {}
+    for b in (1, 8, 32):
+        lg = torch.empty(b, v, device=dev).normal_(0, 2.5, generator=g).bfloat16()
+        u = torch.rand(b, device=dev)
+        tok = torch.empty(b, dtype=torch.int64, device=dev)
+        st = torch.cuda.current_stream().cuda_stream
+        fn = lambda: _lib.check(_lib.lib().mtp_sample_top_k_top_p(lg.data_ptr(), 1, b, v, 0.8, 50, 0.95, u.data_ptr(),
+                                                                  tok.data_ptr(), None, st), "sample")
+        smp[f"B{b}_us"] = round(timer.run(f"sample.b{b}", fn, reps) * 1e3, 1)
+    dec["sample_top_k_top_p"] = smp
     out["decode_c5"] = dec
     del table, wq, wg, wd, step
     # --- Llama-70B tp=8 shard shapes

@@ -32,6 +32,7 @@ namespace {
 constexpr int SP_THREADS = 1024;
 constexpr int SP_WAVES = SP_THREADS / MTP_WAVE;
 constexpr float SP_LOG2E = 1.4426950408889634f;
+constexpr int SP_REP = 8;  // copies of the histogram: lanes of one instruction that hit the same bin are served one after another
 
 // Element access: a row is cut into slots in index order: an unaligned head, 16-byte vectors, a tail.
 template <typename T> struct Row;
@@ -99,11 +100,48 @@ struct Slots {
   }
 };
 
-// probability mass relative to the row maximum, 40 fractional bits
-__device__ __forceinline__ uint64_t sp_mass(float z, float m) {
-  const float e = __builtin_amdgcn_exp2f((z - m) * SP_LOG2E);
-  return (uint64_t)(e * 1099511627776.0f + 0.5f);
+// f(x[EPV], n, j0) for every slot in [s_begin, s_end) taken `stride` apart starting at s_begin + first.  Four
+// loads are issued before the first of them is used: with one load in flight per wave the passes run at
+// the latency of L2, not its bandwidth.
+template <typename T, typename F>
+__device__ __forceinline__ void for_slots(const Slots<T>& sl, int64_t s_begin, int64_t s_end, int first, int stride,
+                                          F&& f) {
+  constexpr int EPV = Row<T>::EPV;
+  int64_t s = s_begin + first;
+  // slots 1..nvec are plain vectors; keep the unrolled part inside them
+  for (; s >= 1 && s + 3 * (int64_t)stride <= sl.nvec && s + 3 * (int64_t)stride < s_end; s += 4 * (int64_t)stride) {
+    u32x4_t v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      v[u] = *reinterpret_cast<const u32x4_t*>(sl.row + sl.head + (s + u * (int64_t)stride - 1) * EPV);
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      float x[EPV];
+      Row<T>::unpack(v[u], x);
+      f(x, EPV, sl.head + (s + u * (int64_t)stride - 1) * EPV);
+    }
+  }
+  for (; s < s_end; s += stride) {
+    float x[EPV];
+    int64_t j0;
+    const int n = sl.load(s, x, j0);
+    f(x, n, j0);
+  }
 }
+
+// Probability mass relative to the row maximum, 40 fractional bits: round(exp(x/T - m) * 2^40) with the
+// exponent argument formed as one fma, x * (log2(e)/T) - m*log2(e).  (The masses only have to be the same
+// numbers in every pass; the filtered logits that leave the kernel are the true quotients x / T.)
+struct Mass {
+  float c1, mc;
+  __device__ __forceinline__ Mass(float temperature, float m) : c1(SP_LOG2E / temperature), mc(m * SP_LOG2E) {}
+  __device__ __forceinline__ uint64_t operator()(float x) const {
+    const float f = __builtin_amdgcn_exp2f(__builtin_fmaf(x, c1, -mc)) * 1099511627776.0f;  // < 2^41
+    const uint32_t hi = (uint32_t)(f * (1.0f / 65536.0f));
+    const float rem = __builtin_fmaf(-(float)hi, 65536.0f, f);  // exact: f has 24 significant bits
+    return ((uint64_t)hi << 16) + (uint32_t)(rem + 0.5f);
+  }
+};
 
 __device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v) {
 #pragma unroll
@@ -177,7 +215,8 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(const T* __restrict_
   constexpr int EPV = Row<T>::EPV, KEY_BITS = Row<T>::KEY_BITS;
   const Slots<T> sl(logits + (int64_t)blockIdx.x * V, V);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  __shared__ uint64_t bins[256];
+  __shared__ uint64_t bins_rep[SP_REP][256];
+  uint64_t* const bins = bins_rep[lane & (SP_REP - 1)];  // this lane's copy; copy 0 holds the sum after fold
   __shared__ float red_f[SP_WAVES];
   __shared__ uint64_t red_u[SP_WAVES];
   __shared__ int sh_bin;
@@ -185,20 +224,19 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(const T* __restrict_
 
   // ---- row maximum of z ---------------------------------------------------
   float m = -INFINITY;
-  for (int64_t s = tid; s < sl.count; s += SP_THREADS) {
-    float x[EPV];
-    int64_t j0;
-    const int n = sl.load(s, x, j0);
+  for_slots(sl, 0, sl.count, tid, SP_THREADS, [&](const float* x, int n, int64_t) {
 #pragma unroll
     for (int e = 0; e < EPV; e++)
-      if (e < n) m = fmaxf(m, x[e] / temperature);
-  }
+      if (e < n) m = fmaxf(m, x[e]);
+  });
   m = wave_max(m);
   if (lane == 0) red_f[wave] = m;
   __syncthreads();
   m = red_f[0];
 #pragma unroll
   for (int w = 1; w < SP_WAVES; w++) m = fmaxf(m, red_f[w]);
+  m = m / temperature;  // x -> x / T is monotone: the maximum of the quotients is the quotient of the maximum
+  const Mass mass(temperature, m);
 
   // ---- top-k: key of the k-th largest element -------------------------------
   uint32_t k_key = 0;  // elements with key < k_key are dropped
@@ -207,25 +245,29 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(const T* __restrict_
     uint64_t want = (uint64_t)top_k;  // rank still to find inside the current prefix
     for (int shift = KEY_BITS - 8; shift >= 0; shift -= 8) {
       __syncthreads();
-      if (tid < 256) bins[tid] = 0;
+      for (int i = tid; i < SP_REP * 256; i += SP_THREADS) (&bins_rep[0][0])[i] = 0;
       __syncthreads();
       const uint32_t hi_mask = shift == KEY_BITS - 8 ? 0u : ~((1u << (shift + 8)) - 1u);
       BinCache cache;
-      for (int64_t s = tid; s < sl.count; s += SP_THREADS) {
-        float x[EPV];
-        int64_t j0;
-        const int n = sl.load(s, x, j0);
+      for_slots(sl, 0, sl.count, tid, SP_THREADS, [&](const float* x, int n, int64_t) {
 #pragma unroll
         for (int e = 0; e < EPV; e++) {
           const uint32_t key = Row<T>::key(x[e], x[e] / temperature);
           if (e < n && (key & hi_mask) == prefix) cache.add(bins, (int)((key >> shift) & 0xff), 1ull);
         }
-      }
+      });
       cache.flush(bins);
+      __syncthreads();
+      if (tid < 256) {
+        uint64_t t = 0;
+#pragma unroll
+        for (int c = 0; c < SP_REP; c++) t += bins_rep[c][tid];
+        bins_rep[0][tid] = t;
+      }
       __syncthreads();
       if (wave == 0) {
         uint64_t above;
-        const int b = scan_bins_desc(bins, want - 1, lane, above);  // first bin with above + bin >= want
+        const int b = scan_bins_desc(bins_rep[0], want - 1, lane, above);  // first bin with above + bin >= want
         if (lane == 0) {
           sh_bin = b;
           sh_above = above;
@@ -246,36 +288,40 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(const T* __restrict_
     bool all = false;
     for (int shift = KEY_BITS - 8; shift >= 0 && !all; shift -= 8) {
       __syncthreads();
-      if (tid < 256) bins[tid] = 0;
+      for (int i = tid; i < SP_REP * 256; i += SP_THREADS) (&bins_rep[0][0])[i] = 0;
       __syncthreads();
       const uint32_t hi_mask = shift == KEY_BITS - 8 ? 0u : ~((1u << (shift + 8)) - 1u);
       BinCache cache;
-      for (int64_t s = tid; s < sl.count; s += SP_THREADS) {
-        float x[EPV];
-        int64_t j0;
-        const int n = sl.load(s, x, j0);
+      for_slots(sl, 0, sl.count, tid, SP_THREADS, [&](const float* x, int n, int64_t) {
 #pragma unroll
         for (int e = 0; e < EPV; e++) {
           const float z = x[e] / temperature;
           const uint32_t key = Row<T>::key(x[e], z);
           if (e < n && key >= k_key && (key & hi_mask) == prefix)
-            cache.add(bins, (int)((key >> shift) & 0xff), sp_mass(z, m));
+            cache.add(bins, (int)((key >> shift) & 0xff), mass(x[e]));
         }
-      }
+      });
       cache.flush(bins);
+      __syncthreads();
+      if (tid < 256) {
+        uint64_t t = 0;
+#pragma unroll
+        for (int c = 0; c < SP_REP; c++) t += bins_rep[c][tid];
+        bins_rep[0][tid] = t;
+      }
       __syncthreads();
       if (wave == 0) {
         if (shift == KEY_BITS - 8) {
           // total mass of the top-k survivors -> the limit in the same fixed point
           uint64_t t = 0;
 #pragma unroll
-          for (int q = 0; q < 4; q++) t += bins[4 * lane + q];
+          for (int q = 0; q < 4; q++) t += bins_rep[0][4 * lane + q];
           t = wave_sum_u64(t);
           const double lim = (double)top_p * (double)t;
           limit = lim >= 1.8e19 ? ~0ull : (uint64_t)lim;
         }
         uint64_t above;
-        const int b = scan_bins_desc(bins, limit, lane, above);
+        const int b = scan_bins_desc(bins_rep[0], limit, lane, above);
         if (lane == 0) {
           sh_bin = b;
           sh_above = above;
@@ -297,16 +343,13 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(const T* __restrict_
   // ---- optional: the filtered logits the reference's top_k_logits returns -------
   if (filtered) {
     float* out = filtered + (int64_t)blockIdx.x * V;
-    for (int64_t s = tid; s < sl.count; s += SP_THREADS) {
-      float x[EPV];
-      int64_t j0;
-      const int n = sl.load(s, x, j0);
+    for_slots(sl, 0, sl.count, tid, SP_THREADS, [&](const float* x, int n, int64_t j0) {
 #pragma unroll
       for (int e = 0; e < EPV; e++) {
         const float z = x[e] / temperature;
         if (e < n) out[j0 + e] = Row<T>::key(x[e], z) >= keep_key ? z : -INFINITY;
       }
-    }
+    });
   }
   if (!tokens) return;
 
@@ -324,17 +367,19 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(const T* __restrict_
 #pragma unroll
     for (int e = 0; e < EPV; e++) {
       const float z = x[e] / temperature;
-      q[e] = (e < n && Row<T>::key(x[e], z) >= keep_key) ? sp_mass(z, m) : 0;
+      q[e] = (e < n && Row<T>::key(x[e], z) >= keep_key) ? mass(x[e]) : 0;
       t += q[e];
     }
     return t;
   };
   uint64_t mine = 0;
-  for (int64_t s = s0 + lane; s < s1; s += 64) {
-    uint64_t q[EPV];
-    int64_t j0;
-    mine += slot_mass(s, q, j0);
-  }
+  for_slots(sl, s0, s1, lane, 64, [&](const float* x, int n, int64_t) {
+#pragma unroll
+    for (int e = 0; e < EPV; e++) {
+      const float z = x[e] / temperature;
+      if (e < n && Row<T>::key(x[e], z) >= keep_key) mine += mass(x[e]);
+    }
+  });
   mine = wave_sum_u64(mine);
   __syncthreads();
   if (lane == 0) red_u[wave] = mine;

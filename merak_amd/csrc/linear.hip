@@ -11,6 +11,8 @@ int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, int64_t M, int6
 int mtp_gemm_generic(const void* A, int64_t sam, int64_t sak, const void* B, int64_t sbn, int64_t sbk,
                      const void* bias, void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, int out_dtype,
                      int accumulate, hipStream_t s);
+int mtp_gemm_f32(int kind, const float* A, int64_t lda, const float* B, int64_t ldb, const float* bias, float* C,
+                 float* rowsum, int64_t ldc, int64_t M, int64_t N, int64_t K, int accumulate, hipStream_t s);
 int mtp_colsum(const void* dy, void* db, int64_t M, int64_t N, int dtype, int out_dtype, int accumulate,
                hipStream_t s);
 int mtp_act_fwd(const void* y, void* act, int64_t M, int64_t N, int dtype, int swiglu, hipStream_t s);
@@ -32,6 +34,12 @@ int check_dims(const char* what, int64_t M, int64_t N, int64_t K, int dtype) {
 bool fast_ok(int64_t rows_ld_a, int64_t rows_ld_b, const void* a, const void* b) {
   return rows_ld_a % 8 == 0 && rows_ld_b % 8 == 0 && aligned16(a) && aligned16(b) && rows_ld_a * 2 * 256 < (1ll << 31) &&
          rows_ld_b * 2 * 256 < (1ll << 31);
+}
+
+// The fp32 MFMA kernel reads 16 bytes per lane: 16-byte aligned bases, row lengths that are multiples of 4
+// floats, and (for the transposed operands, addressed from the matrix origin) matrices below 2 GiB.
+bool f32_fast_ok(const void* a, const void* b, int64_t d0, int64_t d1, int64_t bytes_a, int64_t bytes_b) {
+  return aligned16(a) && aligned16(b) && d0 % 4 == 0 && d1 % 4 == 0 && bytes_a < (1ll << 31) && bytes_b < (1ll << 31);
 }
 
 }  // namespace
@@ -59,6 +67,14 @@ extern "C" int mtp_linear_fwd(const void* x, const void* w, const void* bias, vo
     if (epilogue == MTP_EPI_SWIGLU && !use_bias) use_bias = nullptr;
     return mtp_gemm_bf16_nt(x, w, use_bias, y, act, M, N, K, epi, s);
   }
+  if (dtype == MTP_F32 && f32_fast_ok(x, w, K, K, 0, 0) && K * 4 * 128 < (1ll << 31)) {
+    void* pre32 = y ? y : (epilogue != MTP_EPI_SWIGLU ? act : nullptr);
+    MTP_REQUIRE(pre32, MTP_EUNSUPPORTED, "linear_fwd: this shape needs the pre-activation buffer y");
+    rc = mtp_gemm_f32(0, (const float*)x, K, (const float*)w, K, (const float*)use_bias, (float*)pre32, nullptr, N, M, N, K, 0, s);
+    if (rc) return rc;
+    if (has_act) return mtp_act_fwd(pre32, act, M, N, dtype, epilogue == MTP_EPI_SWIGLU, s);
+    return MTP_OK;
+  }
   // general path: GEMM (+bias) into y, then the activation as a second pass.  Without y the GELU forms
   // run in place in act; SwiGLU's act is half as wide as the pre-activation, so it needs y.
   void* pre = y;
@@ -81,6 +97,8 @@ extern "C" int mtp_linear_dgrad(const void* dy, const void* w, void* dx, int64_t
     rc = mtp_gemm_bf16_dgrad(dy, w, dx, M, N, K, s);
     if (rc != MTP_EUNSUPPORTED) return rc;
   }
+  if (dtype == MTP_F32 && f32_fast_ok(dy, w, N, K, 0, N * K * 4) && N * 4 * 128 < (1ll << 31))
+    return mtp_gemm_f32(1, (const float*)dy, N, (const float*)w, K, nullptr, (float*)dx, nullptr, K, M, K, N, 0, s);
   // dX[m,k] = sum_n dY[m,n] W[n,k]: A = dY (N,1), B(k,n) = W[n*K + k]
   return mtp_gemm_generic(dy, N, 1, w, 1, K, nullptr, dx, K, M, K, N, dtype, dtype, 0, s);
 }
@@ -99,6 +117,11 @@ extern "C" int mtp_linear_wgrad(const void* dy, const void* x, void* dw, void* d
     rc = mtp_gemm_bf16_wgrad(dy, x, dw, M, N, K, dw_dtype, accumulate, s);
     if (rc == MTP_OK && db) return mtp_colsum(dy, db, M, N, dtype, dw_dtype, accumulate, s);
     if (rc != MTP_EUNSUPPORTED) return rc;
+  }
+  if (dtype == MTP_F32 && dw_dtype == MTP_F32 && M > 0 && f32_fast_ok(dy, x, N, K, M * N * 4, M * K * 4)) {
+    // the bias gradient (column sums of dY = row sums of the A operand) rides along in the first tile column
+    return mtp_gemm_f32(2, (const float*)dy, N, (const float*)x, K, nullptr, (float*)dw, (float*)db, K, N, K, M,
+                        accumulate, s);
   }
   // dW[n,k] = sum_m dY[m,n] X[m,k]: A(n,m) = dY[m*N + n], B(k,m) = X[m*K + k]; M == 0 writes zeros
   rc = mtp_gemm_generic(dy, 1, N, x, 1, K, nullptr, dw, K, N, K, M, dtype, dw_dtype, accumulate, s);

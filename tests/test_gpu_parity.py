@@ -363,6 +363,7 @@ def _lin_inputs(m, n, k, dtype, seed, bias=True):
     (torch.bfloat16, 512, 8192, 1024),      # Llama-70B tp=8 o-proj shard
     (torch.bfloat16, 300, 520, 136), (torch.bfloat16, 64, 50, 27), (torch.bfloat16, 1, 8, 8),
     (torch.float32, 100, 77, 33), (torch.float32, 1, 1, 1), (torch.bfloat16, 257, 255, 72),
+    (torch.float32, 300, 520, 136), (torch.float32, 129, 132, 20), (torch.float32, 64, 8, 4), (torch.float32, 3, 260, 4100),
 ])
 def test_linear_fwd_bwd_vs_oracle(gpu, dtype, m, n, k):
     tol = TOL_F32 if dtype == torch.float32 else TOL_BF16

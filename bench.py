@@ -359,7 +359,7 @@ def main():
     # operands of random sign and mantissa): the chip runs against its power limit well below the published peak
     sink = torch.empty(64 * 4096, device=dev)
     st = torch.cuda.current_stream().cuda_stream
-    r_ms = timer.run("mfma_r", lambda: _lib.check(_lib.lib().mtp_mfma_peak(sink.data_ptr(), 4096, 8192, 1, st), "peak"), 3)
+    r_ms = timer.run("mfma_r", lambda: _lib.check(_lib.lib().mtp_mfma_peak(sink.data_ptr(), 4096, 8192, 1, st), "peak"), 12)
     roofline["mfma_loop_random_operands"] = round(4096 * 8192 * 32 * 32 * 16 * 2 / r_ms / 1e9, 1)
     roofline["frac_of_mfma_loop"] = round(dom["tflops"] / roofline["mfma_loop_random_operands"], 4)
     del work, sink

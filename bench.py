@@ -239,6 +239,27 @@ def secondary(dev, timer, reps, with_cpu):
     ebz_ms = timer.run("emb.bwd0", lambda: ops.embedding_bwd(ids, dout, v, 0, v), max(3, reps // 4))
     out["embedding_c4"].update({"bwd_scatter_us": round(eb_ms * 1e3, 1), "bwd_with_zero_fill_us": round(ebz_ms * 1e3, 1)})
     del dout, dtab
+    # --- LM head + cross entropy at the C4 shape: full logits vs one chunk of rows at a time
+    from merak_amd import mpu
+    hid = torch.empty(n, h, dtype=torch.bfloat16, device=dev).normal_(generator=g)
+    def head_ce_unfused():
+        lg, _ = ops.linear_fwd(hid, table, None, ops.EPI_NONE)
+        ops.vocab_ce_fwd_bwd_(lg, tgt, 0, None, 1.0 / n)
+        ops.linear_dgrad(lg, table)
+        ops.linear_wgrad(lg, hid, False)
+    def head_ce_chunked():
+        hh = hid.detach().requires_grad_(True)
+        ww = table.detach().requires_grad_(True)
+        mpu.lm_head_cross_entropy(hh, ww, tgt, chunk_rows=2048).mean().backward()
+    hc = {}
+    for nm, fn in (("full_logits", head_ce_unfused), ("chunks_of_2048_rows", head_ce_chunked)):
+        torch.cuda.synchronize(); torch.cuda.empty_cache(); torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        ms = timer.run(f"headce.{nm}", fn, max(3, reps // 4))
+        hc[nm] = {"ms": round(ms, 3), "peak_extra_GB": round((torch.cuda.max_memory_allocated() - base) / 1e9, 2),
+                  "tflops": round(6.0 * n * h * v / ms / 1e9, 1)}
+    out["lm_head_plus_ce_c4"] = hc
+    del hid
     # --- decode step: QKV, gate/up+SwiGLU, down, LM head + argmax (the table doubles as the LM head)
     mk = lambda nn, kk: torch.empty(nn, kk, device=dev).normal_(0, 0.02, generator=g).bfloat16()
     wq, wg, wd = mk(6144, 4096), mk(2 * 14336, 4096), mk(4096, 14336)

@@ -4,6 +4,7 @@ from .cross_entropy import vocab_parallel_cross_entropy
 from .cross_entropy import vocab_parallel_cross_entropy_partials
 from .cross_entropy import vocab_parallel_cross_entropy_backward_
 from .cross_entropy import vocab_loss_fn
+from .cross_entropy import lm_head_cross_entropy
 
 from .initialize import destroy_model_parallel
 from .initialize import get_model_parallel_group, set_model_parallel_group

@@ -160,3 +160,80 @@ def vocab_parallel_cross_entropy_backward_(vocab_parallel_logits, target, global
     ops.vocab_ce_bwd_(logits_2d, target.reshape(-1), global_row_max.reshape(-1).contiguous(),
                       global_row_sumexp.reshape(-1).contiguous(), grad_output.reshape(-1), vocab_start_index)
     return vocab_parallel_logits
+
+
+class _LMHeadCrossEntropy(torch.autograd.Function):
+    """Vocab-parallel LM head and cross entropy over row chunks: the [tokens, vocab] logits exist one chunk at
+    a time.  Forward already produces the gradients (for an assumed uniform upstream gradient of the
+    per-position losses), as the one-launch cross entropy does."""
+
+    @staticmethod
+    def forward(ctx, hidden, weight, bias, target, assumed_grad, chunk_rows):
+        vocab_start_index, _ = _vocab_range(weight.shape[0])
+        lead = hidden.shape[:-1]
+        h2d = hidden.reshape(-1, hidden.shape[-1])
+        t1d = target.reshape(-1)
+        n = h2d.shape[0]
+        need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        need_b = bias is not None and ctx.needs_input_grad[2]
+        losses = torch.empty((n,), dtype=torch.float32, device=h2d.device)
+        dh = torch.empty_like(h2d) if need_h else None
+        dw = torch.zeros_like(weight) if need_w else None
+        db = torch.zeros_like(bias) if need_b else None
+        epi = ops.EPI_BIAS if bias is not None else ops.EPI_NONE
+        backward_wanted = need_h or need_w or need_b
+        for r0 in range(0, n, chunk_rows):
+            r1 = min(n, r0 + chunk_rows)
+            logits, _ = ops.linear_fwd(h2d[r0:r1], weight, bias, epi)          # layers.py:251-252
+            if backward_wanted:
+                loss_c, _, _, _ = ops.vocab_ce_fwd_bwd_(logits, t1d[r0:r1], vocab_start_index, None, assumed_grad)
+                if need_h:
+                    dh[r0:r1] = ops.linear_dgrad(logits, weight)
+                if need_w or need_b:
+                    ops.linear_wgrad(logits, h2d[r0:r1], need_b, dw=dw if need_w else torch.zeros_like(weight),
+                                     db=db, accumulate=True)
+            else:
+                loss_c, _, _, _ = ops.vocab_ce_fwd(logits, t1d[r0:r1], vocab_start_index)
+            losses[r0:r1] = loss_c
+            del logits
+        ctx.assumed_grad = float(assumed_grad)
+        ctx.lead = lead
+        ctx.save_for_backward(dh, dw, db)
+        return losses.view(*target.shape)
+
+    @staticmethod
+    def backward(ctx, grad_losses):
+        dh, dw, db = ctx.saved_tensors
+        g = grad_losses.reshape(-1)
+        first = g[:1]
+        if not bool((g == first).all()):
+            raise RuntimeError("lm_head_cross_entropy needs one upstream gradient for all positions (a mean or a "
+                               "sum of the losses); weight the positions through the unfused layers instead")
+        ratio = float(first) / ctx.assumed_grad
+        if ratio != 1.0:
+            for t in (dh, dw, db):
+                if t is not None:
+                    t.mul_(ratio)
+        return (dh.view(*ctx.lead, dh.shape[-1]) if dh is not None else None), dw, db, None, None, None
+
+
+def lm_head_cross_entropy(hidden, lm_head, target, loss_scale=1.0, chunk_rows=2048):
+    """Per-position losses of ``vocab_parallel_cross_entropy(lm_head(hidden)[0], target)`` without ever holding
+    the full logits: the head's product, the cross entropy and both of the head's backward products run per
+    chunk of ``chunk_rows`` tokens, so the largest temporary is [chunk_rows, vocab/p].
+
+    ``lm_head``: a ``ColumnParallelLinear(hidden, vocab, gather_output=False)`` (model_parallel.py:143-156) or
+    its weight.  The per-position losses must be reduced with one common factor — ``.mean()`` as the
+    trainer does (merak_trainer.py:325), times ``loss_scale`` if any; that factor is assumed in forward
+    (``loss_scale / n``) and checked in backward.  Weight gradients are accumulated chunk by chunk in the
+    weight's dtype."""
+    weight, bias = (lm_head.weight, lm_head.bias) if isinstance(lm_head, torch.nn.Module) else (lm_head, None)
+    if get_model_parallel_world_size() != 1:
+        raise RuntimeError("lm_head_cross_entropy at tensor-parallel size > 1 needs the MAX/SUM/SUM exchange of "
+                           "cross_entropy.py:33,64,72 between the head and the loss")
+    n = target.numel()
+    if n == 0:
+        return torch.zeros(target.shape, dtype=torch.float32, device=hidden.device)
+    if weight.shape[0] > ops.vocab_ce_fused_max_vocab(hidden.dtype):
+        raise ValueError("vocabulary slice too long for the one-launch cross entropy; use the unfused layers")
+    return _LMHeadCrossEntropy.apply(hidden, weight, bias, target, float(loss_scale) / n, int(chunk_rows))

@@ -266,6 +266,58 @@ def test_ce_one_launch_full_size_llama_vocab(gpu):
     assert torch.equal(x[:64], before)
 
 
+@pytest.mark.parametrize("dtype,n,k,v,chunk,has_bias", [(torch.bfloat16, 300, 256, 5000, 128, False),
+                                                        (torch.bfloat16, 1023, 512, 32000, 512, True),
+                                                        (torch.float32, 96, 64, 1000, 40, True)])
+def test_lm_head_cross_entropy_chunked(gpu, dtype, n, k, v, chunk, has_bias):
+    """LM head + cross entropy per row chunk (the full logits never exist) against the oracle's F.linear
+    followed by the reference cross entropy, forward and both of the head's gradients."""
+    set_args(use_cpu_initialization=True, params_dtype=dtype)
+    torch.manual_seed(4)
+    head = mpu.ColumnParallelLinear(k, v, bias=has_bias, gather_output=False,
+                                    init_method=lambda t: torch.nn.init.normal_(t, 0.0, 0.05))
+    if has_bias:
+        with torch.no_grad():
+            head.bias.normal_(0, 0.05)
+    h = torch.randn(3, n // 3, k, generator=gen(110)).to(dtype)
+    t = torch.randint(0, v, (3, n // 3), generator=gen(111))
+    t[0, 0] = -100
+    hr = h.float().clone().requires_grad_(True)
+    wr = head.weight.detach().float().requires_grad_(True)
+    br = head.bias.detach().float().requires_grad_(True) if has_bias else None
+    logits = R.column_parallel_linear_forward(hr, wr, br)[0]
+    if dtype == torch.bfloat16:                    # the head stores bf16 logits before the loss reads them
+        logits = logits + (logits.detach().bfloat16().float() - logits.detach())
+    ref_loss, _ = R.cross_entropy_fp32(logits.detach().reshape(n, v), t.view(-1), 0, torch.ones(n))
+    lse = torch.logsumexp(logits.reshape(n, v), -1)
+    inr = t.view(-1) >= 0
+    picked = logits.reshape(n, v)[torch.arange(n), t.view(-1).clamp_min(0)]
+    # out-of-range targets: loss = lse - max, and the reference's backward (cross_entropy.py:92-104) is softmax * g,
+    # i.e. the max term is a constant there
+    closed = torch.where(inr, lse - picked, lse - logits.reshape(n, v).max(-1).values.detach())
+    assert rel(closed.detach(), ref_loss) < 1e-5
+    (3.0 * closed.mean()).backward()
+    head.to(gpu)
+    hg = h.to(gpu).requires_grad_(True)
+    losses = mpu.lm_head_cross_entropy(hg, head, t.to(gpu), loss_scale=3.0, chunk_rows=chunk)
+    assert losses.shape == t.shape and losses.dtype == torch.float32
+    assert rel(losses.view(-1), ref_loss) < (TOL_LOSS if dtype == torch.float32 else 1e-4)
+    (3.0 * losses.mean()).backward()
+    tol = TOL_F32 * 5 if dtype == torch.float32 else 2 * TOL_BF16
+    assert rel(hg.grad, hr.grad) < tol and rel(head.weight.grad, wr.grad) < tol
+    if has_bias:
+        assert rel(head.bias.grad, br.grad) < tol
+    # another common factor is rescaled in backward; per-position weights are refused
+    hg2 = h.to(gpu).requires_grad_(True)
+    head.weight.grad = None
+    l2 = mpu.lm_head_cross_entropy(hg2, head, t.to(gpu), chunk_rows=chunk)
+    (5.0 * l2.sum()).backward()
+    assert rel(hg2.grad, hr.grad * (5.0 * n / 3.0)) < tol
+    with pytest.raises(RuntimeError, match="one upstream gradient"):
+        l3 = mpu.lm_head_cross_entropy(h.to(gpu).requires_grad_(True), head, t.to(gpu), chunk_rows=chunk)
+        (l3.view(-1) * torch.arange(n, device=gpu)).sum().backward()
+
+
 # =============================================================================== embedding
 @pytest.mark.parametrize("dtype,v,h", [(torch.bfloat16, 1000, 4096), (torch.float32, 777, 33), (torch.bfloat16, 50, 7),
                                         (torch.float32, 64, 1)])

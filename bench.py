@@ -250,9 +250,9 @@ def secondary(dev, timer, reps, with_cpu):
     def head_ce_chunked():
         hh = hid.detach().requires_grad_(True)
         ww = table.detach().requires_grad_(True)
-        mpu.lm_head_cross_entropy(hh, ww, tgt, chunk_rows=2048).mean().backward()
+        mpu.lm_head_cross_entropy(hh, ww, tgt, chunk_rows=4096).mean().backward()
     hc = {}
-    for nm, fn in (("full_logits", head_ce_unfused), ("chunks_of_2048_rows", head_ce_chunked)):
+    for nm, fn in (("full_logits", head_ce_unfused), ("chunks_of_4096_rows", head_ce_chunked)):
         torch.cuda.synchronize(); torch.cuda.empty_cache(); torch.cuda.reset_peak_memory_stats()
         base = torch.cuda.memory_allocated()
         ms = timer.run(f"headce.{nm}", fn, max(3, reps // 4))

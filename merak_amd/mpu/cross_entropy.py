@@ -217,7 +217,7 @@ class _LMHeadCrossEntropy(torch.autograd.Function):
         return (dh.view(*ctx.lead, dh.shape[-1]) if dh is not None else None), dw, db, None, None, None
 
 
-def lm_head_cross_entropy(hidden, lm_head, target, loss_scale=1.0, chunk_rows=2048):
+def lm_head_cross_entropy(hidden, lm_head, target, loss_scale=1.0, chunk_rows=4096):
     """Per-position losses of ``vocab_parallel_cross_entropy(lm_head(hidden)[0], target)`` without ever holding
     the full logits: the head's product, the cross entropy and both of the head's backward products run per
     chunk of ``chunk_rows`` tokens, so the largest temporary is [chunk_rows, vocab/p].

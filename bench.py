@@ -281,8 +281,10 @@ def secondary(dev, timer, reps, with_cpu):
         u = torch.rand(b, device=dev)
         tok = torch.empty(b, dtype=torch.int64, device=dev)
         st = torch.cuda.current_stream().cuda_stream
+        ws = torch.empty(int(_lib.lib().mtp_sample_workspace_bytes(b)), dtype=torch.uint8, device=dev)
         fn = lambda: _lib.check(_lib.lib().mtp_sample_top_k_top_p(lg.data_ptr(), 1, b, v, 0.8, 50, 0.95, u.data_ptr(),
-                                                                  tok.data_ptr(), None, st), "sample")
+                                                                  tok.data_ptr(), None, ws.data_ptr(), ws.numel(), st),
+                                "sample")
         smp[f"B{b}_us"] = round(timer.run(f"sample.b{b}", fn, reps) * 1e3, 1)
     dec["sample_top_k_top_p"] = smp
     out["decode_c5"] = dec

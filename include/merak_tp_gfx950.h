@@ -228,11 +228,15 @@ int mtp_argmax_rows(const void* logits, int64_t* idx,
  * whose cumulative kept probability, in index order, exceeds uniforms[b].
  * logits: [B,V] f32 or bf16, untouched.  tokens (int64 [B]) and filtered
  * (f32 [B,V]: z where kept, -inf where dropped, what top_k_logits returns) may
- * each be NULL.  Same inputs give the same outputs bit for bit. */
+ * each be NULL.  workspace: device scratch of mtp_sample_workspace_bytes(B)
+ * bytes, 8-byte aligned (the rows are spread over many workgroups and the
+ * passes of the selection are separate launches; their state lives there).
+ * Same inputs give the same outputs bit for bit. */
+int64_t mtp_sample_workspace_bytes(int64_t B);
 int mtp_sample_top_k_top_p(const void* logits, int dtype, int64_t B, int64_t V,
                            float temperature, int top_k, float top_p,
                            const float* uniforms, int64_t* tokens, float* filtered,
-                           void* stream);
+                           void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------
  * Measurement helpers (used by bench.py to state what this GPU can do).

@@ -44,7 +44,8 @@ SIGNATURES = {
     "mtp_gemv_argmax_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "mtp_gemv_argmax": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "mtp_argmax_rows": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
-    "mtp_sample_top_k_top_p": (_int, [_vp, _int, _i64, _i64, C.c_float, _int, C.c_float, _vp, _vp, _vp, _vp]),
+    "mtp_sample_workspace_bytes": (_i64, [_i64]),
+    "mtp_sample_top_k_top_p": (_int, [_vp, _int, _i64, _i64, C.c_float, _int, C.c_float, _vp, _vp, _vp, _vp, _i64, _vp]),
     "mtp_stream_copy": (_int, [_vp, _vp, _i64, _vp]),
     "mtp_mfma_peak": (_int, [_vp, _i64, _i64, _int, _vp]),
 }

@@ -1,5 +1,5 @@
 // Sampling tail of the decode loop for gfx950: temperature, top-k, top-p and
-// one multinomial draw per batch row, in one kernel, one workgroup per row
+// one multinomial draw per batch row
 // (Merak/inference/text_generation_inference.py:35-69 `top_k_logits`, :229-235).
 //
 //   z      = float(logits) / temperature                               (:230-231)
@@ -16,23 +16,45 @@
 // bf16 spacing, never merges two values): 2 passes per threshold; for fp32 it
 // is the 32-bit image of z: 4 passes.  Mass is held as 64-bit fixed point,
 // q = round(exp(z - max) * 2^40), so that integer atomics give sums that do
-// not depend on the order of addition: the kernel is reproducible bit for bit.
+// not depend on the order of addition: the result is reproducible bit for bit.
 // The draw is the inverse CDF in index order on the same integers:
 // token = first j with sum_{i<=j, kept} q_i > floor(u * Q).
 //
-// Every pass re-reads the row with 16-byte loads (L2 resident after the
-// first): 1 (max) + 2 x 2 or 4 (thresholds) + 2 (draw) passes.  Where the
-// reference keeps only some of several exactly equal logits at the top-p
-// boundary (whichever its sort happened to put first), this kernel keeps all
-// of them.
+// The work per element is a few dozen VALU instructions, and a decode batch
+// has few rows, so every row is spread over SG workgroups and every pass is a
+// launch of its own (B * SG workgroups): the per-pass histograms live in a
+// caller-supplied workspace, each launch re-derives the state of the selection
+// from the histograms of the passes before it (a 256-bin scan by one wave), and
+// kernel boundaries are the only synchronisation.  Where the reference keeps
+// only some of several exactly equal logits at the top-p boundary (whichever its
+// sort happened to put first), these kernels keep all of them.
 #include "mtp_common.h"
 
 namespace {
 
-constexpr int SP_THREADS = 1024;
+constexpr int SP_THREADS = 256;
 constexpr int SP_WAVES = SP_THREADS / MTP_WAVE;
+constexpr int SG = 32;       // workgroups per row
+constexpr int SP_MAXPASS = 8;
 constexpr float SP_LOG2E = 1.4426950408889634f;
-constexpr int SP_REP = 8;  // copies of the histogram: lanes of one instruction that hit the same bin are served one after another
+constexpr int SP_REP = 4;    // copies of the LDS histogram: lanes of one instruction that hit the same bin are served one after another
+
+// Per batch row, in the workspace.
+struct RowState {
+  uint32_t max_key;              // order preserving image of the largest logit of the row
+  uint32_t keep_key;             // elements with key >= keep_key survive both filters
+  uint32_t pad[2];
+  uint64_t part[SG];             // kept mass of each chunk of the row, chunks in index order
+  uint64_t hist[SP_MAXPASS][256];  // one histogram per selection pass: top-k passes first, then top-p
+};
+
+__device__ __forceinline__ uint32_t f32_key(float v) {
+  const uint32_t u = v == 0.0f ? 0u : __float_as_uint(v);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float f32_unkey(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k ^ 0x80000000u) : ~k);
+}
 
 // Element access: a row is cut into slots in index order: an unaligned head, 16-byte vectors, a tail.
 template <typename T> struct Row;
@@ -149,25 +171,6 @@ __device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v) {
   return v;
 }
 
-// Histogram updates of one lane: logits of one row share their top key bits, so in the first pass nearly
-// every element lands in the same two or three bins.  Each lane sums runs of equal bins privately and only
-// touches LDS when the bin changes.
-struct BinCache {
-  int bin = -1;
-  uint64_t acc = 0;
-  __device__ __forceinline__ void add(uint64_t* bins, int b, uint64_t v) {
-    if (b != bin) {
-      flush(bins);
-      bin = b;
-    }
-    acc += v;
-  }
-  __device__ __forceinline__ void flush(uint64_t* bins) {
-    if (bin >= 0 && acc) atomicAdd((unsigned long long*)&bins[bin], (unsigned long long)acc);
-    acc = 0;
-  }
-};
-
 // Wave 0 scans 256 bins from the top: the first bin b with above(b) + bin(b) > limit.  Returns b (or -1)
 // to every lane of wave 0 and the sum over the bins above it in `above` (the total when b = -1).
 __device__ __forceinline__ int scan_bins_desc(const uint64_t* bins, uint64_t limit, int lane, uint64_t& above) {
@@ -206,209 +209,221 @@ __device__ __forceinline__ int scan_bins_desc(const uint64_t* bins, uint64_t lim
   return __shfl(found, src, 64);
 }
 
-template <typename T>
-__global__ __launch_bounds__(SP_THREADS) void sample_kernel(const T* __restrict__ logits, int64_t V,
-                                                            float temperature, int top_k, float top_p,
-                                                            const float* __restrict__ uniforms,
-                                                            int64_t* __restrict__ tokens,
-                                                            float* __restrict__ filtered) {
-  constexpr int EPV = Row<T>::EPV, KEY_BITS = Row<T>::KEY_BITS;
-  const Slots<T> sl(logits + (int64_t)blockIdx.x * V, V);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  __shared__ uint64_t bins_rep[SP_REP][256];
-  uint64_t* const bins = bins_rep[lane & (SP_REP - 1)];  // this lane's copy; copy 0 holds the sum after fold
-  __shared__ float red_f[SP_WAVES];
-  __shared__ uint64_t red_u[SP_WAVES];
-  __shared__ int sh_bin;
-  __shared__ uint64_t sh_above;
 
-  // ---- row maximum of z ---------------------------------------------------
+// State of the selection after the first `done` passes, replayed from their histograms by wave 0 and
+// broadcast through LDS.  All threads of the workgroup must call it.
+struct Selection {
+  uint32_t k_key;     // valid once all top-k passes are done (0: no top-k)
+  uint32_t prefix;    // key bits fixed so far in the phase that pass `done` belongs to
+  uint64_t limit;     // top-p: mass that may lie above the threshold inside the current prefix
+  uint64_t want;      // top-k: rank still to find inside the current prefix
+  bool all;           // top-p: the whole mass fits under top_p, nothing is dropped
+};
+
+template <int KEY_BITS>
+__device__ Selection replay(const RowState* st, int done, int top_k_passes, int top_p_passes, int top_k,
+                            float top_p) {
+  __shared__ Selection sh;
+  const int lane = threadIdx.x & 63;
+  if (threadIdx.x < 64) {
+    Selection s{0u, 0u, 0ull, (uint64_t)top_k, false};
+    int pass = 0;
+    for (int lvl = 0; lvl < top_k_passes && pass < done; lvl++, pass++) {
+      const int shift = KEY_BITS - 8 - 8 * lvl;
+      uint64_t above;
+      const int b = scan_bins_desc(st->hist[pass], s.want - 1, lane, above);  // first bin with above + bin >= want
+      s.prefix |= (uint32_t)b << shift;
+      s.want -= above;
+      if (lvl == top_k_passes - 1) {
+        s.k_key = s.prefix;
+        s.prefix = 0;
+      }
+    }
+    for (int lvl = 0; lvl < top_p_passes && pass < done && !s.all; lvl++, pass++) {
+      const int shift = KEY_BITS - 8 - 8 * lvl;
+      if (lvl == 0) {
+        // total mass of the top-k survivors -> the limit in the same fixed point
+        uint64_t t = 0;
+#pragma unroll
+        for (int q = 0; q < 4; q++) t += st->hist[pass][4 * lane + q];
+        t = wave_sum_u64(t);
+        const double lim = (double)top_p * (double)t;
+        s.limit = lim >= 1.8e19 ? ~0ull : (uint64_t)lim;
+      }
+      uint64_t above;
+      const int b = scan_bins_desc(st->hist[pass], s.limit, lane, above);
+      if (b < 0) {
+        s.all = true;
+      } else {
+        s.prefix |= (uint32_t)b << shift;
+        s.limit -= above;
+      }
+    }
+    if (lane == 0) sh = s;
+  }
+  __syncthreads();
+  return sh;
+}
+
+__global__ __launch_bounds__(256) void sample_init_kernel(RowState* __restrict__ st, int64_t words) {
+  uint64_t* p = reinterpret_cast<uint64_t*>(st);
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += stride) p[i] = 0;
+}
+
+// slots [s0, s1) of chunk g of a row
+template <typename T>
+__device__ __forceinline__ void chunk_range(const Slots<T>& sl, int g, int64_t& s0, int64_t& s1) {
+  const int64_t per = (sl.count + SG - 1) / SG;
+  s0 = (int64_t)g * per;
+  s1 = s0 + per < sl.count ? s0 + per : sl.count;
+  if (s0 > s1) s0 = s1;
+}
+
+template <typename T>
+__global__ __launch_bounds__(SP_THREADS) void sample_max_kernel(const T* __restrict__ logits, int64_t V,
+                                                                RowState* __restrict__ state) {
+  constexpr int EPV = Row<T>::EPV;
+  const int b = blockIdx.x / SG, g = blockIdx.x % SG;
+  const Slots<T> sl(logits + (int64_t)b * V, V);
+  int64_t s0, s1;
+  chunk_range(sl, g, s0, s1);
   float m = -INFINITY;
-  for_slots(sl, 0, sl.count, tid, SP_THREADS, [&](const float* x, int n, int64_t) {
+  for_slots(sl, s0, s1, threadIdx.x, SP_THREADS, [&](const float* x, int n, int64_t) {
 #pragma unroll
     for (int e = 0; e < EPV; e++)
       if (e < n) m = fmaxf(m, x[e]);
   });
   m = wave_max(m);
-  if (lane == 0) red_f[wave] = m;
+  if ((threadIdx.x & 63) == 0 && m > -INFINITY) atomicMax(&state[b].max_key, f32_key(m));
+}
+
+// One selection pass over one chunk: histogram of the digit at `pass` of the elements inside the current prefix
+template <typename T>
+__global__ __launch_bounds__(SP_THREADS) void sample_hist_kernel(const T* __restrict__ logits, int64_t V,
+                                                                 float temperature, int top_k, float top_p,
+                                                                 int top_k_passes, int top_p_passes, int pass,
+                                                                 RowState* __restrict__ state) {
+  constexpr int EPV = Row<T>::EPV, KEY_BITS = Row<T>::KEY_BITS;
+  const int b = blockIdx.x / SG, g = blockIdx.x % SG;
+  const int tid = threadIdx.x, lane = tid & 63;
+  RowState* st = state + b;
+  const Selection sel = replay<KEY_BITS>(st, pass, top_k_passes, top_p_passes, top_k, top_p);
+  const bool mass_phase = pass >= top_k_passes;
+  if (mass_phase && sel.all) return;  // nothing more to find
+  const int lvl = mass_phase ? pass - top_k_passes : pass;
+  const int shift = KEY_BITS - 8 - 8 * lvl;
+  const uint32_t hi_mask = lvl == 0 ? 0u : ~((1u << (shift + 8)) - 1u);
+  const uint32_t prefix = sel.prefix, k_key = sel.k_key;
+  const Mass mass(temperature, f32_unkey(st->max_key) / temperature);
+
+  __shared__ uint64_t bins_rep[SP_REP][256];
+  for (int i = tid; i < SP_REP * 256; i += SP_THREADS) (&bins_rep[0][0])[i] = 0;
   __syncthreads();
-  m = red_f[0];
+  uint64_t* const bins = bins_rep[lane & (SP_REP - 1)];
+  const Slots<T> sl(logits + (int64_t)b * V, V);
+  int64_t s0, s1;
+  chunk_range(sl, g, s0, s1);
+  for_slots(sl, s0, s1, tid, SP_THREADS, [&](const float* x, int n, int64_t) {
 #pragma unroll
-  for (int w = 1; w < SP_WAVES; w++) m = fmaxf(m, red_f[w]);
-  m = m / temperature;  // x -> x / T is monotone: the maximum of the quotients is the quotient of the maximum
-  const Mass mass(temperature, m);
-
-  // ---- top-k: key of the k-th largest element -------------------------------
-  uint32_t k_key = 0;  // elements with key < k_key are dropped
-  if (top_k > 0 && top_k < V) {
-    uint32_t prefix = 0;
-    uint64_t want = (uint64_t)top_k;  // rank still to find inside the current prefix
-    for (int shift = KEY_BITS - 8; shift >= 0; shift -= 8) {
-      __syncthreads();
-      for (int i = tid; i < SP_REP * 256; i += SP_THREADS) (&bins_rep[0][0])[i] = 0;
-      __syncthreads();
-      const uint32_t hi_mask = shift == KEY_BITS - 8 ? 0u : ~((1u << (shift + 8)) - 1u);
-      BinCache cache;
-      for_slots(sl, 0, sl.count, tid, SP_THREADS, [&](const float* x, int n, int64_t) {
-#pragma unroll
-        for (int e = 0; e < EPV; e++) {
-          const uint32_t key = Row<T>::key(x[e], x[e] / temperature);
-          if (e < n && (key & hi_mask) == prefix) cache.add(bins, (int)((key >> shift) & 0xff), 1ull);
-        }
-      });
-      cache.flush(bins);
-      __syncthreads();
-      if (tid < 256) {
-        uint64_t t = 0;
-#pragma unroll
-        for (int c = 0; c < SP_REP; c++) t += bins_rep[c][tid];
-        bins_rep[0][tid] = t;
-      }
-      __syncthreads();
-      if (wave == 0) {
-        uint64_t above;
-        const int b = scan_bins_desc(bins_rep[0], want - 1, lane, above);  // first bin with above + bin >= want
-        if (lane == 0) {
-          sh_bin = b;
-          sh_above = above;
-        }
-      }
-      __syncthreads();
-      prefix |= (uint32_t)sh_bin << shift;
-      want -= sh_above;
+    for (int e = 0; e < EPV; e++) {
+      const float z = x[e] / temperature;
+      const uint32_t key = Row<T>::key(x[e], z);
+      if (e < n && (key & hi_mask) == prefix && (!mass_phase || key >= k_key))
+        atomicAdd((unsigned long long*)&bins[(key >> shift) & 0xff], mass_phase ? (unsigned long long)mass(x[e]) : 1ull);
     }
-    k_key = prefix;
-  }
+  });
+  __syncthreads();
+  uint64_t t = 0;
+#pragma unroll
+  for (int c = 0; c < SP_REP; c++) t += bins_rep[c][tid];
+  if (t) atomicAdd((unsigned long long*)&st->hist[pass][tid], (unsigned long long)t);
+}
 
-  // ---- top-p: key of the last token whose predecessors hold <= top_p of the mass ---
-  uint32_t keep_key = k_key;
-  if (top_p > 0.0f) {
-    uint32_t prefix = 0;
-    uint64_t limit = 0;
-    bool all = false;
-    for (int shift = KEY_BITS - 8; shift >= 0 && !all; shift -= 8) {
-      __syncthreads();
-      for (int i = tid; i < SP_REP * 256; i += SP_THREADS) (&bins_rep[0][0])[i] = 0;
-      __syncthreads();
-      const uint32_t hi_mask = shift == KEY_BITS - 8 ? 0u : ~((1u << (shift + 8)) - 1u);
-      BinCache cache;
-      for_slots(sl, 0, sl.count, tid, SP_THREADS, [&](const float* x, int n, int64_t) {
+// Kept mass of every chunk (and the filtered logits, if asked for)
+template <typename T>
+__global__ __launch_bounds__(SP_THREADS) void sample_mass_kernel(const T* __restrict__ logits, int64_t V,
+                                                                 float temperature, int top_k, float top_p,
+                                                                 int top_k_passes, int top_p_passes,
+                                                                 RowState* __restrict__ state,
+                                                                 float* __restrict__ filtered) {
+  constexpr int EPV = Row<T>::EPV, KEY_BITS = Row<T>::KEY_BITS;
+  const int b = blockIdx.x / SG, g = blockIdx.x % SG;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  RowState* st = state + b;
+  const Selection sel = replay<KEY_BITS>(st, top_k_passes + top_p_passes, top_k_passes, top_p_passes, top_k, top_p);
+  uint32_t keep_key = sel.k_key;
+  if (top_p_passes && !sel.all && sel.prefix > keep_key) keep_key = sel.prefix;
+  const Mass mass(temperature, f32_unkey(st->max_key) / temperature);
+  const Slots<T> sl(logits + (int64_t)b * V, V);
+  int64_t s0, s1;
+  chunk_range(sl, g, s0, s1);
+  float* out = filtered ? filtered + (int64_t)b * V : nullptr;
+  uint64_t mine = 0;
+  for_slots(sl, s0, s1, tid, SP_THREADS, [&](const float* x, int n, int64_t j0) {
 #pragma unroll
-        for (int e = 0; e < EPV; e++) {
-          const float z = x[e] / temperature;
-          const uint32_t key = Row<T>::key(x[e], z);
-          if (e < n && key >= k_key && (key & hi_mask) == prefix)
-            cache.add(bins, (int)((key >> shift) & 0xff), mass(x[e]));
-        }
-      });
-      cache.flush(bins);
-      __syncthreads();
-      if (tid < 256) {
-        uint64_t t = 0;
-#pragma unroll
-        for (int c = 0; c < SP_REP; c++) t += bins_rep[c][tid];
-        bins_rep[0][tid] = t;
-      }
-      __syncthreads();
-      if (wave == 0) {
-        if (shift == KEY_BITS - 8) {
-          // total mass of the top-k survivors -> the limit in the same fixed point
-          uint64_t t = 0;
-#pragma unroll
-          for (int q = 0; q < 4; q++) t += bins_rep[0][4 * lane + q];
-          t = wave_sum_u64(t);
-          const double lim = (double)top_p * (double)t;
-          limit = lim >= 1.8e19 ? ~0ull : (uint64_t)lim;
-        }
-        uint64_t above;
-        const int b = scan_bins_desc(bins_rep[0], limit, lane, above);
-        if (lane == 0) {
-          sh_bin = b;
-          sh_above = above;
-          red_u[0] = limit;
-        }
-      }
-      __syncthreads();
-      limit = red_u[0];
-      if (sh_bin < 0) {
-        all = true;  // the whole mass fits under top_p: nothing is dropped (top level only)
-      } else {
-        prefix |= (uint32_t)sh_bin << shift;
-        limit -= sh_above;
-      }
+    for (int e = 0; e < EPV; e++) {
+      const float z = x[e] / temperature;
+      const bool keep = Row<T>::key(x[e], z) >= keep_key;
+      if (e < n && keep) mine += mass(x[e]);
+      if (out && e < n) out[j0 + e] = keep ? z : -INFINITY;
     }
-    if (!all && prefix > keep_key) keep_key = prefix;
-  }
-
-  // ---- optional: the filtered logits the reference's top_k_logits returns -------
-  if (filtered) {
-    float* out = filtered + (int64_t)blockIdx.x * V;
-    for_slots(sl, 0, sl.count, tid, SP_THREADS, [&](const float* x, int n, int64_t j0) {
-#pragma unroll
-      for (int e = 0; e < EPV; e++) {
-        const float z = x[e] / temperature;
-        if (e < n) out[j0 + e] = Row<T>::key(x[e], z) >= keep_key ? z : -INFINITY;
-      }
-    });
-  }
-  if (!tokens) return;
-
-  // ---- draw: inverse CDF in index order.  Wave w owns a contiguous range of slots, a step is 64 slots,
-  // lane l the l-th of them: slot order = index order.
-  const int64_t per_wave = (sl.count + SP_WAVES - 1) / SP_WAVES;
-  const int64_t s0 = (int64_t)wave * per_wave;
-  const int64_t s1 = s0 + per_wave < sl.count ? s0 + per_wave : sl.count;
-  auto slot_mass = [&](int64_t s, uint64_t* q, int64_t& j0) -> uint64_t {  // masses of the kept elements of slot s
-    float x[EPV] = {};
-    int n = 0;
-    j0 = 0;
-    if (s < s1) n = sl.load(s, x, j0);
+  });
+  mine = wave_sum_u64(mine);
+  __shared__ uint64_t red[SP_WAVES];
+  if (lane == 0) red[wave] = mine;
+  __syncthreads();
+  if (tid == 0) {
     uint64_t t = 0;
+#pragma unroll
+    for (int w = 0; w < SP_WAVES; w++) t += red[w];
+    st->part[g] = t;
+    if (g == 0) st->keep_key = keep_key;
+  }
+}
+
+// The draw: one wave per row walks the chunk that holds the target mass
+template <typename T>
+__global__ __launch_bounds__(64) void sample_draw_kernel(const T* __restrict__ logits, int64_t V, float temperature,
+                                                         const float* __restrict__ uniforms,
+                                                         const RowState* __restrict__ state,
+                                                         int64_t* __restrict__ tokens) {
+  constexpr int EPV = Row<T>::EPV;
+  const int b = blockIdx.x, lane = threadIdx.x;
+  const RowState* st = state + b;
+  uint64_t total = 0;
+  for (int g = 0; g < SG; g++) total += st->part[g];
+  // total >= 2^40 (the maximum itself is always kept)
+  float u = uniforms[b];
+  u = u < 0.0f ? 0.0f : u;
+  uint64_t r = (uint64_t)((double)u * (double)total);
+  if (r >= total) r = total - 1;
+  uint64_t run = 0;
+  int pick = 0;
+  for (int g = 0; g < SG; g++) {
+    if (run + st->part[g] > r) {
+      pick = g;
+      break;
+    }
+    run += st->part[g];
+  }
+  const uint32_t keep_key = st->keep_key;
+  const Mass mass(temperature, f32_unkey(st->max_key) / temperature);
+  const Slots<T> sl(logits + (int64_t)b * V, V);
+  int64_t s0, s1;
+  chunk_range(sl, pick, s0, s1);
+  for (int64_t base = s0; base < s1; base += 64) {
+    float x[EPV] = {};
+    int64_t j0 = 0;
+    int n = 0;
+    if (base + lane < s1) n = sl.load(base + lane, x, j0);
+    uint64_t q[EPV], t = 0;
 #pragma unroll
     for (int e = 0; e < EPV; e++) {
       const float z = x[e] / temperature;
       q[e] = (e < n && Row<T>::key(x[e], z) >= keep_key) ? mass(x[e]) : 0;
       t += q[e];
     }
-    return t;
-  };
-  uint64_t mine = 0;
-  for_slots(sl, s0, s1, lane, 64, [&](const float* x, int n, int64_t) {
-#pragma unroll
-    for (int e = 0; e < EPV; e++) {
-      const float z = x[e] / temperature;
-      if (e < n && Row<T>::key(x[e], z) >= keep_key) mine += mass(x[e]);
-    }
-  });
-  mine = wave_sum_u64(mine);
-  __syncthreads();
-  if (lane == 0) red_u[wave] = mine;
-  __syncthreads();
-  uint64_t total = 0;
-#pragma unroll
-  for (int w = 0; w < SP_WAVES; w++) total += red_u[w];
-  // total >= 2^40 (the maximum itself is always kept)
-  float u = uniforms[blockIdx.x];
-  u = u < 0.0f ? 0.0f : u;
-  uint64_t r = (uint64_t)((double)u * (double)total);
-  if (r >= total) r = total - 1;
-  uint64_t before = 0;
-  int pick_wave = -1;
-#pragma unroll
-  for (int w = 0; w < SP_WAVES; w++) {
-    if (pick_wave < 0) {
-      if (before + red_u[w] > r)
-        pick_wave = w;
-      else
-        before += red_u[w];
-    }
-  }
-  if (wave != pick_wave) return;
-  uint64_t run = before;
-  for (int64_t base = s0; base < s1; base += 64) {
-    uint64_t q[EPV];
-    int64_t j0;
-    const uint64_t t = slot_mass(base + lane, q, j0);
     uint64_t incl = t;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
@@ -420,13 +435,13 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(const T* __restrict_
       if (lane == __ffsll((long long)hit) - 1) {
         // the crossing lies inside this lane's slot: walk its elements
         uint64_t acc = run + incl - t;
-        int64_t pick = -1;
+        int64_t tok = -1;
 #pragma unroll
         for (int e = 0; e < EPV; e++) {
           acc += q[e];
-          if (pick < 0 && q[e] > 0 && acc > r) pick = j0 + e;
+          if (tok < 0 && q[e] > 0 && acc > r) tok = j0 + e;
         }
-        tokens[blockIdx.x] = pick;
+        tokens[b] = tok;
       }
       return;
     }
@@ -434,13 +449,39 @@ __global__ __launch_bounds__(SP_THREADS) void sample_kernel(const T* __restrict_
   }
 }
 
+template <typename T>
+int launch_sample(const void* logits, int64_t B, int64_t V, float temperature, int top_k, float top_p,
+                  const float* uniforms, int64_t* tokens, float* filtered, RowState* state, hipStream_t s) {
+  const T* lg = (const T*)logits;
+  const int per_threshold = Row<T>::KEY_BITS / 8;
+  const int kp = (top_k > 0 && top_k < V) ? per_threshold : 0;
+  const int pp = top_p > 0.0f ? per_threshold : 0;
+  const dim3 grid((unsigned)(B * SG)), block(SP_THREADS);
+  const int64_t words = B * (int64_t)(sizeof(RowState) / 8);
+  hipLaunchKernelGGL(sample_init_kernel, dim3((unsigned)((words + 255) / 256 < 1024 ? (words + 255) / 256 : 1024)),
+                     dim3(256), 0, s, state, words);
+  hipLaunchKernelGGL(sample_max_kernel<T>, grid, block, 0, s, lg, V, state);
+  for (int pass = 0; pass < kp + pp; pass++)
+    hipLaunchKernelGGL(sample_hist_kernel<T>, grid, block, 0, s, lg, V, temperature, top_k, top_p, kp, pp, pass, state);
+  hipLaunchKernelGGL(sample_mass_kernel<T>, grid, block, 0, s, lg, V, temperature, top_k, top_p, kp, pp, state,
+                     filtered);
+  if (tokens)
+    hipLaunchKernelGGL(sample_draw_kernel<T>, dim3((unsigned)B), dim3(64), 0, s, lg, V, temperature, uniforms, state,
+                       tokens);
+  MTP_CHECK_LAUNCH("sample");
+  return MTP_OK;
+}
+
 }  // namespace
+
+extern "C" int64_t mtp_sample_workspace_bytes(int64_t B) { return B > 0 ? B * (int64_t)sizeof(RowState) : 0; }
 
 extern "C" int mtp_sample_top_k_top_p(const void* logits, int dtype, int64_t B, int64_t V, float temperature,
                                       int top_k, float top_p, const float* uniforms, int64_t* tokens,
-                                      float* filtered, void* stream) {
+                                      float* filtered, void* workspace, int64_t workspace_bytes, void* stream) {
   MTP_REQUIRE(B >= 0 && V >= 1, MTP_EINVAL, "sample: B=%lld V=%lld", (long long)B, (long long)V);
-  MTP_REQUIRE(B < (1ll << 31) && V < (1ll << 31), MTP_EUNSUPPORTED, "sample: a dimension exceeds 2^31-1");
+  MTP_REQUIRE(B < (1ll << 24) && V < (1ll << 31), MTP_EUNSUPPORTED, "sample: B=%lld or V=%lld too large", (long long)B,
+              (long long)V);
   MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16, MTP_EINVAL, "sample: unknown dtype %d", dtype);
   MTP_REQUIRE(temperature > 0.0f && temperature == temperature, MTP_EINVAL, "sample: temperature must be positive");
   MTP_REQUIRE(top_k >= 0 && top_p >= 0.0f, MTP_EINVAL, "sample: top_k=%d top_p=%g", top_k, (double)top_p);
@@ -449,13 +490,13 @@ extern "C" int mtp_sample_top_k_top_p(const void* logits, int dtype, int64_t B, 
   if (B == 0) return MTP_OK;
   MTP_REQUIRE(logits && (tokens || filtered), MTP_EINVAL, "sample: null pointer");
   MTP_REQUIRE(!tokens || uniforms, MTP_EINVAL, "sample: tokens requested without uniforms");
+  MTP_REQUIRE(workspace && workspace_bytes >= mtp_sample_workspace_bytes(B), MTP_EWORKSPACE,
+              "sample: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)mtp_sample_workspace_bytes(B));
+  MTP_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7) == 0, MTP_EINVAL, "sample: workspace not 8-byte aligned");
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MTP_F32)
-    hipLaunchKernelGGL(sample_kernel<float>, dim3((unsigned)B), dim3(SP_THREADS), 0, s, (const float*)logits, V,
-                       temperature, top_k, top_p, uniforms, tokens, filtered);
-  else
-    hipLaunchKernelGGL(sample_kernel<uint16_t>, dim3((unsigned)B), dim3(SP_THREADS), 0, s, (const uint16_t*)logits, V,
-                       temperature, top_k, top_p, uniforms, tokens, filtered);
-  MTP_CHECK_LAUNCH("sample");
-  return MTP_OK;
+    return launch_sample<float>(logits, B, V, temperature, top_k, top_p, uniforms, tokens, filtered,
+                                (RowState*)workspace, s);
+  return launch_sample<uint16_t>(logits, B, V, temperature, top_k, top_p, uniforms, tokens, filtered,
+                                 (RowState*)workspace, s);
 }

@@ -310,11 +310,12 @@ def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
 
 
 def sample_top_k_top_p(logits: torch.Tensor, temperature: float = 1.0, top_k: int = 0, top_p: float = 0.0,
-                       uniforms: Optional[torch.Tensor] = None, want_filtered: bool = False):
+                       uniforms: Optional[torch.Tensor] = None, want_filtered: bool = False,
+                       workspace: Optional[torch.Tensor] = None):
     """-> (tokens int64 [B] or None, filtered fp32 [B, V] or None).
 
     tokens are drawn when ``uniforms`` (fp32 [B], values in [0, 1)) is given."""
-    dev = _require_gpu(logits, uniforms)
+    dev = _require_gpu(logits, uniforms, workspace)
     if logits.dim() != 2:
         raise ValueError("sample_top_k_top_p takes [B, V] logits")
     logits = _contig(logits)
@@ -329,8 +330,13 @@ def sample_top_k_top_p(logits: torch.Tensor, temperature: float = 1.0, top_k: in
         filtered = torch.empty((B, V), dtype=torch.float32, device=dev)
     if tokens is None and filtered is None:
         raise ValueError("nothing to compute: give uniforms and/or want_filtered=True")
+    lib = _lib.lib()
+    need = int(lib.mtp_sample_workspace_bytes(B))
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty((max(need, 8),), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().mtp_sample_top_k_top_p(_p(logits), _dt(logits), B, V, float(temperature), int(top_k),
-                                                     float(top_p), _p(uniforms), _p(tokens), _p(filtered),
-                                                     _stream(dev)), "mtp_sample_top_k_top_p")
+        _lib.check(lib.mtp_sample_top_k_top_p(_p(logits), _dt(logits), B, V, float(temperature), int(top_k),
+                                              float(top_p), _p(uniforms), _p(tokens), _p(filtered), _p(workspace),
+                                              workspace.numel() * workspace.element_size(), _stream(dev)),
+                   "mtp_sample_top_k_top_p")
     return tokens, filtered

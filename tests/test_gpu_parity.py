@@ -497,7 +497,7 @@ def test_gpt2_small_fp32_full_size(gpu):
 @pytest.mark.parametrize("name,m,k,n", [("llama8b_qkv", 4096, 4096, 6144), ("llama8b_down", 4096, 14336, 4096),
                                          ("llama70b_tp8_qkv", 8192, 8192, 1280), ("llama70b_tp8_oproj", 8192, 1024, 8192)])
 def test_linear_full_size_sampled(gpu, name, m, k, n):
-    """Full BASELINE shapes: oracle on sampled rows of Y, dX and dW; linearity in X over the whole output."""
+    """Full Llama-3-8B and Llama-70B tp=8 shard shapes: oracle on sampled rows of Y, dX and dW; linearity in X over the whole output."""
     g = torch.Generator(device=gpu).manual_seed(1240)
     x = torch.empty(m, k, device=gpu).normal_(generator=g).bfloat16()
     w = torch.empty(n, k, device=gpu).normal_(0, 0.02, generator=g).bfloat16()

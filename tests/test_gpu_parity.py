@@ -656,3 +656,69 @@ def test_sampling_follows_the_distribution_and_api(gpu):
     with pytest.raises(ValueError):
         ops.sample_top_k_top_p(xs[:1])
     assert ops.sample_top_k_top_p(torch.empty(0, 9, device=gpu), 1.0, 0, 0.0, torch.empty(0, device=gpu))[0].numel() == 0
+
+
+# =============================================================================== seeded shape sweeps
+def _sweep_shapes(seed, count, lo, hi, mult):
+    g = torch.Generator().manual_seed(seed)
+    out = []
+    for _ in range(count):
+        m, n, k = (int(torch.randint(lo, hi, (1,), generator=g)) for _ in range(3))
+        out.append((m, max(mult, n // mult * mult), max(mult, k // mult * mult)))
+    return out
+
+
+@pytest.mark.parametrize("dtype,mult", [(torch.bfloat16, 8), (torch.float32, 4), (torch.float32, 1), (torch.bfloat16, 1)])
+def test_linear_shape_sweep(gpu, dtype, mult):
+    """24 seeded shapes per case around the tile edges of every kernel (fast kernels take n, k multiples of
+    8 / 4; anything else goes through the general kernel): forward with bias, dgrad, wgrad with bias gradient."""
+    tol = TOL_F32 if dtype == torch.float32 else TOL_BF16
+    for (m, n, k) in _sweep_shapes(7 + mult, 24, 1, 700, mult):
+        x, w, b, dy = _lin_inputs(m, n, k, dtype, 200 + m + n + k)
+        xf, wf, bf, dyf = x.float(), w.float(), b.float(), dy.float()
+        y, _ = ops.linear_fwd(x.to(gpu), w.to(gpu), b.to(gpu), ops.EPI_BIAS)
+        assert rel(y, R.column_parallel_linear_forward(xf, wf, bf)[0]) < tol, (m, n, k)
+        rdx, rdw, rdb = R.linear_backward(xf, wf, dyf, True)
+        assert rel(ops.linear_dgrad(dy.to(gpu), w.to(gpu)), rdx) < tol, (m, n, k)
+        dw, db = ops.linear_wgrad(dy.to(gpu), x.to(gpu), True)
+        assert rel(dw, rdw) < tol and rel(db, rdb) < tol, (m, n, k)
+
+
+def test_gemv_shape_sweep(gpu):
+    g = torch.Generator().manual_seed(11)
+    for _ in range(24):
+        b = int(torch.randint(1, 33, (1,), generator=g))
+        n = int(torch.randint(1, 3000, (1,), generator=g))
+        k = int(torch.randint(1, 300, (1,), generator=g)) * 8
+        x = torch.randn(b, k, generator=g).bfloat16()
+        w = (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+        ref = F.linear(x.float(), w.float())
+        assert rel(ops.gemv(x.to(gpu), w.to(gpu)), ref) < TOL_BF16, (b, n, k)
+        idx, val = ops.gemv_argmax(x.to(gpu), w.to(gpu))
+        assert torch.equal(idx.cpu(), R.greedy_argmax(ref)), (b, n, k)
+        if n % 2 == 0:
+            sw = ops.gemv(x.to(gpu), w.to(gpu), None, ops.EPI_SWIGLU)
+            y = ref.bfloat16().float()
+            assert rel(sw, F.silu(y[:, : n // 2]) * y[:, n // 2:]) < TOL_BF16, (b, n, k)
+
+
+def test_ce_shape_sweep(gpu):
+    g = torch.Generator().manual_seed(12)
+    for i in range(16):
+        dtype = torch.bfloat16 if i % 2 else torch.float32
+        n = int(torch.randint(1, 40, (1,), generator=g))
+        v = int(torch.randint(1, 70000, (1,), generator=g))
+        start = int(torch.randint(0, 3, (1,), generator=g)) * v
+        x = (torch.randn(n, v, generator=g) * 3).to(dtype)
+        t = torch.randint(0, 3 * v, (n,), generator=g)
+        gr = torch.rand(n, generator=g)
+        ref_loss, ref_grad = R.cross_entropy_fp32(x, t, start, gr)
+        tol = TOL_F32 if dtype == torch.float32 else TOL_BF16
+        a = x.to(gpu)
+        loss, m, s, _ = ops.vocab_ce_fwd(a, t.to(gpu), start)
+        ops.vocab_ce_bwd_(a, t.to(gpu), m, s, gr.to(gpu), start)
+        b2 = x.to(gpu)
+        loss2, *_ = ops.vocab_ce_fwd_bwd_(b2, t.to(gpu), start, gr.to(gpu), 1.0)
+        for lo, gx in ((loss, a), (loss2, b2)):
+            assert (lo.cpu() - ref_loss).abs().max() <= TOL_LOSS * max(ref_loss.abs().max().item(), 0.1), (n, v, dtype)
+            assert rel(gx, ref_grad) < tol, (n, v, dtype)

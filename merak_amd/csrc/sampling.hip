@@ -382,14 +382,17 @@ __global__ __launch_bounds__(SP_THREADS) void sample_mass_kernel(const T* __rest
   }
 }
 
-// The draw: one wave per row walks the chunk that holds the target mass
+// The draw: one workgroup per row finds the chunk that holds the target mass; its 16 waves split that chunk's
+// slots into contiguous ranges, sum them, and the wave whose range holds the target walks it 64 slots at a time.
+constexpr int DR_WAVES = 16;
 template <typename T>
-__global__ __launch_bounds__(64) void sample_draw_kernel(const T* __restrict__ logits, int64_t V, float temperature,
-                                                         const float* __restrict__ uniforms,
-                                                         const RowState* __restrict__ state,
-                                                         int64_t* __restrict__ tokens) {
+__global__ __launch_bounds__(DR_WAVES * 64) void sample_draw_kernel(const T* __restrict__ logits, int64_t V,
+                                                                    float temperature,
+                                                                    const float* __restrict__ uniforms,
+                                                                    const RowState* __restrict__ state,
+                                                                    int64_t* __restrict__ tokens) {
   constexpr int EPV = Row<T>::EPV;
-  const int b = blockIdx.x, lane = threadIdx.x;
+  const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const RowState* st = state + b;
   uint64_t total = 0;
   for (int g = 0; g < SG; g++) total += st->part[g];
@@ -410,20 +413,51 @@ __global__ __launch_bounds__(64) void sample_draw_kernel(const T* __restrict__ l
   const uint32_t keep_key = st->keep_key;
   const Mass mass(temperature, f32_unkey(st->max_key) / temperature);
   const Slots<T> sl(logits + (int64_t)b * V, V);
-  int64_t s0, s1;
-  chunk_range(sl, pick, s0, s1);
-  for (int64_t base = s0; base < s1; base += 64) {
+  int64_t c0, c1;
+  chunk_range(sl, pick, c0, c1);
+  const int64_t per_wave = ((c1 - c0 + DR_WAVES * 64 - 1) / (DR_WAVES * 64)) * 64;  // whole steps of 64 slots
+  int64_t s0 = c0 + (int64_t)wave * per_wave, s1 = s0 + per_wave;
+  if (s0 > c1) s0 = c1;
+  if (s1 > c1) s1 = c1;
+  auto slot_mass = [&](int64_t s, uint64_t* q, int64_t& j0) -> uint64_t {  // masses of the kept elements of slot s
     float x[EPV] = {};
-    int64_t j0 = 0;
     int n = 0;
-    if (base + lane < s1) n = sl.load(base + lane, x, j0);
-    uint64_t q[EPV], t = 0;
+    j0 = 0;
+    if (s < s1) n = sl.load(s, x, j0);
+    uint64_t t = 0;
 #pragma unroll
     for (int e = 0; e < EPV; e++) {
       const float z = x[e] / temperature;
       q[e] = (e < n && Row<T>::key(x[e], z) >= keep_key) ? mass(x[e]) : 0;
       t += q[e];
     }
+    return t;
+  };
+  uint64_t mine = 0;
+  for (int64_t s = s0 + lane; s < s1; s += 64) {
+    uint64_t q[EPV];
+    int64_t j0;
+    mine += slot_mass(s, q, j0);
+  }
+  mine = wave_sum_u64(mine);
+  __shared__ uint64_t red[DR_WAVES];
+  if (lane == 0) red[wave] = mine;
+  __syncthreads();
+  int pick_wave = -1;
+#pragma unroll
+  for (int w = 0; w < DR_WAVES; w++) {
+    if (pick_wave < 0) {
+      if (run + red[w] > r)
+        pick_wave = w;
+      else
+        run += red[w];
+    }
+  }
+  if (wave != pick_wave) return;
+  for (int64_t base = s0; base < s1; base += 64) {
+    uint64_t q[EPV];
+    int64_t j0;
+    const uint64_t t = slot_mass(base + lane, q, j0);
     uint64_t incl = t;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
@@ -466,7 +500,7 @@ int launch_sample(const void* logits, int64_t B, int64_t V, float temperature, i
   hipLaunchKernelGGL(sample_mass_kernel<T>, grid, block, 0, s, lg, V, temperature, top_k, top_p, kp, pp, state,
                      filtered);
   if (tokens)
-    hipLaunchKernelGGL(sample_draw_kernel<T>, dim3((unsigned)B), dim3(64), 0, s, lg, V, temperature, uniforms, state,
+    hipLaunchKernelGGL(sample_draw_kernel<T>, dim3((unsigned)B), dim3(DR_WAVES * 64), 0, s, lg, V, temperature, uniforms, state,
                        tokens);
   MTP_CHECK_LAUNCH("sample");
   return MTP_OK;

@@ -24,6 +24,11 @@ are closed forms, library routines and brute force:
   shard_master_weight     hand-written table for stride 1 and 2 (tests/golden/shard_table.json)
   greedy_argmax           brute-force scan, first index on ties
   VocabUtility / divide   integer closed forms
+  top_k_logits            hand-worked cases (k-th value ties, the token that crosses top_p stays, first token
+                          always stays); transformers' TopKLogitsWarper / TopPLogitsWarper on random logits
+  sample_tail             numpy.searchsorted on the cumulative distribution; draw frequencies over 40000
+                          uniforms against the probabilities (torch.multinomial's own random stream cannot be
+                          reproduced, so the draw takes the uniforms as an argument)
 
 The third-party arithmetic under all of this is PyTorch (the reference pins
 torch>=2.0.0, setup.py:46) and, for the activations, transformers

@@ -237,24 +237,28 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_kernel(const uint16_t* __rest
     multiply();
   }
 
-  // ---- sum the 8 k-slices through LDS, one row group at a time -------------
-  // part_lds[w][nb][j][lane]; fin[b][local row]
-  __shared__ float part_lds[GV_WAVES][NB][4][64];
+  // ---- sum the 8 k-slices through LDS: up to 8 tiles (row group x batch tile) per wave at a time, i.e. one
+  // phase (two barriers) for all but the largest configuration ---------------------------------------------
+  // part_lds[w][group][nb][j][lane]; fin[b][local row]
+  constexpr int GP = (R * NB <= 8) ? R : 8 / NB;  // row groups per phase
+  __shared__ float part_lds[GV_WAVES][GP][NB][4][64];
   __shared__ float fin[16 * NB][16 * R + 1];
 #pragma unroll
-  for (int r = 0; r < R; r++) {
+  for (int r0 = 0; r0 < R; r0 += GP) {
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++)
+    for (int rr = 0; rr < GP; rr++)
 #pragma unroll
-      for (int j = 0; j < 4; j++) part_lds[wave][nb][j][lane] = acc[r][nb][j];
+      for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) part_lds[wave][rr][nb][j][lane] = acc[r0 + rr][nb][j];
     __syncthreads();
-    for (int e = tid; e < NB * 256; e += GV_THREADS) {
-      const int nb = e >> 8, j = (e >> 6) & 3, l = e & 63;
+    for (int e = tid; e < GP * NB * 256; e += GV_THREADS) {
+      const int rr = e / (NB * 256), nb = (e >> 8) % NB, j = (e >> 6) & 3, l = e & 63;
       float s = 0.f;
 #pragma unroll
-      for (int wv = 0; wv < GV_WAVES; wv++) s += part_lds[wv][nb][j][l];
+      for (int wv = 0; wv < GV_WAVES; wv++) s += part_lds[wv][rr][nb][j][l];
       // D[i][b]: lane l, register j holds row i = 4*(l/16)+j, column b = l%16
-      fin[(l & 15) + 16 * nb][16 * r + 4 * (l >> 4) + j] = s;
+      fin[(l & 15) + 16 * nb][16 * (r0 + rr) + 4 * (l >> 4) + j] = s;
     }
     __syncthreads();
   }

@@ -206,7 +206,9 @@ int64_t mtp_gemv_argmax_workspace_bytes(int64_t B, int64_t N, int64_t K);
 /* idx[b] = argmax_n (X[b,:] . W[n,:]) — first index among equal maxima, NaN
  * counts as the maximum (torch.argmax semantics, :227); maxval[b] (may be
  * NULL) receives the winning fp32 logit.  The [B,N] logits are never
- * written to memory. */
+ * written to memory.  "Equal" means equal as computed: rows handled by
+ * different workgroups are summed along k in a different (fixed) order, so
+ * two identical weight rows far apart may differ in the last bit. */
 int mtp_gemv_argmax(const void* x, const void* w,
                     int64_t* idx, float* maxval,
                     void* workspace, int64_t workspace_bytes,

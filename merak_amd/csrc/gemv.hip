@@ -27,8 +27,7 @@
 
 namespace {
 
-constexpr int GV_WAVES = 8;
-constexpr int GV_THREADS = GV_WAVES * MTP_WAVE;
+constexpr int GV_MAX_WAVES = 8;  // waves per workgroup: 8, or 4 for the register-heavy configurations
 
 struct ArgPart {
   float v;
@@ -79,12 +78,15 @@ __device__ __forceinline__ uint32_t rot8_in_row(uint32_t v) {
 }
 
 // MODE 0: store Y (+bias); MODE 1: SwiGLU store; MODE 2: argmax partials
-template <int R, int NB, int MODE, bool GUARD, int D>
-__global__ __launch_bounds__(GV_THREADS) void gemv_kernel(const uint16_t* __restrict__ x,
+// W waves split K.  Configurations whose registers allow only 8 waves per CU run as two independent workgroups of
+// 4 waves rather than one of 8: while one sums its partial tiles and writes its outputs the other keeps streaming.
+template <int R, int NB, int MODE, bool GUARD, int D, int W>
+__global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __restrict__ x,
                                                           const uint16_t* __restrict__ w,
                                                           const uint16_t* __restrict__ bias,
                                                           uint16_t* __restrict__ y, ArgPart* __restrict__ part,
                                                           int B, int64_t N, int64_t K, int rot_mul) {
+  constexpr int GV_WAVES = W, GV_THREADS = W * MTP_WAVE;
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
@@ -142,7 +144,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_kernel(const uint16_t* __rest
   // Every workgroup starts its walk along k at a different pair and wraps around: if all of them began at
   // k = 0 the whole chip would, at any moment, ask for the same few hundred bytes of every row, which
   // (rows being a power-of-two apart) live in the same few memory channels.
-  const int64_t rot = GUARD || (pairs % GV_WAVES) ? 0 : ((int64_t)blockIdx.x * rot_mul) % pairs;
+  // (Summation order along k therefore differs between workgroups: equal weight rows that live in different
+  // workgroups give logits that are equal to rounding, not necessarily bit for bit.)
+  const int64_t rot = GUARD || (pairs % GV_MAX_WAVES) ? 0 : ((int64_t)blockIdx.x * rot_mul) % pairs;
 
   f32x4_t acc[R][NB];
 #pragma unroll
@@ -420,7 +424,7 @@ struct GemvCfg {
   int D;  // k-pairs in flight per wave and step
 };
 
-bool depth_ok(int64_t K, int d) { return d == 1 || (K % 64 == 0 && ((K / 64) % (GV_WAVES * d)) == 0); }
+bool depth_ok(int64_t K, int d) { return d == 1 || (K % 64 == 0 && ((K / 64) % (GV_MAX_WAVES * d)) == 0); }
 
 GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode) {
   const int64_t groups = ((mode == 1 ? N / 2 : N) + 15) / 16 * (mode == 1 ? 2 : 1);
@@ -458,7 +462,8 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   int rot_mul = 1;
   if (const char* e = getenv("MTP_GEMV_ROT")) rot_mul = atoi(e);
 #define GV_LAUNCH(RR, NNB, GG, DD)                                                                              \
-  hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD>), dim3(n_wg), dim3(GV_THREADS), 0, s,                  \
+  hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD, (RR >= 8 ? 4 : 8)>), dim3(n_wg),                       \
+                     dim3((RR >= 8 ? 4 : 8) * MTP_WAVE), 0, s,                                                  \
                      (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part, (int)B, \
                      N, K, rot_mul)
 #define GV_BY_DEPTH(RR, NNB)                                                   \

@@ -46,6 +46,7 @@ struct GemmArgs {
   void* C;             // main output (bf16 or fp32), may be null when C2 carries the result
   void* C2;            // activation output (bf16), epilogue dependent
   const uint16_t* bias;
+  void* rowsum;        // EPI_ROWSUM: [M] sums of the rows of opA(A) over k (bf16 or fp32 like C; (+)= with accumulate)
   int M, N, K;
   int64_t lda, ldb, ldc, ldc2;
   int accumulate;      // C += result
@@ -55,6 +56,10 @@ struct GemmArgs {
 };
 
 enum : int { OUT_BF16 = 0, OUT_F32 = 1 };
+// Plain product that also sums the rows of its A operand along k: with A = dY^T (the wgrad product) those sums
+// are the bias gradient.  Every wave adds up the fragments it feeds to the MFMAs (one v_dot2 per pair of
+// elements, in the shadow of the MFMAs); the first column of tiles writes the result.
+constexpr int EPI_ROWSUM = 18;
 
 // compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{})
 template <int... Is, typename F>
@@ -402,10 +407,24 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   auto read_frags = [&](int stage, int kk, int slot) {
     static_for<NFR>([&](auto u) { read_one(stage, kk, slot, u); });
   };
+  float rsum[TI];
+#pragma unroll
+  for (int i = 0; i < TI; i++) rsum[i] = 0.f;
   auto mfma_one = [&](int slot, auto t_tag) {  // t-th MFMA of a step in shell order
     constexpr int t = decltype(t_tag)::value;
     constexpr int i = shell_pair(t, TI, TJ).i, j = shell_pair(t, TI, TJ).j;
     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[slot][j], af[slot][i], acc[i][j], 0, 0, 0);
+    if constexpr (EPI == EPI_ROWSUM && t < TI) {
+      // the t-th A fragment of this step: 8 k of one row per lane
+      const bf16x8_t a = af[slot][t];
+      const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
+      float r = rsum[t];
+      r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 0, 1), one, r, false);
+      r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 2, 3), one, r, false);
+      r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 4, 5), one, r, false);
+      r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 6, 7), one, r, false);
+      rsum[t] = r;
+    }
   };
   auto mfmas = [&](int slot) {
     static_for<NMF>([&](auto t) { mfma_one(slot, t); });
@@ -504,6 +523,26 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
   __syncthreads();  // the epilogue reuses the tile buffers
   if (p.debug & 2) return;
+
+  if constexpr (EPI == EPI_ROWSUM) {
+    static_assert(NMF >= TI, "every A fragment of a step must meet an MFMA");
+    if (tn == 0 && wn == 0) {
+#pragma unroll
+      for (int i = 0; i < TI; i++) {
+        const float t = rsum[i] + __shfl_xor(rsum[i], 32, 64);  // the two k halves of a row
+        const int row = m0 + wm * (BM / WGM) + 32 * i + l32;
+        if (lh == 0 && row < p.M) {
+          if (OUT == OUT_F32) {
+            float* q = (float*)p.rowsum + row;
+            *q = p.accumulate ? *q + t : t;
+          } else {
+            uint16_t* q = (uint16_t*)p.rowsum + row;
+            *q = f32_to_bf16_bits(p.accumulate ? bf16_bits_to_f32(*q) + t : t);
+          }
+        }
+      }
+    }
+  }
 
   // ---- epilogue ----------------------------------------------------------------
   // acc[i][j][r]: row m = m0 + wm*BM/2 + 32i + l32, column block j, n_local = 8*(r/4) + 4*lh + r%4.
@@ -682,7 +721,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
         flush(i, p.C, p.ldc, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::false_type{}, p.accumulate != 0);
         wave_lds_sync();
       }
-      if (EPI != MTP_EPI_NONE && EPI != MTP_EPI_BIAS) {
+      if (EPI != MTP_EPI_NONE && EPI != MTP_EPI_BIAS && EPI != EPI_ROWSUM) {
 #pragma unroll
         for (int j = 0; j < TJ; j++)
 #pragma unroll

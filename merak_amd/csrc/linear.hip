@@ -6,8 +6,8 @@
 int mtp_gemm_bf16_nt(const void* A, const void* B, const void* bias, void* C, void* C2, int64_t M, int64_t N,
                      int64_t K, int epilogue, hipStream_t s);
 int mtp_gemm_bf16_dgrad(const void* dy, const void* w, void* dx, int64_t M, int64_t N, int64_t K, hipStream_t s);
-int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, int64_t M, int64_t N, int64_t K, int dw_dtype,
-                        int accumulate, hipStream_t s);
+int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
+                        int dw_dtype, int accumulate, hipStream_t s);
 int mtp_gemm_generic(const void* A, int64_t sam, int64_t sak, const void* B, int64_t sbn, int64_t sbk,
                      const void* bias, void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, int out_dtype,
                      int accumulate, hipStream_t s);
@@ -114,8 +114,7 @@ extern "C" int mtp_linear_wgrad(const void* dy, const void* x, void* dw, void* d
   MTP_REQUIRE(M == 0 || (dy && x), MTP_EINVAL, "linear_wgrad: null input");
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MTP_BF16 && M > 0 && fast_ok(N, K, dy, x) && aligned16(dw)) {
-    rc = mtp_gemm_bf16_wgrad(dy, x, dw, M, N, K, dw_dtype, accumulate, s);
-    if (rc == MTP_OK && db) return mtp_colsum(dy, db, M, N, dtype, dw_dtype, accumulate, s);
+    rc = mtp_gemm_bf16_wgrad(dy, x, dw, db, M, N, K, dw_dtype, accumulate, s);
     if (rc != MTP_EUNSUPPORTED) return rc;
   }
   if (dtype == MTP_F32 && dw_dtype == MTP_F32 && M > 0 && f32_fast_ok(dy, x, N, K, M * N * 4, M * K * 4)) {

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTP_ABI_VERSION 2
+#define MTP_ABI_VERSION 3
 
 /* element types */
 #define MTP_F32  0
@@ -239,6 +239,54 @@ int mtp_sample_top_k_top_p(const void* logits, int dtype, int64_t B, int64_t V,
                            float temperature, int top_k, float top_p,
                            const float* uniforms, int64_t* tokens, float* filtered,
                            void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Single-position step with a key/value cache.  The reference's generation
+ * loop re-runs the whole sequence for every new token and keeps one row of
+ * the output (Merak/inference/text_generation_inference.py:199-203, row
+ * picked at :223); for a causal model the same row comes from running only
+ * the new position against cached keys and values.  These are the pieces
+ * of the HF Llama block between the tensor-parallel linears; head_dim is
+ * 128, tensors are bf16 unless stated.
+ * ------------------------------------------------------------------------ */
+/* h = x (+ residual, may be NULL), rounded to the tensor dtype;
+ * residual_out (may be NULL) = h; y = weight * dtype(h * rsqrt(mean(h^2) +
+ * eps)) with the mean and the scaling in fp32 (HF LlamaRMSNorm.forward in
+ * front of which the block's `residual + hidden_states` has been folded).
+ * x, residual, y, residual_out: [rows, dim]; weight: [dim]; dtype f32 or
+ * bf16.  y may alias x; residual_out may alias residual. */
+int mtp_rmsnorm(const void* x, const void* residual, const void* weight,
+                void* y, void* residual_out,
+                int64_t rows, int64_t dim, float eps, int dtype, void* stream);
+
+/* qkv: [B, (n_q_heads + 2 n_kv_heads) * 128], q heads first, then k, then v
+ * (the fused QKV linear's output).  positions: int64 [B], position of the
+ * new token of each row.  Rotary embedding x*cos + rotate_half(x)*sin (HF
+ * apply_rotary_pos_emb) with cos/sin tables [max_positions, 128] of the
+ * tensor dtype; rotated q -> q_out [B, n_q_heads, 128]; rotated k and plain
+ * v -> row positions[b] of k_cache / v_cache [B, n_kv_heads, max_len, 128].
+ * A row whose position lies outside the tables or the cache is left
+ * unwritten (no fault). */
+int mtp_rope_kv_append(const void* qkv, const void* cos_table, const void* sin_table,
+                       const int64_t* positions, void* q_out, void* k_cache, void* v_cache,
+                       int64_t B, int n_q_heads, int n_kv_heads, int head_dim,
+                       int64_t max_len, int64_t max_positions, int dtype, void* stream);
+
+/* out[b,h,:] = softmax_t(scale * q[b,h,:] . K[b,h/g,t,:]) V[b,h/g,t,:] over
+ * t < lens[b] (int64 [B] on the device, clamped to [0, max_len]; a row with
+ * no tokens gives zeros), g = n_q_heads / n_kv_heads <= 16: grouped-query
+ * attention of one new position (HF eager attention: fp32 softmax,
+ * probabilities rounded to bf16 for the product with V).  len_bound: an
+ * upper bound of lens known on the host (<= max_len); it only decides over
+ * how many workgroups a sequence is split.  workspace: device scratch of
+ * mtp_attn_decode_workspace_bytes(B, n_q_heads, n_kv_heads, len_bound)
+ * bytes (may be NULL when that is 0). */
+int64_t mtp_attn_decode_workspace_bytes(int64_t B, int n_q_heads, int n_kv_heads, int64_t len_bound);
+int mtp_attn_decode(const void* q, const void* k_cache, const void* v_cache,
+                    const int64_t* lens, void* out,
+                    void* workspace, int64_t workspace_bytes,
+                    int64_t B, int n_q_heads, int n_kv_heads, int head_dim,
+                    int64_t max_len, int64_t len_bound, float scale, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------
  * Measurement helpers (used by bench.py to state what this GPU can do).

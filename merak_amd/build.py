@@ -30,7 +30,7 @@ SOURCES = [
     "gemm_bf16_fwd.hip",
     "gemm_bf16_dgrad.hip",
     "gemm_bf16_wgrad.hip",
-    "gemm_generic.hip", "gemm_f32.hip",
+    "gemm_generic.hip", "gemm_f32.hip", "decode_attn.hip",
     "linear.hip",
 ]
 

@@ -1,0 +1,139 @@
+"""One new position per sequence through a Llama-shaped model with a key/value cache.
+
+The reference's generation loop pushes the whole token buffer through the
+model for every new token and keeps row ``context_length - 1`` of the output
+(Merak/inference/text_generation_inference.py:199-203,223).  A causal model
+gives the same row from the new position alone once the keys and values of
+the earlier positions are kept, which turns every linear of the block into a
+GEMV that streams its weight once and the attention into one pass over the
+cache.  ``LlamaDecoder.step`` is that row; the greedy pick (:226-227) or the
+sampling tail (:229-235) follows it.
+
+Weights are the tensor-parallel layers' own tensors: the fused QKV and
+gate/up column-parallel weights ([out, in], q heads / k heads / v heads and
+gate rows / up rows stacked along ``out``) and the row-parallel ``o`` and
+``down`` weights.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+
+from .. import ops
+from .greedy import greedy_next_token
+
+
+def rope_tables(head_dim: int, max_positions: int, theta: float = 10000.0, scaling: Optional[dict] = None,
+                dtype: torch.dtype = torch.float32, device=None):
+    """cos / sin tables [max_positions, head_dim] of HF ``LlamaRotaryEmbedding``: default rope type, or
+    ``scaling = {"rope_type": "llama3", "factor", "low_freq_factor", "high_freq_factor",
+    "original_max_position_embeddings"}`` (the Llama-3.1 frequency rescale).  Computed in fp32, then cast."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
+    if scaling is not None and scaling.get("rope_type", "default") != "default":
+        if scaling["rope_type"] != "llama3":
+            raise NotImplementedError(f"rope_type {scaling['rope_type']!r}")
+        factor, low, high = scaling["factor"], scaling["low_freq_factor"], scaling["high_freq_factor"]
+        old_len = scaling["original_max_position_embeddings"]
+        wavelen = 2 * math.pi / inv_freq
+        scaled = torch.where(wavelen > old_len / low, inv_freq / factor, inv_freq)
+        smooth = (old_len / wavelen - low) / (high - low)
+        mid = (1 - smooth) * scaled / factor + smooth * scaled
+        is_mid = ~(wavelen < old_len / high) & ~(wavelen > old_len / low)
+        inv_freq = torch.where(is_mid, mid, scaled)
+    freqs = torch.outer(torch.arange(max_positions).float(), inv_freq)
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return emb.cos().to(dtype=dtype, device=device), emb.sin().to(dtype=dtype, device=device)
+
+
+@dataclass
+class LlamaBlockWeights:
+    input_norm: torch.Tensor   # [H]
+    qkv: torch.Tensor          # [(n_q + 2 n_kv) * head_dim, H]
+    o: torch.Tensor            # [H, n_q * head_dim]
+    post_norm: torch.Tensor    # [H]
+    gate_up: torch.Tensor      # [2 I, H]: gate rows, then up rows
+    down: torch.Tensor         # [H, I]
+
+
+class LlamaDecoder:
+    """Decode-only runner: ``step(tokens)`` appends one token per sequence and returns the next one.
+
+    ``batch`` sequences share one cache allocation [batch, n_kv_heads, max_len, head_dim] per layer; every
+    sequence has its own length (``self.lens``, on the device, so a step never synchronises with the host)."""
+
+    def __init__(self, embed: torch.Tensor, blocks: List[LlamaBlockWeights], final_norm: torch.Tensor,
+                 lm_head: torch.Tensor, n_q_heads: int, n_kv_heads: int, head_dim: int = 128, eps: float = 1e-5,
+                 rope_theta: float = 10000.0, rope_scaling: Optional[dict] = None, max_len: int = 4096,
+                 batch: int = 1):
+        dev, dt = lm_head.device, lm_head.dtype
+        self.embed, self.blocks, self.final_norm, self.lm_head = embed, blocks, final_norm, lm_head
+        self.n_q, self.n_kv, self.head_dim, self.eps = n_q_heads, n_kv_heads, head_dim, eps
+        self.max_len, self.batch = max_len, batch
+        self.cos, self.sin = rope_tables(head_dim, max_len, rope_theta, rope_scaling, dtype=dt, device=dev)
+        self.k_cache = [torch.zeros((batch, n_kv_heads, max_len, head_dim), dtype=dt, device=dev) for _ in blocks]
+        self.v_cache = [torch.zeros((batch, n_kv_heads, max_len, head_dim), dtype=dt, device=dev) for _ in blocks]
+        self.lens = torch.zeros((batch,), dtype=torch.int64, device=dev)
+        self.host_len_bound = 0           # upper bound of self.lens kept on the host
+        from .. import _lib
+        need = _lib.lib().mtp_gemv_argmax_workspace_bytes(batch, lm_head.shape[0], lm_head.shape[1])
+        self.argmax_ws = torch.empty((max(int(need), 8),), dtype=torch.uint8, device=dev)
+        # the number of splits, and with it the need, does not shrink when the length bound grows
+        need = ops.attn_decode_workspace_bytes(batch, n_q_heads, n_kv_heads, max_len)
+        self.attn_ws = torch.empty((max(int(need), 8),), dtype=torch.uint8, device=dev)
+
+    @classmethod
+    def from_hf(cls, model, max_len: int = 4096, batch: int = 1):
+        """From a ``transformers`` ``LlamaForCausalLM`` (weights are concatenated once, not shared)."""
+        cfg = model.config
+        blocks = []
+        for layer in model.model.layers:
+            a, m = layer.self_attn, layer.mlp
+            blocks.append(LlamaBlockWeights(
+                layer.input_layernorm.weight.data,
+                torch.cat([a.q_proj.weight.data, a.k_proj.weight.data, a.v_proj.weight.data]).contiguous(),
+                a.o_proj.weight.data.contiguous(), layer.post_attention_layernorm.weight.data,
+                torch.cat([m.gate_proj.weight.data, m.up_proj.weight.data]).contiguous(),
+                m.down_proj.weight.data.contiguous()))
+        rp = getattr(cfg, "rope_parameters", None) or getattr(cfg, "rope_scaling", None) or {}
+        theta = rp.get("rope_theta", getattr(cfg, "rope_theta", 10000.0))
+        scaling = rp if rp.get("rope_type", "default") != "default" else None
+        head_dim = getattr(cfg, "head_dim", None) or cfg.hidden_size // cfg.num_attention_heads
+        return cls(model.model.embed_tokens.weight.data, blocks, model.model.norm.weight.data,
+                   model.lm_head.weight.data, cfg.num_attention_heads, cfg.num_key_value_heads, head_dim,
+                   cfg.rms_norm_eps, theta, scaling, max_len, batch)
+
+    def reset(self):
+        self.lens.zero_()
+        self.host_len_bound = 0
+
+    def hidden(self, tokens: torch.Tensor) -> torch.Tensor:
+        """Appends ``tokens`` (int64 [batch]) and returns the final-norm output [batch, H] of their position."""
+        if self.host_len_bound >= self.max_len:
+            raise RuntimeError(f"key/value cache full ({self.max_len} positions)")
+        positions = self.lens.clone()
+        self.lens += 1
+        self.host_len_bound += 1
+        x = ops.embedding_gather(tokens, self.embed, 0, self.embed.shape[0])
+        residual = None
+        B = x.shape[0]
+        for w, kc, vc in zip(self.blocks, self.k_cache, self.v_cache):
+            h, residual = ops.rmsnorm(x, w.input_norm, self.eps, residual, want_residual=True)
+            qkv = ops.gemv(h, w.qkv)
+            q = ops.rope_kv_append(qkv, self.cos, self.sin, positions, kc, vc, self.n_q)
+            a = ops.attn_decode(q, kc, vc, self.lens, len_bound=self.host_len_bound, workspace=self.attn_ws)
+            o = ops.gemv(a.view(B, -1), w.o)
+            h, residual = ops.rmsnorm(o, w.post_norm, self.eps, residual, want_residual=True)
+            act = ops.gemv(h, w.gate_up, None, ops.EPI_SWIGLU)
+            x = ops.gemv(act, w.down)
+        return ops.rmsnorm(x, self.final_norm, self.eps, residual)
+
+    def logits(self, tokens: torch.Tensor) -> torch.Tensor:
+        """The row the reference slices out at :223 (fp32 accumulation, model dtype)."""
+        return ops.gemv(self.hidden(tokens), self.lm_head)
+
+    def step(self, tokens: torch.Tensor) -> torch.Tensor:
+        """Greedy next token per sequence (:226-227); the [batch, vocab] logits are never written."""
+        return greedy_next_token(self.hidden(tokens), self.lm_head, self.argmax_ws)

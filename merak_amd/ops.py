@@ -340,3 +340,86 @@ def sample_top_k_top_p(logits: torch.Tensor, temperature: float = 1.0, top_k: in
                                               workspace.numel() * workspace.element_size(), _stream(dev)),
                    "mtp_sample_top_k_top_p")
     return tokens, filtered
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None,
+            want_residual: bool = False):
+    """-> y, or (y, h) with ``want_residual``: h = x (+ residual), y = weight * (h * rsqrt(mean(h^2) + eps))."""
+    dev = _require_gpu(x, weight, residual)
+    x = _contig(x)
+    dim = x.shape[-1]
+    if weight.shape != (dim,) or weight.dtype != x.dtype:
+        raise ValueError(f"rmsnorm: weight {tuple(weight.shape)} {weight.dtype} for rows of {dim} {x.dtype}")
+    if residual is not None:
+        residual = _contig(residual)
+        if residual.shape != x.shape or residual.dtype != x.dtype:
+            raise ValueError("rmsnorm: residual must match x")
+    y = torch.empty_like(x)
+    h = torch.empty_like(x) if want_residual else None
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_rmsnorm(_p(x), _p(residual), _p(_contig(weight)), _p(y), _p(h), x.numel() // dim, dim,
+                                          float(eps), _dt(x), _stream(dev)), "mtp_rmsnorm")
+    return (y, h) if want_residual else y
+
+
+def rope_kv_append(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: torch.Tensor, positions: torch.Tensor,
+                   k_cache: torch.Tensor, v_cache: torch.Tensor, n_q_heads: int) -> torch.Tensor:
+    """Rotates the new q and k heads of ``qkv`` [B, (n_q + 2 n_kv) * 128], writes k and v into row
+    ``positions[b]`` of the caches [B, n_kv, max_len, 128] and returns the rotated q [B, n_q, 128]."""
+    dev = _require_gpu(qkv, cos_table, sin_table, positions, k_cache, v_cache)
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("rope_kv_append: caches must be contiguous [B, n_kv_heads, max_len, head_dim] of one shape")
+    B, n_kv, max_len, hd = k_cache.shape
+    qkv = _contig(qkv)
+    if qkv.shape != (B, (n_q_heads + 2 * n_kv) * hd):
+        raise ValueError(f"rope_kv_append: qkv {tuple(qkv.shape)} for {n_q_heads}+2*{n_kv} heads of {hd}")
+    if cos_table.shape != sin_table.shape or cos_table.dim() != 2 or cos_table.shape[1] != hd:
+        raise ValueError("rope_kv_append: cos / sin tables must be [max_positions, head_dim]")
+    for t in (cos_table, sin_table, k_cache, v_cache):
+        if t.dtype != qkv.dtype:
+            raise ValueError("rope_kv_append: all tensors must share the dtype of qkv")
+    if positions.dtype != torch.int64 or positions.numel() != B:
+        raise ValueError("rope_kv_append: positions must be int64 [B]")
+    q = torch.empty((B, n_q_heads, hd), dtype=qkv.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_rope_kv_append(_p(qkv), _p(_contig(cos_table)), _p(_contig(sin_table)),
+                                                 _p(_contig(positions)), _p(q), _p(k_cache), _p(v_cache), B,
+                                                 n_q_heads, n_kv, hd, max_len, cos_table.shape[0], _dt(qkv),
+                                                 _stream(dev)), "mtp_rope_kv_append")
+    return q
+
+
+def attn_decode_workspace_bytes(B: int, n_q_heads: int, n_kv_heads: int, len_bound: int) -> int:
+    return int(_lib.lib().mtp_attn_decode_workspace_bytes(B, n_q_heads, n_kv_heads, len_bound))
+
+
+def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, lens: torch.Tensor,
+                scale: Optional[float] = None, len_bound: Optional[int] = None,
+                workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention of one new position per row over the first ``lens[b]`` cached tokens.
+    q [B, n_q, 128], caches [B, n_kv, max_len, 128] -> [B, n_q, 128]."""
+    dev = _require_gpu(q, k_cache, v_cache, lens, workspace)
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("attn_decode: caches must be contiguous [B, n_kv_heads, max_len, head_dim] of one shape")
+    B, n_kv, max_len, hd = k_cache.shape
+    q = _contig(q)
+    if q.dim() != 3 or q.shape[0] != B or q.shape[2] != hd:
+        raise ValueError(f"attn_decode: q {tuple(q.shape)} against caches {tuple(k_cache.shape)}")
+    if not (q.dtype == k_cache.dtype == v_cache.dtype):
+        raise ValueError("attn_decode: q and the caches must share a dtype")
+    if lens.dtype != torch.int64 or lens.numel() != B:
+        raise ValueError("attn_decode: lens must be int64 [B]")
+    n_q = q.shape[1]
+    len_bound = max_len if len_bound is None else int(len_bound)
+    scale = hd ** -0.5 if scale is None else float(scale)
+    lib = _lib.lib()
+    need = int(lib.mtp_attn_decode_workspace_bytes(B, n_q, n_kv, len_bound))
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty((need,), dtype=torch.uint8, device=dev)
+    out = torch.empty_like(q)
+    wbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    with torch.cuda.device(dev):
+        _lib.check(lib.mtp_attn_decode(_p(q), _p(k_cache), _p(v_cache), _p(_contig(lens)), _p(out), _p(workspace),
+                                       wbytes, B, n_q, n_kv, hd, max_len, len_bound, scale, _dt(q), _stream(dev)),
+                   "mtp_attn_decode")
+    return out

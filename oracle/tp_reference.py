@@ -293,3 +293,80 @@ def sample_tail(logits, temperature, top_k, top_p, uniforms):
     target = uniforms.double().view(-1, 1) * cdf[:, -1:]
     tokens = (cdf <= target).sum(-1).clamp_max(logits.shape[-1] - 1)             # :235 (see above)
     return tokens, probs
+
+
+# --------------------------------------------------------------------------- one position against a cache
+# The generation loop feeds the whole token buffer through the model for every new token and keeps row
+# context_length-1 of the output (Merak/inference/text_generation_inference.py:199-203,223).  The functions
+# below compute that row for an HF Llama block (the model family the reference's examples wrap) from the new
+# position alone plus the keys and values of the earlier ones; they are pinned against transformers' own
+# LlamaDecoderLayer / LlamaModel run over the full sequence (tests/test_oracle_pins.py).
+def rms_norm(x, weight, eps, residual=None):
+    """HF LlamaRMSNorm.forward with the block's ``residual + hidden_states`` in front: returns (y, h)."""
+    h = x if residual is None else residual + x
+    hf = h.float()
+    variance = hf.pow(2).mean(-1, keepdim=True)
+    return weight * (hf * torch.rsqrt(variance + eps)).to(x.dtype), h
+
+
+def rotate_half(x):
+    """HF modeling_llama.rotate_half."""
+    x1, x2 = x[..., : x.shape[-1] // 2], x[..., x.shape[-1] // 2:]
+    return torch.cat((-x2, x1), dim=-1)
+
+
+def rope_tables(head_dim, max_positions, theta=10000.0, dtype=torch.float32):
+    """cos / sin [max_positions, head_dim] of HF LlamaRotaryEmbedding with the default rope type:
+    inv_freq = theta^(-2i/d), angles = position x inv_freq, both halves of the last dim hold the same angles."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
+    freqs = torch.outer(torch.arange(max_positions).float(), inv_freq)
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+def apply_rope(x, cos, sin):
+    """HF apply_rotary_pos_emb for one position per row: x [B, heads, d], cos / sin [B, d]."""
+    return x * cos[:, None, :] + rotate_half(x) * sin[:, None, :]
+
+
+def attn_decode(q, k_cache, v_cache, lens, scale=None):
+    """Grouped-query attention of one new position (HF eager_attention_forward with repeat_kv, no mask needed:
+    every cached token is in the past): q [B, n_q, d], caches [B, n_kv, max_len, d], lens [B] -> [B, n_q, d]."""
+    B, n_q, d = q.shape
+    n_kv = k_cache.shape[1]
+    g = n_q // n_kv
+    scale = d ** -0.5 if scale is None else scale
+    out = torch.zeros_like(q)
+    for b in range(B):
+        n = int(lens[b])
+        if n == 0:
+            continue
+        k = k_cache[b, :, :n].repeat_interleave(g, dim=0)          # [n_q, n, d]
+        v = v_cache[b, :, :n].repeat_interleave(g, dim=0)
+        w = torch.einsum("hd,hnd->hn", q[b], k) * scale
+        w = F.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
+        out[b] = torch.einsum("hn,hnd->hd", w, v)
+    return out
+
+
+def llama_block_step(x, residual, positions, lens, w, k_cache, v_cache, cos_table, sin_table, n_q_heads, eps):
+    """One position per row through an HF LlamaDecoderLayer.  ``x`` is what the previous block's MLP returned
+    (or the embedding), ``residual`` the stream it has to be added to (None for the first block); returns the
+    same pair for the next block.  ``w``: input_norm, qkv [(n_q + 2 n_kv) d, H], o [H, n_q d],
+    post_norm, gate_up [2 I, H] (gate rows first), down [H, I].  Writes the new key / value at ``positions``."""
+    B = x.shape[0]
+    n_kv, d = k_cache.shape[1], k_cache.shape[3]
+    h, res = rms_norm(x, w["input_norm"], eps, residual)
+    qkv = F.linear(h, w["qkv"]).view(B, n_q_heads + 2 * n_kv, d)
+    cos, sin = cos_table[positions], sin_table[positions]
+    q = apply_rope(qkv[:, :n_q_heads], cos, sin)
+    k = apply_rope(qkv[:, n_q_heads:n_q_heads + n_kv], cos, sin)
+    v = qkv[:, n_q_heads + n_kv:]
+    for b in range(B):
+        k_cache[b, :, positions[b]] = k[b]
+        v_cache[b, :, positions[b]] = v[b]
+    a = attn_decode(q, k_cache, v_cache, lens)
+    o = F.linear(a.reshape(B, -1), w["o"])
+    h2, res2 = rms_norm(o, w["post_norm"], eps, res)
+    act = swiglu(F.linear(h2, w["gate_up"]))
+    return F.linear(act, w["down"]), res2

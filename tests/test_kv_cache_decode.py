@@ -1,0 +1,240 @@
+"""GPU parity of the cached single-position step (RMSNorm, rotary + cache append, attention over the cache,
+the whole Llama block and model) against the CPU oracle, through the C ABI.
+
+Tolerances: bf16 results 1e-2 relative (norm-wise) against the oracle's fp32 arithmetic on the same bf16
+inputs; fp32 RMSNorm 1e-4; copies (the value rows of the cache, untouched cache rows) bit-exact.
+"""
+import os
+
+import pytest
+import torch
+
+from merak_amd import ops
+from merak_amd.inference import LlamaDecoder, rope_tables
+from oracle import tp_reference as R
+
+pytestmark = pytest.mark.gpu
+TOL_F32, TOL_BF16 = 1e-4, 1e-2
+
+
+def rel(got, ref):
+    got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
+    return ((got - ref).norm() / ref.norm().clamp_min(1e-300)).item()
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(4321 + seed)
+
+
+@pytest.mark.parametrize("dtype,rows,dim", [(torch.bfloat16, 1, 4096), (torch.bfloat16, 32, 4096), (torch.bfloat16, 5, 1000),
+                                            (torch.float32, 3, 768), (torch.bfloat16, 2, 8192), (torch.float32, 1, 7)])
+def test_rmsnorm(gpu, dtype, rows, dim):
+    g = gen(1)
+    x = (torch.randn(rows, dim, generator=g) * 3).to(dtype)
+    r = torch.randn(rows, dim, generator=g).to(dtype)
+    w = (torch.rand(dim, generator=g) + 0.5).to(dtype)
+    tol = TOL_F32 if dtype == torch.float32 else TOL_BF16
+    y = ops.rmsnorm(x.to(gpu), w.to(gpu), 1e-5)
+    assert y.dtype == dtype and rel(y, R.rms_norm(x.float(), w.float(), 1e-5)[0]) < tol
+    y, h = ops.rmsnorm(x.to(gpu), w.to(gpu), 1e-5, r.to(gpu), want_residual=True)
+    ref_y, ref_h = R.rms_norm(x.float(), w.float(), 1e-5, r.float())
+    assert torch.equal(h.cpu(), (r + x))            # the sum is rounded as the tensor expression rounds it
+    assert rel(y, ref_y) < tol
+    with pytest.raises(ValueError):
+        ops.rmsnorm(x.to(gpu), w[:-1].to(gpu), 1e-5)
+
+
+@pytest.mark.parametrize("B,n_q,n_kv", [(1, 32, 8), (5, 8, 1), (32, 4, 4)])
+def test_rope_kv_append(gpu, B, n_q, n_kv):
+    g = gen(2)
+    d, L = 128, 64
+    qkv = torch.randn(B, (n_q + 2 * n_kv) * d, generator=g).bfloat16()
+    cos, sin = rope_tables(d, L, 500000.0, dtype=torch.bfloat16)
+    pos = torch.randint(0, L, (B,), generator=g)
+    kc0 = torch.randn(B, n_kv, L, d, generator=g).bfloat16()
+    vc0 = torch.randn(B, n_kv, L, d, generator=g).bfloat16()
+    kc, vc = kc0.to(gpu), vc0.to(gpu)
+    q = ops.rope_kv_append(qkv.to(gpu), cos.to(gpu), sin.to(gpu), pos.to(gpu), kc, vc, n_q)
+    heads = qkv.float().view(B, n_q + 2 * n_kv, d)
+    cf, sf = cos.float()[pos], sin.float()[pos]
+    assert rel(q, R.apply_rope(heads[:, :n_q], cf, sf)) < TOL_BF16
+    ref_k = R.apply_rope(heads[:, n_q:n_q + n_kv], cf, sf)
+    kc, vc = kc.cpu(), vc.cpu()
+    for b in range(B):
+        p = int(pos[b])
+        assert rel(kc[b, :, p], ref_k[b]) < TOL_BF16
+        assert torch.equal(vc[b, :, p], qkv.view(B, -1, d)[b, n_q + n_kv:])        # values are copied
+        keep = torch.ones(L, dtype=torch.bool)
+        keep[p] = False
+        assert torch.equal(kc[b][:, keep], kc0[b][:, keep]) and torch.equal(vc[b][:, keep], vc0[b][:, keep])
+    # a position outside the cache leaves everything as it was
+    kc, vc = kc0.to(gpu), vc0.to(gpu)
+    ops.rope_kv_append(qkv.to(gpu), cos.to(gpu), sin.to(gpu), torch.full((B,), L, dtype=torch.int64, device=gpu), kc, vc,
+                       n_q)
+    assert torch.equal(kc.cpu(), kc0) and torch.equal(vc.cpu(), vc0)
+
+
+def _attn_case(gpu, B, n_q, n_kv, max_len, lens, seed, scale_v=1.0):
+    g = gen(seed)
+    d = 128
+    q = torch.randn(B, n_q, d, generator=g).bfloat16()
+    kc = torch.randn(B, n_kv, max_len, d, generator=g).bfloat16()
+    vc = (torch.randn(B, n_kv, max_len, d, generator=g) * scale_v).bfloat16()
+    lens = torch.tensor(lens, dtype=torch.int64)
+    ref = R.attn_decode(q.float(), kc.float(), vc.float(), lens)
+    # whatever lies behind the valid prefix must not be read into the result
+    for b in range(B):
+        kc[b, :, int(lens[b]):] = float("nan")
+        vc[b, :, int(lens[b]):] = float("nan")
+    return q.to(gpu), kc.to(gpu), vc.to(gpu), lens.to(gpu), ref
+
+
+@pytest.mark.parametrize("n_q,n_kv", [(32, 8), (8, 1), (16, 16), (16, 1)])
+@pytest.mark.parametrize("lens", [[1], [31], [32], [33], [128], [777], [2048]])
+def test_attn_decode_lengths_and_groups(gpu, n_q, n_kv, lens):
+    q, kc, vc, dl, ref = _attn_case(gpu, 1, n_q, n_kv, 2048, lens, seed=3)
+    out = ops.attn_decode(q, kc, vc, dl, len_bound=max(lens))
+    assert out.shape == q.shape and out.dtype == torch.bfloat16
+    assert rel(out, ref) < TOL_BF16
+
+
+@pytest.mark.parametrize("splits", ["1", "3", "16", "64"])
+def test_attn_decode_ragged_batch_any_split_count(gpu, splits, monkeypatch):
+    lens = [1000, 1, 0, 64, 513, 37]
+    q, kc, vc, dl, ref = _attn_case(gpu, 6, 32, 8, 1024, lens, seed=4)
+    monkeypatch.setenv("MTP_ATTN_SPLITS", splits)
+    out = ops.attn_decode(q, kc, vc, dl)
+    assert torch.count_nonzero(out[2]) == 0                      # no tokens: zeros
+    for b in range(6):
+        if lens[b]:
+            assert rel(out[b], ref[b]) < TOL_BF16, (b, lens[b])
+    # one token: exactly its value row
+    assert torch.equal(out[1].cpu().view(8, 4, 128), vc[1, :, 0].cpu()[:, None, :].expand(8, 4, 128))
+
+
+def test_attn_decode_sharp_and_flat_softmax(gpu):
+    """A query that matches one key far better than the rest returns that key's value; zero queries average."""
+    g = gen(5)
+    B, n_q, n_kv, L, d = 2, 8, 2, 500, 128
+    kc = torch.randn(B, n_kv, L, d, generator=g).bfloat16()
+    vc = torch.randn(B, n_kv, L, d, generator=g).bfloat16()
+    q = torch.zeros(B, n_q, d).bfloat16()
+    q[0] = (kc[0, :, 321].float() * 8).bfloat16().repeat_interleave(4, 0)      # scores ~ 8 |k|^2 / sqrt(d) ~ 90
+    lens = torch.tensor([L, L])
+    out = ops.attn_decode(q.to(gpu), kc.to(gpu), vc.to(gpu), lens.to(gpu)).cpu()
+    assert rel(out[0], vc[0, :, 321].repeat_interleave(4, 0)) < TOL_BF16
+    assert rel(out[1], vc[1].float().mean(1).repeat_interleave(4, 0)) < TOL_BF16
+    ref = R.attn_decode(q.float(), kc.float(), vc.float(), lens)
+    assert rel(out, ref) < TOL_BF16
+
+
+def test_attn_decode_llama8b_shape_long_context(gpu):
+    """32 sequences of up to 8192 tokens, 32 q / 8 kv heads: checked on a sample of (sequence, head) pairs
+    against the oracle, and through invariance: permuting the cached tokens of a sequence (keys and values
+    together) must not change its output beyond rounding."""
+    g = gen(6)
+    B, n_q, n_kv, L, d = 32, 32, 8, 8192, 128
+    kc = torch.randn(B, n_kv, L, d, generator=g, dtype=torch.bfloat16).to(gpu)
+    vc = torch.randn(B, n_kv, L, d, generator=g, dtype=torch.bfloat16).to(gpu)
+    q = torch.randn(B, n_q, d, generator=g).bfloat16().to(gpu)
+    lens = torch.randint(4000, L + 1, (B,), generator=g)
+    lens[0], lens[1] = L, 4097
+    out = ops.attn_decode(q, kc, vc, lens.to(gpu))
+    for b in (0, 1, 17, 31):
+        ref = R.attn_decode(q[b:b + 1].float().cpu(), kc[b:b + 1].float().cpu(), vc[b:b + 1].float().cpu(), lens[b:b + 1])
+        assert rel(out[b], ref[0]) < TOL_BF16, b
+    n = int(lens[5])
+    perm = torch.randperm(n, generator=g).to(gpu)
+    kc[5, :, :n] = kc[5][:, perm]
+    vc[5, :, :n] = vc[5][:, perm]
+    again = ops.attn_decode(q, kc, vc, lens.to(gpu))
+    assert rel(again[5], out[5]) < TOL_BF16
+    assert torch.equal(again[6], out[6])                     # untouched sequences: bit for bit the same
+
+
+def test_attn_decode_rejects_bad_arguments(gpu):
+    q = torch.zeros(2, 8, 128, dtype=torch.bfloat16, device=gpu)
+    kc = torch.zeros(2, 2, 64, 128, dtype=torch.bfloat16, device=gpu)
+    lens = torch.ones(2, dtype=torch.int64, device=gpu)
+    ops.attn_decode(q, kc, kc.clone(), lens)
+    with pytest.raises(ValueError):
+        ops.attn_decode(q, kc, kc.clone()[:, :, :32], lens)                      # cache shapes differ
+    with pytest.raises(ValueError):
+        ops.attn_decode(q, kc, kc.clone(), lens.int())                            # lens must be int64
+    with pytest.raises(RuntimeError, match="head_dim"):
+        ops.attn_decode(q[:, :, :64].contiguous(), kc[..., :64].contiguous(), kc[..., :64].contiguous(), lens)
+    with pytest.raises(RuntimeError, match="q heads per kv head"):
+        ops.attn_decode(torch.zeros(2, 34, 128, dtype=torch.bfloat16, device=gpu), kc, kc.clone(), lens)
+    with pytest.raises(RuntimeError, match="len_bound"):
+        ops.attn_decode(q, kc, kc.clone(), lens, len_bound=65)
+
+
+def _tiny_model(seed):
+    from transformers import LlamaConfig, LlamaForCausalLM
+    torch.manual_seed(seed)
+    cfg = LlamaConfig(hidden_size=512, intermediate_size=1024, num_attention_heads=4, num_key_value_heads=2,
+                      head_dim=128, num_hidden_layers=2, vocab_size=1000, max_position_embeddings=128,
+                      rope_theta=10000.0, rms_norm_eps=1e-5, attn_implementation="eager", tie_word_embeddings=False)
+    model = LlamaForCausalLM(cfg).eval()
+    for p_ in model.parameters():
+        if p_.dim() == 1:
+            p_.data.uniform_(0.5, 1.5)
+        p_.data = p_.data.bfloat16().float()          # values a bf16 copy holds exactly
+    return cfg, model
+
+
+def test_llama_decoder_matches_full_sequence_forward(gpu):
+    """Token by token with the cache on the GPU == what the generation loop computes: the full-sequence forward
+    of the library model (fp32, CPU, same bf16-representable weights), row context_length-1 (:223)."""
+    cfg, model = _tiny_model(7)
+    B, T = 3, 40
+    ids = torch.randint(0, cfg.vocab_size, (B, T), generator=gen(7))
+    with torch.no_grad():
+        full = model(input_ids=ids).logits                              # [B, T, V] fp32
+    dec = LlamaDecoder.from_hf(model.bfloat16().to(gpu), max_len=64, batch=B)
+    worst = 0.0
+    for t in range(T):
+        logits = dec.logits(ids[:, t].to(gpu))
+        worst = max(worst, rel(logits, full[:, t]))
+    assert worst < 2 * TOL_BF16, worst            # two blocks of bf16 rounding on top of each other
+    assert dec.lens.tolist() == [T] * B
+    # greedy pick of the fused LM head == argmax of the materialised logits of the same step
+    dec.reset()
+    for t in range(5):
+        tok = dec.step(ids[:, t].to(gpu))
+        dec.lens -= 1                                 # run the same position again, now with logits written
+        dec.host_len_bound -= 1
+        lg = dec.logits(ids[:, t].to(gpu))
+        top2 = lg.float().topk(2, dim=-1).values
+        clear = (top2[:, 0] - top2[:, 1]) > 1e-2 * top2[:, 0].abs()
+        assert torch.equal(tok[clear].cpu(), lg.argmax(-1)[clear].cpu())
+
+
+def test_block_step_vs_oracle_llama8b_shape(gpu):
+    """One Llama-3-8B block (H 4096, 32/8 heads, I 14336), 8 sequences with 1000-3000 cached tokens."""
+    g = gen(8)
+    B, H, n_q, n_kv, d, I, L = 8, 4096, 32, 8, 128, 14336, 3072
+    def w(*shape, std=0.02):
+        return (torch.randn(*shape, generator=g) * std).bfloat16()
+    wt = {"input_norm": (torch.rand(H, generator=g) + 0.5).bfloat16(), "qkv": w((n_q + 2 * n_kv) * d, H),
+          "o": w(H, n_q * d), "post_norm": (torch.rand(H, generator=g) + 0.5).bfloat16(), "gate_up": w(2 * I, H),
+          "down": w(H, I)}
+    x, res = torch.randn(B, H, generator=g).bfloat16(), torch.randn(B, H, generator=g).bfloat16()
+    kc, vc = torch.randn(B, n_kv, L, d, generator=g).bfloat16(), torch.randn(B, n_kv, L, d, generator=g).bfloat16()
+    pos = torch.randint(1000, 3000, (B,), generator=g)
+    cos, sin = rope_tables(d, L, 500000.0, dtype=torch.bfloat16)
+    kf, vf = kc.float(), vc.float()
+    ref_x, ref_res = R.llama_block_step(x.float(), res.float(), pos, pos + 1, {k: v.float() for k, v in wt.items()}, kf,
+                                        vf, cos.float(), sin.float(), n_q, 1e-5)
+    G = {k: v.to(gpu) for k, v in wt.items()}
+    kc, vc = kc.to(gpu), vc.to(gpu)
+    h, r1 = ops.rmsnorm(x.to(gpu), G["input_norm"], 1e-5, res.to(gpu), want_residual=True)
+    q = ops.rope_kv_append(ops.gemv(h, G["qkv"]), cos.to(gpu), sin.to(gpu), pos.to(gpu), kc, vc, n_q)
+    a = ops.attn_decode(q, kc, vc, (pos + 1).to(gpu), len_bound=3000)
+    o = ops.gemv(a.view(B, -1), G["o"])
+    h2, r2 = ops.rmsnorm(o, G["post_norm"], 1e-5, r1, want_residual=True)
+    out = ops.gemv(ops.gemv(h2, G["gate_up"], None, ops.EPI_SWIGLU), G["down"])
+    assert rel(r2, ref_res) < TOL_BF16
+    assert rel(out, ref_x) < 2 * TOL_BF16
+    for b in range(B):
+        assert rel(kc[b, :, int(pos[b])], kf[b, :, int(pos[b])]) < TOL_BF16

@@ -275,3 +275,98 @@ def test_sample_tail_is_inverse_cdf_and_follows_the_distribution():
     toks, pr = R.sample_tail(one.expand(40000, 30).clone(), 1.0, 8, 0.0, us)
     freq = torch.bincount(toks, minlength=30).double() / 40000
     assert (freq - pr[0]).abs().max() < 0.01 and int((pr[0] > 0).sum()) == 8
+
+
+# ---- one position against a key/value cache: pinned on transformers' own Llama block over the full sequence ----
+ROPE_THETA = 10000.0
+
+
+def _tiny_llama(seed=11, layers=2):
+    from transformers import LlamaConfig
+    from transformers.models.llama import modeling_llama as ML
+    torch.manual_seed(seed)
+    cfg = LlamaConfig(hidden_size=256, intermediate_size=384, num_attention_heads=4, num_key_value_heads=2,
+                      head_dim=64, num_hidden_layers=layers, vocab_size=211, max_position_embeddings=64,
+                      rope_theta=ROPE_THETA, rms_norm_eps=1e-5, attn_implementation="eager", attention_bias=False,
+                      mlp_bias=False)
+    model = ML.LlamaModel(cfg).eval()
+    for p_ in model.parameters():      # norm weights away from 1 so that a dropped weight would show
+        if p_.dim() == 1:
+            p_.data.uniform_(0.5, 1.5)
+    return cfg, model
+
+
+def _block_weights(layer):
+    a, m = layer.self_attn, layer.mlp
+    return {"input_norm": layer.input_layernorm.weight.data,
+            "qkv": torch.cat([a.q_proj.weight, a.k_proj.weight, a.v_proj.weight]).data,
+            "o": a.o_proj.weight.data, "post_norm": layer.post_attention_layernorm.weight.data,
+            "gate_up": torch.cat([m.gate_proj.weight, m.up_proj.weight]).data, "down": m.down_proj.weight.data}
+
+
+def test_cached_step_equals_full_sequence_forward_of_the_library_model():
+    """Stepping position by position with a cache gives, at every position, the row the full-sequence forward
+    of transformers' LlamaModel gives there (rows of two different lengths in one batch)."""
+    cfg, model = _tiny_llama()
+    B, T = 2, 9
+    ids = torch.randint(0, cfg.vocab_size, (B, T), generator=torch.Generator().manual_seed(3))
+    with torch.no_grad():
+        full = model(input_ids=ids).last_hidden_state                        # [B, T, H]
+    d, n_q, n_kv = cfg.head_dim, cfg.num_attention_heads, cfg.num_key_value_heads
+    cos_t, sin_t = R.rope_tables(d, 64, ROPE_THETA)
+    kc = [torch.zeros(B, n_kv, 16, d) for _ in model.layers]
+    vc = [torch.zeros(B, n_kv, 16, d) for _ in model.layers]
+    with torch.no_grad():
+        for t in range(T):
+            pos = torch.full((B,), t, dtype=torch.int64)
+            x, res = model.embed_tokens(ids[:, t]), None
+            for li, layer in enumerate(model.layers):
+                x, res = R.llama_block_step(x, res, pos, pos + 1, _block_weights(layer), kc[li], vc[li], cos_t,
+                                            sin_t, n_q, cfg.rms_norm_eps)
+            y, _ = R.rms_norm(x, model.norm.weight.data, cfg.rms_norm_eps, res)
+            assert torch.allclose(y, full[:, t], atol=2e-5, rtol=1e-4), t
+
+
+def test_cached_step_pieces_against_library_routines():
+    from transformers.models.llama import modeling_llama as ML
+    cfg, model = _tiny_llama(layers=1)
+    g = torch.Generator().manual_seed(4)
+    # RMSNorm: the library module; the residual is added first
+    x, r = torch.randn(3, 256, generator=g), torch.randn(3, 256, generator=g)
+    norm = model.layers[0].input_layernorm
+    y, h = R.rms_norm(x, norm.weight.data, cfg.rms_norm_eps, r)
+    assert torch.equal(h, r + x) and torch.allclose(y, norm(r + x))
+    # closed form on a constant row: every element c -> weight * c / sqrt(c^2 + eps)
+    c = torch.full((1, 256), 3.0)
+    assert torch.allclose(R.rms_norm(c, norm.weight.data, 1e-5)[0], norm.weight.data * 3.0 / math.sqrt(9.0 + 1e-5))
+    # rotary tables and rotation: the library's rotary module and apply_rotary_pos_emb
+    rot = ML.LlamaRotaryEmbedding(cfg)
+    pos = torch.tensor([[0, 5, 17]])
+    cos, sin = rot(torch.zeros(1, 3, 256), pos)
+    cos_t, sin_t = R.rope_tables(cfg.head_dim, 64, ROPE_THETA)
+    assert torch.allclose(cos[0], cos_t[pos[0]]) and torch.allclose(sin[0], sin_t[pos[0]])
+    q = torch.randn(1, 4, 3, 64, generator=g)                             # [batch, heads, positions, d]
+    k = torch.randn(1, 2, 3, 64, generator=g)
+    qe, ke = ML.apply_rotary_pos_emb(q, k, cos, sin)
+    mine = R.apply_rope(q[0].transpose(0, 1), cos_t[pos[0]], sin_t[pos[0]])   # rows = positions
+    assert torch.allclose(mine, qe[0].transpose(0, 1), atol=1e-6)
+    # a rotation keeps the norm of every (i, i + d/2) pair; position 0 is the identity
+    assert torch.allclose(mine.norm(dim=-1), q[0].transpose(0, 1).norm(dim=-1), rtol=1e-5)
+    assert torch.equal(R.apply_rope(q[0, :, :1].transpose(0, 1), cos_t[:1], sin_t[:1]), q[0, :, :1].transpose(0, 1))
+    # attention: torch's scaled_dot_product_attention over the valid prefix, kv heads repeated per group
+    B, n_q, n_kv, d, L = 3, 8, 2, 32, 20
+    qq = torch.randn(B, n_q, d, generator=g)
+    kc, vc = torch.randn(B, n_kv, L, d, generator=g), torch.randn(B, n_kv, L, d, generator=g)
+    lens = torch.tensor([20, 1, 7])
+    got = R.attn_decode(qq, kc, vc, lens)
+    for b in range(B):
+        n = int(lens[b])
+        kk = kc[b, :, :n].repeat_interleave(n_q // n_kv, 0)
+        vv = vc[b, :, :n].repeat_interleave(n_q // n_kv, 0)
+        ref = F.scaled_dot_product_attention(qq[b][:, None], kk, vv)[:, 0]
+        assert torch.allclose(got[b], ref, atol=1e-5)
+    assert torch.allclose(got[1], vc[1, :, 0].repeat_interleave(4, 0))     # one token: its value comes back
+    # junk beyond lens must not matter
+    kc2, vc2 = kc.clone(), vc.clone()
+    kc2[2, :, 7:], vc2[2, :, 7:] = 1e4, float("nan")
+    assert torch.equal(R.attn_decode(qq, kc2, vc2, lens)[2], got[2])

@@ -280,13 +280,31 @@ int mtp_rope_kv_append(const void* qkv, const void* cos_table, const void* sin_t
  * upper bound of lens known on the host (<= max_len); it only decides over
  * how many workgroups a sequence is split.  workspace: device scratch of
  * mtp_attn_decode_workspace_bytes(B, n_q_heads, n_kv_heads, len_bound)
- * bytes (may be NULL when that is 0). */
+ * bytes, 16-byte aligned (may be NULL when that is 0).  ITS FIRST
+ * 4 * B * n_kv_heads BYTES MUST BE ZERO before the first launch that uses
+ * it; every launch leaves them zero again (they count the splits of a
+ * sequence that have delivered, the last one merges).  Launches that share a
+ * workspace must not overlap. */
 int64_t mtp_attn_decode_workspace_bytes(int64_t B, int n_q_heads, int n_kv_heads, int64_t len_bound);
 int mtp_attn_decode(const void* q, const void* k_cache, const void* v_cache,
                     const int64_t* lens, void* out,
                     void* workspace, int64_t workspace_bytes,
                     int64_t B, int n_q_heads, int n_kv_heads, int head_dim,
                     int64_t max_len, int64_t len_bound, float scale, int dtype, void* stream);
+
+/* mtp_rope_kv_append followed by mtp_attn_decode with lens = positions + 1,
+ * as one launch: the new query and key are rotated in registers, the new
+ * key and value are appended to the caches and enter the softmax straight
+ * from the QKV projection's output; the cached rows below positions[b] are
+ * read as in mtp_attn_decode.  A row whose position lies outside the cache
+ * or the tables appends nothing and gives zeros.  len_bound bounds
+ * positions + 1.  Same workspace rules. */
+int mtp_attn_decode_append(const void* qkv, const void* cos_table, const void* sin_table,
+                           const int64_t* positions, void* k_cache, void* v_cache, void* out,
+                           void* workspace, int64_t workspace_bytes,
+                           int64_t B, int n_q_heads, int n_kv_heads, int head_dim,
+                           int64_t max_len, int64_t max_positions, int64_t len_bound,
+                           float scale, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------
  * Measurement helpers (used by bench.py to state what this GPU can do).

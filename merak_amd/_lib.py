@@ -50,6 +50,8 @@ SIGNATURES = {
     "mtp_rope_kv_append": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _int, _vp]),
     "mtp_attn_decode_workspace_bytes": (_i64, [_i64, _int, _int, _i64]),
     "mtp_attn_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _int, _i64, _i64, C.c_float, _int, _vp]),
+    "mtp_attn_decode_append": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _int, _i64, _i64, _i64,
+                                      C.c_float, _int, _vp]),
     "mtp_stream_copy": (_int, [_vp, _vp, _i64, _vp]),
     "mtp_mfma_peak": (_int, [_vp, _i64, _i64, _int, _vp]),
 }

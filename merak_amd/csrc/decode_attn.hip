@@ -34,27 +34,66 @@ namespace {
 constexpr int AD_D = 128;                      // head dimension
 constexpr int AD_TILE = 32;                    // tokens per tile
 constexpr int AD_ITEM = AD_TILE * AD_D * 2;    // bytes of the K (or V) rows of one tile
-constexpr int AD_RING = 4;                     // ring slots per wave
-constexpr int AD_WAVES = 4;
+constexpr int AD_MAX_WAVES = 8;
 constexpr int AD_PART = AD_D + 2;              // floats per partial result: O[128], max, sum
 constexpr int AD_MAX_GROUP = 16;
 
 struct AttnArgs {
-  const uint16_t* q;      // [B, n_q_heads, 128]
-  const uint16_t* k;      // [B, n_kv_heads, max_len, 128]
-  const uint16_t* v;
-  const int64_t* lens;    // [B] tokens to attend to (the new one included)
+  const uint16_t* q;      // [B, n_q_heads, 128]                       (plain form)
+  uint16_t* k;            // [B, n_kv_heads, max_len, 128]
+  uint16_t* v;
+  const int64_t* lens;    // [B] tokens to attend to                   (plain form)
   uint16_t* out;          // [B, n_q_heads, 128]
   float* part;            // [B, n_q_heads, splits, AD_PART] when splits > 1
+  int32_t* arrived;       // [B, n_kv_heads] zero between launches: splits that have delivered their partial
   int n_q_heads, n_kv_heads, group;
   int64_t max_len;
   int splits;
+  int rot_mul;            // tile rotation per workgroup index
   float scale_log2e;      // softmax scale * log2(e)
+  // appending form: the new position comes straight from the QKV projection
+  const uint16_t* qkv;        // [B, (n_q_heads + 2 n_kv_heads) * 128]
+  const uint16_t* cos_t;      // [max_positions, 128]
+  const uint16_t* sin_t;
+  const int64_t* positions;   // [B] position of the new token = number of tokens already cached
+  int64_t max_positions;
 };
+
+// x * cos + rotate_half(x) * sin for 8 elements of one head: `own` holds dims d .. d+7, `other` the dims
+// 64 away, sign = -1 for d < 64 (rotate_half = cat(-x[64:], x[:64])).  Every product is rounded to bf16
+// before the sum, and the sum again, as the bf16 tensor expression rounds.
+__device__ __forceinline__ u32x4_t rope8(u32x4_t own, u32x4_t other, u32x4_t c, u32x4_t s, float sign) {
+  u32x4_t r;
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    const float a0 = bf16_lo(own[e]) * bf16_lo(c[e]), a1 = bf16_hi(own[e]) * bf16_hi(c[e]);
+    const float b0 = sign * bf16_lo(other[e]) * bf16_lo(s[e]), b1 = sign * bf16_hi(other[e]) * bf16_hi(s[e]);
+    const uint32_t pa = pack_bf16x2(a0, a1), pb = pack_bf16x2(b0, b1);
+    r[e] = pack_bf16x2(bf16_lo(pa) + bf16_lo(pb), bf16_hi(pa) + bf16_hi(pb));
+  }
+  return r;
+}
+
+// dma16 with the streaming (non-temporal) hint: the cache rows are read once per launch
+__device__ __forceinline__ void dma16_nt(rsrc_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff));
+}
+
+// device-scope accesses: served at the level all XCDs share
+__device__ __forceinline__ void coherent_store(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float coherent_load(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 __device__ __forceinline__ void wait_vm(int items_after) {
   // every item is 8 DMA instructions; "memory": LDS reads below must not move above the wait
   switch (items_after) {
+    case 5: asm volatile("s_waitcnt vmcnt(40)" ::: "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(32)" ::: "memory"); break;
     case 3: asm volatile("s_waitcnt vmcnt(24)" ::: "memory"); break;
     case 2: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
     case 1: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
@@ -62,6 +101,8 @@ __device__ __forceinline__ void wait_vm(int items_after) {
   }
 }
 
+// AD_WAVES waves with AD_RING ring slots each: 32 KiB of LDS per wave with 4 slots, 48 KiB with 6
+template <bool APPEND, int AD_WAVES, int AD_RING, bool NT>
 __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
   __shared__ __attribute__((aligned(1024))) char lds[AD_WAVES * AD_RING * AD_ITEM];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -70,25 +111,62 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
   const int G = p.group;
   const int h = lane & 15, q = lane >> 4;
 
-  int64_t len = p.lens[b];
-  len = len < 0 ? 0 : (len > p.max_len ? p.max_len : len);
+  // tokens to read from the cache; the appending form adds the new one from registers
+  int64_t len;
+  bool fresh = false;     // this row has a new token to rotate, append and attend to
+  int64_t pos = 0;
+  if (APPEND) {
+    pos = p.positions[b];
+    fresh = pos >= 0 && pos < p.max_len && pos < p.max_positions;
+    len = fresh ? pos : 0;
+  } else {
+    len = p.lens[b];
+    len = len < 0 ? 0 : (len > p.max_len ? p.max_len : len);
+  }
   const int tiles = (int)((len + AD_TILE - 1) / AD_TILE);
   const int tps = (tiles + p.splits - 1) / p.splits;
   const int tile_lo = split * tps;
   const int tile_hi = tile_lo + tps < tiles ? tile_lo + tps : tiles;
-  const int first = tile_lo + wave;
-  const int n_my = tile_hi > first ? (tile_hi - first + AD_WAVES - 1) / AD_WAVES : 0;
+  // The workgroup's tiles are taken in rotated order, by an amount that differs between workgroups: the
+  // sequences start a multiple of the cache's row stride apart, and workgroups walking them in step would
+  // all be on the same memory channels at the same time.  (The recurrence does not care about the order.)
+  const int n_wg = tile_hi > tile_lo ? tile_hi - tile_lo : 0;
+  const int wg_lin = ((int)b * p.n_kv_heads + kvh) * p.splits + split;
+  const int rot = n_wg > 0 ? (int)(((int64_t)wg_lin * p.rot_mul) % n_wg) : 0;
+  const int n_my = n_wg > wave ? (n_wg - wave + AD_WAVES - 1) / AD_WAVES : 0;
+  auto tile_of = [&](int i) {      // i-th tile of this wave
+    int j = wave + AD_WAVES * i + rot;
+    if (j >= n_wg) j -= n_wg;
+    return tile_lo + j;
+  };
   const int n_items = 2 * n_my;
 
   // this lane's share of Q^T as MFMA B operand: head h, dims 32c + 8q .. +7
   bf16x8_t qf[4];
+  u32x4_t cs[4], sn[4];   // appending form: cos / sin of this lane's dims at the new position
   {
-    const uint16_t* qrow = p.q + ((int64_t)b * p.n_q_heads + (int64_t)kvh * G + (h < G ? h : 0)) * AD_D;
+    const int64_t heads_row = APPEND ? (int64_t)b * (p.n_q_heads + 2 * p.n_kv_heads) : (int64_t)b * p.n_q_heads;
+    const uint16_t* qrow = (APPEND ? p.qkv : p.q) + (heads_row + (int64_t)kvh * G + (h < G ? h : 0)) * AD_D;
+    u32x4_t raw[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) raw[c] = *reinterpret_cast<const u32x4_t*>(qrow + 32 * c + 8 * q);
+    if (APPEND) {
+      const int64_t trow = (fresh ? pos : 0) * AD_D;
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        cs[c] = *reinterpret_cast<const u32x4_t*>(p.cos_t + trow + 32 * c + 8 * q);
+        sn[c] = *reinterpret_cast<const u32x4_t*>(p.sin_t + trow + 32 * c + 8 * q);
+      }
+      u32x4_t rot[4];
+#pragma unroll
+      for (int c = 0; c < 4; c++) rot[c] = rope8(raw[c], raw[c ^ 2], cs[c], sn[c], c < 2 ? -1.0f : 1.0f);
+#pragma unroll
+      for (int c = 0; c < 4; c++) raw[c] = rot[c];
+    }
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-      u32x4_t raw = *reinterpret_cast<const u32x4_t*>(qrow + 32 * c + 8 * q);
-      if (h >= G) raw = u32x4_t{0, 0, 0, 0};
-      qf[c] = __builtin_bit_cast(bf16x8_t, raw);
+      if (h >= G) raw[c] = u32x4_t{0, 0, 0, 0};
+      qf[c] = __builtin_bit_cast(bf16x8_t, raw[c]);
     }
   }
 
@@ -107,12 +185,17 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
   auto issue = [&](int it) {
     // the slot's earlier contents have been read: keep those reads in front of the DMA, and wait for them
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    const int64_t tok0 = (int64_t)(first + AD_WAVES * (it >> 1)) * AD_TILE;
+    const int64_t tok0 = (int64_t)tile_of(it >> 1) * AD_TILE;
     const char* base = reinterpret_cast<const char*>((it & 1) ? p.v : p.k) + (head_rows + tok0) * (AD_D * 2);
     const rsrc_t r = make_rsrc(base, (len - tok0) * (AD_D * 2));
-    const uint32_t slot = ring0 + (it & (AD_RING - 1)) * AD_ITEM;
+    const uint32_t slot = ring0 + (it % AD_RING) * AD_ITEM;
 #pragma unroll
-    for (int j = 0; j < 8; j++) dma16(r, slot + j * 1024, voff[j & 3] + (j >> 2) * 4096, 0);
+    for (int j = 0; j < 8; j++) {
+      if (NT)
+        dma16_nt(r, slot + j * 1024, voff[j & 3] + (j >> 2) * 4096, 0);
+      else
+        dma16(r, slot + j * 1024, voff[j & 3] + (j >> 2) * 4096, 0);
+    }
   };
 
   // fragment addresses inside a slot
@@ -129,19 +212,58 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
 #pragma unroll
   for (int dt = 0; dt < 8; dt++) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  if (n_items > 0) issue(0);
-  if (n_items > 1) issue(1);
-  if (n_items > 2) issue(2);
+  constexpr int AHEAD = AD_RING - 1;     // items in flight while one is used
+#pragma unroll
+  for (int it = 0; it < AHEAD; it++)
+    if (it < n_items) issue(it);
+
+  if (APPEND && fresh && split == 0 && wave == 0) {
+    // The new token: rotate its key, append key and value to the cache, and start the recurrence from it
+    // (score s, probability 1, O = v).  No workgroup reads row `pos` of the cache in this launch.
+    const uint16_t* krow = p.qkv + ((int64_t)b * (p.n_q_heads + 2 * p.n_kv_heads) + p.n_q_heads + kvh) * AD_D;
+    const uint16_t* vrow_new = krow + (int64_t)p.n_kv_heads * AD_D;
+    u32x4_t kraw[4], krot[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) kraw[c] = *reinterpret_cast<const u32x4_t*>(krow + 32 * c + 8 * q);
+#pragma unroll
+    for (int c = 0; c < 4; c++) krot[c] = rope8(kraw[c], kraw[c ^ 2], cs[c], sn[c], c < 2 ? -1.0f : 1.0f);
+    float dot = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      const u32x4_t qq = __builtin_bit_cast(u32x4_t, qf[c]);
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        dot += bf16_lo(qq[e]) * bf16_lo(krot[c][e]) + bf16_hi(qq[e]) * bf16_hi(krot[c][e]);
+    }
+    dot += __shfl_xor(dot, 16, 64);
+    dot += __shfl_xor(dot, 32, 64);
+    m_run = dot * p.scale_log2e;
+    l_run = q == 0 ? 1.0f : 0.0f;          // summed over the four lanes of a head at the end
+    uint16_t* kdst = p.k + (head_rows + pos) * AD_D;
+    uint16_t* vdst = p.v + (head_rows + pos) * AD_D;
+#pragma unroll
+    for (int dt = 0; dt < 8; dt++) {
+      const u32x2_t vv = *reinterpret_cast<const u32x2_t*>(vrow_new + 16 * dt + 4 * q);
+      o[dt] = f32x4_t{bf16_lo(vv[0]), bf16_hi(vv[0]), bf16_lo(vv[1]), bf16_hi(vv[1])};
+    }
+    if (h == 0) {
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        *reinterpret_cast<u32x4_t*>(kdst + 32 * c + 8 * q) = krot[c];
+        *reinterpret_cast<u32x4_t*>(vdst + 32 * c + 8 * q) = *reinterpret_cast<const u32x4_t*>(vrow_new + 32 * c + 8 * q);
+      }
+    }
+  }
 
   for (int i = 0; i < n_my; i++) {
     // ---- K: scores of 32 tokens for the heads of the group ----
     {
       const int it = 2 * i;
-      if (it + 3 < n_items) issue(it + 3);
+      if (it + AHEAD < n_items) issue(it + AHEAD);
       const int after = n_items - 1 - it;
-      wait_vm(after < 3 ? after : 3);
+      wait_vm(after < AHEAD ? after : AHEAD);
     }
-    const char* kslot = ring + ((2 * i) & (AD_RING - 1)) * AD_ITEM;
+    const char* kslot = ring + ((2 * i) % AD_RING) * AD_ITEM;
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int c = 0; c < 4; c++) {
@@ -152,7 +274,7 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
       s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qf[c], s1, 0, 0, 0);
     }
     // this lane: head h, tokens 4q + j (s0) and 16 + 4q + j (s1) of the tile
-    const int64_t valid = len - (int64_t)(first + AD_WAVES * i) * AD_TILE;
+    const int64_t valid = len - (int64_t)tile_of(i) * AD_TILE;
     float x0[4], x1[4];
     float mx = -INFINITY;
 #pragma unroll
@@ -183,11 +305,11 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
     // ---- V: O^T += V^T P^T ----
     {
       const int it = 2 * i + 1;
-      if (it + 3 < n_items) issue(it + 3);
+      if (it + AHEAD < n_items) issue(it + AHEAD);
       const int after = n_items - 1 - it;
-      wait_vm(after < 3 ? after : 3);
+      wait_vm(after < AHEAD ? after : AHEAD);
     }
-    const char* vslot = ring + ((2 * i + 1) & (AD_RING - 1)) * AD_ITEM;
+    const char* vslot = ring + ((2 * i + 1) % AD_RING) * AD_ITEM;
 #pragma unroll
     for (int dt = 0; dt < 8; dt++) {
       const char* a = vslot + vrow + (uint32_t)(((2 * dt + vc0) ^ (vt & 15)) << 4);
@@ -236,34 +358,68 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
       p.out[hq * AD_D + d] = f32_to_bf16_bits(l > 0.0f ? acc / l : 0.0f);
     } else {
       float* dst = p.part + (hq * p.splits + split) * AD_PART;
-      dst[d] = acc;
+      coherent_store(dst + d, acc);
       if (d == 0) {
-        dst[AD_D] = mstar;
-        dst[AD_D + 1] = l;
+        coherent_store(dst + AD_D, mstar);
+        coherent_store(dst + AD_D + 1, l);
       }
     }
   }
+  if (p.splits == 1) return;
+
+  // The split that delivers last merges all of them.  Partials travel through device-coherent stores and
+  // loads (they bypass the per-XCD L2), so no cache write-back or invalidate is needed: a workgroup waits for
+  // its stores to be acknowledged, then bumps the counter; whoever sees the counter full reads afterwards.
+  __shared__ int last_one;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (tid == 0) {
+    int32_t* cnt = p.arrived + (int64_t)b * p.n_kv_heads + kvh;
+    const int seen = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last_one = seen == p.splits - 1;
+    if (last_one) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+  }
+  __syncthreads();
+  if (!last_one) return;
+  for (int idx = tid; idx < G * AD_D; idx += AD_WAVES * 64) {
+    const int hh = idx >> 7, d = idx & (AD_D - 1);
+    const int64_t hq = (int64_t)b * p.n_q_heads + (int64_t)kvh * G + hh;
+    const float* src = p.part + hq * p.splits * AD_PART;
+    // 16 splits at a time, all their loads in flight together; running (max, sum, O) across the chunks
+    float mstar = -INFINITY, acc = 0.0f, l = 0.0f;
+    for (int s0 = 0; s0 < p.splits; s0 += 16) {
+      float ms[16], av[16], lv[16];
+#pragma unroll
+      for (int u = 0; u < 16; u++) {
+        const bool ok = s0 + u < p.splits;
+        const float* one = src + (ok ? s0 + u : s0) * AD_PART;
+        ms[u] = coherent_load(one + AD_D);
+        av[u] = coherent_load(one + d);
+        lv[u] = coherent_load(one + AD_D + 1);
+        if (!ok) ms[u] = -INFINITY;
+      }
+      float mnew = mstar;
+#pragma unroll
+      for (int u = 0; u < 16; u++) mnew = fmaxf(mnew, ms[u]);
+      if (mnew == -INFINITY) continue;
+      const float keep = __builtin_amdgcn_exp2f(mstar - mnew);
+      acc *= keep;
+      l *= keep;
+#pragma unroll
+      for (int u = 0; u < 16; u++) {
+        const float f = ms[u] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ms[u] - mnew);
+        acc += (ms[u] == -INFINITY ? 0.0f : av[u]) * f;
+        l += (ms[u] == -INFINITY ? 0.0f : lv[u]) * f;
+      }
+      mstar = mnew;
+    }
+    p.out[hq * AD_D + d] = f32_to_bf16_bits(l > 0.0f ? acc / l : 0.0f);
+  }
 }
 
-__global__ __launch_bounds__(AD_WAVES * 64) void attn_decode_kernel(const AttnArgs p) { attn_decode_body(p); }
-
-// out[b, hq, :] from the per-split partials
-__global__ __launch_bounds__(AD_D) void attn_merge_kernel(const float* __restrict__ part, uint16_t* __restrict__ out,
-                                                          int splits) {
-  const int64_t hq = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
-  const int d = threadIdx.x;
-  const float* src = part + hq * splits * AD_PART;
-  float mstar = -INFINITY;
-  for (int s = 0; s < splits; s++) mstar = fmaxf(mstar, src[s * AD_PART + AD_D]);
-  float acc = 0.0f, l = 0.0f;
-  for (int s = 0; s < splits; s++) {
-    const float ms = src[s * AD_PART + AD_D];
-    if (ms == -INFINITY) continue;
-    const float f = __builtin_amdgcn_exp2f(ms - mstar);
-    acc += src[s * AD_PART + d] * f;
-    l += src[s * AD_PART + AD_D + 1] * f;
-  }
-  out[hq * AD_D + d] = f32_to_bf16_bits(l > 0.0f ? acc / l : 0.0f);
+template <bool APPEND, int AD_WAVES, int AD_RING, bool NT>
+__global__ __launch_bounds__(AD_WAVES * 64) void attn_decode_kernel(const AttnArgs p) {
+  attn_decode_body<APPEND, AD_WAVES, AD_RING, NT>(p);
 }
 
 // ---- RMSNorm with the residual add in front of it ---------------------------------------------------
@@ -280,10 +436,10 @@ template <> struct Elem<float> {
   static __device__ __forceinline__ float store(float f) { return f; }
 };
 
+// General form: any dim, two passes over the row (the second re-reads it), element at a time.
 template <typename T>
-__global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ residual,
-                                                      const T* __restrict__ weight, T* __restrict__ y,
-                                                      T* __restrict__ residual_out, int64_t dim, float eps) {
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const T* x, const T* residual, const T* weight, T* y,
+                                                      T* residual_out, int64_t dim, float eps) {
   const int64_t row = blockIdx.x;
   const T* xr = x + row * dim;
   const T* rr = residual ? residual + row * dim : nullptr;
@@ -294,18 +450,102 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, c
   for (int64_t i = threadIdx.x; i < dim; i += 256) {
     float hval = Elem<T>::load(xr[i]);
     if (rr) hval = Elem<T>::load(Elem<T>::store(hval + Elem<T>::load(rr[i])));
-    if (hr) hr[i] = Elem<T>::store(hval);
     ss += hval * hval;
   }
   ss = wave_sum(ss);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
   __syncthreads();
   const float inv = rsqrtf((red[0] + red[1] + red[2] + red[3]) / (float)dim + eps);
+  // a thread reads and writes the same elements in both passes, so y may alias x and residual_out residual
   for (int64_t i = threadIdx.x; i < dim; i += 256) {
     float hval = Elem<T>::load(xr[i]);
     if (rr) hval = Elem<T>::load(Elem<T>::store(hval + Elem<T>::load(rr[i])));
     const float n = Elem<T>::load(Elem<T>::store(hval * inv));
+    if (hr) hr[i] = Elem<T>::store(hval);
     yr[i] = Elem<T>::store(Elem<T>::load(weight[i]) * n);
+  }
+}
+
+// Fast form: the row sits in registers between the two passes, 16 bytes per access, up to NV accesses per
+// thread (dim <= 256 * NV * elements per 16 bytes).  All loads of a thread come before its stores.
+template <typename T> struct Vec16;
+template <> struct Vec16<uint16_t> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void unpack(u32x4_t v, float* f) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      f[2 * e] = bf16_lo(v[e]);
+      f[2 * e + 1] = bf16_hi(v[e]);
+    }
+  }
+  static __device__ __forceinline__ u32x4_t pack(const float* f) {
+    return u32x4_t{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7])};
+  }
+  static __device__ __forceinline__ float round(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+};
+template <> struct Vec16<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void unpack(u32x4_t v, float* f) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) f[e] = __uint_as_float(v[e]);
+  }
+  static __device__ __forceinline__ u32x4_t pack(const float* f) {
+    return u32x4_t{__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
+  }
+  static __device__ __forceinline__ float round(float f) { return f; }
+};
+
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const T* x, const T* residual, const T* weight, T* y,
+                                                          T* residual_out, int64_t dim, float eps) {
+  using V = Vec16<T>;
+  constexpr int N = V::N;
+  const int64_t row = blockIdx.x;
+  const int nvec = (int)(dim / N);
+  const u32x4_t* xv = reinterpret_cast<const u32x4_t*>(x + row * dim);
+  const u32x4_t* rv = residual ? reinterpret_cast<const u32x4_t*>(residual + row * dim) : nullptr;
+  const u32x4_t* wv = reinterpret_cast<const u32x4_t*>(weight);
+  u32x4_t* hv = residual_out ? reinterpret_cast<u32x4_t*>(residual_out + row * dim) : nullptr;
+  u32x4_t* yv = reinterpret_cast<u32x4_t*>(y + row * dim);
+  __shared__ float red[4];
+  u32x4_t xin[NV], rin[NV], win[NV];
+#pragma unroll
+  for (int j = 0; j < NV; j++) {
+    const int i = threadIdx.x + 256 * j;
+    xin[j] = rin[j] = win[j] = u32x4_t{0u, 0u, 0u, 0u};
+    if (i < nvec) {
+      xin[j] = xv[i];
+      if (rv) rin[j] = rv[i];
+      win[j] = wv[i];
+    }
+  }
+  float hval[NV][N];
+  float ss = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NV; j++) {
+    float r[N];
+    V::unpack(xin[j], hval[j]);
+    V::unpack(rin[j], r);
+#pragma unroll
+    for (int e = 0; e < N; e++) {
+      if (rv) hval[j][e] = V::round(hval[j][e] + r[e]);
+      ss += hval[j][e] * hval[j][e];
+    }
+  }
+  ss = wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float inv = rsqrtf((red[0] + red[1] + red[2] + red[3]) / (float)dim + eps);
+#pragma unroll
+  for (int j = 0; j < NV; j++) {
+    const int i = threadIdx.x + 256 * j;
+    if (i >= nvec) continue;
+    float g[N], out[N];
+    V::unpack(win[j], g);
+#pragma unroll
+    for (int e = 0; e < N; e++) out[e] = g[e] * V::round(hval[j][e] * inv);
+    if (hv) hv[i] = V::pack(hval[j]);
+    yv[i] = V::pack(out);
   }
 }
 
@@ -356,8 +596,9 @@ int pick_splits(int64_t B, int n_kv, int64_t len_bound) {
     if (v >= 1) return v;
   }
   const int64_t tiles = (len_bound + AD_TILE - 1) / AD_TILE;
-  const int64_t by_len = (tiles + 2 * AD_WAVES - 1) / (2 * AD_WAVES);   // at least two tiles per wave
-  const int64_t by_grid = (1024 + B * n_kv - 1) / (B * n_kv);           // about four workgroups per CU slot
+  const int64_t by_len = (tiles + 2 * AD_MAX_WAVES - 1) / (2 * AD_MAX_WAVES);   // at least two tiles per wave
+  // about one workgroup per CU: a workgroup's start-up and its merge are paid once per split
+  const int64_t by_grid = (256 + B * n_kv / 2) / (B * n_kv);
   int64_t s = by_len < by_grid ? by_len : by_grid;
   if (s < 1) s = 1;
   if (s > 256) s = 256;
@@ -366,56 +607,109 @@ int pick_splits(int64_t B, int n_kv, int64_t len_bound) {
 
 }  // namespace
 
+namespace {
+int64_t counter_bytes(int64_t B, int n_kv) { return (B * n_kv * (int64_t)sizeof(int32_t) + 255) / 256 * 256; }
+
+int64_t workspace_need(int64_t B, int n_q, int n_kv, int splits) {
+  if (splits <= 1) return 0;
+  return counter_bytes(B, n_kv) + B * n_q * (int64_t)splits * AD_PART * (int64_t)sizeof(float);
+}
+
+// checks shared by the two forms; fills what they have in common and launches
+int launch_attn(bool append, AttnArgs a, const char* what, void* workspace, int64_t workspace_bytes, int64_t B,
+                int n_q_heads, int n_kv_heads, int head_dim, int64_t max_len, int64_t len_bound, float scale, int dtype,
+                void* stream) {
+  MTP_REQUIRE(dtype == MTP_BF16, MTP_EUNSUPPORTED, "%s: bf16 only", what);
+  MTP_REQUIRE(head_dim == AD_D, MTP_EUNSUPPORTED, "%s: head_dim %d (128 supported)", what, head_dim);
+  MTP_REQUIRE(B >= 0 && n_q_heads > 0 && n_kv_heads > 0 && n_q_heads % n_kv_heads == 0, MTP_EINVAL,
+              "%s: B=%lld heads %d/%d", what, (long long)B, n_q_heads, n_kv_heads);
+  const int group = n_q_heads / n_kv_heads;
+  MTP_REQUIRE(group <= AD_MAX_GROUP, MTP_EUNSUPPORTED, "%s: %d q heads per kv head (at most %d)", what, group,
+              AD_MAX_GROUP);
+  MTP_REQUIRE(max_len > 0 && len_bound > 0 && len_bound <= max_len, MTP_EINVAL, "%s: max_len=%lld len_bound=%lld", what,
+              (long long)max_len, (long long)len_bound);
+  MTP_REQUIRE(B <= 65535 && n_kv_heads <= 65535, MTP_EINVAL, "%s: grid too large", what);
+  if (B == 0) return MTP_OK;
+  MTP_REQUIRE(a.k && a.v && a.out, MTP_EINVAL, "%s: null pointer", what);
+  MTP_REQUIRE(((uintptr_t)a.k | (uintptr_t)a.v | (uintptr_t)a.q | (uintptr_t)a.qkv | (uintptr_t)a.cos_t |
+               (uintptr_t)a.sin_t) % 16 == 0,
+              MTP_EINVAL, "%s: tensors must be 16-byte aligned", what);
+  const int splits = pick_splits(B, n_kv_heads, len_bound);
+  const int64_t need = workspace_need(B, n_q_heads, n_kv_heads, splits);
+  MTP_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && (uintptr_t)workspace % 16 == 0), MTP_EINVAL,
+              "%s: workspace %lld bytes, need %lld (16-byte aligned)", what, (long long)workspace_bytes,
+              (long long)need);
+  a.arrived = static_cast<int32_t*>(workspace);
+  a.part = need ? reinterpret_cast<float*>(static_cast<char*>(workspace) + counter_bytes(B, n_kv_heads)) : nullptr;
+  a.n_q_heads = n_q_heads;
+  a.n_kv_heads = n_kv_heads;
+  a.group = group;
+  a.max_len = max_len;
+  a.splits = splits;
+  a.rot_mul = 1;
+  if (const char* e = getenv("MTP_ATTN_ROT")) a.rot_mul = atoi(e);
+  a.scale_log2e = scale * 1.4426950408889634f;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(splits, n_kv_heads, (unsigned)B);
+  int cfg = 0;
+  if (const char* e = getenv("MTP_ATTN_CFG")) cfg = atoi(e);
+#define MTP_ATTN_LAUNCH(W, R, NT)                                                                  \
+  do {                                                                                             \
+    if (append)                                                                                    \
+      hipLaunchKernelGGL((attn_decode_kernel<true, W, R, NT>), grid, dim3(W * 64), 0, s, a);       \
+    else                                                                                           \
+      hipLaunchKernelGGL((attn_decode_kernel<false, W, R, NT>), grid, dim3(W * 64), 0, s, a);      \
+  } while (0)
+  if (cfg == 1)
+    MTP_ATTN_LAUNCH(8, 2, false);
+  else if (cfg == 2)
+    MTP_ATTN_LAUNCH(4, 4, true);
+  else
+    MTP_ATTN_LAUNCH(8, 2, true);
+#undef MTP_ATTN_LAUNCH
+  MTP_CHECK_LAUNCH(what);
+  return MTP_OK;
+}
+}  // namespace
+
 extern "C" int64_t mtp_attn_decode_workspace_bytes(int64_t B, int n_q_heads, int n_kv_heads, int64_t len_bound) {
   if (B <= 0 || n_q_heads <= 0 || n_kv_heads <= 0 || len_bound <= 0) return 0;
-  return B * n_q_heads * (int64_t)pick_splits(B, n_kv_heads, len_bound) * AD_PART * (int64_t)sizeof(float);
+  return workspace_need(B, n_q_heads, n_kv_heads, pick_splits(B, n_kv_heads, len_bound));
 }
 
 extern "C" int mtp_attn_decode(const void* q, const void* k_cache, const void* v_cache, const int64_t* lens, void* out,
                                void* workspace, int64_t workspace_bytes, int64_t B, int n_q_heads, int n_kv_heads,
                                int head_dim, int64_t max_len, int64_t len_bound, float scale, int dtype,
                                void* stream) {
-  MTP_REQUIRE(dtype == MTP_BF16, MTP_EUNSUPPORTED, "attn_decode: bf16 only");
-  MTP_REQUIRE(head_dim == AD_D, MTP_EUNSUPPORTED, "attn_decode: head_dim %d (128 supported)", head_dim);
-  MTP_REQUIRE(B >= 0 && n_q_heads > 0 && n_kv_heads > 0 && n_q_heads % n_kv_heads == 0, MTP_EINVAL,
-              "attn_decode: B=%lld heads %d/%d", (long long)B, n_q_heads, n_kv_heads);
-  const int group = n_q_heads / n_kv_heads;
-  MTP_REQUIRE(group <= AD_MAX_GROUP, MTP_EUNSUPPORTED, "attn_decode: %d q heads per kv head (at most %d)", group,
-              AD_MAX_GROUP);
-  MTP_REQUIRE(max_len > 0 && len_bound > 0 && len_bound <= max_len, MTP_EINVAL,
-              "attn_decode: max_len=%lld len_bound=%lld", (long long)max_len, (long long)len_bound);
-  MTP_REQUIRE(B <= 65535 && n_kv_heads <= 65535, MTP_EINVAL, "attn_decode: grid too large");
-  if (B == 0) return MTP_OK;
-  MTP_REQUIRE(q && k_cache && v_cache && lens && out, MTP_EINVAL, "attn_decode: null pointer");
-  MTP_REQUIRE(((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0, MTP_EINVAL,
-              "attn_decode: q and the caches must be 16-byte aligned");
-  const int splits = pick_splits(B, n_kv_heads, len_bound);
-  if (splits > 1) {
-    const int64_t need = B * n_q_heads * (int64_t)splits * AD_PART * (int64_t)sizeof(float);
-    MTP_REQUIRE(workspace && workspace_bytes >= need, MTP_EINVAL, "attn_decode: workspace %lld bytes, need %lld",
-                (long long)workspace_bytes, (long long)need);
-  }
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  AttnArgs a;
+  MTP_REQUIRE(B == 0 || (q && lens), MTP_EINVAL, "attn_decode: null pointer");
+  AttnArgs a = {};
   a.q = static_cast<const uint16_t*>(q);
-  a.k = static_cast<const uint16_t*>(k_cache);
-  a.v = static_cast<const uint16_t*>(v_cache);
+  a.k = static_cast<uint16_t*>(const_cast<void*>(k_cache));     // only read in this form
+  a.v = static_cast<uint16_t*>(const_cast<void*>(v_cache));
   a.lens = lens;
   a.out = static_cast<uint16_t*>(out);
-  a.part = static_cast<float*>(workspace);
-  a.n_q_heads = n_q_heads;
-  a.n_kv_heads = n_kv_heads;
-  a.group = group;
-  a.max_len = max_len;
-  a.splits = splits;
-  a.scale_log2e = scale * 1.4426950408889634f;
-  hipLaunchKernelGGL(attn_decode_kernel, dim3(splits, n_kv_heads, (unsigned)B), dim3(AD_WAVES * 64), 0, s, a);
-  MTP_CHECK_LAUNCH("attn_decode");
-  if (splits > 1) {
-    hipLaunchKernelGGL(attn_merge_kernel, dim3(n_q_heads, (unsigned)B), dim3(AD_D), 0, s, a.part, a.out, splits);
-    MTP_CHECK_LAUNCH("attn_merge");
-  }
-  return MTP_OK;
+  return launch_attn(false, a, "attn_decode", workspace, workspace_bytes, B, n_q_heads, n_kv_heads, head_dim, max_len,
+                     len_bound, scale, dtype, stream);
+}
+
+extern "C" int mtp_attn_decode_append(const void* qkv, const void* cos_table, const void* sin_table,
+                                      const int64_t* positions, void* k_cache, void* v_cache, void* out,
+                                      void* workspace, int64_t workspace_bytes, int64_t B, int n_q_heads,
+                                      int n_kv_heads, int head_dim, int64_t max_len, int64_t max_positions,
+                                      int64_t len_bound, float scale, int dtype, void* stream) {
+  MTP_REQUIRE(B == 0 || (qkv && cos_table && sin_table && positions), MTP_EINVAL, "attn_decode_append: null pointer");
+  MTP_REQUIRE(max_positions > 0, MTP_EINVAL, "attn_decode_append: max_positions=%lld", (long long)max_positions);
+  AttnArgs a = {};
+  a.qkv = static_cast<const uint16_t*>(qkv);
+  a.cos_t = static_cast<const uint16_t*>(cos_table);
+  a.sin_t = static_cast<const uint16_t*>(sin_table);
+  a.positions = positions;
+  a.max_positions = max_positions;
+  a.k = static_cast<uint16_t*>(k_cache);
+  a.v = static_cast<uint16_t*>(v_cache);
+  a.out = static_cast<uint16_t*>(out);
+  return launch_attn(true, a, "attn_decode_append", workspace, workspace_bytes, B, n_q_heads, n_kv_heads, head_dim,
+                     max_len, len_bound, scale, dtype, stream);
 }
 
 extern "C" int mtp_rmsnorm(const void* x, const void* residual, const void* weight, void* y, void* residual_out,
@@ -426,15 +720,28 @@ extern "C" int mtp_rmsnorm(const void* x, const void* residual, const void* weig
   if (rows == 0) return MTP_OK;
   MTP_REQUIRE(x && weight && y, MTP_EINVAL, "rmsnorm: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const int epv = dtype == MTP_BF16 ? 8 : 4;
+  const bool aligned = ((uintptr_t)x | (uintptr_t)residual | (uintptr_t)weight | (uintptr_t)y |
+                        (uintptr_t)residual_out) % 16 == 0;
+  const int64_t nvec = dim / epv;
+  const bool fast = aligned && dim % epv == 0 && nvec <= 256 * 8;
+  const dim3 grid((unsigned)rows), block(256);
+#define MTP_RMS_LAUNCH(T, KERNEL)                                                                            \
+  hipLaunchKernelGGL(KERNEL, grid, block, 0, s, static_cast<const T*>(x), static_cast<const T*>(residual), \
+                     static_cast<const T*>(weight), static_cast<T*>(y), static_cast<T*>(residual_out), dim, eps)
+#define MTP_RMS_PICK(T)                                                \
+  do {                                                                 \
+    if (!fast) MTP_RMS_LAUNCH(T, rmsnorm_kernel<T>);                   \
+    else if (nvec <= 256 * 2) MTP_RMS_LAUNCH(T, (rmsnorm_vec_kernel<T, 2>)); \
+    else if (nvec <= 256 * 4) MTP_RMS_LAUNCH(T, (rmsnorm_vec_kernel<T, 4>)); \
+    else MTP_RMS_LAUNCH(T, (rmsnorm_vec_kernel<T, 8>));                \
+  } while (0)
   if (dtype == MTP_BF16)
-    hipLaunchKernelGGL(rmsnorm_kernel<uint16_t>, dim3((unsigned)rows), dim3(256), 0, s,
-                       static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(residual),
-                       static_cast<const uint16_t*>(weight), static_cast<uint16_t*>(y),
-                       static_cast<uint16_t*>(residual_out), dim, eps);
+    MTP_RMS_PICK(uint16_t);
   else
-    hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3((unsigned)rows), dim3(256), 0, s, static_cast<const float*>(x),
-                       static_cast<const float*>(residual), static_cast<const float*>(weight), static_cast<float*>(y),
-                       static_cast<float*>(residual_out), dim, eps);
+    MTP_RMS_PICK(float);
+#undef MTP_RMS_PICK
+#undef MTP_RMS_LAUNCH
   MTP_CHECK_LAUNCH("rmsnorm");
   return MTP_OK;
 }

@@ -81,8 +81,7 @@ class LlamaDecoder:
         need = _lib.lib().mtp_gemv_argmax_workspace_bytes(batch, lm_head.shape[0], lm_head.shape[1])
         self.argmax_ws = torch.empty((max(int(need), 8),), dtype=torch.uint8, device=dev)
         # the number of splits, and with it the need, does not shrink when the length bound grows
-        need = ops.attn_decode_workspace_bytes(batch, n_q_heads, n_kv_heads, max_len)
-        self.attn_ws = torch.empty((max(int(need), 8),), dtype=torch.uint8, device=dev)
+        self.attn_ws = ops.attn_workspace(batch, n_q_heads, n_kv_heads, max_len, dev)
 
     @classmethod
     def from_hf(cls, model, max_len: int = 4096, batch: int = 1):
@@ -113,8 +112,7 @@ class LlamaDecoder:
         """Appends ``tokens`` (int64 [batch]) and returns the final-norm output [batch, H] of their position."""
         if self.host_len_bound >= self.max_len:
             raise RuntimeError(f"key/value cache full ({self.max_len} positions)")
-        positions = self.lens.clone()
-        self.lens += 1
+        positions = self.lens             # tokens cached so far = position of the new one
         self.host_len_bound += 1
         x = ops.embedding_gather(tokens, self.embed, 0, self.embed.shape[0])
         residual = None
@@ -122,12 +120,13 @@ class LlamaDecoder:
         for w, kc, vc in zip(self.blocks, self.k_cache, self.v_cache):
             h, residual = ops.rmsnorm(x, w.input_norm, self.eps, residual, want_residual=True)
             qkv = ops.gemv(h, w.qkv)
-            q = ops.rope_kv_append(qkv, self.cos, self.sin, positions, kc, vc, self.n_q)
-            a = ops.attn_decode(q, kc, vc, self.lens, len_bound=self.host_len_bound, workspace=self.attn_ws)
+            a = ops.attn_decode_append(qkv, self.cos, self.sin, positions, kc, vc, self.n_q,
+                                       len_bound=self.host_len_bound, workspace=self.attn_ws)
             o = ops.gemv(a.view(B, -1), w.o)
             h, residual = ops.rmsnorm(o, w.post_norm, self.eps, residual, want_residual=True)
             act = ops.gemv(h, w.gate_up, None, ops.EPI_SWIGLU)
             x = ops.gemv(act, w.down)
+        self.lens += 1
         return ops.rmsnorm(x, self.final_norm, self.eps, residual)
 
     def logits(self, tokens: torch.Tensor) -> torch.Tensor:

@@ -393,6 +393,20 @@ def attn_decode_workspace_bytes(B: int, n_q_heads: int, n_kv_heads: int, len_bou
     return int(_lib.lib().mtp_attn_decode_workspace_bytes(B, n_q_heads, n_kv_heads, len_bound))
 
 
+def attn_workspace(B: int, n_q_heads: int, n_kv_heads: int, len_bound: int, device) -> torch.Tensor:
+    """Zero-filled scratch for ``attn_decode`` / ``attn_decode_append`` (the kernels need its head zero before
+    the first use and leave it zero)."""
+    return torch.zeros((max(attn_decode_workspace_bytes(B, n_q_heads, n_kv_heads, len_bound), 16),), dtype=torch.uint8,
+                       device=device)
+
+
+def _attn_workspace(workspace, B, n_q, n_kv, len_bound, dev):
+    need = attn_decode_workspace_bytes(B, n_q, n_kv, len_bound)
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = attn_workspace(B, n_q, n_kv, len_bound, dev)
+    return workspace
+
+
 def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, lens: torch.Tensor,
                 scale: Optional[float] = None, len_bound: Optional[int] = None,
                 workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -413,13 +427,44 @@ def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, l
     len_bound = max_len if len_bound is None else int(len_bound)
     scale = hd ** -0.5 if scale is None else float(scale)
     lib = _lib.lib()
-    need = int(lib.mtp_attn_decode_workspace_bytes(B, n_q, n_kv, len_bound))
-    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
-        workspace = torch.empty((need,), dtype=torch.uint8, device=dev)
+    workspace = _attn_workspace(workspace, B, n_q, n_kv, len_bound, dev)
     out = torch.empty_like(q)
     wbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     with torch.cuda.device(dev):
         _lib.check(lib.mtp_attn_decode(_p(q), _p(k_cache), _p(v_cache), _p(_contig(lens)), _p(out), _p(workspace),
                                        wbytes, B, n_q, n_kv, hd, max_len, len_bound, scale, _dt(q), _stream(dev)),
                    "mtp_attn_decode")
+    return out
+
+
+def attn_decode_append(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: torch.Tensor, positions: torch.Tensor,
+                       k_cache: torch.Tensor, v_cache: torch.Tensor, n_q_heads: int, scale: Optional[float] = None,
+                       len_bound: Optional[int] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``rope_kv_append`` then ``attn_decode`` over ``positions + 1`` tokens, as one launch.
+    ``workspace``: from ``attn_workspace`` (zero-filled once, reusable)."""
+    dev = _require_gpu(qkv, cos_table, sin_table, positions, k_cache, v_cache, workspace)
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("attn_decode_append: caches must be contiguous [B, n_kv_heads, max_len, head_dim] of one shape")
+    B, n_kv, max_len, hd = k_cache.shape
+    qkv = _contig(qkv)
+    if qkv.shape != (B, (n_q_heads + 2 * n_kv) * hd):
+        raise ValueError(f"attn_decode_append: qkv {tuple(qkv.shape)} for {n_q_heads}+2*{n_kv} heads of {hd}")
+    if cos_table.shape != sin_table.shape or cos_table.dim() != 2 or cos_table.shape[1] != hd:
+        raise ValueError("attn_decode_append: cos / sin tables must be [max_positions, head_dim]")
+    for t in (cos_table, sin_table, k_cache, v_cache):
+        if t.dtype != qkv.dtype:
+            raise ValueError("attn_decode_append: all tensors must share the dtype of qkv")
+    if positions.dtype != torch.int64 or positions.numel() != B:
+        raise ValueError("attn_decode_append: positions must be int64 [B]")
+    len_bound = max_len if len_bound is None else int(len_bound)
+    scale = hd ** -0.5 if scale is None else float(scale)
+    workspace = _attn_workspace(workspace, B, n_q_heads, n_kv, len_bound, dev)
+    out = torch.empty((B, n_q_heads, hd), dtype=qkv.dtype, device=dev)
+    wbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_attn_decode_append(_p(qkv), _p(_contig(cos_table)), _p(_contig(sin_table)),
+                                                     _p(_contig(positions)), _p(k_cache), _p(v_cache), _p(out),
+                                                     _p(workspace), wbytes, B, n_q_heads, n_kv, hd, max_len,
+                                                     cos_table.shape[0], len_bound, scale, _dt(qkv), _stream(dev)),
+                   "mtp_attn_decode_append")
     return out

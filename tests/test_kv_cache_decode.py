@@ -152,6 +152,45 @@ def test_attn_decode_llama8b_shape_long_context(gpu):
     assert torch.equal(again[6], out[6])                     # untouched sequences: bit for bit the same
 
 
+@pytest.mark.parametrize("B,n_q,n_kv,L", [(1, 32, 8, 2048), (7, 8, 1, 300), (32, 32, 8, 1024), (3, 16, 16, 64)])
+def test_attn_decode_append_equals_append_then_attend(gpu, B, n_q, n_kv, L):
+    """The one-launch form against rotary/append followed by attention (and so, through the tests of those,
+    against the oracle): same cache contents bit for bit, same attention output up to summation order."""
+    g = gen(9)
+    d = 128
+    qkv = torch.randn(B, (n_q + 2 * n_kv) * d, generator=g).bfloat16().to(gpu)
+    cos, sin = (t.to(gpu) for t in rope_tables(d, L, 500000.0, dtype=torch.bfloat16))
+    pos = torch.randint(0, L, (B,), generator=g)
+    pos[0] = L - 1
+    if B > 2:
+        pos[1], pos[2] = 0, L                      # nothing cached yet; outside the cache
+    kc0 = torch.randn(B, n_kv, L, d, generator=g).bfloat16()
+    vc0 = torch.randn(B, n_kv, L, d, generator=g).bfloat16()
+    k1, v1, k2, v2 = kc0.to(gpu), vc0.to(gpu), kc0.to(gpu), vc0.to(gpu)
+    q = ops.rope_kv_append(qkv, cos, sin, pos.to(gpu), k1, v1, n_q)
+    ref = ops.attn_decode(q, k1, v1, (pos + 1).clamp_max(L).to(gpu))
+    ws = ops.attn_workspace(B, n_q, n_kv, L, gpu)
+    for _ in range(2):                              # the workspace is reusable as the launch leaves it
+        out = ops.attn_decode_append(qkv, cos, sin, pos.to(gpu), k2, v2, n_q, workspace=ws)
+        assert torch.equal(k1, k2) and torch.equal(v1, v2)
+        for b in range(B):
+            if int(pos[b]) < L:
+                assert rel(out[b], ref[b]) < TOL_BF16, (b, int(pos[b]))
+            else:
+                assert torch.count_nonzero(out[b]) == 0
+    if B > 2:
+        assert torch.equal(out[1].cpu().view(n_kv, n_q // n_kv, d),
+                           qkv[1].view(-1, d)[n_q + n_kv:].cpu()[:, None, :].expand(n_kv, n_q // n_kv, d))
+    # and straight against the oracle for one row
+    heads = qkv[0].float().cpu().view(1, n_q + 2 * n_kv, d)
+    cf, sf = cos.float().cpu()[pos[:1]], sin.float().cpu()[pos[:1]]
+    kf, vf = kc0[:1].float(), vc0[:1].float()
+    kf[0, :, pos[0]] = R.apply_rope(heads[:, n_q:n_q + n_kv], cf, sf)[0]
+    vf[0, :, pos[0]] = heads[0, n_q + n_kv:]
+    want = R.attn_decode(R.apply_rope(heads[:, :n_q], cf, sf), kf, vf, pos[:1] + 1)
+    assert rel(out[0], want[0]) < TOL_BF16
+
+
 def test_attn_decode_rejects_bad_arguments(gpu):
     q = torch.zeros(2, 8, 128, dtype=torch.bfloat16, device=gpu)
     kc = torch.zeros(2, 2, 64, 128, dtype=torch.bfloat16, device=gpu)

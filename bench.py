@@ -173,6 +173,56 @@ def cpu_baseline(sample_tokens):
                       f"reference's order, median of 3 ({sec:.2f} s/step); cpu: {model}"}
 
 
+def kv_cache_decode(dev, timer, reps, table):
+    """Attention over the cache alone (algorithmic bytes: the K and V rows of every cached token, once), and
+    whole-model steps (32 blocks + LM head with fused argmax; bytes: all weights + the cached rows)."""
+    from merak_amd import ops, _lib
+    from merak_amd.inference import LlamaBlockWeights, LlamaDecoder
+    n_q, n_kv, d, H, I, layers = 32, 8, 128, 4096, 14336, 32
+    res = {}
+    st = torch.cuda.current_stream().cuda_stream
+    att = {}
+    for B, L in ((32, 8192), (8, 8192), (1, 8192)):
+        kc = torch.empty(B, n_kv, L, d, dtype=torch.bfloat16, device=dev).normal_()
+        vc = torch.empty(B, n_kv, L, d, dtype=torch.bfloat16, device=dev).normal_()
+        q = torch.randn(B, n_q, d, device=dev).bfloat16()
+        lens = torch.full((B,), L, dtype=torch.int64, device=dev)
+        ws = ops.attn_workspace(B, n_q, n_kv, L, dev)
+        o = torch.empty_like(q)
+        fn = lambda: _lib.check(_lib.lib().mtp_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), lens.data_ptr(),
+                                                           o.data_ptr(), ws.data_ptr(), ws.numel(), B, n_q, n_kv, d, L,
+                                                           L, d ** -0.5, 1, st), "attn")
+        # ten launches per timed region: one launch is shorter than the host's launch path at the small sizes
+        ms = timer.run(f"attn.b{B}", lambda: [fn() for _ in range(10)], max(3, reps // 2)) / 10
+        by = 2.0 * B * n_kv * L * d * 2
+        att[f"B{B}_L{L}"] = {"us": round(ms * 1e3, 1), "GBs": round(by / ms / 1e6, 1),
+                             "frac_hbm_peak": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        del kc, vc
+    res["attention"] = att
+    mk = lambda *shape: torch.empty(*shape, device=dev).normal_(0, 0.02).bfloat16()
+    ones = torch.ones(H, device=dev).bfloat16()
+    blocks = [LlamaBlockWeights(ones, mk((n_q + 2 * n_kv) * d, H), mk(H, n_q * d), ones, mk(2 * I, H), mk(H, I))
+              for _ in range(layers)]
+    wbytes = sum(t.numel() * 2 for b in blocks for t in (b.qkv, b.o, b.gate_up, b.down)) + table.numel() * 2
+    for B, L in ((1, 2048), (8, 2048), (32, 2048), (32, 8192)):
+        dec = LlamaDecoder(table, blocks, ones, table, n_q, n_kv, d, 1e-5, 500000.0, None, L + 8, B)
+        for c in dec.k_cache + dec.v_cache:
+            c.normal_()
+        tok = torch.randint(0, table.shape[0], (B,), device=dev)
+
+        def one():
+            dec.lens.fill_(L)
+            dec.host_len_bound = L
+            dec.step(tok)
+
+        ms = timer.run(f"kvdecode.b{B}.l{L}", one, max(3, reps // 4))
+        by = wbytes + 2.0 * layers * B * n_kv * L * d * 2
+        res[f"model_B{B}_L{L}"] = {"ms_per_token_step": round(ms, 3), "tokens_per_s": round(B / ms * 1e3, 1),
+                                   "GBs": round(by / ms / 1e6, 1), "frac_hbm_peak": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        del dec
+    return res
+
+
 def secondary(dev, timer, reps, with_cpu):
     from merak_amd import ops, _lib
     from oracle import tp_reference as R
@@ -288,7 +338,10 @@ def secondary(dev, timer, reps, with_cpu):
         smp[f"B{b}_us"] = round(timer.run(f"sample.b{b}", fn, reps) * 1e3, 1)
     dec["sample_top_k_top_p"] = smp
     out["decode_c5"] = dec
-    del table, wq, wg, wd, step
+    del wq, wg, wd, step
+    # --- the same step with attention over a key/value cache: one Llama-3-8B position per sequence
+    out["decode_with_kv_cache_llama8b"] = kv_cache_decode(dev, timer, reps, table)
+    del table
     # --- Llama-70B tp=8 shard shapes
     w3 = build_linear_workload(dev, LLAMA70B_TP8, 8192, 100)
     ms3 = timer.run("c3.step", lambda: linear_step(w3), max(3, reps // 2))

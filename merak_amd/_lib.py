@@ -46,6 +46,8 @@ SIGNATURES = {
     "mtp_argmax_rows": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "mtp_sample_workspace_bytes": (_i64, [_i64]),
     "mtp_sample_top_k_top_p": (_int, [_vp, _int, _i64, _i64, C.c_float, _int, C.c_float, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "mtp_gemv_workspace_bytes": (_i64, [_i64, _i64, _i64, _int]),
+    "mtp_gemv_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "mtp_rmsnorm": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, C.c_float, _int, _vp]),
     "mtp_rope_kv_append": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _int, _vp]),
     "mtp_attn_decode_workspace_bytes": (_i64, [_i64, _int, _int, _i64]),

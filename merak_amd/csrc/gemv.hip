@@ -85,7 +85,12 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
                                                           const uint16_t* __restrict__ w,
                                                           const uint16_t* __restrict__ bias,
                                                           uint16_t* __restrict__ y, ArgPart* __restrict__ part,
-                                                          int B, int64_t N, int64_t K, int rot_mul) {
+                                                          int B, int64_t N, int64_t K, int rot_mul, int64_t ld,
+                                                          float* __restrict__ kpart, int32_t* __restrict__ karrived) {
+  // K is the extent along k that this workgroup covers and ld the row stride of X and W: with gridDim.y > 1
+  // the k range is cut into gridDim.y slices of K elements, one workgroup per (row block, slice); the
+  // slices' partial sums meet in `kpart` and the slice that delivers last adds them up in slice order.
+  const int64_t koff = (int64_t)blockIdx.y * K;
   constexpr int GV_WAVES = W, GV_THREADS = W * MTP_WAVE;
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -113,15 +118,15 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
     }
     if (row0 >= lim) row0 = lim - 1;                 // a group entirely past the end reads the last row
     const int last = (int)(lim - 1 - row0);          // >= 0: largest valid row offset inside this group
-    wbase[r] = w + row0 * K;
+    wbase[r] = w + row0 * ld + koff;
     if (GUARD) {
       const int ra = li < last ? li : last;
-      offa[r] = (uint32_t)(ra * K + 8 * lg);
+      offa[r] = (uint32_t)(ra * ld + 8 * lg);
       offb[r] = offa[r] + 32;
     } else {
       const int ra = (li & 7) < last ? (li & 7) : last, rb = 8 + (li & 7) < last ? 8 + (li & 7) : last;
-      offa[r] = (uint32_t)(ra * K + 32 * (li >> 3) + 8 * lg);
-      offb[r] = (uint32_t)(rb * K + 32 * (1 - (li >> 3)) + 8 * lg);
+      offa[r] = (uint32_t)(ra * ld + 32 * (li >> 3) + 8 * lg);
+      offb[r] = (uint32_t)(rb * ld + 32 * (1 - (li >> 3)) + 8 * lg);
     }
   }
   const uint16_t* xp[NB];
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   for (int nb = 0; nb < NB; nb++) {
     int b = li + 16 * nb;
     if (b >= B) b = B - 1;
-    xp[nb] = x + (int64_t)b * K + 8 * lg;
+    xp[nb] = x + (int64_t)b * ld + koff + 8 * lg;
   }
 
   // This wave's k range, in pairs of 32-element steps: a pair covers 64 elements = one 128-byte line of
@@ -146,7 +151,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   // (rows being a power-of-two apart) live in the same few memory channels.
   // (Summation order along k therefore differs between workgroups: equal weight rows that live in different
   // workgroups give logits that are equal to rounding, not necessarily bit for bit.)
-  const int64_t rot = GUARD || (pairs % GV_MAX_WAVES) ? 0 : ((int64_t)blockIdx.x * rot_mul) % pairs;
+  const int64_t rot = GUARD || (pairs % GV_MAX_WAVES) ? 0 : ((int64_t)(blockIdx.x + blockIdx.y) * rot_mul) % pairs;
 
   f32x4_t acc[R][NB];
 #pragma unroll
@@ -263,6 +268,38 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
       for (int wv = 0; wv < GV_WAVES; wv++) s += part_lds[wv][rr][nb][j][l];
       // D[i][b]: lane l, register j holds row i = 4*(l/16)+j, column b = l%16
       fin[(l & 15) + 16 * nb][16 * (r0 + rr) + 4 * (l >> 4) + j] = s;
+    }
+    __syncthreads();
+  }
+
+  if (MODE != 2 && gridDim.y > 1) {
+    // k slices: hand the partial over with device-scope stores, count arrivals; the last slice to arrive sums
+    // all of them in slice order (its own included, read back), so the result does not depend on who is last
+    constexpr int FIN = 16 * R;
+    const int S = gridDim.y, cnt = B * FIN;
+    float* mine = kpart + ((int64_t)blockIdx.x * S + blockIdx.y) * cnt;
+    for (int e = tid; e < cnt; e += GV_THREADS)
+      __hip_atomic_store(mine + e, fin[e / FIN][e % FIN], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    __shared__ int last_one;
+    if (tid == 0) {
+      const int seen = __hip_atomic_fetch_add(karrived + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      last_one = seen == S - 1;
+      if (last_one) __hip_atomic_store(karrived + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!last_one) return;
+    const float* all = kpart + (int64_t)blockIdx.x * S * cnt;
+    for (int e = tid; e < cnt; e += GV_THREADS) {
+      float v[8];
+#pragma unroll
+      for (int sl = 0; sl < 8; sl++)
+        v[sl] = sl < S ? __hip_atomic_load(all + (int64_t)sl * cnt + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+      float sum = v[0];
+#pragma unroll
+      for (int sl = 1; sl < 8; sl++) sum += v[sl];
+      fin[e / FIN][e % FIN] = sum;
     }
     __syncthreads();
   }
@@ -422,17 +459,35 @@ __global__ __launch_bounds__(256) void argmax_rows_kernel(const T* __restrict__ 
 struct GemvCfg {
   int R;  // 16-row groups per workgroup
   int D;  // k-pairs in flight per wave and step
+  int S;  // slices along k, one workgroup each (needs a workspace); 1 = the workgroup walks all of k
 };
+constexpr int GV_MAX_SLICES = 8;
 
 bool depth_ok(int64_t K, int d) { return d == 1 || (K % 64 == 0 && ((K / 64) % (GV_MAX_WAVES * d)) == 0); }
 
-GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode) {
+GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode, bool may_split = false) {
   const int64_t groups = ((mode == 1 ? N / 2 : N) + 15) / 16 * (mode == 1 ? 2 : 1);
   // Bytes in flight are what a bandwidth-bound kernel lives on: R*D k-pairs (2 KiB each) per wave.  Large
   // matrices take them as rows (X is re-read from L2 once per 16*R rows, which is what batches above 16
   // care about); matrices with few row groups keep every CU busy by going deeper along k instead.
   // Measured on 128256x4096, 28672x4096, 6144x4096, 4096x14336, 8192x3584 and 1280x8192 at B = 1, 8, 32.
-  GemvCfg c{B > 16 ? 8 : 4, 1};
+  GemvCfg c{B > 16 ? 8 : 4, 1, 1};
+  // Above 16 batch rows X is read twice per 16 R weight rows: halving R until there are enough workgroups
+  // makes the L2 -> CU traffic of X a multiple of the weight stream.  With a workspace the rows stay and k is
+  // cut instead (each slice reads only its part of X); every wave of a slice gets the same number of pairs.
+  // Measured (B = 16 and 32): 4096x14336 gains 17-23 %, matrices with K = 4096 lose (too little k per slice to
+  // pay for the hand-over), batches up to 8 gain nothing.
+  if (may_split && mode != 2 && K % 64 == 0 && groups / c.R < 190) {
+    int want = (B > 8 && K >= 8192) ? 0 : -1;
+    if (const char* e = getenv("MTP_GEMV_S")) want = atoi(e);
+    const int waves = c.R >= 8 ? 4 : GV_MAX_WAVES;
+    for (int sl = 2; want >= 0 && sl <= GV_MAX_SLICES; sl *= 2) {
+      if ((K / 64) % (sl * waves) != 0 || (want == 0 && K / 64 / (sl * waves) < 6)) break;
+      c.S = sl;
+      if (want ? sl >= want : groups / c.R * sl >= 190) break;
+    }
+    if (c.S > 1) return c;
+  }
   while (c.R > 1 && groups / c.R < 190) c.R >>= 1;
   if (mode == 1 && c.R < 2) c.R = 2;
   c.D = (B > 16 || c.R >= 4) ? 1 : 2;
@@ -450,9 +505,12 @@ GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode) {
   return c;
 }
 
+// bytes of the arrival counters in front of the partial sums: one per 16 rows covers every configuration
+int64_t gemv_counter_bytes(int64_t N) { return ((N + 15) / 16 * (int64_t)sizeof(int32_t) + 255) / 256 * 256; }
+
 template <int MODE>
 int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart* part, int64_t B, int64_t N,
-                int64_t K, GemvCfg cfg, hipStream_t s, unsigned* n_wg_out) {
+                int64_t K, GemvCfg cfg, hipStream_t s, unsigned* n_wg_out, void* workspace = nullptr) {
   const int R = cfg.R;
   const int64_t rows_per_wg = (MODE == 1) ? 8 * R : 16 * R;
   const int64_t span = (MODE == 1) ? N / 2 : N;
@@ -461,14 +519,20 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   const int NB = B > 16 ? 2 : 1;
   int rot_mul = 1;
   if (const char* e = getenv("MTP_GEMV_ROT")) rot_mul = atoi(e);
+  // k slices: counters first (one per row block, zero between launches), then the partial sums
+  const int S = workspace ? cfg.S : 1;
+  int32_t* karrived = static_cast<int32_t*>(workspace);
+  float* kpart = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + gemv_counter_bytes(N)) : nullptr;
+  const int64_t k_slice = K / S;
 #define GV_LAUNCH(RR, NNB, GG, DD)                                                                              \
-  hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD, (RR >= 8 ? 4 : 8)>), dim3(n_wg),                       \
+  hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD, (RR >= 8 ? 4 : 8)>), dim3(n_wg, S),                    \
                      dim3((RR >= 8 ? 4 : 8) * MTP_WAVE), 0, s,                                                  \
                      (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part, (int)B, \
-                     N, K, rot_mul)
+                     N, k_slice, rot_mul, K, kpart, karrived)
 #define GV_BY_DEPTH(RR, NNB)                                                   \
   do {                                                                         \
     if (K % 64 != 0) GV_LAUNCH(RR, NNB, true, 1);                              \
+    else if (S > 1) GV_LAUNCH(RR, NNB, false, 1);                              \
     else if (RR * 4 <= 4 && cfg.D == 4) GV_LAUNCH(RR, NNB, false, (RR * 4 <= 4 ? 4 : 1)); \
     else if (RR * 2 <= 4 && cfg.D == 2) GV_LAUNCH(RR, NNB, false, (RR * 2 <= 4 ? 2 : 1)); \
     else GV_LAUNCH(RR, NNB, false, 1);                                         \
@@ -503,8 +567,17 @@ int check_gemv_args(const char* what, const void* x, const void* w, int64_t B, i
 
 }  // namespace
 
-extern "C" int mtp_gemv(const void* x, const void* w, const void* bias, void* y, int64_t B, int64_t N, int64_t K,
-                        int epilogue, void* stream) {
+extern "C" int64_t mtp_gemv_workspace_bytes(int64_t B, int64_t N, int64_t K, int epilogue) {
+  if (B < 1 || B > 32 || N < 1 || K < 1) return 0;
+  const GemvCfg c = pick_gemv_cfg(B, N, K, epilogue == MTP_EPI_SWIGLU ? 1 : 0, true);
+  if (c.S <= 1) return 0;
+  // every row block leaves B x (its rows) partial sums per slice; row blocks may overhang N by one block
+  const int64_t rows = (N + 16 * c.R - 1) / (16 * c.R) * (16 * c.R) + (epilogue == MTP_EPI_SWIGLU ? 16 * c.R : 0);
+  return gemv_counter_bytes(N) + (int64_t)c.S * B * rows * (int64_t)sizeof(float);
+}
+
+extern "C" int mtp_gemv_ws(const void* x, const void* w, const void* bias, void* y, void* workspace,
+                           int64_t workspace_bytes, int64_t B, int64_t N, int64_t K, int epilogue, void* stream) {
   int rc = check_gemv_args("gemv", x, w, B, N, K);
   if (rc) return rc;
   MTP_REQUIRE(y, MTP_EINVAL, "gemv: null output");
@@ -512,12 +585,22 @@ extern "C" int mtp_gemv(const void* x, const void* w, const void* bias, void* y,
               "gemv: epilogue %d not supported", epilogue);
   MTP_REQUIRE(epilogue != MTP_EPI_BIAS || bias, MTP_EINVAL, "gemv: MTP_EPI_BIAS without bias");
   hipStream_t s = (hipStream_t)stream;
-  if (epilogue == MTP_EPI_SWIGLU) {
+  const int mode = epilogue == MTP_EPI_SWIGLU ? 1 : 0;
+  // without a workspace (or with one too small for the slices) every workgroup walks all of k
+  const int64_t need = workspace ? mtp_gemv_workspace_bytes(B, N, K, epilogue) : 0;
+  const bool split = need > 0 && workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0;
+  const GemvCfg cfg = pick_gemv_cfg(B, N, K, mode, split);
+  if (mode == 1) {
     MTP_REQUIRE(N % 2 == 0, MTP_EINVAL, "gemv: SwiGLU needs an even N, got %lld", (long long)N);
-    return launch_gemv<1>(x, w, bias, y, nullptr, B, N, K, pick_gemv_cfg(B, N, K, 1), s, nullptr);
+    return launch_gemv<1>(x, w, bias, y, nullptr, B, N, K, cfg, s, nullptr, split ? workspace : nullptr);
   }
-  return launch_gemv<0>(x, w, epilogue == MTP_EPI_NONE ? nullptr : bias, y, nullptr, B, N, K,
-                        pick_gemv_cfg(B, N, K, 0), s, nullptr);
+  return launch_gemv<0>(x, w, epilogue == MTP_EPI_NONE ? nullptr : bias, y, nullptr, B, N, K, cfg, s, nullptr,
+                        split ? workspace : nullptr);
+}
+
+extern "C" int mtp_gemv(const void* x, const void* w, const void* bias, void* y, int64_t B, int64_t N, int64_t K,
+                        int epilogue, void* stream) {
+  return mtp_gemv_ws(x, w, bias, y, nullptr, 0, B, N, K, epilogue, stream);
 }
 
 extern "C" int64_t mtp_gemv_argmax_workspace_bytes(int64_t B, int64_t N, int64_t K) {

@@ -57,10 +57,22 @@ class DecodeStep:
         from .. import _lib
         need = _lib.lib().mtp_gemv_argmax_workspace_bytes(max_batch, w_lm_head.shape[0], w_lm_head.shape[1])
         self.workspace = torch.empty((need,), dtype=torch.uint8, device=w_lm_head.device)
+        # scratch of the linears that are cut along k at this batch size (the launches follow each other)
+        self.max_batch = max_batch
+        self._gemv_ws = {}
+
+    def _ws(self, batch: int):
+        if batch not in self._gemv_ws:
+            need = [ops.gemv_workspace(batch, w.shape[0], w.shape[1], e, w.device)
+                    for w, e in ((self.w_qkv, ops.EPI_NONE), (self.w_gate_up, ops.EPI_SWIGLU), (self.w_down, ops.EPI_NONE))]
+            need = [t for t in need if t is not None]
+            self._gemv_ws[batch] = max(need, key=lambda t: t.numel()) if need else None
+        return self._gemv_ws[batch]
 
     def __call__(self, x: torch.Tensor):
-        qkv = ops.gemv(x, self.w_qkv)
-        h = ops.gemv(x, self.w_gate_up, None, ops.EPI_SWIGLU)
-        out = ops.gemv(h, self.w_down)
+        ws = self._ws(x.shape[0])
+        qkv = ops.gemv(x, self.w_qkv, workspace=ws)
+        h = ops.gemv(x, self.w_gate_up, None, ops.EPI_SWIGLU, workspace=ws)
+        out = ops.gemv(h, self.w_down, workspace=ws)
         token = greedy_next_token(out, self.w_lm_head, self.workspace)
         return qkv, out, token

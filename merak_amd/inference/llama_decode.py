@@ -82,6 +82,12 @@ class LlamaDecoder:
         self.argmax_ws = torch.empty((max(int(need), 8),), dtype=torch.uint8, device=dev)
         # the number of splits, and with it the need, does not shrink when the length bound grows
         self.attn_ws = ops.attn_workspace(batch, n_q_heads, n_kv_heads, max_len, dev)
+        w0 = blocks[0]
+        need = [ops.gemv_workspace(batch, w.shape[0], w.shape[1], e, dev)
+                for w, e in ((w0.qkv, ops.EPI_NONE), (w0.o, ops.EPI_NONE), (w0.gate_up, ops.EPI_SWIGLU),
+                             (w0.down, ops.EPI_NONE), (lm_head, ops.EPI_NONE))]
+        need = [t for t in need if t is not None]
+        self.gemv_ws = max(need, key=lambda t: t.numel()) if need else None
 
     @classmethod
     def from_hf(cls, model, max_len: int = 4096, batch: int = 1):
@@ -119,19 +125,19 @@ class LlamaDecoder:
         B = x.shape[0]
         for w, kc, vc in zip(self.blocks, self.k_cache, self.v_cache):
             h, residual = ops.rmsnorm(x, w.input_norm, self.eps, residual, want_residual=True)
-            qkv = ops.gemv(h, w.qkv)
+            qkv = ops.gemv(h, w.qkv, workspace=self.gemv_ws)
             a = ops.attn_decode_append(qkv, self.cos, self.sin, positions, kc, vc, self.n_q,
                                        len_bound=self.host_len_bound, workspace=self.attn_ws)
-            o = ops.gemv(a.view(B, -1), w.o)
+            o = ops.gemv(a.view(B, -1), w.o, workspace=self.gemv_ws)
             h, residual = ops.rmsnorm(o, w.post_norm, self.eps, residual, want_residual=True)
-            act = ops.gemv(h, w.gate_up, None, ops.EPI_SWIGLU)
-            x = ops.gemv(act, w.down)
+            act = ops.gemv(h, w.gate_up, None, ops.EPI_SWIGLU, workspace=self.gemv_ws)
+            x = ops.gemv(act, w.down, workspace=self.gemv_ws)
         self.lens += 1
         return ops.rmsnorm(x, self.final_norm, self.eps, residual)
 
     def logits(self, tokens: torch.Tensor) -> torch.Tensor:
         """The row the reference slices out at :223 (fp32 accumulation, model dtype)."""
-        return ops.gemv(self.hidden(tokens), self.lm_head)
+        return ops.gemv(self.hidden(tokens), self.lm_head, workspace=self.gemv_ws)
 
     def step(self, tokens: torch.Tensor) -> torch.Tensor:
         """Greedy next token per sequence (:226-227); the [batch, vocab] logits are never written."""

@@ -267,16 +267,26 @@ def vocab_ce_rescale_(grad2d: torch.Tensor, grad_rows: torch.Tensor, assumed: fl
 
 
 # --------------------------------------------------------------------------- decode
-def gemv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE) -> torch.Tensor:
-    dev = _require_gpu(x, w, bias)
+def gemv_workspace(B: int, N: int, K: int, epilogue: int, device) -> Optional[torch.Tensor]:
+    """Zero-filled scratch for ``gemv(..., workspace=)`` or None when this shape runs without one.  One
+    workspace serves any number of launches that do not overlap (take the largest need)."""
+    need = int(_lib.lib().mtp_gemv_workspace_bytes(B, N, K, epilogue))
+    return torch.zeros((need,), dtype=torch.uint8, device=device) if need else None
+
+
+def gemv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE,
+         workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    dev = _require_gpu(x, w, bias, workspace)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise TypeError("gemv is bf16 only")
     B, K = x.shape
     N = w.shape[0]
     x, w = _contig(x), _contig(w)
     y = torch.empty((B, N // 2 if epilogue == EPI_SWIGLU else N), dtype=torch.bfloat16, device=dev)
+    wbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().mtp_gemv(_p(x), _p(w), _p(bias), _p(y), B, N, K, epilogue, _stream(dev)), "mtp_gemv")
+        _lib.check(_lib.lib().mtp_gemv_ws(_p(x), _p(w), _p(bias), _p(y), _p(workspace), wbytes, B, N, K, epilogue,
+                                          _stream(dev)), "mtp_gemv")
     return y
 
 

@@ -551,6 +551,37 @@ def test_gemv_and_fused_argmax(gpu, b, n, k):
     assert torch.equal(greedy_from_logits(ref.to(gpu)).cpu(), R.greedy_argmax(ref))
 
 
+@pytest.mark.parametrize("b,n,k,epi,force,cut", [
+    (32, 4096, 14336, "none", None, True), (17, 4096, 14336, "bias", None, True), (9, 1280, 8192, "none", None, True),
+    (32, 4096, 4096, "none", None, False), (8, 4096, 14336, "none", None, False),      # small k / small batch: uncut
+    (32, 6144, 4096, "bias", "4", True), (32, 2048, 4096, "swiglu", "8", True), (24, 1000, 1024, "none", "2", True),
+    (3, 4096, 4096, "none", "8", True)])
+def test_gemv_cut_along_k_with_workspace(gpu, monkeypatch, b, n, k, epi, force, cut):
+    """Few-row matrices with a long k run, above 8 batch rows, as k slices whose partial sums meet in a
+    workspace (other shapes only when forced): same numbers as the oracle, the same bits on every run, and a
+    workspace that can be used again as it is left."""
+    if force:
+        monkeypatch.setenv("MTP_GEMV_S", force)
+    g = gen(31)
+    x = torch.randn(b, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.02).bfloat16()
+    bias = (torch.randn(n, generator=g) * 0.1).bfloat16() if epi == "bias" else None
+    e = {"none": ops.EPI_NONE, "bias": ops.EPI_BIAS, "swiglu": ops.EPI_SWIGLU}[epi]
+    ref = F.linear(x.float(), w.float(), None if bias is None else bias.float())
+    if epi == "swiglu":
+        ref = R.swiglu(ref.bfloat16().float())
+    ws = ops.gemv_workspace(b, n, k, e, gpu)
+    assert (ws is not None) == cut
+    xg, wg, bg = x.to(gpu), w.to(gpu), None if bias is None else bias.to(gpu)
+    y1 = ops.gemv(xg, wg, bg, e, workspace=ws)
+    y2 = ops.gemv(xg, wg, bg, e, workspace=ws)
+    assert rel(y1, ref) < TOL_BF16
+    assert torch.equal(y1, y2)
+    if ws is not None:
+        assert rel(ops.gemv(xg, wg, bg, e), y1) < TOL_BF16 / 4        # against the uncut form
+        assert int(ws[:4 * ((n + 15) // 16)].count_nonzero()) == 0       # counters are back at zero
+
+
 def test_argmax_ties_and_nan(gpu):
     k, n = 256, 999
     x = torch.randn(4, k, generator=gen(92)).bfloat16()

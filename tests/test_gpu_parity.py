@@ -817,3 +817,42 @@ def test_training_loop_matches_stock_pytorch(gpu, dtype):
     tol = 1e-4 if dtype == torch.float32 else 3e-2
     assert all(abs(a - b_) <= tol * abs(b_) for a, b_ in zip(losses, ref_losses)), (losses, ref_losses)
     assert ref_losses[-1] < ref_losses[0] - 0.05, "the reference loop itself must be learning"
+
+
+def test_tagged_model_rebuilt_onto_the_gfx950_layers(gpu):
+    """The reference's sequence (feature lists -> set_mp_attr -> module rebuild, mp_attrs.py:43-202,
+    model_parallel.py:87-99) at tensor-parallel degree 1: the rebuilt MLP, given the original weights, computes
+    what the stock torch modules compute, forward and backward."""
+    from merak_amd.tensor_parallel import (set_tp_layer_lists, set_mp_attr, rebuild_module, reset_tp_layer_lists,
+                                           init_method_normal, scaled_init_method_normal, ColPara, RowPara)
+
+    class MLP(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc_in, self.fc_out = torch.nn.Linear(256, 1024), torch.nn.Linear(1024, 256)
+
+        def forward(self, x):
+            return self.fc_out(F.gelu(self.fc_in(x), approximate="tanh"))
+
+    torch.manual_seed(5)
+    stock = MLP()
+    x = torch.randn(3, 50, 256)
+    xs = x.clone().requires_grad_(True)
+    ref = stock(xs)
+    ref.backward(torch.ones_like(ref))
+    reset_tp_layer_lists()
+    set_tp_layer_lists(col_para_list=["fc_in"], row_para_list=["fc_out"])
+    set_args(use_cpu_initialization=True, params_dtype=torch.float32)
+    mine = rebuild_module(set_mp_attr(MLP(), 1), 1, init_method_normal(0.02), scaled_init_method_normal(0.02, 1))
+    reset_tp_layer_lists()
+    assert isinstance(mine.fc_in, ColPara) and isinstance(mine.fc_out, RowPara)
+    missing = mine.load_state_dict({k.replace("fc_in.", "fc_in.col_linear.").replace("fc_out.", "fc_out.row_linear."): v
+                                    for k, v in stock.state_dict().items()})
+    assert not missing.missing_keys and not missing.unexpected_keys
+    mine.to(gpu)
+    xg = x.to(gpu).requires_grad_(True)
+    out = mine(xg)
+    out.backward(torch.ones_like(out))
+    assert rel(out, ref) < TOL_F32 and rel(xg.grad, xs.grad) < TOL_F32
+    assert rel(mine.fc_in.weight.grad, stock.fc_in.weight.grad) < TOL_F32
+    assert rel(mine.fc_out.bias.grad, stock.fc_out.bias.grad) < TOL_F32

@@ -157,3 +157,112 @@ def test_vocab_utility_matches_oracle(per, world, data):
     got = mpu.VocabUtility.vocab_range_from_global_vocab_size(per * world, rank, world)
     assert got == R.vocab_range_from_global_vocab_size(per * world, rank, world) == (rank * per, rank * per + per)
     assert mpu.divide(per * world, world) == per
+
+
+def test_rope_tables_default_and_llama3_scaling_match_the_library():
+    """cos / sin tables of the decoder against transformers' LlamaRotaryEmbedding (default rope type and the
+    Llama-3.1 frequency rescale)."""
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaRotaryEmbedding
+    from merak_amd.inference import rope_tables
+    scaling = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+               "original_max_position_embeddings": 8192, "rope_theta": 500000.0}
+    pos = torch.tensor([[0, 1, 17, 4095, 8191, 20000]])
+    for params in ({"rope_type": "default", "rope_theta": 10000.0}, scaling):
+        cfg = LlamaConfig(hidden_size=512, num_attention_heads=4, head_dim=128, num_hidden_layers=1, vocab_size=32,
+                          intermediate_size=64, max_position_embeddings=32768, rope_parameters=dict(params))
+        cos, sin = LlamaRotaryEmbedding(cfg)(torch.zeros(1, pos.shape[1], 512), pos)
+        mine_cos, mine_sin = rope_tables(128, 20001, params["rope_theta"],
+                                         params if params["rope_type"] != "default" else None)
+        assert torch.allclose(mine_cos[pos[0]], cos[0], atol=2e-4), params["rope_type"]
+        assert torch.allclose(mine_sin[pos[0]], sin[0], atol=2e-4), params["rope_type"]
+    with pytest.raises(NotImplementedError):
+        rope_tables(128, 16, 10000.0, {"rope_type": "yarn"})
+
+
+# ---- feature lists -> tags -> rebuilt layers (mp_attrs.py:43-202, model_parallel.py:87-99) ----
+class _ToyAttn(nn.Module):
+    def __init__(self, h):
+        super().__init__()
+        self.c_attn, self.c_proj = nn.Linear(h, 3 * h), nn.Linear(h, h)
+        self.num_heads, self.split_size = 4, h
+
+
+class _ToyMLP(nn.Module):
+    def __init__(self, h):
+        super().__init__()
+        self.fc_in, self.fc_out = nn.Linear(h, 4 * h), nn.Linear(4 * h, h, bias=False)
+
+    def forward(self, x):
+        return self.fc_out(torch.nn.functional.gelu(self.fc_in(x), approximate="tanh"))
+
+
+class _ToyModel(nn.Module):
+    def __init__(self, h=64, v=100):
+        super().__init__()
+        self.wte = nn.Embedding(v, h)
+        self.blocks = nn.ModuleList([nn.ModuleDict({"attn": _ToyAttn(h), "mlp": _ToyMLP(h)}) for _ in range(2)])
+        self.head_scale = nn.Parameter(torch.ones(8, h))
+
+
+def test_feature_lists_tag_and_rebuild_like_the_reference():
+    from merak_amd.tensor_parallel import (set_tp_layer_lists, set_mp_attr, rebuild_module, mp_is_setted,
+                                           get_tp_attr_list, reset_tp_layer_lists)
+    reset_tp_layer_lists()
+    assert not mp_is_setted()
+    with pytest.raises(AssertionError, match="at least one kind of tp list"):
+        set_tp_layer_lists(col_para_list=["c_attn"])                 # column names need row names (:181-183)
+    set_tp_layer_lists(col_para_list=["c_attn", "fc_in"], row_para_list=["c_proj", "fc_out"],
+                       weight_change_list=[("wte", 0), ("head_scale", 0)])
+    assert mp_is_setted() and get_tp_attr_list() == []
+    m = set_mp_attr(_ToyModel(), 2)
+    b0 = m.blocks[0]
+    assert (b0["attn"].c_attn.mp_attr, b0["attn"].c_attn.out_features, b0["attn"].c_attn.in_features) == ("col", 96, 64)
+    assert (b0["attn"].c_proj.mp_attr, b0["attn"].c_proj.in_features) == ("row", 32)
+    assert (b0["mlp"].fc_in.mp_attr, b0["mlp"].fc_in.out_features) == ("col", 128)
+    assert (b0["mlp"].fc_out.mp_attr, b0["mlp"].fc_out.in_features) == ("row", 128)
+    assert (b0["attn"].num_heads, b0["attn"].split_size) == (2, 32)         # default attribute list (:26-27)
+    assert m.wte.weight.shape == (50, 64) and m.wte.num_embeddings == 50    # module weight cut along dim 0
+    assert m.head_scale.shape == (4, 64)                                    # bare parameter cut along dim 0
+    mpu.set_model_parallel_world_size(2)
+    mpu.set_model_parallel_rank(1)
+    rebuild_module(m, 2, init_method_normal(0.02), scaled_init_method_normal(0.02, 2))
+    for blk in m.blocks:
+        assert isinstance(blk["attn"].c_attn, ColPara) and isinstance(blk["mlp"].fc_in, ColPara)
+        assert isinstance(blk["attn"].c_proj, RowPara) and isinstance(blk["mlp"].fc_out, RowPara)
+        assert blk["attn"].c_attn.weight.shape == (96, 64) and blk["attn"].c_proj.weight.shape == (64, 32)
+        assert blk["mlp"].fc_in.weight.shape == (128, 64) and blk["mlp"].fc_out.weight.shape == (64, 128)
+        assert blk["mlp"].fc_out.bias is None and blk["mlp"].fc_in.bias.shape == (128,)
+    assert "blocks.1.mlp.fc_in.col_linear.weight" in m.state_dict()
+    # attributes that do not divide are refused with the reference's message (:140-141)
+    reset_tp_layer_lists()
+    set_tp_layer_lists(col_para_list=["c_attn"], row_para_list=["c_proj"], tp_attr_list=["num_heads"])
+    with pytest.raises(AssertionError, match="mp attr set error, num_heads"):
+        set_mp_attr(_ToyModel(), 3)
+    reset_tp_layer_lists()
+
+
+def test_input_output_ratio_table_tags_linear_and_conv1d():
+    from transformers.pytorch_utils import Conv1D
+    from merak_amd.tensor_parallel import set_tp_layer_lists, set_mp_attr, reset_tp_layer_lists, rebuild_module
+    reset_tp_layer_lists()
+    set_tp_layer_lists(input_output_mapping=[(1, 4, "col"), (4, 1, "row"), (1, 3, "col")])
+
+    class GPT2ish(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.c_fc, self.c_proj, self.c_attn = Conv1D(256, 64), Conv1D(64, 256), Conv1D(192, 64)   # (nf, nx)
+            self.lin_up, self.lin_same = nn.Linear(64, 256), nn.Linear(64, 64)
+
+    m = set_mp_attr(GPT2ish(), 4)
+    assert (m.c_fc.mp_attr, m.c_fc.in_features, m.c_fc.out_features) == ("col", 64, 64)
+    assert (m.c_proj.mp_attr, m.c_proj.in_features, m.c_proj.out_features) == ("row", 64, 64)
+    assert (m.c_attn.mp_attr, m.c_attn.out_features) == ("col", 48)
+    assert (m.lin_up.mp_attr, m.lin_up.out_features) == ("col", 64) and not hasattr(m.lin_same, "mp_attr")
+    mpu.set_model_parallel_world_size(4)
+    rebuild_module(m, 4, init_method_normal(0.02), scaled_init_method_normal(0.02, 1))
+    assert isinstance(m.c_fc, ColPara) and m.c_fc.weight.shape == (64, 64)          # [out/p, in]
+    assert isinstance(m.c_proj, RowPara) and m.c_proj.weight.shape == (64, 64)      # [out, in/p]
+    assert isinstance(m.c_attn, ColPara) and m.c_attn.weight.shape == (48, 64)
+    assert isinstance(m.lin_same, nn.Linear)                                        # untagged: left alone
+    reset_tp_layer_lists()

@@ -648,6 +648,7 @@ int launch_attn(bool append, AttnArgs a, const char* what, void* workspace, int6
   a.splits = splits;
   a.rot_mul = 1;
   if (const char* e = getenv("MTP_ATTN_ROT")) a.rot_mul = atoi(e);
+  if (a.rot_mul < 0) a.rot_mul = 0;   // taken modulo the tile count: must not go negative
   a.scale_log2e = scale * 1.4426950408889634f;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(splits, n_kv_heads, (unsigned)B);

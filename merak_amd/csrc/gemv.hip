@@ -86,7 +86,8 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
                                                           const uint16_t* __restrict__ bias,
                                                           uint16_t* __restrict__ y, ArgPart* __restrict__ part,
                                                           int B, int64_t N, int64_t K, int rot_mul, int64_t ld,
-                                                          float* __restrict__ kpart, int32_t* __restrict__ karrived) {
+                                                          float* __restrict__ kpart, int32_t* __restrict__ karrived,
+                                                          int flags) {
   // K is the extent along k that this workgroup covers and ld the row stride of X and W: with gridDim.y > 1
   // the k range is cut into gridDim.y slices of K elements, one workgroup per (row block, slice); the
   // slices' partial sums meet in `kpart` and the slice that delivers last adds them up in slice order.
@@ -169,7 +170,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
     // Walking both at the same k makes the two streams evict each other's open page, so the up rows walk
     // half a row ahead (XS = 2 sets of X fragments, one per k position).
     constexpr int XS = (MODE == 1 && !GUARD && NB == 1) ? 2 : 1;
-    const int64_t up_shift = (XS == 2 && pairs % GV_WAVES == 0) ? ((pairs / 2) & ~(int64_t)(GV_WAVES - 1)) : 0;
+    const int64_t up_shift = (XS == 2 && pairs % GV_WAVES == 0 && !(flags & 1)) ? ((pairs / 2) & ~(int64_t)(GV_WAVES - 1)) : 0;
     bf16x8_t a_cur[D][R][2], b_cur[D][XS][NB][2];
     // GUARD: K is not a multiple of 64, the last pair is partly (or half) past the end of the rows
     auto load_set = [&](int64_t pq0, bf16x8_t (&a)[D][R][2], bf16x8_t (&b)[D][XS][NB][2]) {
@@ -519,6 +520,9 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   const int NB = B > 16 ? 2 : 1;
   int rot_mul = 1;
   if (const char* e = getenv("MTP_GEMV_ROT")) rot_mul = atoi(e);
+  if (rot_mul < 0) rot_mul = 0;   // the rotation is taken modulo the number of pairs: it must not go negative
+  int flags = 0;                  // bit 0: SwiGLU up rows walk in step with the gate rows (measurement only)
+  if (const char* e = getenv("MTP_GEMV_NOSHIFT")) flags |= atoi(e) ? 1 : 0;
   // k slices: counters first (one per row block, zero between launches), then the partial sums
   const int S = workspace ? cfg.S : 1;
   int32_t* karrived = static_cast<int32_t*>(workspace);
@@ -528,7 +532,7 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD, (RR >= 8 ? 4 : 8)>), dim3(n_wg, S),                    \
                      dim3((RR >= 8 ? 4 : 8) * MTP_WAVE), 0, s,                                                  \
                      (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part, (int)B, \
-                     N, k_slice, rot_mul, K, kpart, karrived)
+                     N, k_slice, rot_mul, K, kpart, karrived, flags)
 #define GV_BY_DEPTH(RR, NNB)                                                   \
   do {                                                                         \
     if (K % 64 != 0) GV_LAUNCH(RR, NNB, true, 1);                              \

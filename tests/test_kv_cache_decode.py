@@ -277,3 +277,16 @@ def test_block_step_vs_oracle_llama8b_shape(gpu):
     assert rel(out, ref_x) < 2 * TOL_BF16
     for b in range(B):
         assert rel(kc[b, :, int(pos[b])], kf[b, :, int(pos[b])]) < TOL_BF16
+
+
+def test_negative_rotation_knobs_are_clamped(gpu, monkeypatch):
+    """The measurement knobs that rotate the walk order are taken modulo a count on the device: negative values
+    from the environment are clamped on the host (they used to turn into negative offsets)."""
+    monkeypatch.setenv("MTP_GEMV_ROT", "-3")
+    monkeypatch.setenv("MTP_ATTN_ROT", "-5")
+    g = gen(12)
+    x = torch.randn(4, 1024, generator=g).bfloat16()
+    w = (torch.randn(512, 1024, generator=g) * 0.05).bfloat16()
+    assert rel(ops.gemv(x.to(gpu), w.to(gpu)), torch.nn.functional.linear(x.float(), w.float())) < TOL_BF16
+    q, kc, vc, dl, ref = _attn_case(gpu, 2, 8, 2, 512, [512, 100], seed=12)
+    assert rel(ops.attn_decode(q, kc, vc, dl), ref) < TOL_BF16

@@ -219,6 +219,23 @@ def kv_cache_decode(dev, timer, reps, table):
         by = wbytes + 2.0 * layers * B * n_kv * L * d * 2
         res[f"model_B{B}_L{L}"] = {"ms_per_token_step": round(ms, 3), "tokens_per_s": round(B / ms * 1e3, 1),
                                    "GBs": round(by / ms / 1e6, 1), "frac_hbm_peak": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        if B == 1:
+            # host wall clock per token, launches from Python against one HIP graph replay
+            def wall(n=20):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n):
+                    one()
+                torch.cuda.synchronize()
+                return (time.perf_counter() - t0) / n * 1e3
+            eager_ms = wall()
+            dec.lens.fill_(L)
+            dec.host_len_bound = L
+            dec.capture()
+            graph_ms = wall()
+            res[f"model_B{B}_L{L}"].update({"wall_ms_python_launches": round(eager_ms, 3),
+                                            "wall_ms_hip_graph": round(graph_ms, 3),
+                                            "tokens_per_s_hip_graph_wall": round(B / graph_ms * 1e3, 1)})
         del dec
     return res
 

@@ -114,20 +114,16 @@ class LlamaDecoder:
         self.lens.zero_()
         self.host_len_bound = 0
 
-    def hidden(self, tokens: torch.Tensor) -> torch.Tensor:
-        """Appends ``tokens`` (int64 [batch]) and returns the final-norm output [batch, H] of their position."""
-        if self.host_len_bound >= self.max_len:
-            raise RuntimeError(f"key/value cache full ({self.max_len} positions)")
+    def _hidden(self, tokens: torch.Tensor, len_bound: int) -> torch.Tensor:
         positions = self.lens             # tokens cached so far = position of the new one
-        self.host_len_bound += 1
         x = ops.embedding_gather(tokens, self.embed, 0, self.embed.shape[0])
         residual = None
         B = x.shape[0]
         for w, kc, vc in zip(self.blocks, self.k_cache, self.v_cache):
             h, residual = ops.rmsnorm(x, w.input_norm, self.eps, residual, want_residual=True)
             qkv = ops.gemv(h, w.qkv, workspace=self.gemv_ws)
-            a = ops.attn_decode_append(qkv, self.cos, self.sin, positions, kc, vc, self.n_q,
-                                       len_bound=self.host_len_bound, workspace=self.attn_ws)
+            a = ops.attn_decode_append(qkv, self.cos, self.sin, positions, kc, vc, self.n_q, len_bound=len_bound,
+                                       workspace=self.attn_ws)
             o = ops.gemv(a.view(B, -1), w.o, workspace=self.gemv_ws)
             h, residual = ops.rmsnorm(o, w.post_norm, self.eps, residual, want_residual=True)
             act = ops.gemv(h, w.gate_up, None, ops.EPI_SWIGLU, workspace=self.gemv_ws)
@@ -135,10 +131,46 @@ class LlamaDecoder:
         self.lens += 1
         return ops.rmsnorm(x, self.final_norm, self.eps, residual)
 
+    def capture(self):
+        """Records one step (all blocks, final norm, LM head with argmax) into a HIP graph; ``hidden`` / ``logits``
+        / ``step`` replay it from then on, which takes the ~230 launches of a step off the Python path.
+        Sequence lengths live on the device, so the same graph serves every later position; the attention is
+        recorded with the split count of a full cache."""
+        dev = self.lm_head.device
+        self._tokens_in = torch.zeros((self.batch,), dtype=torch.int64, device=dev)
+        saved = self.lens.clone()
+        cur = torch.cuda.current_stream(dev)
+        side = torch.cuda.Stream(dev)
+        side.wait_stream(cur)
+        with torch.cuda.stream(side):       # two real steps first (they write cache rows that later tokens overwrite)
+            for _ in range(2):
+                greedy_next_token(self._hidden(self._tokens_in, self.max_len), self.lm_head, self.argmax_ws)
+            self.lens.copy_(saved)
+        cur.wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self._hidden_out = self._hidden(self._tokens_in, self.max_len)
+            self._token_out = greedy_next_token(self._hidden_out, self.lm_head, self.argmax_ws)
+        self._graph = graph
+
+    def hidden(self, tokens: torch.Tensor) -> torch.Tensor:
+        """Appends ``tokens`` (int64 [batch]) and returns the final-norm output [batch, H] of their position."""
+        if self.host_len_bound >= self.max_len:
+            raise RuntimeError(f"key/value cache full ({self.max_len} positions)")
+        self.host_len_bound += 1
+        if getattr(self, "_graph", None) is not None:
+            self._tokens_in.copy_(tokens)
+            self._graph.replay()
+            return self._hidden_out
+        return self._hidden(tokens, self.host_len_bound)
+
     def logits(self, tokens: torch.Tensor) -> torch.Tensor:
         """The row the reference slices out at :223 (fp32 accumulation, model dtype)."""
         return ops.gemv(self.hidden(tokens), self.lm_head, workspace=self.gemv_ws)
 
     def step(self, tokens: torch.Tensor) -> torch.Tensor:
         """Greedy next token per sequence (:226-227); the [batch, vocab] logits are never written."""
-        return greedy_next_token(self.hidden(tokens), self.lm_head, self.argmax_ws)
+        h = self.hidden(tokens)
+        if getattr(self, "_graph", None) is not None:
+            return self._token_out.clone()
+        return greedy_next_token(h, self.lm_head, self.argmax_ws)

@@ -536,6 +536,48 @@ def test_module_surface_on_gpu(gpu):
     assert empty.shape == (0, 64)
 
 
+def test_modules_cast_to_bf16_after_construction(gpu):
+    """The reference builds its parameters in fp32 (or fp16) and turns the model to bf16 afterwards with
+    ``module.bfloat16()`` (amp_engine.py:130-139, pipeline/module.py:189-190): the layers, embedding and loss
+    must work on parameters that changed dtype after the constructor ran."""
+    set_args(use_cpu_initialization=True, params_dtype=torch.float32)
+    torch.manual_seed(3)
+    init = lambda t: torch.nn.init.normal_(t, 0.0, 0.02)
+
+    class Tiny(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.emb = mpu.VocabParallelEmbedding(300, 128, init_method=init)
+            self.col = mpu.ColumnParallelLinear(128, 512, gather_output=False, init_method=init)
+            self.row = mpu.RowParallelLinear(512, 128, input_is_parallel=True, init_method=init)
+            self.head = mpu.ColumnParallelLinear(128, 300, bias=False, gather_output=False, init_method=init)
+
+        def forward(self, ids, labels):
+            h = self.emb(ids)
+            h = h + self.row(F.gelu(self.col(h)[0], approximate="tanh"))[0]
+            return mpu.vocab_parallel_cross_entropy(self.head(h)[0], labels).mean()
+
+    m = Tiny()
+    assert m.col.weight.dtype == torch.float32
+    ref = {k: v.detach().clone() for k, v in m.state_dict().items()}
+    m = m.to(gpu).bfloat16()
+    assert all(p.dtype == torch.bfloat16 and p.is_cuda for p in m.parameters())
+    ids = torch.randint(0, 300, (4, 9), generator=gen(81))
+    labels = torch.randint(0, 300, (4, 9), generator=gen(82))
+    loss = m(ids.to(gpu), labels.to(gpu))
+    loss.backward()
+    # stock torch on the bf16-rounded weights, fp32 arithmetic
+    w = {k: v.bfloat16().float().requires_grad_(True) for k, v in ref.items()}
+    h = F.embedding(ids, w["emb.weight"])
+    h = h + F.linear(F.gelu(F.linear(h, w["col.weight"], w["col.bias"]), approximate="tanh"), w["row.weight"], w["row.bias"])
+    want = F.cross_entropy(F.linear(h, w["head.weight"]).view(-1, 300), labels.view(-1))
+    want.backward()
+    assert abs(loss.item() - want.item()) < 2e-2 * abs(want.item())
+    for name, p_ in m.named_parameters():
+        assert p_.grad is not None and p_.grad.dtype == torch.bfloat16, name
+        assert rel(p_.grad, w[name].grad) < 3 * TOL_BF16, name          # bf16 activations through three layers
+
+
 # =============================================================================== decode
 @pytest.mark.parametrize("b,n,k", [(1, 64, 256), (8, 1000, 512), (32, 4096, 1024), (5, 130, 4104), (17, 77, 40),
                                     (32, 6144, 4096), (8, 4096, 14336)])

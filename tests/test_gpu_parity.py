@@ -898,3 +898,31 @@ def test_tagged_model_rebuilt_onto_the_gfx950_layers(gpu):
     assert rel(out, ref) < TOL_F32 and rel(xg.grad, xs.grad) < TOL_F32
     assert rel(mine.fc_in.weight.grad, stock.fc_in.weight.grad) < TOL_F32
     assert rel(mine.fc_out.bias.grad, stock.fc_out.bias.grad) < TOL_F32
+
+
+def test_greedy_pick_over_a_vocab_sharded_lm_head(gpu):
+    """Eight ranks' vocab slices of an LM head, each through the fused GEMV + argmax: one (max value, local index)
+    pair per row and rank, combined on the host the way an all-gather would allow (largest value, lowest rank on
+    equality), gives the full head's pick."""
+    g = gen(77)
+    B, V, K, p = 8, 8 * 1003, 512, 8
+    x = torch.randn(B, K, generator=g).bfloat16()
+    w = (torch.randn(V, K, generator=g) * 0.05).bfloat16()
+    w[5000] = w[1200]                                            # an exact tie across two ranks' slices
+    x[3] = (w[1200].float() * 4).bfloat16()                      # row 3 picks the tied rows
+    full_idx, full_val = ops.gemv_argmax(x.to(gpu), w.to(gpu))
+    vals, idxs = [], []
+    for r in range(p):
+        lo, hi = R.vocab_range_from_global_vocab_size(V, r, p)
+        i, v = ops.gemv_argmax(x.to(gpu), w[lo:hi].contiguous().to(gpu))
+        vals.append(v.cpu())
+        idxs.append(i.cpu() + lo)
+    vals, idxs = torch.stack(vals), torch.stack(idxs)            # [ranks, B]
+    win = vals.argmax(0)                                         # first (lowest) rank among equal maxima
+    got = idxs[win, torch.arange(B)]
+    ref = R.greedy_argmax(F.linear(x.float(), w.float()))
+    clear = torch.ones(B, dtype=torch.bool)
+    clear[3] = False
+    assert torch.equal(got[clear], ref[clear]) and torch.equal(full_idx.cpu()[clear], ref[clear])
+    assert int(got[3]) in (1200, 5000) and int(ref[3]) == 1200   # the tie: equal to rounding across workgroups
+    assert torch.allclose(vals.max(0).values, full_val.cpu(), rtol=1e-5)

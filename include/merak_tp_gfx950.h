@@ -27,9 +27,13 @@ extern "C" {
 
 #define MTP_ABI_VERSION 3
 
-/* element types */
+/* element types.  MTP_F16 (IEEE half, what the reference's --fp16 sets as
+ * params_dtype, Merak/merak_args/args.py:584-585) is taken by the linear
+ * layers, the activation backward, the embedding and the cross entropy
+ * entry points; the decode entry points take bf16 (and f32 where stated). */
 #define MTP_F32  0
 #define MTP_BF16 1
+#define MTP_F16  2
 
 /* error codes */
 #define MTP_OK            0
@@ -54,8 +58,8 @@ int mtp_device_arch(char* buf, int len);
 
 /* ------------------------------------------------------------------------
  * Linear layers.  All matrices are row-major and dense (leading dimension
- * = number of columns).  dtype is the element type of X, W, Y, dY, dX and
- * bias; accumulation is always fp32.
+ * = number of columns).  dtype (f32, bf16 or f16) is the element type of X,
+ * W, Y, dY, dX and bias; accumulation is always fp32.
  * ------------------------------------------------------------------------ */
 
 /* Y[M,N] = X[M,K] W[N,K]^T (+ bias[N]) with an optional fused activation.
@@ -85,7 +89,7 @@ int mtp_linear_dgrad(const void* dy, const void* w, void* dx,
 
 /* dW[N,K] (+)= dY[M,N]^T X[M,K]; db[N] (+)= sum_m dY[m,:]  — the weight and
  * bias gradients of F.linear.  dw_dtype selects the element type of dW and
- * db (MTP_F32 lets the caller keep an fp32 main gradient); accumulate != 0
+ * db: dtype itself, or MTP_F32 (an fp32 main gradient); accumulate != 0
  * adds into the existing contents instead of overwriting.  db may be NULL. */
 int mtp_linear_wgrad(const void* dy, const void* x, void* dw, void* db,
                      int64_t M, int64_t N, int64_t K,
@@ -115,8 +119,8 @@ int mtp_embedding_gather(const int64_t* ids, const void* table, void* out,
                          int32_t* oob_count, void* stream);
 
 /* Dense gradient of the lookup: dtable[ids[i]-vocab_start,:] += dout[i,:]
- * for in-range ids; dtable is [rows,dim] of dtable_dtype (fp32, or bf16 for
- * bf16 dout).  This is the embedding_dense_backward ATen runs behind
+ * for in-range ids; dtable is [rows,dim] of dtable_dtype (fp32, or the
+ * 16-bit dtype of dout).  This is the embedding_dense_backward ATen runs behind
  * F.embedding (layers.py:156).  Tokens that share an id are summed in
  * ascending token order in fp32 and added to the table row once, so the
  * result is reproducible bit for bit.  The caller zeroes dtable first unless

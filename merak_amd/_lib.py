@@ -17,7 +17,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmerak_tp_gfx950.so"
 
-MTP_F32, MTP_BF16 = 0, 1
+MTP_F32, MTP_BF16, MTP_F16 = 0, 1, 2
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_SWIGLU, EPI_GELU = 0, 1, 2, 3, 4
 ABI_VERSION = 3
 

@@ -6,7 +6,7 @@
 namespace {
 
 // ---- activation backward ---------------------------------------------------
-// T = float or uint16_t (bf16 bits); one thread handles one 16-byte vector.
+// T = float, uint16_t (bf16 bits) or f16s (IEEE half bits); one thread handles one 16-byte vector.
 template <typename T> struct Io;
 template <> struct Io<float> {
   static constexpr int EPV = 4;
@@ -32,6 +32,20 @@ template <> struct Io<uint16_t> {
   }
   __device__ static __forceinline__ float ld(const uint16_t* p) { return bf16_bits_to_f32(*p); }
   __device__ static __forceinline__ void st(uint16_t* p, float v) { *p = f32_to_bf16_bits(v); }
+};
+
+template <> struct Io<f16s> {
+  static constexpr int EPV = 8;
+  using H = X16<true>;
+  __device__ static __forceinline__ void unpack(const u32x4_t& v, float* f) {
+    f[0] = H::lo(v.x); f[1] = H::hi(v.x); f[2] = H::lo(v.y); f[3] = H::hi(v.y);
+    f[4] = H::lo(v.z); f[5] = H::hi(v.z); f[6] = H::lo(v.w); f[7] = H::hi(v.w);
+  }
+  __device__ static __forceinline__ u32x4_t pack(const float* f) {
+    return u32x4_t{H::pack2(f[0], f[1]), H::pack2(f[2], f[3]), H::pack2(f[4], f[5]), H::pack2(f[6], f[7])};
+  }
+  __device__ static __forceinline__ float ld(const f16s* p) { return H::from_bits(p->bits); }
+  __device__ static __forceinline__ void st(f16s* p, float v) { p->bits = H::to_bits(v); }
 };
 
 template <typename T>
@@ -170,7 +184,8 @@ unsigned grid_for(int64_t work_items) {
 extern "C" int mtp_activation_bwd(const void* dact, const void* y, void* dy, int64_t M, int64_t N, int dtype,
                                   int epilogue, void* stream) {
   MTP_REQUIRE(M >= 0 && N >= 1, MTP_EINVAL, "activation_bwd: M=%lld N=%lld", (long long)M, (long long)N);
-  MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16, MTP_EINVAL, "activation_bwd: unknown dtype %d", dtype);
+  MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16 || dtype == MTP_F16, MTP_EINVAL, "activation_bwd: unknown dtype %d",
+              dtype);
   if (M == 0) return MTP_OK;
   MTP_REQUIRE(dact && y && dy, MTP_EINVAL, "activation_bwd: null pointer");
   hipStream_t s = (hipStream_t)stream;
@@ -181,6 +196,9 @@ extern "C" int mtp_activation_bwd(const void* dact, const void* y, void* dy, int
     if (dtype == MTP_F32)
       hipLaunchKernelGGL(gelu_bwd_kernel<float>, dim3(grid_for(n / 4 + 1)), dim3(256), 0, s, (const float*)dact,
                          (const float*)y, (float*)dy, n);
+    else if (dtype == MTP_F16)
+      hipLaunchKernelGGL(gelu_bwd_kernel<f16s>, dim3(grid_for(n / 8 + 1)), dim3(256), 0, s, (const f16s*)dact,
+                         (const f16s*)y, (f16s*)dy, n);
     else
       hipLaunchKernelGGL(gelu_bwd_kernel<uint16_t>, dim3(grid_for(n / 8 + 1)), dim3(256), 0, s,
                          (const uint16_t*)dact, (const uint16_t*)y, (uint16_t*)dy, n);
@@ -197,6 +215,13 @@ extern "C" int mtp_activation_bwd(const void* dact, const void* y, void* dy, int
       else
         hipLaunchKernelGGL((swiglu_bwd_kernel<float, false>), dim3(grid_for(M * H)), dim3(256), 0, s,
                            (const float*)dact, (const float*)y, (float*)dy, M, H);
+    } else if (dtype == MTP_F16) {
+      if (vec)
+        hipLaunchKernelGGL((swiglu_bwd_kernel<f16s, true>), dim3(grid_for(M * H / 8)), dim3(256), 0, s,
+                           (const f16s*)dact, (const f16s*)y, (f16s*)dy, M, H);
+      else
+        hipLaunchKernelGGL((swiglu_bwd_kernel<f16s, false>), dim3(grid_for(M * H)), dim3(256), 0, s,
+                           (const f16s*)dact, (const f16s*)y, (f16s*)dy, M, H);
     } else {
       if (vec)
         hipLaunchKernelGGL((swiglu_bwd_kernel<uint16_t, true>), dim3(grid_for(M * H / 8)), dim3(256), 0, s,

@@ -68,6 +68,14 @@ __global__ __launch_bounds__(256) void embedding_link_kernel(const int64_t* __re
   if (tid == 0) link[i] = TokenLink{first_after == INT32_MAX ? -1 : first_after, dup ? 0 : 1};
 }
 
+// element <-> float for float, uint16_t (bf16 bits) and f16s (IEEE half bits)
+__device__ __forceinline__ float elem_f32(float v) { return v; }
+__device__ __forceinline__ float elem_f32(uint16_t v) { return bf16_bits_to_f32(v); }
+__device__ __forceinline__ float elem_f32(f16s v) { return X16<true>::from_bits(v.bits); }
+__device__ __forceinline__ void elem_set(float* p, float v) { *p = v; }
+__device__ __forceinline__ void elem_set(uint16_t* p, float v) { *p = f32_to_bf16_bits(v); }
+__device__ __forceinline__ void elem_set(f16s* p, float v) { p->bits = X16<true>::to_bits(v); }
+
 template <typename T, typename TO>
 __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t* __restrict__ ids,
                                                             const T* __restrict__ dout, TO* __restrict__ dtable,
@@ -81,20 +89,10 @@ __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t* __res
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   for (int j = i; j >= 0; j = link[j].next) {
     const T* src = dout + (int64_t)j * dim + c0;
-    for (int e = 0; e < nc; e++) {
-      if constexpr (sizeof(T) == 2)
-        acc[e] += bf16_bits_to_f32(src[e]);
-      else
-        acc[e] += src[e];
-    }
+    for (int e = 0; e < nc; e++) acc[e] += elem_f32(src[e]);
   }
   TO* dst = dtable + (ids[i] - vocab_start) * dim + c0;
-  for (int e = 0; e < nc; e++) {
-    if constexpr (sizeof(TO) == 2)
-      dst[e] = f32_to_bf16_bits(bf16_bits_to_f32(dst[e]) + acc[e]);
-    else
-      dst[e] += acc[e];
-  }
+  for (int e = 0; e < nc; e++) elem_set(dst + e, elem_f32(dst[e]) + acc[e]);
 }
 
 template <typename V>
@@ -140,8 +138,9 @@ extern "C" int mtp_embedding_bwd(const int64_t* ids, const void* dout, void* dta
   MTP_REQUIRE(n_ids >= 0 && dim >= 1, MTP_EINVAL, "embedding_bwd: n_ids=%lld dim=%lld", (long long)n_ids,
               (long long)dim);
   MTP_REQUIRE(n_ids < (1ll << 31), MTP_EUNSUPPORTED, "embedding_bwd: n_ids=%lld exceeds 2^31-1", (long long)n_ids);
-  MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16, MTP_EINVAL, "embedding_bwd: unknown dtype %d", dtype);
-  MTP_REQUIRE(dtable_dtype == MTP_F32 || dtable_dtype == MTP_BF16, MTP_EINVAL,
+  MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16 || dtype == MTP_F16, MTP_EINVAL, "embedding_bwd: unknown dtype %d",
+              dtype);
+  MTP_REQUIRE(dtable_dtype == MTP_F32 || dtable_dtype == MTP_BF16 || dtable_dtype == MTP_F16, MTP_EINVAL,
               "embedding_bwd: unknown dtable_dtype %d", dtable_dtype);
   if (n_ids == 0) return MTP_OK;
   MTP_REQUIRE(ids && dout && dtable && workspace, MTP_EINVAL, "embedding_bwd: null pointer");
@@ -166,8 +165,15 @@ extern "C" int mtp_embedding_bwd(const int64_t* ids, const void* dout, void* dta
   else if (dtype == MTP_BF16 && dtable_dtype == MTP_BF16)
     hipLaunchKernelGGL((embedding_bwd_kernel<uint16_t, uint16_t>), grid, block, 0, s, ids, (const uint16_t*)dout,
                        (uint16_t*)dtable, link, dim, vocab_start);
+  else if (dtype == MTP_F16 && dtable_dtype == MTP_F32)
+    hipLaunchKernelGGL((embedding_bwd_kernel<f16s, float>), grid, block, 0, s, ids, (const f16s*)dout, (float*)dtable,
+                       link, dim, vocab_start);
+  else if (dtype == MTP_F16 && dtable_dtype == MTP_F16)
+    hipLaunchKernelGGL((embedding_bwd_kernel<f16s, f16s>), grid, block, 0, s, ids, (const f16s*)dout, (f16s*)dtable,
+                       link, dim, vocab_start);
   else
-    MTP_REQUIRE(false, MTP_EUNSUPPORTED, "embedding_bwd: fp32 gradients into a bf16 table are not supported");
+    MTP_REQUIRE(false, MTP_EUNSUPPORTED, "embedding_bwd: the table gradient is fp32 or of the dtype of dout (%d -> %d)",
+                dtype, dtable_dtype);
   MTP_CHECK_LAUNCH("embedding_bwd");
   return MTP_OK;
 }

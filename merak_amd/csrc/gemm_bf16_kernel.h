@@ -294,8 +294,9 @@ template <int ROWS, int NW> struct OperandOf<LAY_COL, ROWS, NW> { using type = C
 
 // The body lives in a __device__ function: it uses inline assembly operands that the host pass over a
 // __global__ function would trip on.
-template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT, int NW>
+template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16>
 __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
+  using X = X16<F16>;   // element type of A, B, bias and the 16-bit outputs: bf16 or IEEE half
   static_assert(EPI != MTP_EPI_SWIGLU || BLAY == LAY_ROW, "the SwiGLU row interleave is a forward (row B) feature");
   static_assert(NW == 4 || NW == 8, "4 waves (2x2) or 8 waves (2x4) per workgroup");
   constexpr int WGM = 2, WGN = NW / 2;                         // wave grid over the tile
@@ -413,17 +414,10 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   auto mfma_one = [&](int slot, auto t_tag) {  // t-th MFMA of a step in shell order
     constexpr int t = decltype(t_tag)::value;
     constexpr int i = shell_pair(t, TI, TJ).i, j = shell_pair(t, TI, TJ).j;
-    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[slot][j], af[slot][i], acc[i][j], 0, 0, 0);
+    acc[i][j] = X::mfma32(bfr[slot][j], af[slot][i], acc[i][j]);
     if constexpr (EPI == EPI_ROWSUM && t < TI) {
       // the t-th A fragment of this step: 8 k of one row per lane
-      const bf16x8_t a = af[slot][t];
-      const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
-      float r = rsum[t];
-      r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 0, 1), one, r, false);
-      r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 2, 3), one, r, false);
-      r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 4, 5), one, r, false);
-      r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 6, 7), one, r, false);
-      rsum[t] = r;
+      rsum[t] = X::sum8(af[slot][t], rsum[t]);
     }
   };
   auto mfmas = [&](int slot) {
@@ -537,7 +531,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
             *q = p.accumulate ? *q + t : t;
           } else {
             uint16_t* q = (uint16_t*)p.rowsum + row;
-            *q = f32_to_bf16_bits(p.accumulate ? bf16_bits_to_f32(*q) + t : t);
+            *q = X::to_bits(p.accumulate ? X::from_bits(*q) + t : t);
           }
         }
       }
@@ -602,10 +596,10 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
               v.z = __float_as_uint(__uint_as_float(v.z) + __uint_as_float(o.z));
               v.w = __float_as_uint(__uint_as_float(v.w) + __uint_as_float(o.w));
             } else {
-              v.x = pack_bf16x2(bf16_lo(v.x) + bf16_lo(o.x), bf16_hi(v.x) + bf16_hi(o.x));
-              v.y = pack_bf16x2(bf16_lo(v.y) + bf16_lo(o.y), bf16_hi(v.y) + bf16_hi(o.y));
-              v.z = pack_bf16x2(bf16_lo(v.z) + bf16_lo(o.z), bf16_hi(v.z) + bf16_hi(o.z));
-              v.w = pack_bf16x2(bf16_lo(v.w) + bf16_lo(o.w), bf16_hi(v.w) + bf16_hi(o.w));
+              v.x = X::pack2(X::lo(v.x) + X::lo(o.x), X::hi(v.x) + X::hi(o.x));
+              v.y = X::pack2(X::lo(v.y) + X::lo(o.y), X::hi(v.y) + X::hi(o.y));
+              v.z = X::pack2(X::lo(v.z) + X::lo(o.z), X::hi(v.z) + X::hi(o.z));
+              v.w = X::pack2(X::lo(v.w) + X::lo(o.w), X::hi(v.w) + X::hi(o.w));
             }
           }
           __builtin_nontemporal_store(v, q);  // written once, read by a later kernel: keep it out of the way of A/B in L2
@@ -638,10 +632,10 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
               v.z = __float_as_uint(__uint_as_float(v.z) + __uint_as_float(o.z));
               v.w = __float_as_uint(__uint_as_float(v.w) + __uint_as_float(o.w));
             } else {
-              v.x = pack_bf16x2(bf16_lo(v.x) + bf16_lo(o.x), bf16_hi(v.x) + bf16_hi(o.x));
-              v.y = pack_bf16x2(bf16_lo(v.y) + bf16_lo(o.y), bf16_hi(v.y) + bf16_hi(o.y));
-              v.z = pack_bf16x2(bf16_lo(v.z) + bf16_lo(o.z), bf16_hi(v.z) + bf16_hi(o.z));
-              v.w = pack_bf16x2(bf16_lo(v.w) + bf16_lo(o.w), bf16_hi(v.w) + bf16_hi(o.w));
+              v.x = X::pack2(X::lo(v.x) + X::lo(o.x), X::hi(v.x) + X::hi(o.x));
+              v.y = X::pack2(X::lo(v.y) + X::lo(o.y), X::hi(v.y) + X::hi(o.y));
+              v.z = X::pack2(X::lo(v.z) + X::lo(o.z), X::hi(v.z) + X::hi(o.z));
+              v.w = X::pack2(X::lo(v.w) + X::lo(o.w), X::hi(v.w) + X::hi(o.w));
             }
           }
           *reinterpret_cast<u32x4_t*>(gp) = v;
@@ -656,8 +650,8 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
             } else {
               uint16_t* q = reinterpret_cast<uint16_t*>(gp) + e;
               const uint32_t pr = w4[e >> 1];
-              const float nv = (e & 1) ? bf16_hi(pr) : bf16_lo(pr);
-              *q = f32_to_bf16_bits(accumulate ? bf16_bits_to_f32(*q) + nv : nv);
+              const float nv = (e & 1) ? X::hi(pr) : X::lo(pr);
+              *q = X::to_bits(accumulate ? X::from_bits(*q) + nv : nv);
             }
           }
         }
@@ -680,7 +674,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
               const int col = cb + 8 * g + 4 * lh + e;
-              b4[e] = col < lim_of_block(j) ? bf16_bits_to_f32(p.bias[col]) : 0.f;
+              b4[e] = col < lim_of_block(j) ? X::from_bits(p.bias[col]) : 0.f;
             }
           }
         }
@@ -708,7 +702,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
 #pragma unroll
       for (int j = 0; j < TJ; j++)
 #pragma unroll
-        for (int q = 0; q < 8; q++) pk[j][q] = pack_bf16x2(pre[j][2 * q], pre[j][2 * q + 1]);
+        for (int q = 0; q < 8; q++) pk[j][q] = X::pack2(pre[j][2 * q], pre[j][2 * q + 1]);
       if (p.C) {
 #pragma unroll
         for (int j = 0; j < TJ; j++)
@@ -726,8 +720,8 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
         for (int j = 0; j < TJ; j++)
 #pragma unroll
           for (int q = 0; q < 8; q++) {
-            pre[j][2 * q] = bf16_lo(pk[j][q]);
-            pre[j][2 * q + 1] = bf16_hi(pk[j][q]);
+            pre[j][2 * q] = X::lo(pk[j][q]);
+            pre[j][2 * q + 1] = X::hi(pk[j][q]);
           }
       }
       if constexpr (EPI == MTP_EPI_BIAS_GELU || EPI == MTP_EPI_GELU) {
@@ -735,8 +729,8 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
         for (int j = 0; j < TJ; j++)
 #pragma unroll
           for (int g = 0; g < 4; g++) {
-            u32x2_t v = {pack_bf16x2(gelu_new_f(pre[j][4 * g]), gelu_new_f(pre[j][4 * g + 1])),
-                         pack_bf16x2(gelu_new_f(pre[j][4 * g + 2]), gelu_new_f(pre[j][4 * g + 3]))};
+            u32x2_t v = {X::pack2(gelu_new_f(pre[j][4 * g]), gelu_new_f(pre[j][4 * g + 1])),
+                         X::pack2(gelu_new_f(pre[j][4 * g + 2]), gelu_new_f(pre[j][4 * g + 3]))};
             *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
           }
         wave_lds_sync();
@@ -752,7 +746,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
             float a4[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) a4[e] = silu_f(pre[j][4 * g + e]) * pre[j + HJ][4 * g + e];
-            u32x2_t v = {pack_bf16x2(a4[0], a4[1]), pack_bf16x2(a4[2], a4[3])};
+            u32x2_t v = {X::pack2(a4[0], a4[1]), X::pack2(a4[2], a4[3])};
             *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
           }
         wave_lds_sync();
@@ -765,9 +759,9 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   }
 }
 
-template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT, int NW>
+template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16>
 __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs p) {
-  gemm_bf16_body<BM, BN, ALAY, BLAY, EPI, OUT, NW>(p);
+  gemm_bf16_body<BM, BN, ALAY, BLAY, EPI, OUT, NW, F16>(p);
 }
 
 // ---------------------------------------------------------------------------
@@ -829,7 +823,7 @@ int pick_config(const GemmArgs& a) {
   return best;
 }
 
-template <int C, int ALAY, int BLAY, int EPI, int OUT>
+template <int C, int ALAY, int BLAY, int EPI, int OUT, bool F16>
 int launch_cfg(const GemmArgs& a, hipStream_t s) {
   if constexpr (!cfg_valid<EPI>(C)) {
     mtp_set_error("gemm_bf16: tile configuration %d cannot serve this epilogue", C);
@@ -840,27 +834,33 @@ int launch_cfg(const GemmArgs& a, hipStream_t s) {
     const int span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
     const int bn_span = (EPI == MTP_EPI_SWIGLU) ? BN / 2 : BN;
     const int tiles_n = (span + bn_span - 1) / bn_span;
-    hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, NW>), dim3((unsigned)(tiles_m * tiles_n)),
+    hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, NW, F16>), dim3((unsigned)(tiles_m * tiles_n)),
                        dim3(NW * 64), 0, s, a);
     MTP_CHECK_LAUNCH("gemm_bf16");
     return MTP_OK;
   }
 }
 
-template <int ALAY, int BLAY, int EPI, int OUT>
-int launch(GemmArgs a, hipStream_t s) {
+template <int ALAY, int BLAY, int EPI, int OUT, bool F16>
+int launch_typed(GemmArgs a, hipStream_t s) {
   if (const char* e = getenv("MTP_GEMM_DEBUG")) a.debug = atoi(e);
   int c = pick_config<EPI>(a);
   if (!cfg_valid<EPI>(c)) c = 0;
   switch (c) {
-    case 0: return launch_cfg<0, ALAY, BLAY, EPI, OUT>(a, s);
-    case 1: return launch_cfg<1, ALAY, BLAY, EPI, OUT>(a, s);
-    case 2: return launch_cfg<2, ALAY, BLAY, EPI, OUT>(a, s);
-    case 3: return launch_cfg<3, ALAY, BLAY, EPI, OUT>(a, s);
-    case 4: return launch_cfg<4, ALAY, BLAY, EPI, OUT>(a, s);
-    case 5: return launch_cfg<5, ALAY, BLAY, EPI, OUT>(a, s);
+    case 0: return launch_cfg<0, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 1: return launch_cfg<1, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 2: return launch_cfg<2, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 3: return launch_cfg<3, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 4: return launch_cfg<4, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 5: return launch_cfg<5, ALAY, BLAY, EPI, OUT, F16>(a, s);
   }
   return MTP_EINVAL;
+}
+
+// f16 != 0: the 16-bit tensors (A, B, bias, and C / C2 / rowsum unless OUT_F32) are IEEE half instead of bf16
+template <int ALAY, int BLAY, int EPI, int OUT>
+int launch(const GemmArgs& a, hipStream_t s, int f16) {
+  return f16 ? launch_typed<ALAY, BLAY, EPI, OUT, true>(a, s) : launch_typed<ALAY, BLAY, EPI, OUT, false>(a, s);
 }
 
 }  // namespace

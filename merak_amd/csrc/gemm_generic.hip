@@ -33,9 +33,11 @@ struct GenArgs {
 template <typename T> __device__ __forceinline__ float ld_elem(const T* p);
 template <> __device__ __forceinline__ float ld_elem<float>(const float* p) { return *p; }
 template <> __device__ __forceinline__ float ld_elem<uint16_t>(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+template <> __device__ __forceinline__ float ld_elem<f16s>(const f16s* p) { return X16<true>::from_bits(p->bits); }
 template <typename T> __device__ __forceinline__ void st_elem(T* p, float v);
 template <> __device__ __forceinline__ void st_elem<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void st_elem<uint16_t>(uint16_t* p, float v) { *p = f32_to_bf16_bits(v); }
+template <> __device__ __forceinline__ void st_elem<f16s>(f16s* p, float v) { p->bits = X16<true>::to_bits(v); }
 
 // Each thread stages 8 elements of the A tile and 8 of the B tile per k-tile:
 // tile = 128 rows x 16 k = 2048 elements / 256 threads.
@@ -205,7 +207,7 @@ int launch_generic(const GenArgs& a, hipStream_t s) {
 
 }  // namespace
 
-// dtype/out_dtype: MTP_F32 or MTP_BF16
+// dtype: MTP_F32, MTP_BF16 or MTP_F16; out_dtype: the same or MTP_F32
 int mtp_gemm_generic(const void* A, int64_t sam, int64_t sak, const void* B, int64_t sbn, int64_t sbk,
                      const void* bias, void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, int out_dtype,
                      int accumulate, hipStream_t s) {
@@ -217,6 +219,8 @@ int mtp_gemm_generic(const void* A, int64_t sam, int64_t sak, const void* B, int
   if (dtype == MTP_F32 && out_dtype == MTP_F32) return launch_generic<float, float>(a, s);
   if (dtype == MTP_BF16 && out_dtype == MTP_BF16) return launch_generic<uint16_t, uint16_t>(a, s);
   if (dtype == MTP_BF16 && out_dtype == MTP_F32) return launch_generic<uint16_t, float>(a, s);
+  if (dtype == MTP_F16 && out_dtype == MTP_F16) return launch_generic<f16s, f16s>(a, s);
+  if (dtype == MTP_F16 && out_dtype == MTP_F32) return launch_generic<f16s, float>(a, s);
   mtp_set_error("gemm_generic: dtype %d -> %d not supported", dtype, out_dtype);
   return MTP_EUNSUPPORTED;
 }
@@ -230,6 +234,12 @@ int mtp_colsum(const void* dy, void* db, int64_t M, int64_t N, int dtype, int ou
   else if (dtype == MTP_BF16 && out_dtype == MTP_BF16)
     hipLaunchKernelGGL((colsum_kernel<uint16_t, uint16_t>), dim3(blocks), dim3(256), 0, s, (const uint16_t*)dy,
                        (uint16_t*)db, (int)M, (int)N, accumulate);
+  else if (dtype == MTP_F16 && out_dtype == MTP_F16)
+    hipLaunchKernelGGL((colsum_kernel<f16s, f16s>), dim3(blocks), dim3(256), 0, s, (const f16s*)dy, (f16s*)db, (int)M,
+                       (int)N, accumulate);
+  else if (dtype == MTP_F16 && out_dtype == MTP_F32)
+    hipLaunchKernelGGL((colsum_kernel<f16s, float>), dim3(blocks), dim3(256), 0, s, (const f16s*)dy, (float*)db, (int)M,
+                       (int)N, accumulate);
   else if (dtype == MTP_BF16 && out_dtype == MTP_F32)
     hipLaunchKernelGGL((colsum_kernel<uint16_t, float>), dim3(blocks), dim3(256), 0, s, (const uint16_t*)dy,
                        (float*)db, (int)M, (int)N, accumulate);
@@ -249,6 +259,9 @@ int mtp_act_fwd(const void* y, void* act, int64_t M, int64_t N, int dtype, int s
   if (dtype == MTP_F32)
     hipLaunchKernelGGL(act_fwd_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, s, (const float*)y, (float*)act,
                        M, N, swiglu);
+  else if (dtype == MTP_F16)
+    hipLaunchKernelGGL(act_fwd_kernel<f16s>, dim3((unsigned)blocks), dim3(256), 0, s, (const f16s*)y, (f16s*)act, M, N,
+                       swiglu);
   else
     hipLaunchKernelGGL(act_fwd_kernel<uint16_t>, dim3((unsigned)blocks), dim3(256), 0, s, (const uint16_t*)y,
                        (uint16_t*)act, M, N, swiglu);

@@ -3,11 +3,13 @@
 // tensors and every bf16 shape the fast kernel does not take.
 #include "mtp_common.h"
 
+// f16 != 0: the 16-bit tensors are IEEE half instead of bf16 (same kernel, other MFMA and conversions)
 int mtp_gemm_bf16_nt(const void* A, const void* B, const void* bias, void* C, void* C2, int64_t M, int64_t N,
-                     int64_t K, int epilogue, hipStream_t s);
-int mtp_gemm_bf16_dgrad(const void* dy, const void* w, void* dx, int64_t M, int64_t N, int64_t K, hipStream_t s);
+                     int64_t K, int epilogue, int f16, hipStream_t s);
+int mtp_gemm_bf16_dgrad(const void* dy, const void* w, void* dx, int64_t M, int64_t N, int64_t K, int f16,
+                        hipStream_t s);
 int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
-                        int dw_dtype, int accumulate, hipStream_t s);
+                        int dw_dtype, int accumulate, int f16, hipStream_t s);
 int mtp_gemm_generic(const void* A, int64_t sam, int64_t sak, const void* B, int64_t sbn, int64_t sbk,
                      const void* bias, void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, int out_dtype,
                      int accumulate, hipStream_t s);
@@ -26,7 +28,8 @@ int check_dims(const char* what, int64_t M, int64_t N, int64_t K, int dtype) {
               (long long)K);
   MTP_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), MTP_EUNSUPPORTED,
               "%s: a dimension exceeds 2^31-1", what);
-  MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16, MTP_EINVAL, "%s: unknown dtype %d", what, dtype);
+  MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16 || dtype == MTP_F16, MTP_EINVAL, "%s: unknown dtype %d", what,
+              dtype);
   return MTP_OK;
 }
 
@@ -62,10 +65,11 @@ extern "C" int mtp_linear_fwd(const void* x, const void* w, const void* bias, vo
   hipStream_t s = (hipStream_t)stream;
   const void* use_bias = (epilogue == MTP_EPI_NONE || epilogue == MTP_EPI_GELU) ? nullptr : bias;
 
-  if (dtype == MTP_BF16 && fast_ok(K, K, x, w) && N * K * 2 < (1ll << 31)) {
+  const bool is16 = dtype == MTP_BF16 || dtype == MTP_F16;
+  if (is16 && fast_ok(K, K, x, w) && N * K * 2 < (1ll << 31)) {
     int epi = epilogue;
     if (epilogue == MTP_EPI_SWIGLU && !use_bias) use_bias = nullptr;
-    return mtp_gemm_bf16_nt(x, w, use_bias, y, act, M, N, K, epi, s);
+    return mtp_gemm_bf16_nt(x, w, use_bias, y, act, M, N, K, epi, dtype == MTP_F16, s);
   }
   if (dtype == MTP_F32 && f32_fast_ok(x, w, K, K, 0, 0) && K * 4 * 128 < (1ll << 31)) {
     void* pre32 = y ? y : (epilogue != MTP_EPI_SWIGLU ? act : nullptr);
@@ -93,8 +97,8 @@ extern "C" int mtp_linear_dgrad(const void* dy, const void* w, void* dx, int64_t
   if (M == 0) return MTP_OK;
   MTP_REQUIRE(dy && w && dx, MTP_EINVAL, "linear_dgrad: null pointer");
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == MTP_BF16 && fast_ok(N, K, dy, w) && aligned16(dx)) {
-    rc = mtp_gemm_bf16_dgrad(dy, w, dx, M, N, K, s);
+  if ((dtype == MTP_BF16 || dtype == MTP_F16) && fast_ok(N, K, dy, w) && aligned16(dx)) {
+    rc = mtp_gemm_bf16_dgrad(dy, w, dx, M, N, K, dtype == MTP_F16, s);
     if (rc != MTP_EUNSUPPORTED) return rc;
   }
   if (dtype == MTP_F32 && f32_fast_ok(dy, w, N, K, 0, N * K * 4) && N * 4 * 128 < (1ll << 31))
@@ -107,14 +111,13 @@ extern "C" int mtp_linear_wgrad(const void* dy, const void* x, void* dw, void* d
                                 int dtype, int dw_dtype, int accumulate, void* stream) {
   int rc = check_dims("linear_wgrad", M, N, K, dtype);
   if (rc) return rc;
-  MTP_REQUIRE(dw_dtype == MTP_F32 || dw_dtype == MTP_BF16, MTP_EINVAL, "linear_wgrad: unknown dw_dtype %d", dw_dtype);
-  MTP_REQUIRE(!(dtype == MTP_F32 && dw_dtype == MTP_BF16), MTP_EUNSUPPORTED,
-              "linear_wgrad: fp32 inputs with bf16 gradients are not supported");
+  MTP_REQUIRE(dw_dtype == MTP_F32 || dw_dtype == dtype, MTP_EUNSUPPORTED,
+              "linear_wgrad: gradients are fp32 or of the inputs' dtype (inputs %d, dw %d)", dtype, dw_dtype);
   MTP_REQUIRE(dw, MTP_EINVAL, "linear_wgrad: null dw");
   MTP_REQUIRE(M == 0 || (dy && x), MTP_EINVAL, "linear_wgrad: null input");
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == MTP_BF16 && M > 0 && fast_ok(N, K, dy, x) && aligned16(dw)) {
-    rc = mtp_gemm_bf16_wgrad(dy, x, dw, db, M, N, K, dw_dtype, accumulate, s);
+  if ((dtype == MTP_BF16 || dtype == MTP_F16) && M > 0 && fast_ok(N, K, dy, x) && aligned16(dw)) {
+    rc = mtp_gemm_bf16_wgrad(dy, x, dw, db, M, N, K, dw_dtype, accumulate, dtype == MTP_F16, s);
     if (rc != MTP_EUNSUPPORTED) return rc;
   }
   if (dtype == MTP_F32 && dw_dtype == MTP_F32 && M > 0 && f32_fast_ok(dy, x, N, K, M * N * 4, M * K * 4)) {

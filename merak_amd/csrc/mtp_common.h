@@ -35,6 +35,56 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return (uint16_t)(pack_bf16x2(f, 0.0f) & 0xffffu); }
 
+// storage type of IEEE half tensors in templates (bf16 tensors travel as uint16_t)
+struct f16s {
+  uint16_t bits;
+};
+
+// ---- the two 16-bit element types of the MFMA kernels: bf16 (F16 = false) and IEEE half (F16 = true) ---------
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+template <bool F16> struct X16;
+template <> struct X16<false> {
+  static __device__ __forceinline__ float lo(uint32_t p) { return bf16_lo(p); }
+  static __device__ __forceinline__ float hi(uint32_t p) { return bf16_hi(p); }
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) { return pack_bf16x2(a, b); }
+  static __device__ __forceinline__ uint16_t to_bits(float f) { return f32_to_bf16_bits(f); }
+  static __device__ __forceinline__ float from_bits(uint16_t b) { return bf16_bits_to_f32(b); }
+  static __device__ __forceinline__ f32x16_t mfma32(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  // r + the sum of the 8 elements of a (v_dot2 against ones)
+  static __device__ __forceinline__ float sum8(bf16x8_t a, float r) {
+    const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
+    r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 0, 1), one, r, false);
+    r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 2, 3), one, r, false);
+    r = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 4, 5), one, r, false);
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 6, 7), one, r, false);
+  }
+};
+template <> struct X16<true> {
+  static __device__ __forceinline__ float lo(uint32_t p) { return (float)__builtin_bit_cast(f16x2_t, p)[0]; }
+  static __device__ __forceinline__ float hi(uint32_t p) { return (float)__builtin_bit_cast(f16x2_t, p)[1]; }
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    const f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));   // round to nearest even
+  }
+  static __device__ __forceinline__ uint16_t to_bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+  static __device__ __forceinline__ float from_bits(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+  static __device__ __forceinline__ f32x16_t mfma32(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0,
+                                                  0);
+  }
+  static __device__ __forceinline__ float sum8(bf16x8_t a, float r) {
+    const f16x8_t h = __builtin_bit_cast(f16x8_t, a);
+    const f16x2_t one = {(_Float16)1.0f, (_Float16)1.0f};
+    r = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 0, 1), one, r, false);
+    r = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 2, 3), one, r, false);
+    r = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 4, 5), one, r, false);
+    return __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 6, 7), one, r, false);
+  }
+};
+
 // ---- wave64 reductions (butterfly over ds_bpermute-free shuffles) ---------
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll

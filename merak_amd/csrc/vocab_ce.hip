@@ -53,6 +53,23 @@ template <> struct Elem<uint16_t> {  // bf16 bits
   }
 };
 
+template <> struct Elem<f16s> {  // IEEE half bits
+  static constexpr int EPV = 8;
+  using H = X16<true>;
+  __device__ static __forceinline__ float ld(const f16s* p) { return H::from_bits(p->bits); }
+  __device__ static __forceinline__ void st(f16s* p, float v) { p->bits = H::to_bits(v); }
+  __device__ static __forceinline__ void unpack(const u32x4_t& v, float* f) {
+    f[0] = H::lo(v.x); f[1] = H::hi(v.x); f[2] = H::lo(v.y); f[3] = H::hi(v.y);
+    f[4] = H::lo(v.z); f[5] = H::hi(v.z); f[6] = H::lo(v.w); f[7] = H::hi(v.w);
+  }
+  __device__ static __forceinline__ u32x4_t pack(const float* f) {
+    u32x4_t v;
+    v.x = H::pack2(f[0], f[1]); v.y = H::pack2(f[2], f[3]);
+    v.z = H::pack2(f[4], f[5]); v.w = H::pack2(f[6], f[7]);
+    return v;
+  }
+};
+
 // Split a row of V elements starting at p into [0,head) scalar, nvec aligned
 // 16-byte vectors, and a scalar tail.
 template <typename T>
@@ -469,6 +486,10 @@ extern "C" int mtp_vocab_ce_fwd(const void* logits, const int64_t* target, float
     MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL, "vocab_ce_fwd: bf16 logits not 2-byte aligned");
     hipLaunchKernelGGL(vocab_ce_fwd_kernel<uint16_t>, grid, block, 0, s, (const uint16_t*)logits, target, loss,
                        row_max, row_sumexp, pred, vocab, vocab_start);
+  } else if (dtype == MTP_F16) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL, "vocab_ce_fwd: fp16 logits not 2-byte aligned");
+    hipLaunchKernelGGL(vocab_ce_fwd_kernel<f16s>, grid, block, 0, s, (const f16s*)logits, target, loss, row_max,
+                       row_sumexp, pred, vocab, vocab_start);
   } else {
     MTP_REQUIRE(false, MTP_EINVAL, "vocab_ce_fwd: unknown dtype %d", dtype);
   }
@@ -496,6 +517,10 @@ extern "C" int mtp_vocab_ce_bwd(void* logits, const int64_t* target, const float
     MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL, "vocab_ce_bwd: bf16 logits not 2-byte aligned");
     hipLaunchKernelGGL(vocab_ce_bwd_kernel<uint16_t>, grid, block, 0, s, (uint16_t*)logits, target, row_max,
                        row_sumexp, grad_out, vocab, vocab_start);
+  } else if (dtype == MTP_F16) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL, "vocab_ce_bwd: fp16 logits not 2-byte aligned");
+    hipLaunchKernelGGL(vocab_ce_bwd_kernel<f16s>, grid, block, 0, s, (f16s*)logits, target, row_max, row_sumexp,
+                       grad_out, vocab, vocab_start);
   } else {
     MTP_REQUIRE(false, MTP_EINVAL, "vocab_ce_bwd: unknown dtype %d", dtype);
   }
@@ -505,7 +530,7 @@ extern "C" int mtp_vocab_ce_bwd(void* logits, const int64_t* target, const float
 
 extern "C" int64_t mtp_vocab_ce_fwd_bwd_max_vocab(int dtype) {
   if (dtype == MTP_F32) return 20ll * FU_THREADS * Elem<float>::EPV;
-  if (dtype == MTP_BF16) return 20ll * FU_THREADS * Elem<uint16_t>::EPV;
+  if (dtype == MTP_BF16 || dtype == MTP_F16) return 20ll * FU_THREADS * Elem<uint16_t>::EPV;
   return 0;
 }
 
@@ -530,6 +555,11 @@ extern "C" int mtp_vocab_ce_fwd_bwd(void* logits, const int64_t* target, const f
                 "vocab_ce_fwd_bwd: bf16 logits not 2-byte aligned");
     rc = dispatch_fused<uint16_t>(logits, target, grad_rows, grad_scale, loss, row_max, row_sumexp, pred, n_rows,
                                   vocab, vocab_start, s);
+  } else if (dtype == MTP_F16) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL,
+                "vocab_ce_fwd_bwd: fp16 logits not 2-byte aligned");
+    rc = dispatch_fused<f16s>(logits, target, grad_rows, grad_scale, loss, row_max, row_sumexp, pred, n_rows, vocab,
+                              vocab_start, s);
   } else {
     MTP_REQUIRE(false, MTP_EINVAL, "vocab_ce_fwd_bwd: unknown dtype %d", dtype);
   }
@@ -555,6 +585,9 @@ extern "C" int mtp_vocab_ce_rescale(void* grad, const float* grad_rows, float as
   } else if (dtype == MTP_BF16) {
     MTP_REQUIRE((reinterpret_cast<uintptr_t>(grad) & 1) == 0, MTP_EINVAL, "vocab_ce_rescale: bf16 buffer not 2-byte aligned");
     hipLaunchKernelGGL(vocab_ce_rescale_kernel<uint16_t>, grid, block, 0, s, (uint16_t*)grad, grad_rows, assumed, vocab);
+  } else if (dtype == MTP_F16) {
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(grad) & 1) == 0, MTP_EINVAL, "vocab_ce_rescale: fp16 buffer not 2-byte aligned");
+    hipLaunchKernelGGL(vocab_ce_rescale_kernel<f16s>, grid, block, 0, s, (f16s*)grad, grad_rows, assumed, vocab);
   } else {
     MTP_REQUIRE(false, MTP_EINVAL, "vocab_ce_rescale: unknown dtype %d", dtype);
   }

@@ -13,9 +13,9 @@ import torch
 
 from . import _lib
 from ._lib import (EPI_BIAS, EPI_BIAS_GELU, EPI_GELU, EPI_NONE, EPI_SWIGLU,
-                   MTP_BF16, MTP_F32)
+                   MTP_BF16, MTP_F16, MTP_F32)
 
-_DTYPES = {torch.float32: MTP_F32, torch.bfloat16: MTP_BF16}
+_DTYPES = {torch.float32: MTP_F32, torch.bfloat16: MTP_BF16, torch.float16: MTP_F16}
 _arch_ok = {}
 
 
@@ -23,7 +23,7 @@ def _dt(t: torch.Tensor) -> int:
     try:
         return _DTYPES[t.dtype]
     except KeyError:
-        raise TypeError(f"merak_amd kernels take float32 or bfloat16 tensors, got {t.dtype}") from None
+        raise TypeError(f"merak_amd kernels take float32, bfloat16 or float16 tensors, got {t.dtype}") from None
 
 
 def _require_gpu(*ts: torch.Tensor) -> torch.device:

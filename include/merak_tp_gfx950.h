@@ -25,12 +25,10 @@
 extern "C" {
 #endif
 
-#define MTP_ABI_VERSION 3
+#define MTP_ABI_VERSION 4
 
-/* element types.  MTP_F16 (IEEE half, what the reference's --fp16 sets as
- * params_dtype, Merak/merak_args/args.py:584-585) is taken by the linear
- * layers, the activation backward, the embedding and the cross entropy
- * entry points; the decode entry points take bf16 (and f32 where stated). */
+/* element types.  MTP_F16 is IEEE half, what the reference's --fp16 sets as
+ * params_dtype (Merak/merak_args/args.py:584-585). */
 #define MTP_F32  0
 #define MTP_BF16 1
 #define MTP_F16  2
@@ -196,13 +194,13 @@ int mtp_vocab_ce_rescale(void* grad, const float* grad_rows, float assumed,
 /* ------------------------------------------------------------------------
  * Decode step (Merak/inference/text_generation_inference.py:223,226-227):
  * a handful of single-token activation rows through a linear layer, and the
- * greedy pick over the LM-head row.  bf16 only, B <= 32, K % 8 == 0.
+ * greedy pick over the LM-head row.  dtype bf16 or f16, B <= 32, K % 8 == 0.
  * ------------------------------------------------------------------------ */
 
 /* Y[B,N] = X[B,K] W[N,K]^T (+bias) ; epilogue NONE, BIAS or SWIGLU
  * (SWIGLU: y is [B,N/2] = silu(gate)*up with W = [gate rows | up rows]). */
 int mtp_gemv(const void* x, const void* w, const void* bias, void* y,
-             int64_t B, int64_t N, int64_t K, int epilogue, void* stream);
+             int64_t B, int64_t N, int64_t K, int epilogue, int dtype, void* stream);
 
 /* mtp_gemv with device scratch.  Matrices with few rows at B > 16 are cut
  * along k into slices that run as separate workgroups (each reads only its
@@ -216,7 +214,7 @@ int mtp_gemv(const void* x, const void* w, const void* bias, void* y,
 int64_t mtp_gemv_workspace_bytes(int64_t B, int64_t N, int64_t K, int epilogue);
 int mtp_gemv_ws(const void* x, const void* w, const void* bias, void* y,
                 void* workspace, int64_t workspace_bytes,
-                int64_t B, int64_t N, int64_t K, int epilogue, void* stream);
+                int64_t B, int64_t N, int64_t K, int epilogue, int dtype, void* stream);
 
 /* Bytes of device scratch mtp_gemv_argmax needs for this shape. */
 int64_t mtp_gemv_argmax_workspace_bytes(int64_t B, int64_t N, int64_t K);
@@ -230,9 +228,9 @@ int64_t mtp_gemv_argmax_workspace_bytes(int64_t B, int64_t N, int64_t K);
 int mtp_gemv_argmax(const void* x, const void* w,
                     int64_t* idx, float* maxval,
                     void* workspace, int64_t workspace_bytes,
-                    int64_t B, int64_t N, int64_t K, void* stream);
+                    int64_t B, int64_t N, int64_t K, int dtype, void* stream);
 
-/* Row-wise argmax of materialised logits [B,V] (dtype f32 or bf16): the
+/* Row-wise argmax of materialised logits [B,V] (dtype f32, bf16 or f16): the
  * literal torch.argmax(logits, dim=-1) of :227. */
 int mtp_argmax_rows(const void* logits, int64_t* idx,
                     int64_t B, int64_t V, int dtype, void* stream);
@@ -246,7 +244,7 @@ int mtp_argmax_rows(const void* logits, int64_t* idx,
  * probability softmax(z kept).  The draw replaces torch.multinomial's private
  * random stream by the caller's uniforms[b] in [0,1): token = first index
  * whose cumulative kept probability, in index order, exceeds uniforms[b].
- * logits: [B,V] f32 or bf16, untouched.  tokens (int64 [B]) and filtered
+ * logits: [B,V] f32, bf16 or f16, untouched.  tokens (int64 [B]) and filtered
  * (f32 [B,V]: z where kept, -inf where dropped, what top_k_logits returns) may
  * each be NULL.  workspace: device scratch of mtp_sample_workspace_bytes(B)
  * bytes, 8-byte aligned (the rows are spread over many workgroups and the
@@ -265,14 +263,14 @@ int mtp_sample_top_k_top_p(const void* logits, int dtype, int64_t B, int64_t V,
  * picked at :223); for a causal model the same row comes from running only
  * the new position against cached keys and values.  These are the pieces
  * of the HF Llama block between the tensor-parallel linears; head_dim is
- * 128, tensors are bf16 unless stated.
+ * 128, dtype is bf16 or f16 (f32 too where stated).
  * ------------------------------------------------------------------------ */
 /* h = x (+ residual, may be NULL), rounded to the tensor dtype;
  * residual_out (may be NULL) = h; y = weight * dtype(h * rsqrt(mean(h^2) +
  * eps)) with the mean and the scaling in fp32 (HF LlamaRMSNorm.forward in
  * front of which the block's `residual + hidden_states` has been folded).
- * x, residual, y, residual_out: [rows, dim]; weight: [dim]; dtype f32 or
- * bf16.  y may alias x; residual_out may alias residual. */
+ * x, residual, y, residual_out: [rows, dim]; weight: [dim]; dtype f32,
+ * bf16 or f16.  y may alias x; residual_out may alias residual. */
 int mtp_rmsnorm(const void* x, const void* residual, const void* weight,
                 void* y, void* residual_out,
                 int64_t rows, int64_t dim, float eps, int dtype, void* stream);
@@ -294,7 +292,7 @@ int mtp_rope_kv_append(const void* qkv, const void* cos_table, const void* sin_t
  * t < lens[b] (int64 [B] on the device, clamped to [0, max_len]; a row with
  * no tokens gives zeros), g = n_q_heads / n_kv_heads <= 16: grouped-query
  * attention of one new position (HF eager attention: fp32 softmax,
- * probabilities rounded to bf16 for the product with V).  len_bound: an
+ * probabilities rounded to the tensor dtype for the product with V).  len_bound: an
  * upper bound of lens known on the host (<= max_len); it only decides over
  * how many workgroups a sequence is split.  workspace: device scratch of
  * mtp_attn_decode_workspace_bytes(B, n_q_heads, n_kv_heads, len_bound)

@@ -62,14 +62,19 @@ struct AttnArgs {
 // x * cos + rotate_half(x) * sin for 8 elements of one head: `own` holds dims d .. d+7, `other` the dims
 // 64 away, sign = -1 for d < 64 (rotate_half = cat(-x[64:], x[:64])).  Every product is rounded to bf16
 // before the sum, and the sum again, as the bf16 tensor expression rounds.
+template <bool F16>
 __device__ __forceinline__ u32x4_t rope8(u32x4_t own, u32x4_t other, u32x4_t c, u32x4_t s, float sign) {
+  using X = X16<F16>;
   u32x4_t r;
 #pragma unroll
   for (int e = 0; e < 4; e++) {
-    const float a0 = bf16_lo(own[e]) * bf16_lo(c[e]), a1 = bf16_hi(own[e]) * bf16_hi(c[e]);
-    const float b0 = sign * bf16_lo(other[e]) * bf16_lo(s[e]), b1 = sign * bf16_hi(other[e]) * bf16_hi(s[e]);
-    const uint32_t pa = pack_bf16x2(a0, a1), pb = pack_bf16x2(b0, b1);
-    r[e] = pack_bf16x2(bf16_lo(pa) + bf16_lo(pb), bf16_hi(pa) + bf16_hi(pb));
+    float a0 = X::lo(own[e]) * X::lo(c[e]), a1 = X::hi(own[e]) * X::hi(c[e]);
+    float b0 = sign * X::lo(other[e]) * X::lo(s[e]), b1 = sign * X::hi(other[e]) * X::hi(s[e]);
+    // the products exist as fp32 values here: with half tensors the compiler otherwise narrows the whole
+    // expression to packed half arithmetic and folds one rounded product into a fused multiply-add
+    asm volatile("" : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1));
+    const uint32_t pa = X::pack2(a0, a1), pb = X::pack2(b0, b1);
+    r[e] = X::pack2(X::lo(pa) + X::lo(pb), X::hi(pa) + X::hi(pb));
   }
   return r;
 }
@@ -102,8 +107,9 @@ __device__ __forceinline__ void wait_vm(int items_after) {
 }
 
 // AD_WAVES waves with AD_RING ring slots each: 32 KiB of LDS per wave with 4 slots, 48 KiB with 6
-template <bool APPEND, int AD_WAVES, int AD_RING, bool NT>
+template <bool APPEND, int AD_WAVES, int AD_RING, bool NT, bool F16>
 __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
+  using X = X16<F16>;   // bf16 or IEEE half
   __shared__ __attribute__((aligned(1024))) char lds[AD_WAVES * AD_RING * AD_ITEM];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -159,7 +165,7 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
       }
       u32x4_t rot[4];
 #pragma unroll
-      for (int c = 0; c < 4; c++) rot[c] = rope8(raw[c], raw[c ^ 2], cs[c], sn[c], c < 2 ? -1.0f : 1.0f);
+      for (int c = 0; c < 4; c++) rot[c] = rope8<F16>(raw[c], raw[c ^ 2], cs[c], sn[c], c < 2 ? -1.0f : 1.0f);
 #pragma unroll
       for (int c = 0; c < 4; c++) raw[c] = rot[c];
     }
@@ -226,14 +232,14 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
 #pragma unroll
     for (int c = 0; c < 4; c++) kraw[c] = *reinterpret_cast<const u32x4_t*>(krow + 32 * c + 8 * q);
 #pragma unroll
-    for (int c = 0; c < 4; c++) krot[c] = rope8(kraw[c], kraw[c ^ 2], cs[c], sn[c], c < 2 ? -1.0f : 1.0f);
+    for (int c = 0; c < 4; c++) krot[c] = rope8<F16>(kraw[c], kraw[c ^ 2], cs[c], sn[c], c < 2 ? -1.0f : 1.0f);
     float dot = 0.0f;
 #pragma unroll
     for (int c = 0; c < 4; c++) {
       const u32x4_t qq = __builtin_bit_cast(u32x4_t, qf[c]);
 #pragma unroll
       for (int e = 0; e < 4; e++)
-        dot += bf16_lo(qq[e]) * bf16_lo(krot[c][e]) + bf16_hi(qq[e]) * bf16_hi(krot[c][e]);
+        dot += X::lo(qq[e]) * X::lo(krot[c][e]) + X::hi(qq[e]) * X::hi(krot[c][e]);
     }
     dot += __shfl_xor(dot, 16, 64);
     dot += __shfl_xor(dot, 32, 64);
@@ -244,7 +250,7 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
 #pragma unroll
     for (int dt = 0; dt < 8; dt++) {
       const u32x2_t vv = *reinterpret_cast<const u32x2_t*>(vrow_new + 16 * dt + 4 * q);
-      o[dt] = f32x4_t{bf16_lo(vv[0]), bf16_hi(vv[0]), bf16_lo(vv[1]), bf16_hi(vv[1])};
+      o[dt] = f32x4_t{X::lo(vv[0]), X::hi(vv[0]), X::lo(vv[1]), X::hi(vv[1])};
     }
     if (h == 0) {
 #pragma unroll
@@ -270,8 +276,8 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
       const uint32_t off = krow + (uint32_t)(((4 * c + q) ^ h) << 4);
       const bf16x8_t a0 = *reinterpret_cast<const bf16x8_t*>(kslot + off);
       const bf16x8_t a1 = *reinterpret_cast<const bf16x8_t*>(kslot + off + 16 * 256);
-      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[c], s0, 0, 0, 0);
-      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qf[c], s1, 0, 0, 0);
+      s0 = X::mfma16(a0, qf[c], s0);
+      s1 = X::mfma16(a1, qf[c], s1);
     }
     // this lane: head h, tokens 4q + j (s0) and 16 + 4q + j (s1) of the tile
     const int64_t valid = len - (int64_t)tile_of(i) * AD_TILE;
@@ -296,8 +302,8 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
       psum += x0[j] + x1[j];
     }
     l_run = l_run * alpha + psum;
-    const u32x4_t praw = {pack_bf16x2(x0[0], x0[1]), pack_bf16x2(x0[2], x0[3]), pack_bf16x2(x1[0], x1[1]),
-                          pack_bf16x2(x1[2], x1[3])};
+    const u32x4_t praw = {X::pack2(x0[0], x0[1]), X::pack2(x0[2], x0[3]), X::pack2(x1[0], x1[1]),
+                          X::pack2(x1[2], x1[3])};
     const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, praw);
 #pragma unroll
     for (int dt = 0; dt < 8; dt++) o[dt] *= alpha;
@@ -318,7 +324,7 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
       const bf16x4_t hi =
           __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4_t __attribute__((address_space(3)))*)(a + 16 * 256));
       const bf16x8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
+      o[dt] = X::mfma16(vf, pf, o[dt]);
     }
   }
 
@@ -355,7 +361,7 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
     }
     const int64_t hq = (int64_t)b * p.n_q_heads + (int64_t)kvh * G + hh;
     if (p.splits == 1) {
-      p.out[hq * AD_D + d] = f32_to_bf16_bits(l > 0.0f ? acc / l : 0.0f);
+      p.out[hq * AD_D + d] = X::to_bits(l > 0.0f ? acc / l : 0.0f);
     } else {
       float* dst = p.part + (hq * p.splits + split) * AD_PART;
       coherent_store(dst + d, acc);
@@ -413,13 +419,13 @@ __device__ __forceinline__ void attn_decode_body(const AttnArgs& p) {
       }
       mstar = mnew;
     }
-    p.out[hq * AD_D + d] = f32_to_bf16_bits(l > 0.0f ? acc / l : 0.0f);
+    p.out[hq * AD_D + d] = X::to_bits(l > 0.0f ? acc / l : 0.0f);
   }
 }
 
-template <bool APPEND, int AD_WAVES, int AD_RING, bool NT>
+template <bool APPEND, int AD_WAVES, int AD_RING, bool NT, bool F16>
 __global__ __launch_bounds__(AD_WAVES * 64) void attn_decode_kernel(const AttnArgs p) {
-  attn_decode_body<APPEND, AD_WAVES, AD_RING, NT>(p);
+  attn_decode_body<APPEND, AD_WAVES, AD_RING, NT, F16>(p);
 }
 
 // ---- RMSNorm with the residual add in front of it ---------------------------------------------------
@@ -430,6 +436,10 @@ template <typename T> struct Elem;
 template <> struct Elem<uint16_t> {
   static __device__ __forceinline__ float load(uint16_t v) { return bf16_bits_to_f32(v); }
   static __device__ __forceinline__ uint16_t store(float f) { return f32_to_bf16_bits(f); }
+};
+template <> struct Elem<f16s> {
+  static __device__ __forceinline__ float load(f16s v) { return X16<true>::from_bits(v.bits); }
+  static __device__ __forceinline__ f16s store(float f) { return f16s{X16<true>::to_bits(f)}; }
 };
 template <> struct Elem<float> {
   static __device__ __forceinline__ float load(float v) { return v; }
@@ -482,6 +492,21 @@ template <> struct Vec16<uint16_t> {
     return u32x4_t{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7])};
   }
   static __device__ __forceinline__ float round(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+};
+template <> struct Vec16<f16s> {
+  static constexpr int N = 8;
+  using H = X16<true>;
+  static __device__ __forceinline__ void unpack(u32x4_t v, float* f) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      f[2 * e] = H::lo(v[e]);
+      f[2 * e + 1] = H::hi(v[e]);
+    }
+  }
+  static __device__ __forceinline__ u32x4_t pack(const float* f) {
+    return u32x4_t{H::pack2(f[0], f[1]), H::pack2(f[2], f[3]), H::pack2(f[4], f[5]), H::pack2(f[6], f[7])};
+  }
+  static __device__ __forceinline__ float round(float f) { return H::from_bits(H::to_bits(f)); }
 };
 template <> struct Vec16<float> {
   static constexpr int N = 4;
@@ -553,6 +578,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const T* x, const T* r
 // qkv [B, (n_q + 2 n_kv) * 128]: q heads, then k heads, then v heads (the fused QKV linear's output).
 // HF apply_rotary_pos_emb: x * cos + rotate_half(x) * sin with rotate_half(x) = cat(-x[64:], x[:64]);
 // cos / sin are tables [max_positions, 128] in the tensor dtype, indexed by the token's position.
+template <bool F16>
 __global__ __launch_bounds__(64) void rope_append_kernel(const uint16_t* __restrict__ qkv,
                                                          const uint16_t* __restrict__ cos_t,
                                                          const uint16_t* __restrict__ sin_t,
@@ -560,6 +586,7 @@ __global__ __launch_bounds__(64) void rope_append_kernel(const uint16_t* __restr
                                                          uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache,
                                                          uint16_t* __restrict__ v_cache, int n_q, int n_kv,
                                                          int64_t max_len, int64_t max_positions) {
+  using X = X16<F16>;
   const int head = blockIdx.x, b = blockIdx.y, j = threadIdx.x;
   const int64_t pos = positions[b];
   const uint16_t* src = qkv + ((int64_t)b * (n_q + 2 * n_kv) + head) * AD_D;
@@ -571,14 +598,18 @@ __global__ __launch_bounds__(64) void rope_append_kernel(const uint16_t* __restr
     return;
   }
   if (pos < 0 || pos >= max_positions) return;
-  const float x1 = bf16_bits_to_f32(src[j]), x2 = bf16_bits_to_f32(src[j + 64]);
+  const float x1 = X::from_bits(src[j]), x2 = X::from_bits(src[j + 64]);
   const uint16_t* cr = cos_t + pos * AD_D;
   const uint16_t* sr = sin_t + pos * AD_D;
-  const float c1 = bf16_bits_to_f32(cr[j]), c2 = bf16_bits_to_f32(cr[j + 64]);
-  const float s1 = bf16_bits_to_f32(sr[j]), s2 = bf16_bits_to_f32(sr[j + 64]);
-  // each product is rounded to bf16 before the sum, as the bf16 tensor expression does
-  const float r1 = bf16_bits_to_f32(f32_to_bf16_bits(x1 * c1)) + bf16_bits_to_f32(f32_to_bf16_bits(-x2 * s1));
-  const float r2 = bf16_bits_to_f32(f32_to_bf16_bits(x2 * c2)) + bf16_bits_to_f32(f32_to_bf16_bits(x1 * s2));
+  const float c1 = X::from_bits(cr[j]), c2 = X::from_bits(cr[j + 64]);
+  const float s1 = X::from_bits(sr[j]), s2 = X::from_bits(sr[j + 64]);
+  // each product is rounded to the tensor dtype before the sum, as the tensor expression does.  The products are
+  // pinned as fp32 values: with half tensors the compiler otherwise narrows the arithmetic to half and folds one
+  // of the rounded products into a fused multiply-add.
+  float a1 = x1 * c1, a2 = x2 * c2, b1 = -x2 * s1, b2 = x1 * s2;
+  asm volatile("" : "+v"(a1), "+v"(a2), "+v"(b1), "+v"(b2));
+  const uint32_t pa = X::pack2(a1, a2), pb = X::pack2(b1, b2);
+  const uint32_t pr = X::pack2(X::lo(pa) + X::lo(pb), X::hi(pa) + X::hi(pb));
   uint16_t* dst;
   if (head < n_q) {
     dst = q_out + ((int64_t)b * n_q + head) * AD_D;
@@ -586,8 +617,8 @@ __global__ __launch_bounds__(64) void rope_append_kernel(const uint16_t* __restr
     if (pos >= max_len) return;
     dst = k_cache + (((int64_t)b * n_kv + (head - n_q)) * max_len + pos) * AD_D;
   }
-  dst[j] = f32_to_bf16_bits(r1);
-  dst[j + 64] = f32_to_bf16_bits(r2);
+  dst[j] = (uint16_t)(pr & 0xffffu);
+  dst[j + 64] = (uint16_t)(pr >> 16);
 }
 
 int pick_splits(int64_t B, int n_kv, int64_t len_bound) {
@@ -619,7 +650,7 @@ int64_t workspace_need(int64_t B, int n_q, int n_kv, int splits) {
 int launch_attn(bool append, AttnArgs a, const char* what, void* workspace, int64_t workspace_bytes, int64_t B,
                 int n_q_heads, int n_kv_heads, int head_dim, int64_t max_len, int64_t len_bound, float scale, int dtype,
                 void* stream) {
-  MTP_REQUIRE(dtype == MTP_BF16, MTP_EUNSUPPORTED, "%s: bf16 only", what);
+  MTP_REQUIRE(dtype == MTP_BF16 || dtype == MTP_F16, MTP_EUNSUPPORTED, "%s: dtype %d (bf16 or f16)", what, dtype);
   MTP_REQUIRE(head_dim == AD_D, MTP_EUNSUPPORTED, "%s: head_dim %d (128 supported)", what, head_dim);
   MTP_REQUIRE(B >= 0 && n_q_heads > 0 && n_kv_heads > 0 && n_q_heads % n_kv_heads == 0, MTP_EINVAL,
               "%s: B=%lld heads %d/%d", what, (long long)B, n_q_heads, n_kv_heads);
@@ -654,12 +685,17 @@ int launch_attn(bool append, AttnArgs a, const char* what, void* workspace, int6
   const dim3 grid(splits, n_kv_heads, (unsigned)B);
   int cfg = 0;
   if (const char* e = getenv("MTP_ATTN_CFG")) cfg = atoi(e);
-#define MTP_ATTN_LAUNCH(W, R, NT)                                                                  \
-  do {                                                                                             \
-    if (append)                                                                                    \
-      hipLaunchKernelGGL((attn_decode_kernel<true, W, R, NT>), grid, dim3(W * 64), 0, s, a);       \
-    else                                                                                           \
-      hipLaunchKernelGGL((attn_decode_kernel<false, W, R, NT>), grid, dim3(W * 64), 0, s, a);      \
+  const bool f16 = dtype == MTP_F16;
+#define MTP_ATTN_LAUNCH(W, R, NT)                                                                        \
+  do {                                                                                                   \
+    if (append && f16)                                                                                   \
+      hipLaunchKernelGGL((attn_decode_kernel<true, W, R, NT, true>), grid, dim3(W * 64), 0, s, a);       \
+    else if (append)                                                                                     \
+      hipLaunchKernelGGL((attn_decode_kernel<true, W, R, NT, false>), grid, dim3(W * 64), 0, s, a);      \
+    else if (f16)                                                                                        \
+      hipLaunchKernelGGL((attn_decode_kernel<false, W, R, NT, true>), grid, dim3(W * 64), 0, s, a);      \
+    else                                                                                                 \
+      hipLaunchKernelGGL((attn_decode_kernel<false, W, R, NT, false>), grid, dim3(W * 64), 0, s, a);     \
   } while (0)
   if (cfg == 1)
     MTP_ATTN_LAUNCH(8, 2, false);
@@ -715,13 +751,13 @@ extern "C" int mtp_attn_decode_append(const void* qkv, const void* cos_table, co
 
 extern "C" int mtp_rmsnorm(const void* x, const void* residual, const void* weight, void* y, void* residual_out,
                            int64_t rows, int64_t dim, float eps, int dtype, void* stream) {
-  MTP_REQUIRE(dtype == MTP_BF16 || dtype == MTP_F32, MTP_EINVAL, "rmsnorm: dtype %d", dtype);
+  MTP_REQUIRE(dtype == MTP_BF16 || dtype == MTP_F32 || dtype == MTP_F16, MTP_EINVAL, "rmsnorm: dtype %d", dtype);
   MTP_REQUIRE(rows >= 0 && dim > 0 && rows <= 0x7fffffffll, MTP_EINVAL, "rmsnorm: rows=%lld dim=%lld", (long long)rows,
               (long long)dim);
   if (rows == 0) return MTP_OK;
   MTP_REQUIRE(x && weight && y, MTP_EINVAL, "rmsnorm: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int epv = dtype == MTP_BF16 ? 8 : 4;
+  const int epv = dtype == MTP_F32 ? 4 : 8;
   const bool aligned = ((uintptr_t)x | (uintptr_t)residual | (uintptr_t)weight | (uintptr_t)y |
                         (uintptr_t)residual_out) % 16 == 0;
   const int64_t nvec = dim / epv;
@@ -739,6 +775,8 @@ extern "C" int mtp_rmsnorm(const void* x, const void* residual, const void* weig
   } while (0)
   if (dtype == MTP_BF16)
     MTP_RMS_PICK(uint16_t);
+  else if (dtype == MTP_F16)
+    MTP_RMS_PICK(f16s);
   else
     MTP_RMS_PICK(float);
 #undef MTP_RMS_PICK
@@ -751,7 +789,7 @@ extern "C" int mtp_rope_kv_append(const void* qkv, const void* cos_table, const 
                                   const int64_t* positions, void* q_out, void* k_cache, void* v_cache, int64_t B,
                                   int n_q_heads, int n_kv_heads, int head_dim, int64_t max_len, int64_t max_positions,
                                   int dtype, void* stream) {
-  MTP_REQUIRE(dtype == MTP_BF16, MTP_EUNSUPPORTED, "rope_kv_append: bf16 only");
+  MTP_REQUIRE(dtype == MTP_BF16 || dtype == MTP_F16, MTP_EUNSUPPORTED, "rope_kv_append: dtype %d (bf16 or f16)", dtype);
   MTP_REQUIRE(head_dim == AD_D, MTP_EUNSUPPORTED, "rope_kv_append: head_dim %d (128 supported)", head_dim);
   MTP_REQUIRE(B >= 0 && B <= 65535 && n_q_heads > 0 && n_kv_heads > 0 && max_len > 0 && max_positions > 0, MTP_EINVAL,
               "rope_kv_append: B=%lld heads %d/%d max_len=%lld", (long long)B, n_q_heads, n_kv_heads,
@@ -760,11 +798,17 @@ extern "C" int mtp_rope_kv_append(const void* qkv, const void* cos_table, const 
   MTP_REQUIRE(qkv && cos_table && sin_table && positions && q_out && k_cache && v_cache, MTP_EINVAL,
               "rope_kv_append: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(rope_append_kernel, dim3(n_q_heads + 2 * n_kv_heads, (unsigned)B), dim3(64), 0, s,
-                     static_cast<const uint16_t*>(qkv), static_cast<const uint16_t*>(cos_table),
-                     static_cast<const uint16_t*>(sin_table), positions, static_cast<uint16_t*>(q_out),
-                     static_cast<uint16_t*>(k_cache), static_cast<uint16_t*>(v_cache), n_q_heads, n_kv_heads, max_len,
-                     max_positions);
+  const dim3 grid(n_q_heads + 2 * n_kv_heads, (unsigned)B), block(64);
+#define MTP_ROPE_ARGS                                                                                       \
+  static_cast<const uint16_t*>(qkv), static_cast<const uint16_t*>(cos_table),                               \
+      static_cast<const uint16_t*>(sin_table), positions, static_cast<uint16_t*>(q_out),                    \
+      static_cast<uint16_t*>(k_cache), static_cast<uint16_t*>(v_cache), n_q_heads, n_kv_heads, max_len,     \
+      max_positions
+  if (dtype == MTP_F16)
+    hipLaunchKernelGGL(rope_append_kernel<true>, grid, block, 0, s, MTP_ROPE_ARGS);
+  else
+    hipLaunchKernelGGL(rope_append_kernel<false>, grid, block, 0, s, MTP_ROPE_ARGS);
+#undef MTP_ROPE_ARGS
   MTP_CHECK_LAUNCH("rope_kv_append");
   return MTP_OK;
 }

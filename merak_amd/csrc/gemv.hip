@@ -24,6 +24,7 @@
 // bit-reproducible run to run.
 #include "mtp_common.h"
 #include <stdlib.h>
+#include <type_traits>
 
 namespace {
 
@@ -80,7 +81,7 @@ __device__ __forceinline__ uint32_t rot8_in_row(uint32_t v) {
 // MODE 0: store Y (+bias); MODE 1: SwiGLU store; MODE 2: argmax partials
 // W waves split K.  Configurations whose registers allow only 8 waves per CU run as two independent workgroups of
 // 4 waves rather than one of 8: while one sums its partial tiles and writes its outputs the other keeps streaming.
-template <int R, int NB, int MODE, bool GUARD, int D, int W>
+template <int R, int NB, int MODE, bool GUARD, int D, int W, bool F16>
 __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __restrict__ x,
                                                           const uint16_t* __restrict__ w,
                                                           const uint16_t* __restrict__ bias,
@@ -92,6 +93,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   // the k range is cut into gridDim.y slices of K elements, one workgroup per (row block, slice); the
   // slices' partial sums meet in `kpart` and the slice that delivers last adds them up in slice order.
   const int64_t koff = (int64_t)blockIdx.y * K;
+  using X = X16<F16>;   // bf16 or IEEE half: the MFMA and the conversions of the epilogue
   constexpr int GV_WAVES = W, GV_THREADS = W * MTP_WAVE;
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -215,8 +217,8 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
           const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
 #pragma unroll
           for (int nb = 0; nb < NB; nb++) {
-            acc[r][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(h0, b_cur[d][xs][nb][0], acc[r][nb], 0, 0, 0);
-            acc[r][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(h1, b_cur[d][xs][nb][1], acc[r][nb], 0, 0, 0);
+            acc[r][nb] = X::mfma16(h0, b_cur[d][xs][nb][0], acc[r][nb]);
+            acc[r][nb] = X::mfma16(h1, b_cur[d][xs][nb][1], acc[r][nb]);
           }
         }
     };
@@ -312,8 +314,8 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
       const int64_t n = n0 + rl;
       if (n < N) {
         float v = fin[b][rl];
-        if (bias) v += bf16_bits_to_f32(bias[n]);
-        y[(int64_t)b * N + n] = f32_to_bf16_bits(v);
+        if (bias) v += X::from_bits(bias[n]);
+        y[(int64_t)b * N + n] = X::to_bits(v);
       }
     }
   } else if (MODE == 1) {
@@ -324,13 +326,13 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
       if (jn < half) {
         float gate = fin[b][rl], up = fin[b][8 * R + rl];
         if (bias) {
-          gate += bf16_bits_to_f32(bias[jn]);
-          up += bf16_bits_to_f32(bias[half + jn]);
+          gate += X::from_bits(bias[jn]);
+          up += X::from_bits(bias[half + jn]);
         }
         // round the pre-activations to bf16 first, as the unfused layer stack would
-        gate = bf16_bits_to_f32(f32_to_bf16_bits(gate));
-        up = bf16_bits_to_f32(f32_to_bf16_bits(up));
-        y[(int64_t)b * half + jn] = f32_to_bf16_bits(silu_f(gate) * up);
+        gate = X::from_bits(X::to_bits(gate));
+        up = X::from_bits(X::to_bits(up));
+        y[(int64_t)b * half + jn] = X::to_bits(silu_f(gate) * up);
       }
     }
   } else {
@@ -415,7 +417,9 @@ __global__ __launch_bounds__(256) void argmax_rows_kernel(const T* __restrict__ 
   bool have = false;
   for (int64_t j = threadIdx.x; j < V; j += 256) {
     float v;
-    if constexpr (sizeof(T) == 2)
+    if constexpr (std::is_same<T, f16s>::value)
+      v = X16<true>::from_bits(rp[j].bits);
+    else if constexpr (sizeof(T) == 2)
       v = bf16_bits_to_f32(rp[j]);
     else
       v = rp[j];
@@ -511,7 +515,7 @@ int64_t gemv_counter_bytes(int64_t N) { return ((N + 15) / 16 * (int64_t)sizeof(
 
 template <int MODE>
 int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart* part, int64_t B, int64_t N,
-                int64_t K, GemvCfg cfg, hipStream_t s, unsigned* n_wg_out, void* workspace = nullptr) {
+                int64_t K, GemvCfg cfg, hipStream_t s, unsigned* n_wg_out, bool f16, void* workspace = nullptr) {
   const int R = cfg.R;
   const int64_t rows_per_wg = (MODE == 1) ? 8 * R : 16 * R;
   const int64_t span = (MODE == 1) ? N / 2 : N;
@@ -528,11 +532,16 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   int32_t* karrived = static_cast<int32_t*>(workspace);
   float* kpart = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + gemv_counter_bytes(N)) : nullptr;
   const int64_t k_slice = K / S;
-#define GV_LAUNCH(RR, NNB, GG, DD)                                                                              \
-  hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD, (RR >= 8 ? 4 : 8)>), dim3(n_wg, S),                    \
+#define GV_LAUNCH_T(RR, NNB, GG, DD, FF)                                                                        \
+  hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD, (RR >= 8 ? 4 : 8), FF>), dim3(n_wg, S),                \
                      dim3((RR >= 8 ? 4 : 8) * MTP_WAVE), 0, s,                                                  \
                      (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part, (int)B, \
                      N, k_slice, rot_mul, K, kpart, karrived, flags)
+#define GV_LAUNCH(RR, NNB, GG, DD)                 \
+  do {                                             \
+    if (f16) GV_LAUNCH_T(RR, NNB, GG, DD, true);   \
+    else GV_LAUNCH_T(RR, NNB, GG, DD, false);      \
+  } while (0)
 #define GV_BY_DEPTH(RR, NNB)                                                   \
   do {                                                                         \
     if (K % 64 != 0) GV_LAUNCH(RR, NNB, true, 1);                              \
@@ -554,11 +563,13 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   }
 #undef GV_BY_DEPTH
 #undef GV_LAUNCH
+#undef GV_LAUNCH_T
   MTP_CHECK_LAUNCH("gemv");
   return MTP_OK;
 }
 
-int check_gemv_args(const char* what, const void* x, const void* w, int64_t B, int64_t N, int64_t K) {
+int check_gemv_args(const char* what, const void* x, const void* w, int64_t B, int64_t N, int64_t K, int dtype) {
+  MTP_REQUIRE(dtype == MTP_BF16 || dtype == MTP_F16, MTP_EUNSUPPORTED, "%s: dtype %d (bf16 or f16)", what, dtype);
   MTP_REQUIRE(B >= 1 && B <= 32, MTP_EUNSUPPORTED, "%s: B=%lld outside [1,32]", what, (long long)B);
   MTP_REQUIRE(N >= 1 && K >= 1, MTP_EINVAL, "%s: N=%lld K=%lld", what, (long long)N, (long long)K);
   MTP_REQUIRE(N < (1ll << 31), MTP_EUNSUPPORTED, "%s: N=%lld exceeds 2^31-1", what, (long long)N);
@@ -581,8 +592,10 @@ extern "C" int64_t mtp_gemv_workspace_bytes(int64_t B, int64_t N, int64_t K, int
 }
 
 extern "C" int mtp_gemv_ws(const void* x, const void* w, const void* bias, void* y, void* workspace,
-                           int64_t workspace_bytes, int64_t B, int64_t N, int64_t K, int epilogue, void* stream) {
-  int rc = check_gemv_args("gemv", x, w, B, N, K);
+                           int64_t workspace_bytes, int64_t B, int64_t N, int64_t K, int epilogue, int dtype,
+                           void* stream) {
+  int rc = check_gemv_args("gemv", x, w, B, N, K, dtype);
+  const bool f16 = dtype == MTP_F16;
   if (rc) return rc;
   MTP_REQUIRE(y, MTP_EINVAL, "gemv: null output");
   MTP_REQUIRE(epilogue == MTP_EPI_NONE || epilogue == MTP_EPI_BIAS || epilogue == MTP_EPI_SWIGLU, MTP_EINVAL,
@@ -596,15 +609,15 @@ extern "C" int mtp_gemv_ws(const void* x, const void* w, const void* bias, void*
   const GemvCfg cfg = pick_gemv_cfg(B, N, K, mode, split);
   if (mode == 1) {
     MTP_REQUIRE(N % 2 == 0, MTP_EINVAL, "gemv: SwiGLU needs an even N, got %lld", (long long)N);
-    return launch_gemv<1>(x, w, bias, y, nullptr, B, N, K, cfg, s, nullptr, split ? workspace : nullptr);
+    return launch_gemv<1>(x, w, bias, y, nullptr, B, N, K, cfg, s, nullptr, f16, split ? workspace : nullptr);
   }
-  return launch_gemv<0>(x, w, epilogue == MTP_EPI_NONE ? nullptr : bias, y, nullptr, B, N, K, cfg, s, nullptr,
+  return launch_gemv<0>(x, w, epilogue == MTP_EPI_NONE ? nullptr : bias, y, nullptr, B, N, K, cfg, s, nullptr, f16,
                         split ? workspace : nullptr);
 }
 
 extern "C" int mtp_gemv(const void* x, const void* w, const void* bias, void* y, int64_t B, int64_t N, int64_t K,
-                        int epilogue, void* stream) {
-  return mtp_gemv_ws(x, w, bias, y, nullptr, 0, B, N, K, epilogue, stream);
+                        int epilogue, int dtype, void* stream) {
+  return mtp_gemv_ws(x, w, bias, y, nullptr, 0, B, N, K, epilogue, dtype, stream);
 }
 
 extern "C" int64_t mtp_gemv_argmax_workspace_bytes(int64_t B, int64_t N, int64_t K) {
@@ -615,8 +628,8 @@ extern "C" int64_t mtp_gemv_argmax_workspace_bytes(int64_t B, int64_t N, int64_t
 }
 
 extern "C" int mtp_gemv_argmax(const void* x, const void* w, int64_t* idx, float* maxval, void* workspace,
-                               int64_t workspace_bytes, int64_t B, int64_t N, int64_t K, void* stream) {
-  int rc = check_gemv_args("gemv_argmax", x, w, B, N, K);
+                               int64_t workspace_bytes, int64_t B, int64_t N, int64_t K, int dtype, void* stream) {
+  int rc = check_gemv_args("gemv_argmax", x, w, B, N, K, dtype);
   if (rc) return rc;
   MTP_REQUIRE(idx && workspace, MTP_EINVAL, "gemv_argmax: null pointer");
   MTP_REQUIRE(workspace_bytes >= mtp_gemv_argmax_workspace_bytes(B, N, K), MTP_EWORKSPACE,
@@ -625,7 +638,8 @@ extern "C" int mtp_gemv_argmax(const void* x, const void* w, int64_t* idx, float
   MTP_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7) == 0, MTP_EINVAL, "gemv_argmax: workspace not 8-byte aligned");
   hipStream_t s = (hipStream_t)stream;
   unsigned n_wg = 0;
-  rc = launch_gemv<2>(x, w, nullptr, nullptr, (ArgPart*)workspace, B, N, K, pick_gemv_cfg(B, N, K, 2), s, &n_wg);
+  rc = launch_gemv<2>(x, w, nullptr, nullptr, (ArgPart*)workspace, B, N, K, pick_gemv_cfg(B, N, K, 2), s, &n_wg,
+                      dtype == MTP_F16);
   if (rc) return rc;
   hipLaunchKernelGGL(argmax_finish_kernel, dim3((unsigned)B), dim3(256), 0, s, (const ArgPart*)workspace, (int)n_wg, (int)B,
                      idx, maxval);
@@ -644,6 +658,8 @@ extern "C" int mtp_argmax_rows(const void* logits, int64_t* idx, int64_t B, int6
   else if (dtype == MTP_BF16)
     hipLaunchKernelGGL(argmax_rows_kernel<uint16_t>, dim3((unsigned)B), dim3(256), 0, s, (const uint16_t*)logits,
                        idx, V);
+  else if (dtype == MTP_F16)
+    hipLaunchKernelGGL(argmax_rows_kernel<f16s>, dim3((unsigned)B), dim3(256), 0, s, (const f16s*)logits, idx, V);
   else
     MTP_REQUIRE(false, MTP_EINVAL, "argmax_rows: unknown dtype %d", dtype);
   MTP_CHECK_LAUNCH("argmax_rows");

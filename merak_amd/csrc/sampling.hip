@@ -84,6 +84,21 @@ template <> struct Row<uint16_t> {
   }
 };
 
+template <> struct Row<f16s> {
+  static constexpr int EPV = 8, KEY_BITS = 16;
+  using H = X16<true>;
+  __device__ static __forceinline__ float ld(const f16s* p) { return H::from_bits(p->bits); }
+  __device__ static __forceinline__ void unpack(const u32x4_t& v, float* f) {
+    f[0] = H::lo(v.x); f[1] = H::hi(v.x); f[2] = H::lo(v.y); f[3] = H::hi(v.y);
+    f[4] = H::lo(v.z); f[5] = H::hi(v.z); f[6] = H::lo(v.w); f[7] = H::hi(v.w);
+  }
+  // 16-bit image of the half logit itself (the conversion back is exact): x -> x / T is increasing on it
+  __device__ static __forceinline__ uint32_t key(float x, float z) {
+    const uint32_t u = x == 0.0f ? 0u : (uint32_t)H::to_bits(x);
+    return (u & 0x8000u) ? (~u & 0xffffu) : (u | 0x8000u);
+  }
+};
+
 template <typename T>
 struct Slots {
   const T* row;
@@ -516,7 +531,7 @@ extern "C" int mtp_sample_top_k_top_p(const void* logits, int dtype, int64_t B, 
   MTP_REQUIRE(B >= 0 && V >= 1, MTP_EINVAL, "sample: B=%lld V=%lld", (long long)B, (long long)V);
   MTP_REQUIRE(B < (1ll << 24) && V < (1ll << 31), MTP_EUNSUPPORTED, "sample: B=%lld or V=%lld too large", (long long)B,
               (long long)V);
-  MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16, MTP_EINVAL, "sample: unknown dtype %d", dtype);
+  MTP_REQUIRE(dtype == MTP_F32 || dtype == MTP_BF16 || dtype == MTP_F16, MTP_EINVAL, "sample: unknown dtype %d", dtype);
   MTP_REQUIRE(temperature > 0.0f && temperature == temperature, MTP_EINVAL, "sample: temperature must be positive");
   MTP_REQUIRE(top_k >= 0 && top_p >= 0.0f, MTP_EINVAL, "sample: top_k=%d top_p=%g", top_k, (double)top_p);
   // torch.topk in the reference (:50) refuses k beyond the row length
@@ -531,6 +546,9 @@ extern "C" int mtp_sample_top_k_top_p(const void* logits, int dtype, int64_t B, 
   if (dtype == MTP_F32)
     return launch_sample<float>(logits, B, V, temperature, top_k, top_p, uniforms, tokens, filtered,
                                 (RowState*)workspace, s);
+  if (dtype == MTP_F16)
+    return launch_sample<f16s>(logits, B, V, temperature, top_k, top_p, uniforms, tokens, filtered,
+                               (RowState*)workspace, s);
   return launch_sample<uint16_t>(logits, B, V, temperature, top_k, top_p, uniforms, tokens, filtered,
                                  (RowState*)workspace, s);
 }

@@ -274,27 +274,32 @@ def gemv_workspace(B: int, N: int, K: int, epilogue: int, device) -> Optional[to
     return torch.zeros((need,), dtype=torch.uint8, device=device) if need else None
 
 
+def _decode_dtype(what: str, *ts: torch.Tensor) -> torch.dtype:
+    dt = ts[0].dtype
+    if dt not in (torch.bfloat16, torch.float16) or any(t.dtype != dt for t in ts if t is not None):
+        raise TypeError(f"{what} takes bfloat16 or float16 tensors of one dtype, got {[t.dtype for t in ts if t is not None]}")
+    return dt
+
+
 def gemv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE,
          workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     dev = _require_gpu(x, w, bias, workspace)
-    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
-        raise TypeError("gemv is bf16 only")
+    dt = _decode_dtype("gemv", x, w, bias)
     B, K = x.shape
     N = w.shape[0]
     x, w = _contig(x), _contig(w)
-    y = torch.empty((B, N // 2 if epilogue == EPI_SWIGLU else N), dtype=torch.bfloat16, device=dev)
+    y = torch.empty((B, N // 2 if epilogue == EPI_SWIGLU else N), dtype=dt, device=dev)
     wbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().mtp_gemv_ws(_p(x), _p(w), _p(bias), _p(y), _p(workspace), wbytes, B, N, K, epilogue,
-                                          _stream(dev)), "mtp_gemv")
+                                          _DTYPES[dt], _stream(dev)), "mtp_gemv")
     return y
 
 
 def gemv_argmax(x: torch.Tensor, w: torch.Tensor, workspace: Optional[torch.Tensor] = None):
     """-> (idx int64 [B], maxval fp32 [B]) without materialising the logits."""
     dev = _require_gpu(x, w, workspace)
-    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
-        raise TypeError("gemv_argmax is bf16 only")
+    dt = _decode_dtype("gemv_argmax", x, w)
     B, K = x.shape
     N = w.shape[0]
     x, w = _contig(x), _contig(w)
@@ -305,7 +310,7 @@ def gemv_argmax(x: torch.Tensor, w: torch.Tensor, workspace: Optional[torch.Tens
     val = torch.empty((B,), dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().mtp_gemv_argmax(_p(x), _p(w), _p(idx), _p(val), _p(workspace), workspace.numel(), B, N, K,
-                                              _stream(dev)), "mtp_gemv_argmax")
+                                              _DTYPES[dt], _stream(dev)), "mtp_gemv_argmax")
     return idx, val
 
 

@@ -26,7 +26,7 @@ def test_header_symbols_are_exported_and_bound():
 
 def test_loader_and_versions():
     lib = _lib.lib()
-    assert lib.mtp_abi_version() == _lib.ABI_VERSION == 3
+    assert lib.mtp_abi_version() == _lib.ABI_VERSION == 4
     hdr = open(os.path.join(ROOT, "include", "merak_tp_gfx950.h")).read()
     assert f"#define MTP_ABI_VERSION {_lib.ABI_VERSION}" in hdr
     for name, val in (("MTP_F32", _lib.MTP_F32), ("MTP_BF16", _lib.MTP_BF16), ("MTP_EPI_NONE", _lib.EPI_NONE),
@@ -42,8 +42,10 @@ def test_argument_errors_are_reported_without_a_device():
     assert lib.mtp_vocab_ce_fwd(None, None, None, None, None, None, 4, 0, 0, 0, None) == -1
     assert b"vocab" in lib.mtp_last_error()
     assert lib.mtp_linear_fwd(None, None, None, None, None, 4, 4, 4, 7, 0, None) == -1
-    assert lib.mtp_gemv(None, None, None, None, 33, 8, 8, 0, None) == -2
+    assert lib.mtp_gemv(None, None, None, None, 33, 8, 8, 0, 1, None) == -2
     assert b"B=33" in lib.mtp_last_error()
+    assert lib.mtp_gemv(None, None, None, None, 4, 8, 8, 0, 0, None) == -2          # fp32 is not a decode dtype
+    assert b"dtype 0" in lib.mtp_last_error()
     assert lib.mtp_stream_copy(None, None, 24, None) == -1
 
 

@@ -135,3 +135,68 @@ def test_fp16_params_dtype_model_trains_like_stock_torch(gpu):
     for name, p_ in mods.named_parameters():
         assert p_.grad.dtype == H and torch.isfinite(p_.grad).all(), name
         assert rel(p_.grad, ref[name].grad) < 1e-2, name                    # fp16 activations through three layers
+
+
+# ---- the decode kernels in IEEE half ----
+@pytest.mark.parametrize("b,n,k,epi", [(1, 4096, 4096, "none"), (8, 1000, 512, "bias"), (32, 2048, 1024, "swiglu"),
+                                       (32, 4096, 14336, "none"), (5, 130, 4104, "none")])
+def test_gemv_and_fused_argmax_fp16(gpu, b, n, k, epi):
+    g = gen(21)
+    x = torch.randn(b, k, generator=g).to(H)
+    w = (torch.randn(n, k, generator=g) * 0.02).to(H)
+    bias = (torch.randn(n, generator=g) * 0.1).to(H) if epi == "bias" else None
+    e = {"none": ops.EPI_NONE, "bias": ops.EPI_BIAS, "swiglu": ops.EPI_SWIGLU}[epi]
+    ref = F.linear(x.float(), w.float(), None if bias is None else bias.float())
+    ws = ops.gemv_workspace(b, n, k, e, gpu)
+    y = ops.gemv(x.to(gpu), w.to(gpu), None if bias is None else bias.to(gpu), e, workspace=ws)
+    assert y.dtype == H and rel(y, R.swiglu(ref.to(H).float()) if epi == "swiglu" else ref) < TOL_F16
+    if epi == "none":
+        idx, val = ops.gemv_argmax(x.to(gpu), w.to(gpu))
+        top2 = ref.topk(2, dim=-1).values
+        clear = (top2[:, 0] - top2[:, 1]) > 1e-3 * top2[:, 0].abs()
+        assert torch.equal(idx.cpu()[clear], ref.argmax(-1)[clear])
+        assert torch.allclose(val.cpu(), ref.max(-1).values, rtol=1e-3, atol=1e-4)
+    with pytest.raises(TypeError):
+        ops.gemv(x.to(gpu), w.bfloat16().to(gpu))                 # mixed 16-bit dtypes
+
+
+def test_rmsnorm_rope_attention_fp16(gpu):
+    from merak_amd.inference import rope_tables
+    g = gen(22)
+    x, r = (torch.randn(4, 4096, generator=g) * 2).to(H), torch.randn(4, 4096, generator=g).to(H)
+    wn = (torch.rand(4096, generator=g) + 0.5).to(H)
+    y, h = ops.rmsnorm(x.to(gpu), wn.to(gpu), 1e-5, r.to(gpu), want_residual=True)
+    ref_y, _ = R.rms_norm(x.float(), wn.float(), 1e-5, r.float())
+    assert torch.equal(h.cpu(), r + x) and rel(y, ref_y) < TOL_F16
+    B, n_q, n_kv, d, L = 3, 8, 2, 128, 700
+    qkv = torch.randn(B, (n_q + 2 * n_kv) * d, generator=g).to(H)
+    kc0, vc0 = torch.randn(B, n_kv, L, d, generator=g).to(H), torch.randn(B, n_kv, L, d, generator=g).to(H)
+    cos, sin = rope_tables(d, L, 500000.0, dtype=H)
+    pos = torch.tensor([699, 0, 300])
+    heads = qkv.float().view(B, n_q + 2 * n_kv, d)
+    cf, sf = cos.float()[pos], sin.float()[pos]
+    kf, vf = kc0.float(), vc0.float()
+    for b in range(B):
+        kf[b, :, pos[b]] = R.apply_rope(heads[:, n_q:n_q + n_kv], cf, sf)[b]
+        vf[b, :, pos[b]] = heads[b, n_q + n_kv:]
+    want = R.attn_decode(R.apply_rope(heads[:, :n_q], cf, sf), kf, vf, pos + 1)
+    k1, v1, k2, v2 = kc0.to(gpu), vc0.to(gpu), kc0.to(gpu), vc0.to(gpu)
+    out = ops.attn_decode_append(qkv.to(gpu), cos.to(gpu), sin.to(gpu), pos.to(gpu), k1, v1, n_q)
+    assert out.dtype == H and rel(out, want) < TOL_F16
+    q = ops.rope_kv_append(qkv.to(gpu), cos.to(gpu), sin.to(gpu), pos.to(gpu), k2, v2, n_q)
+    assert torch.equal(k1, k2) and torch.equal(v1, v2)
+    assert rel(ops.attn_decode(q, k2, v2, (pos + 1).to(gpu)), want) < TOL_F16
+
+
+def test_sampling_and_argmax_rows_fp16(gpu):
+    g = gen(23)
+    logits = (torch.randn(4, 5000, generator=g) * 3).to(H)
+    u = torch.rand(4, generator=g)
+    ref_tok, ref_probs = R.sample_tail(logits.clone(), 0.7, 40, 0.9, u)
+    tok, filt = ops.sample_top_k_top_p(logits.to(gpu), 0.7, 40, 0.9, u.to(gpu), want_filtered=True)
+    ref_filt = R.top_k_logits(logits.float() / 0.7, 40, 0.9)
+    kept, ref_kept = filt.cpu() > -float("inf"), ref_filt > -float("inf")
+    assert (kept | ~ref_kept).all()                                  # ties at the top-p boundary may only add
+    assert torch.equal(filt.cpu()[ref_kept], ref_filt[ref_kept])
+    assert int((tok.cpu() == ref_tok).sum()) >= 3
+    assert torch.equal(ops.argmax_rows(logits.to(gpu)).cpu(), logits.float().argmax(-1))

@@ -137,7 +137,7 @@ def test_ce_empty_and_errors(gpu):
     with pytest.raises(ValueError, match="contiguous"):
         ops.vocab_ce_fwd(torch.randn(4, 8, device=gpu)[:, ::2], torch.zeros(4, dtype=torch.int64, device=gpu), 0)
     with pytest.raises(TypeError):
-        ops.vocab_ce_fwd(torch.randn(2, 4, device=gpu).half(), torch.zeros(2, dtype=torch.int64, device=gpu), 0)
+        ops.vocab_ce_fwd(torch.randn(2, 4, device=gpu).double(), torch.zeros(2, dtype=torch.int64, device=gpu), 0)
 
 
 def test_ce_full_size_llama_vocab(gpu):

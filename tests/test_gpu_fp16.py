@@ -200,3 +200,28 @@ def test_sampling_and_argmax_rows_fp16(gpu):
     assert torch.equal(filt.cpu()[ref_kept], ref_filt[ref_kept])
     assert int((tok.cpu() == ref_tok).sum()) >= 3
     assert torch.equal(ops.argmax_rows(logits.to(gpu)).cpu(), logits.float().argmax(-1))
+
+
+def test_llama_decoder_fp16_matches_full_sequence_forward(gpu):
+    """The cached decoder on an fp16 model against the fp32 full-sequence forward of the library model."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from merak_amd.inference import LlamaDecoder
+    torch.manual_seed(31)
+    cfg = LlamaConfig(hidden_size=512, intermediate_size=1024, num_attention_heads=4, num_key_value_heads=2,
+                      head_dim=128, num_hidden_layers=2, vocab_size=1000, max_position_embeddings=128,
+                      rope_theta=10000.0, rms_norm_eps=1e-5, attn_implementation="eager", tie_word_embeddings=False)
+    model = LlamaForCausalLM(cfg).eval()
+    for p_ in model.parameters():
+        if p_.dim() == 1:
+            p_.data.uniform_(0.5, 1.5)
+        p_.data = p_.data.to(H).float()
+    ids = torch.randint(0, cfg.vocab_size, (2, 24), generator=gen(31))
+    with torch.no_grad():
+        full = model(input_ids=ids).logits
+    dec = LlamaDecoder.from_hf(model.half().to(gpu), max_len=32, batch=2)
+    worst = 0.0
+    for t in range(24):
+        lg = dec.logits(ids[:, t].to(gpu))
+        assert lg.dtype == H
+        worst = max(worst, rel(lg, full[:, t]))
+    assert worst < 4 * TOL_F16, worst

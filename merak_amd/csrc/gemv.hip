@@ -78,7 +78,14 @@ __device__ __forceinline__ uint32_t rot8_in_row(uint32_t v) {
   return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xf, 0xf, false);
 }
 
-// MODE 0: store Y (+bias); MODE 1: SwiGLU store; MODE 2: argmax partials
+// MODE 0: store Y (+bias); MODE 1: SwiGLU store; MODE 2: argmax partials;
+// MODE 3: SwiGLU with mixed row groups: rows 0-7 of a 16-row MFMA tile are gate rows, rows 8-15 the matching up
+// rows, so a workgroup may own any number R of groups (8 R gate rows and their up rows) and the workgroup count can
+// be made a multiple of the CU count (R = 7 gives exactly 256 workgroups for 14336 gate rows; with R = 4 the 448
+// workgroups leave a quarter of the CUs with half the bytes in flight: 5.4 instead of 6.4 TB/s).  Load A fetches the
+// gate rows of a k-pair, load B the up rows half a row further along k (the two sit a large power of two apart in
+// memory, see below), so a tile mixes two k positions: it is multiplied twice, once with X at either position,
+// into two accumulators, and each lane keeps the one whose rows it owns.
 // W waves split K.  Configurations whose registers allow only 8 waves per CU run as two independent workgroups of
 // 4 waves rather than one of 8: while one sums its partial tiles and writes its outputs the other keeps streaming.
 template <int R, int NB, int MODE, bool GUARD, int D, int W, bool F16>
@@ -111,7 +118,10 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
 #pragma unroll
   for (int r = 0; r < R; r++) {
     int64_t row0, lim;
-    if (MODE == 1) {
+    if (MODE == 3) {
+      row0 = (int64_t)blockIdx.x * (8 * R) + 8 * r;
+      lim = half;
+    } else if (MODE == 1) {
       const int64_t j0 = (int64_t)blockIdx.x * (8 * R);
       row0 = (r < R / 2) ? j0 + 16 * r : half + j0 + 16 * (r - R / 2);
       lim = (r < R / 2) ? half : N;
@@ -126,6 +136,12 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
       const int ra = li < last ? li : last;
       offa[r] = (uint32_t)(ra * ld + 8 * lg);
       offb[r] = offa[r] + 32;
+    } else if (MODE == 3) {
+      // load A: gate row row0 + li%8; load B: the up row of the same index, `half` rows further down (the host
+      // checks that this offset fits 32 bits)
+      const int ra = (li & 7) < last ? (li & 7) : last;
+      offa[r] = (uint32_t)(ra * ld + 32 * (li >> 3) + 8 * lg);
+      offb[r] = (uint32_t)((half + ra) * ld + 32 * (1 - (li >> 3)) + 8 * lg);
     } else {
       const int ra = (li & 7) < last ? (li & 7) : last, rb = 8 + (li & 7) < last ? 8 + (li & 7) : last;
       offa[r] = (uint32_t)(ra * ld + 32 * (li >> 3) + 8 * lg);
@@ -156,11 +172,16 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   // workgroups give logits that are equal to rounding, not necessarily bit for bit.)
   const int64_t rot = GUARD || (pairs % GV_MAX_WAVES) ? 0 : ((int64_t)(blockIdx.x + blockIdx.y) * rot_mul) % pairs;
 
+  static_assert(MODE != 3 || (NB == 1 && !GUARD && D == 1), "mixed SwiGLU groups: one batch tile, K % 64 == 0, depth 1");
+  constexpr bool MIX = MODE == 3;
   f32x4_t acc[R][NB];
+  f32x4_t acc_up[MIX ? R : 1];   // MIX: the products with X at the up rows' k position
 #pragma unroll
   for (int r = 0; r < R; r++)
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) acc[r][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int r = 0; r < (MIX ? R : 1); r++) acc_up[r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const bool low = li < 8;
 
   // D pairs (8 apart) per step: with few rows per workgroup this is what keeps enough bytes in flight.
@@ -171,7 +192,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
     // shapes a large power of two apart, i.e. in the same memory channel and bank but another DRAM page.
     // Walking both at the same k makes the two streams evict each other's open page, so the up rows walk
     // half a row ahead (XS = 2 sets of X fragments, one per k position).
-    constexpr int XS = (MODE == 1 && !GUARD && NB == 1) ? 2 : 1;
+    constexpr int XS = ((MODE == 1 || MODE == 3) && !GUARD && NB == 1) ? 2 : 1;
     const int64_t up_shift = (XS == 2 && pairs % GV_WAVES == 0 && !(flags & 1)) ? ((pairs / 2) & ~(int64_t)(GV_WAVES - 1)) : 0;
     bf16x8_t a_cur[D][R][2], b_cur[D][XS][NB][2];
     // GUARD: K is not a multiple of 64, the last pair is partly (or half) past the end of the rows
@@ -185,6 +206,11 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
         const int64_t ks[2] = {pr * 64, pu * 64};
 #pragma unroll
         for (int r = 0; r < R; r++) {
+          if (MIX) {   // gate rows at the pair itself, up rows at the shifted pair
+            a[d][r][0] = load_frag_nt(wbase[r] + ks[0] + offa[r], true);
+            a[d][r][1] = load_frag_nt(wbase[r] + ks[1] + offb[r], true);
+            continue;
+          }
           const int64_t k = ks[(XS == 2 && r >= R / 2) ? 1 : 0];
           a[d][r][0] = load_frag_nt(wbase[r] + k + offa[r], !GUARD || (k + 8 * lg < K));
           a[d][r][1] = load_frag_nt(wbase[r] + k + offb[r], !GUARD || (k + 32 + 8 * lg < K));
@@ -213,6 +239,14 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
             u32x4_t rt;
             rt.x = rot8_in_row(t.x); rt.y = rot8_in_row(t.y); rt.z = rot8_in_row(t.z); rt.w = rot8_in_row(t.w);
             h1 = __builtin_bit_cast(bf16x8_t, rt);
+          }
+          if (MIX) {
+            // rows 0-7 (gate) belong to k position 0, rows 8-15 (up) to position 1: both products, two accumulators
+            acc[r][0] = X::mfma16(h0, b_cur[d][0][0][0], acc[r][0]);
+            acc[r][0] = X::mfma16(h1, b_cur[d][0][0][1], acc[r][0]);
+            acc_up[r] = X::mfma16(h0, b_cur[d][XS - 1][0][0], acc_up[r]);
+            acc_up[r] = X::mfma16(h1, b_cur[d][XS - 1][0][1], acc_up[r]);
+            continue;
           }
           const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
 #pragma unroll
@@ -247,6 +281,12 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
       }
     }
     multiply();
+  }
+
+  if (MIX) {
+    // D[i][b]: lane groups 0 and 1 hold rows 0-7 (gate, from acc), groups 2 and 3 rows 8-15 (up, from acc_up)
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r][0] = lg < 2 ? acc[r][0] : acc_up[r];
   }
 
   // ---- sum the 8 k-slices through LDS: up to 8 tiles (row group x batch tile) per wave at a time, i.e. one
@@ -307,7 +347,25 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
     __syncthreads();
   }
 
-  if (MODE == 0) {
+  if (MODE == 3) {
+    // fin[b][16 r + i]: i < 8 gate row j0 + 8 r + i, i >= 8 the up row of gate row j0 + 8 r + i - 8
+    const int64_t j0 = (int64_t)blockIdx.x * (8 * R);
+    for (int e = tid; e < B * 8 * R; e += GV_THREADS) {
+      const int b = e / (8 * R), rl = e - b * (8 * R);
+      const int64_t jn = j0 + rl;
+      if (jn < half) {
+        const int col = 16 * (rl >> 3) + (rl & 7);
+        float gate = fin[b][col], up = fin[b][col + 8];
+        if (bias) {
+          gate += X::from_bits(bias[jn]);
+          up += X::from_bits(bias[half + jn]);
+        }
+        gate = X::from_bits(X::to_bits(gate));
+        up = X::from_bits(X::to_bits(up));
+        y[(int64_t)b * half + jn] = X::to_bits(silu_f(gate) * up);
+      }
+    }
+  } else if (MODE == 0) {
     const int64_t n0 = (int64_t)blockIdx.x * (16 * R);
     for (int e = tid; e < B * 16 * R; e += GV_THREADS) {
       const int b = e / (16 * R), rl = e - b * (16 * R);
@@ -568,6 +626,63 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   return MTP_OK;
 }
 
+// SwiGLU with mixed row groups (MODE 3): how many groups per workgroup.  0 = this shape keeps MODE 1.
+// Every CU should hold the same number of bytes in flight: prefer the R whose workgroup count fills whole
+// layers of 256 workgroups best, then the larger R (fewer reductions); too few workgroups are not an option.
+int pick_mixed_groups(int64_t B, int64_t N, int64_t K) {
+  const int64_t half = N / 2;
+  if (B > 16 || K % 64 != 0 || (K / 64) % GV_MAX_WAVES != 0 || (half + 64) * K >= (1ll << 32)) return 0;
+  if (const char* e = getenv("MTP_GEMV_MIX")) {
+    const int r = atoi(e);
+    return r >= 1 && r <= 7 ? r : 0;
+  }
+  const int64_t groups = (half + 7) / 8;
+  int best = 0;
+  double best_eff = 0.0;
+  for (int r = 1; r <= 7; r++) {
+    const int64_t wgs = (groups + r - 1) / r;
+    if (wgs < 200) continue;
+    const double eff = (double)wgs / (double)((wgs + 255) / 256 * 256);
+    if (eff >= best_eff - 1e-9) {
+      best_eff = eff;
+      best = r;
+    }
+  }
+  return best_eff >= 0.9 ? best : 0;   // MODE 1 with R = 4 reaches 0.875 on the usual shapes
+}
+
+int launch_gemv_mixed(const void* x, const void* w, const void* bias, void* y, int64_t B, int64_t N, int64_t K, int R,
+                      hipStream_t s, bool f16) {
+  const int64_t half = N / 2;
+  const unsigned n_wg = (unsigned)((half + 8 * R - 1) / (8 * R));
+  int rot_mul = 1;
+  if (const char* e = getenv("MTP_GEMV_ROT")) rot_mul = atoi(e);
+  if (rot_mul < 0) rot_mul = 0;
+#define GVM_T(RR, FF)                                                                                              \
+  hipLaunchKernelGGL((gemv_kernel<RR, 1, 3, false, 1, GV_MAX_WAVES, FF>), dim3(n_wg), dim3(GV_MAX_WAVES * MTP_WAVE), 0, \
+                     s, (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y,              \
+                     (ArgPart*)nullptr, (int)B, N, K, rot_mul, K, (float*)nullptr, (int32_t*)nullptr, 0)
+#define GVM(RR)                  \
+  case RR:                       \
+    if (f16) GVM_T(RR, true);    \
+    else GVM_T(RR, false);       \
+    break
+  switch (R) {
+    GVM(1);
+    GVM(2);
+    GVM(3);
+    GVM(4);
+    GVM(5);
+    GVM(6);
+    GVM(7);
+    default: mtp_set_error("gemv: %d mixed row groups", R); return MTP_EINVAL;
+  }
+#undef GVM
+#undef GVM_T
+  MTP_CHECK_LAUNCH("gemv");
+  return MTP_OK;
+}
+
 int check_gemv_args(const char* what, const void* x, const void* w, int64_t B, int64_t N, int64_t K, int dtype) {
   MTP_REQUIRE(dtype == MTP_BF16 || dtype == MTP_F16, MTP_EUNSUPPORTED, "%s: dtype %d (bf16 or f16)", what, dtype);
   MTP_REQUIRE(B >= 1 && B <= 32, MTP_EUNSUPPORTED, "%s: B=%lld outside [1,32]", what, (long long)B);
@@ -609,6 +724,7 @@ extern "C" int mtp_gemv_ws(const void* x, const void* w, const void* bias, void*
   const GemvCfg cfg = pick_gemv_cfg(B, N, K, mode, split);
   if (mode == 1) {
     MTP_REQUIRE(N % 2 == 0, MTP_EINVAL, "gemv: SwiGLU needs an even N, got %lld", (long long)N);
+    if (const int mixed = pick_mixed_groups(B, N, K)) return launch_gemv_mixed(x, w, bias, y, B, N, K, mixed, s, f16);
     return launch_gemv<1>(x, w, bias, y, nullptr, B, N, K, cfg, s, nullptr, f16, split ? workspace : nullptr);
   }
   return launch_gemv<0>(x, w, epilogue == MTP_EPI_NONE ? nullptr : bias, y, nullptr, B, N, K, cfg, s, nullptr, f16,

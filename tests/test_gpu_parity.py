@@ -926,3 +926,21 @@ def test_greedy_pick_over_a_vocab_sharded_lm_head(gpu):
     assert torch.equal(got[clear], ref[clear]) and torch.equal(full_idx.cpu()[clear], ref[clear])
     assert int(got[3]) in (1200, 5000) and int(ref[3]) == 1200   # the tie: equal to rounding across workgroups
     assert torch.allclose(vals.max(0).values, full_val.cpu(), rtol=1e-5)
+
+
+@pytest.mark.parametrize("mix", ["1", "2", "3", "4", "5", "6", "7", None])
+@pytest.mark.parametrize("b,half,k,with_bias", [(1, 14336, 4096, False), (8, 1000, 1024, True), (16, 56, 512, False),
+                                                (3, 3584, 8192, False)])
+def test_gemv_swiglu_mixed_row_groups(gpu, monkeypatch, mix, b, half, k, with_bias):
+    """SwiGLU GEMV whose 16-row tiles hold 8 gate rows and their 8 up rows, for every number of groups per
+    workgroup (forced) and for the automatic choice: same result as the oracle, ragged ends included."""
+    if mix is not None:
+        monkeypatch.setenv("MTP_GEMV_MIX", mix)
+    g = gen(41)
+    x = torch.randn(b, k, generator=g).bfloat16()
+    w = (torch.randn(2 * half, k, generator=g) * 0.03).bfloat16()
+    bias = (torch.randn(2 * half, generator=g) * 0.1).bfloat16() if with_bias else None
+    pre = F.linear(x.float(), w.float(), None if bias is None else bias.float()).bfloat16().float()
+    y = ops.gemv(x.to(gpu), w.to(gpu), None if bias is None else bias.to(gpu), ops.EPI_SWIGLU)
+    assert y.shape == (b, half) and rel(y, R.swiglu(pre)) < TOL_BF16
+    assert torch.equal(y, ops.gemv(x.to(gpu), w.to(gpu), None if bias is None else bias.to(gpu), ops.EPI_SWIGLU))

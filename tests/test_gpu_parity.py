@@ -944,3 +944,19 @@ def test_gemv_swiglu_mixed_row_groups(gpu, monkeypatch, mix, b, half, k, with_bi
     y = ops.gemv(x.to(gpu), w.to(gpu), None if bias is None else bias.to(gpu), ops.EPI_SWIGLU)
     assert y.shape == (b, half) and rel(y, R.swiglu(pre)) < TOL_BF16
     assert torch.equal(y, ops.gemv(x.to(gpu), w.to(gpu), None if bias is None else bias.to(gpu), ops.EPI_SWIGLU))
+
+
+def test_gemv_swiglu_seeded_sweep(gpu):
+    """30 seeded SwiGLU GEMV shapes (any batch up to 32, ragged halves, k multiples of 8) against the oracle."""
+    g = gen(43)
+    for case in range(30):
+        b = int(torch.randint(1, 33, (1,), generator=g))
+        half = int(torch.randint(1, 3000, (1,), generator=g))
+        k = 8 * int(torch.randint(1, 600, (1,), generator=g))
+        if case % 3 == 0:
+            k = 512 * int(torch.randint(1, 9, (1,), generator=g))           # the shapes the mixed row groups take
+        x = torch.randn(b, k, generator=g).bfloat16()
+        w = (torch.randn(2 * half, k, generator=g) * 0.03).bfloat16()
+        pre = F.linear(x.float(), w.float()).bfloat16().float()
+        y = ops.gemv(x.to(gpu), w.to(gpu), None, ops.EPI_SWIGLU)
+        assert rel(y, R.swiglu(pre)) < TOL_BF16, (case, b, half, k)

@@ -323,3 +323,45 @@ def test_llama_decoder_graph_replay_matches_eager(gpu):
     top2 = le.topk(2, dim=-1).values
     clear = (top2[:, 0] - top2[:, 1]) > 1e-2 * top2[:, 0].abs()
     assert tok_g.shape == (B,) and torch.equal(tok_g[clear], le.argmax(-1)[clear])
+
+
+def test_attn_decode_seeded_sweep(gpu):
+    """40 seeded cases over batch, head grouping, cache capacity, ragged lengths and dtype, plain and appending
+    forms, against the oracle."""
+    g = gen(50)
+    worst = 0.0
+    for case in range(40):
+        B = int(torch.randint(1, 9, (1,), generator=g))
+        group = [1, 2, 4, 8, 16][int(torch.randint(0, 5, (1,), generator=g))]
+        n_kv = int(torch.randint(1, 5, (1,), generator=g))
+        n_q = n_kv * group
+        max_len = int(torch.randint(1, 1200, (1,), generator=g))
+        dt = torch.bfloat16 if case % 2 == 0 else torch.float16
+        tol = TOL_BF16 if dt == torch.bfloat16 else 2e-3
+        lens = torch.randint(0, max_len + 1, (B,), generator=g)
+        q = torch.randn(B, n_q, 128, generator=g).to(dt)
+        kc = torch.randn(B, n_kv, max_len, 128, generator=g).to(dt)
+        vc = torch.randn(B, n_kv, max_len, 128, generator=g).to(dt)
+        ref = R.attn_decode(q.float(), kc.float(), vc.float(), lens)
+        out = ops.attn_decode(q.to(gpu), kc.to(gpu), vc.to(gpu), lens.to(gpu))
+        for b in range(B):
+            if int(lens[b]) == 0:
+                assert torch.count_nonzero(out[b]) == 0, (case, b)
+            else:
+                e = rel(out[b], ref[b])
+                worst = max(worst, e / tol)
+                assert e < tol, (case, b, B, n_q, n_kv, max_len, int(lens[b]), dt)
+        # the appending form at positions lens - 1 reproduces the same output when the cache row and qkv agree
+        pos = (lens - 1).clamp_min(0)
+        heads = torch.cat([q, torch.stack([kc[b, :, pos[b]] for b in range(B)]),
+                           torch.stack([vc[b, :, pos[b]] for b in range(B)])], dim=1)       # [B, n_q + 2 n_kv, 128]
+        ident_cos = torch.ones(max_len, 128).to(dt)                                         # rotation by zero
+        ident_sin = torch.zeros(max_len, 128).to(dt)
+        k2, v2 = kc.to(gpu), vc.to(gpu)
+        out2 = ops.attn_decode_append(heads.reshape(B, -1).to(gpu), ident_cos.to(gpu), ident_sin.to(gpu), pos.to(gpu),
+                                      k2, v2, n_q)
+        assert torch.equal(k2.cpu(), kc) and torch.equal(v2.cpu(), vc)                      # rewrote the same rows
+        for b in range(B):
+            if int(lens[b]) > 0:
+                assert rel(out2[b], ref[b]) < tol, ("append", case, b)
+    assert worst < 1.0

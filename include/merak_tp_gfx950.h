@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTP_ABI_VERSION 4
+#define MTP_ABI_VERSION 5
 
 /* element types.  MTP_F16 is IEEE half, what the reference's --fp16 sets as
  * params_dtype (Merak/merak_args/args.py:584-585). */
@@ -215,6 +215,29 @@ int64_t mtp_gemv_workspace_bytes(int64_t B, int64_t N, int64_t K, int epilogue);
 int mtp_gemv_ws(const void* x, const void* w, const void* bias, void* y,
                 void* workspace, int64_t workspace_bytes,
                 int64_t B, int64_t N, int64_t K, int epilogue, int dtype, void* stream);
+
+/* mtp_gemv_ws with what a decoder block puts around its linears (HF
+ * LlamaDecoderLayer.forward: `residual + hidden_states`, LlamaRMSNorm in
+ * front of the QKV and the gate/up projections), so that a block is five
+ * launches and the normalised row is never stored:
+ *   norm_weight != NULL: X is the residual stream and the product is taken
+ *     with RMSNorm(X) = norm_weight * dtype(x * rsqrt(mean_k x^2 + eps));
+ *     sumsq_in [B, K/16] fp32 holds the sums of squares of X per 16 elements
+ *     (what sumsq_out of the producing call wrote).  Every workgroup keeps
+ *     RMSNorm(X) in its LDS: K % 512 == 0, K <= 8192, B K <= 8 x 4096 elements
+ *     (mtp_gemv_norm_fits(B, K) == 1); both pointers 16-byte aligned; the
+ *     product is not cut along k.
+ *   residual != NULL ([B,N], epilogue NONE or BIAS):
+ *     y = dtype(dtype(W x + bias) + residual); y may be residual itself.
+ *   sumsq_out != NULL ([B, ceil(N/16)] fp32, epilogue NONE or BIAS): sum of
+ *     the squares of the stored y per batch row and 16 output rows.
+ * All three NULL: exactly mtp_gemv_ws. */
+int mtp_gemv_norm_fits(int64_t B, int64_t K);
+int mtp_gemv_fused(const void* x, const void* w, const void* bias, void* y,
+                   const void* norm_weight, const float* sumsq_in, float eps,
+                   const void* residual, float* sumsq_out,
+                   void* workspace, int64_t workspace_bytes,
+                   int64_t B, int64_t N, int64_t K, int epilogue, int dtype, void* stream);
 
 /* Bytes of device scratch mtp_gemv_argmax needs for this shape. */
 int64_t mtp_gemv_argmax_workspace_bytes(int64_t B, int64_t N, int64_t K);

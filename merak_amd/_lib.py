@@ -19,7 +19,7 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmerak_tp_gfx950.so"
 
 MTP_F32, MTP_BF16, MTP_F16 = 0, 1, 2
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_SWIGLU, EPI_GELU = 0, 1, 2, 3, 4
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _i64, _int, _vp = C.c_int64, C.c_int, C.c_void_p
 
@@ -48,6 +48,9 @@ SIGNATURES = {
     "mtp_sample_top_k_top_p": (_int, [_vp, _int, _i64, _i64, C.c_float, _int, C.c_float, _vp, _vp, _vp, _vp, _i64, _vp]),
     "mtp_gemv_workspace_bytes": (_i64, [_i64, _i64, _i64, _int]),
     "mtp_gemv_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
+    "mtp_gemv_norm_fits": (_int, [_i64, _i64]),
+    "mtp_gemv_fused": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, C.c_float, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int,
+                              _int, _vp]),
     "mtp_rmsnorm": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, C.c_float, _int, _vp]),
     "mtp_rope_kv_append": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _i64, _i64, _int, _vp]),
     "mtp_attn_decode_workspace_bytes": (_i64, [_i64, _int, _int, _i64]),

@@ -78,6 +78,21 @@ __device__ __forceinline__ uint32_t rot8_in_row(uint32_t v) {
   return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xf, 0xf, false);
 }
 
+// What a decoder block fuses around its linears.  NORM (template flag): X is the residual stream and the kernel
+// multiplies by RMSNorm(X) instead: y = W (g * dtype(x * rstd_b)), rstd_b = rsqrt(mean_k x[b,k]^2 + eps), with the
+// sum of squares handed over as partial sums per 16 elements (the producer below writes exactly those).  Every
+// workgroup builds RMSNorm(X) in its LDS while its first weights are on their way (up to 8 rows of 4096 elements,
+// see gemv_norm_fits) and takes its X fragments from there; the normalised rows never go to memory.
+// `residual` (plain stores only): y = dtype(dtype(W x + bias) + residual), the model's `residual + hidden_states`;
+// `sumsq_out`: per batch row and per 16 output rows, the sum of the squares of what was stored.
+struct GemvFuse {
+  const uint16_t* norm_w;    // NORM: RMSNorm weight [K]
+  const float* sumsq_in;     // NORM: [B, K / 16]
+  float eps;
+  const uint16_t* residual;  // [B, N] or null
+  float* sumsq_out;          // [B, ceil(N / 16)] or null
+};
+
 // MODE 0: store Y (+bias); MODE 1: SwiGLU store; MODE 2: argmax partials;
 // MODE 3: SwiGLU with mixed row groups: rows 0-7 of a 16-row MFMA tile are gate rows, rows 8-15 the matching up
 // rows, so a workgroup may own any number R of groups (8 R gate rows and their up rows) and the workgroup count can
@@ -88,14 +103,15 @@ __device__ __forceinline__ uint32_t rot8_in_row(uint32_t v) {
 // into two accumulators, and each lane keeps the one whose rows it owns.
 // W waves split K.  Configurations whose registers allow only 8 waves per CU run as two independent workgroups of
 // 4 waves rather than one of 8: while one sums its partial tiles and writes its outputs the other keeps streaming.
-template <int R, int NB, int MODE, bool GUARD, int D, int W, bool F16>
+template <int R, int NB, int MODE, bool GUARD, int D, int W, bool F16, bool NORM, bool PP>
 __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __restrict__ x,
                                                           const uint16_t* __restrict__ w,
                                                           const uint16_t* __restrict__ bias,
                                                           uint16_t* __restrict__ y, ArgPart* __restrict__ part,
                                                           int B, int64_t N, int64_t K, int rot_mul, int64_t ld,
                                                           float* __restrict__ kpart, int32_t* __restrict__ karrived,
-                                                          int flags) {
+                                                          int flags, const GemvFuse fz) {
+  static_assert(!NORM || (!GUARD && MODE != 2), "the norm prologue needs K % 64 == 0 and a stored output");
   // K is the extent along k that this workgroup covers and ld the row stride of X and W: with gridDim.y > 1
   // the k range is cut into gridDim.y slices of K elements, one workgroup per (row block, slice); the
   // slices' partial sums meet in `kpart` and the slice that delivers last adds them up in slice order.
@@ -187,100 +203,244 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   // D pairs (8 apart) per step: with few rows per workgroup this is what keeps enough bytes in flight.
   // The host only picks D > 1 when every wave's share of the pairs is a multiple of D.
   const int64_t n_it = ((pairs - p0 + GV_WAVES - 1) / GV_WAVES) / D;
-  if (n_it > 0) {
-    // SwiGLU: the "up" rows sit exactly N/2 rows below the "gate" rows of the same workgroup, for the usual
-    // shapes a large power of two apart, i.e. in the same memory channel and bank but another DRAM page.
-    // Walking both at the same k makes the two streams evict each other's open page, so the up rows walk
-    // half a row ahead (XS = 2 sets of X fragments, one per k position).
-    constexpr int XS = ((MODE == 1 || MODE == 3) && !GUARD && NB == 1) ? 2 : 1;
-    const int64_t up_shift = (XS == 2 && pairs % GV_WAVES == 0 && !(flags & 1)) ? ((pairs / 2) & ~(int64_t)(GV_WAVES - 1)) : 0;
-    bf16x8_t a_cur[D][R][2], b_cur[D][XS][NB][2];
-    // GUARD: K is not a multiple of 64, the last pair is partly (or half) past the end of the rows
-    auto load_set = [&](int64_t pq0, bf16x8_t (&a)[D][R][2], bf16x8_t (&b)[D][XS][NB][2]) {
+  // SwiGLU: the "up" rows sit exactly N/2 rows below the "gate" rows of the same workgroup, for the usual
+  // shapes a large power of two apart, i.e. in the same memory channel and bank but another DRAM page.
+  // Walking both at the same k makes the two streams evict each other's open page, so the up rows walk
+  // half a row ahead (XS = 2 sets of X fragments, one per k position).
+  constexpr int XS = ((MODE == 1 || MODE == 3) && !GUARD && NB == 1) ? 2 : 1;
+  const int64_t up_shift = (XS == 2 && pairs % GV_WAVES == 0 && !(flags & 1)) ? ((pairs / 2) & ~(int64_t)(GV_WAVES - 1)) : 0;
+  // Operand registers of one step.  PP: two such sets used in turn, the next step's requests go out before the
+  // current step's operands are waited for.  Otherwise one set is rotated by copying, which the compiler folds
+  // into the requests themselves: each goes out right behind the last MFMA that read its register.
+  bf16x8_t a_s0[D][R][2], b_s0[D][XS][NB][2];
+  bf16x8_t a_s1[D][R][2], b_s1[D][XS][NB][2];
+  // NORM: RMSNorm(X) is built once per workgroup in LDS, rows padded so that the 16-byte fragment reads of four
+  // batch rows fall into different banks
+  constexpr int XL_PAD = 32, XL_ELEMS = 8 * (4096 + XL_PAD);
+  [[maybe_unused]] const int xl_ld = (int)K + XL_PAD;
+  __shared__ uint16_t x_lds[NORM ? XL_ELEMS : 8];
+  const int b_row = li < B ? li : B - 1;
+  // GUARD: K is not a multiple of 64, the last pair is partly (or half) past the end of the rows
+  auto pair_k = [&](int64_t pq0, int d, int64_t (&ks)[2]) {
+    int64_t pr = pq0 + d * GV_WAVES;
+    if (pr >= pairs) pr -= pairs;
+    int64_t pu = pr + up_shift;
+    if (pu >= pairs) pu -= pairs;
+    ks[0] = pr * 64;
+    ks[1] = pu * 64;
+  };
+  auto load_w = [&](int64_t pq0, bf16x8_t (&a)[D][R][2]) {
 #pragma unroll
-      for (int d = 0; d < D; d++) {
-        int64_t pr = pq0 + d * GV_WAVES;
-        if (pr >= pairs) pr -= pairs;
-        int64_t pu = pr + up_shift;
-        if (pu >= pairs) pu -= pairs;
-        const int64_t ks[2] = {pr * 64, pu * 64};
+    for (int d = 0; d < D; d++) {
+      int64_t ks[2];
+      pair_k(pq0, d, ks);
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-          if (MIX) {   // gate rows at the pair itself, up rows at the shifted pair
-            a[d][r][0] = load_frag_nt(wbase[r] + ks[0] + offa[r], true);
-            a[d][r][1] = load_frag_nt(wbase[r] + ks[1] + offb[r], true);
-            continue;
-          }
-          const int64_t k = ks[(XS == 2 && r >= R / 2) ? 1 : 0];
-          a[d][r][0] = load_frag_nt(wbase[r] + k + offa[r], !GUARD || (k + 8 * lg < K));
-          a[d][r][1] = load_frag_nt(wbase[r] + k + offb[r], !GUARD || (k + 32 + 8 * lg < K));
+      for (int r = 0; r < R; r++) {
+        if (MIX) {   // gate rows at the pair itself, up rows at the shifted pair
+          a[d][r][0] = load_frag_nt(wbase[r] + ks[0] + offa[r], true);
+          a[d][r][1] = load_frag_nt(wbase[r] + ks[1] + offb[r], true);
+          continue;
         }
-#pragma unroll
-        for (int xs = 0; xs < XS; xs++)
-#pragma unroll
-          for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-            for (int hf = 0; hf < 2; hf++)
-              b[d][xs][nb][hf] = load_frag(xp[nb] + ks[xs] + 32 * hf, !GUARD || (ks[xs] + 32 * hf + 8 * lg < K));
-      }
-    };
-    auto multiply = [&]() {
-#pragma unroll
-      for (int d = 0; d < D; d++)
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-          // GUARD: a[0] / a[1] are the halves themselves.  Otherwise pick them per lane out of loads A and
-          // B; the second half then sits 8 lanes away inside its group of 16 (row i^8 at position i): one
-          // DPP rotation per register puts it in place.
-          bf16x8_t h0 = a_cur[d][r][0], h1 = a_cur[d][r][1];
-          if (!GUARD) {
-            h0 = low ? a_cur[d][r][0] : a_cur[d][r][1];
-            const u32x4_t t = __builtin_bit_cast(u32x4_t, low ? a_cur[d][r][1] : a_cur[d][r][0]);
-            u32x4_t rt;
-            rt.x = rot8_in_row(t.x); rt.y = rot8_in_row(t.y); rt.z = rot8_in_row(t.z); rt.w = rot8_in_row(t.w);
-            h1 = __builtin_bit_cast(bf16x8_t, rt);
-          }
-          if (MIX) {
-            // rows 0-7 (gate) belong to k position 0, rows 8-15 (up) to position 1: both products, two accumulators
-            acc[r][0] = X::mfma16(h0, b_cur[d][0][0][0], acc[r][0]);
-            acc[r][0] = X::mfma16(h1, b_cur[d][0][0][1], acc[r][0]);
-            acc_up[r] = X::mfma16(h0, b_cur[d][XS - 1][0][0], acc_up[r]);
-            acc_up[r] = X::mfma16(h1, b_cur[d][XS - 1][0][1], acc_up[r]);
-            continue;
-          }
-          const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
-#pragma unroll
-          for (int nb = 0; nb < NB; nb++) {
-            acc[r][nb] = X::mfma16(h0, b_cur[d][xs][nb][0], acc[r][nb]);
-            acc[r][nb] = X::mfma16(h1, b_cur[d][xs][nb][1], acc[r][nb]);
-          }
-        }
-    };
-    int64_t pq = p0 + rot;  // first pair of the step in flight; pairs % 8 == 0 whenever rot != 0, so wrapping keeps the wave's residue
-    if (pq >= pairs) pq -= pairs;
-    load_set(pq, a_cur, b_cur);
-    // all but the last step: fetch the next one (unconditionally: it exists), multiply the current one
-    for (int64_t it = 1; it < n_it; it++) {
-      bf16x8_t a_nxt[D][R][2], b_nxt[D][XS][NB][2];
-      pq += GV_WAVES * D;
-      if (pq >= pairs) pq -= pairs;
-      load_set(pq, a_nxt, b_nxt);
-      multiply();
-#pragma unroll
-      for (int d = 0; d < D; d++) {
-#pragma unroll
-        for (int r = 0; r < R; r++)
-#pragma unroll
-          for (int hf = 0; hf < 2; hf++) a_cur[d][r][hf] = a_nxt[d][r][hf];
-#pragma unroll
-        for (int xs = 0; xs < XS; xs++)
-#pragma unroll
-          for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-            for (int hf = 0; hf < 2; hf++) b_cur[d][xs][nb][hf] = b_nxt[d][xs][nb][hf];
+        const int64_t k = ks[(XS == 2 && r >= R / 2) ? 1 : 0];
+        a[d][r][0] = load_frag_nt(wbase[r] + k + offa[r], !GUARD || (k + 8 * lg < K));
+        a[d][r][1] = load_frag_nt(wbase[r] + k + offb[r], !GUARD || (k + 32 + 8 * lg < K));
       }
     }
-    multiply();
+  };
+  auto load_x = [&](int64_t pq0, bf16x8_t (&b)[D][XS][NB][2]) {
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+      int64_t ks[2];
+      pair_k(pq0, d, ks);
+#pragma unroll
+      for (int xs = 0; xs < XS; xs++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+          for (int hf = 0; hf < 2; hf++) {
+            if constexpr (NORM)
+              b[d][xs][nb][hf] = *reinterpret_cast<const bf16x8_t*>(&x_lds[b_row * xl_ld + (int)ks[xs] + 32 * hf + 8 * lg]);
+            else
+              b[d][xs][nb][hf] = load_frag(xp[nb] + ks[xs] + 32 * hf, !GUARD || (ks[xs] + 32 * hf + 8 * lg < K));
+          }
+    }
+  };
+  auto load_set = [&](int64_t pq0, bf16x8_t (&a)[D][R][2], bf16x8_t (&b)[D][XS][NB][2]) {
+    load_w(pq0, a);
+    load_x(pq0, b);
+  };
+  auto multiply = [&](bf16x8_t (&a_cur)[D][R][2], bf16x8_t (&b_cur)[D][XS][NB][2]) {
+#pragma unroll
+    for (int d = 0; d < D; d++)
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        // GUARD: a[0] / a[1] are the halves themselves.  Otherwise pick them per lane out of loads A and
+        // B; the second half then sits 8 lanes away inside its group of 16 (row i^8 at position i): one
+        // DPP rotation per register puts it in place.
+        bf16x8_t h0 = a_cur[d][r][0], h1 = a_cur[d][r][1];
+        if (!GUARD) {
+          h0 = low ? a_cur[d][r][0] : a_cur[d][r][1];
+          const u32x4_t t = __builtin_bit_cast(u32x4_t, low ? a_cur[d][r][1] : a_cur[d][r][0]);
+          u32x4_t rt;
+          rt.x = rot8_in_row(t.x); rt.y = rot8_in_row(t.y); rt.z = rot8_in_row(t.z); rt.w = rot8_in_row(t.w);
+          h1 = __builtin_bit_cast(bf16x8_t, rt);
+        }
+        if (MIX) {
+          // rows 0-7 (gate) belong to k position 0, rows 8-15 (up) to position 1: both products, two accumulators
+          acc[r][0] = X::mfma16(h0, b_cur[d][0][0][0], acc[r][0]);
+          acc[r][0] = X::mfma16(h1, b_cur[d][0][0][1], acc[r][0]);
+          acc_up[r] = X::mfma16(h0, b_cur[d][XS - 1][0][0], acc_up[r]);
+          acc_up[r] = X::mfma16(h1, b_cur[d][XS - 1][0][1], acc_up[r]);
+          continue;
+        }
+        const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+          acc[r][nb] = X::mfma16(h0, b_cur[d][xs][nb][0], acc[r][nb]);
+          acc[r][nb] = X::mfma16(h1, b_cur[d][xs][nb][1], acc[r][nb]);
+        }
+      }
+  };
+
+  // NORM prologue, part 1: everything it reads is asked for before the first weights, folded after them, so
+  // that the reduction, the normalisation and their two barriers sit inside the latency of that first request.
+  //  * the row statistics: 16 lanes per batch row add up its partial sums of squares (16 bytes per load);
+  //  * the rows themselves: thread t owns the 16-byte pieces t, t + 512, ... of every row and the matching
+  //    pieces of the norm weight (B K <= 8 x 4096 elements: at most 8 pieces of X per thread).
+  static_assert(!NORM || (NB == 1 && W == 8 && !GUARD && MODE != 2), "norm prologue: up to 8 rows, 512 threads, K % 64 == 0");
+  constexpr int SQ_LOADS = 8, XV = 8;
+  [[maybe_unused]] f32x4_t sv[SQ_LOADS];
+  [[maybe_unused]] u32x4_t xv[XV], gv[XV];
+  [[maybe_unused]] const int sq_nq = (int)(K >> 6);   // 16-byte groups of partial sums per row: (K / 16) / 4
+  [[maybe_unused]] const int sq_b = tid >> 4, sq_sub = tid & 15;
+  [[maybe_unused]] const int kvecs = (int)(K >> 3), kv_per = (kvecs + GV_THREADS - 1) / GV_THREADS;   // pieces per row / thread
+  if constexpr (NORM) {
+    const f32x4_t* sp = reinterpret_cast<const f32x4_t*>(fz.sumsq_in + (int64_t)(sq_b < B ? sq_b : 0) * (K >> 4));
+#pragma unroll
+    for (int u = 0; u < SQ_LOADS; u++) {   // no branches: out-of-range lanes read element 0 and drop it later
+      const int q = sq_sub + 16 * u;
+      sv[u] = sp[q < sq_nq ? q : 0];
+    }
+#pragma unroll
+    for (int u = 0; u < XV; u++) {         // piece u: k-vector u % kv_per of batch row u / kv_per
+      const int j = u % kv_per, b = u / kv_per;
+      const int kv = tid + GV_THREADS * j;
+      const bool ok = b < B && kv < kvecs;
+      xv[u] = reinterpret_cast<const u32x4_t*>(x + (int64_t)(ok ? b : 0) * ld)[ok ? kv : 0];
+      gv[u] = reinterpret_cast<const u32x4_t*>(fz.norm_w)[ok ? kv : 0];
+    }
+  }
+
+  int64_t pq = p0 + rot;  // first pair of the step in flight; pairs % 8 == 0 whenever rot != 0, so wrapping keeps the wave's residue
+  if (pq >= pairs) pq -= pairs;
+  // (NORM: the host only launches with an equal, non-zero share of pairs for every wave; leaving the condition
+  // out keeps the wait for the prologue's loads from covering these younger requests as well)
+  if (NORM || n_it > 0) load_w(pq, a_s0);
+  if constexpr (NORM) __builtin_amdgcn_sched_barrier(0);   // nothing of the prologue is waited for before this point
+  if constexpr (!NORM) {
+    if (n_it > 0) load_x(pq, b_s0);
+  } else {
+    // part 2: scale of every row, then the normalised rows into LDS
+    __shared__ float rstd_lds[32];
+    {
+      float s = 0.f;
+#pragma unroll
+      for (int u = 0; u < SQ_LOADS; u++)
+        if (sq_b < B && sq_sub + 16 * u < sq_nq) s += (sv[u][0] + sv[u][1]) + (sv[u][2] + sv[u][3]);
+      // the same order in all 16 lanes of a row: every lane ends with the same bits
+      s += __shfl_xor(s, 8, 64);
+      s += __shfl_xor(s, 4, 64);
+      s += __shfl_xor(s, 2, 64);
+      s += __shfl_xor(s, 1, 64);
+      if (sq_sub == 0) rstd_lds[sq_b] = sq_b < B ? rsqrtf(s / (float)K + fz.eps) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < XV; u++) {
+      const int j = u % kv_per, b = u / kv_per;
+      const int kv = tid + GV_THREADS * j;
+      if (b < B && kv < kvecs) {
+        const float rs = rstd_lds[b];
+        u32x4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          // g * dtype(x * rstd): the scaling in fp32, rounded to the tensor dtype, the product with the weight in
+          // the tensor dtype (HF LlamaRMSNorm.forward)
+          const uint32_t n = X::pack2(X::lo(xv[u][e]) * rs, X::hi(xv[u][e]) * rs);
+          o[e] = X::pack2(X::lo(gv[u][e]) * X::lo(n), X::hi(gv[u][e]) * X::hi(n));
+        }
+        *reinterpret_cast<u32x4_t*>(&x_lds[b * xl_ld + 8 * kv]) = o;
+      }
+    }
+    __syncthreads();
+    load_x(pq, b_s0);
+  }
+
+  if (n_it > 0) {
+    auto advance = [&]() {
+      pq += GV_WAVES * D;
+      if (pq >= pairs) pq -= pairs;
+    };
+    if constexpr (PP) {
+      // set 0 holds the oldest step that has not been multiplied yet
+      int64_t it = 1;
+      for (; it + 1 < n_it; it += 2) {
+        advance();
+        load_set(pq, a_s1, b_s1);
+        __builtin_amdgcn_sched_barrier(0);   // requests first, then the wait for the older set
+        multiply(a_s0, b_s0);
+        advance();
+        load_set(pq, a_s0, b_s0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(a_s1, b_s1);
+      }
+      if (it < n_it) {
+        advance();
+        load_set(pq, a_s1, b_s1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(a_s0, b_s0);
+        multiply(a_s1, b_s1);
+      } else {
+        multiply(a_s0, b_s0);
+      }
+    } else {
+      for (int64_t it = 1; it < n_it; it++) {
+        advance();
+        load_set(pq, a_s1, b_s1);
+        multiply(a_s0, b_s0);
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+#pragma unroll
+          for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) a_s0[d][r][hf] = a_s1[d][r][hf];
+#pragma unroll
+          for (int xs = 0; xs < XS; xs++)
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+              for (int hf = 0; hf < 2; hf++) b_s0[d][xs][nb][hf] = b_s1[d][xs][nb][hf];
+        }
+      }
+      multiply(a_s0, b_s0);
+    }
+  }
+
+  // MODE 0 stores B x 16 R values, EPT per thread at most.  The residual values they are added to are asked for
+  // here, ahead of the reduction below, and all of a thread's loads come before its stores (y may be the
+  // residual tensor itself: a thread reads and writes the same elements).
+  constexpr int EPT = (16 * NB * 16 * R + GV_THREADS - 1) / GV_THREADS;
+  [[maybe_unused]] uint16_t rres[EPT];
+  if constexpr (MODE == 0) {
+    if (fz.residual) {
+#pragma unroll
+      for (int i = 0; i < EPT; i++) {
+        const int e = i * GV_THREADS + tid;
+        const int b = e / (16 * R), rl = e - b * (16 * R);
+        const int64_t n = (int64_t)blockIdx.x * (16 * R) + rl;
+        rres[i] = (e < B * 16 * R && n < N) ? fz.residual[(int64_t)b * N + n] : (uint16_t)0;
+      }
+    }
   }
 
   if (MIX) {
@@ -366,14 +526,33 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
       }
     }
   } else if (MODE == 0) {
+    // 16 consecutive lanes hold 16 consecutive output rows of one batch row: their squares meet in one
+    // partial sum (fixed butterfly order), which is what the norm prologue of the next linear adds up
     const int64_t n0 = (int64_t)blockIdx.x * (16 * R);
-    for (int e = tid; e < B * 16 * R; e += GV_THREADS) {
-      const int b = e / (16 * R), rl = e - b * (16 * R);
+    const int total = B * 16 * R;
+    const int64_t parts_out = (N + 15) >> 4;
+#pragma unroll
+    for (int i = 0; i < EPT; i++) {
+      const int e = i * GV_THREADS + tid;
+      const bool on = e < total;
+      const int b = on ? e / (16 * R) : 0, rl = on ? e - b * (16 * R) : 0;
       const int64_t n = n0 + rl;
-      if (n < N) {
+      float sq = 0.f;
+      if (on && n < N) {
         float v = fin[b][rl];
         if (bias) v += X::from_bits(bias[n]);
-        y[(int64_t)b * N + n] = X::to_bits(v);
+        uint16_t out = X::to_bits(v);
+        if (fz.residual) out = X::to_bits(X::from_bits(out) + X::from_bits(rres[i]));
+        y[(int64_t)b * N + n] = out;
+        const float f = X::from_bits(out);
+        sq = f * f;
+      }
+      if (fz.sumsq_out && i * GV_THREADS < total) {   // (uniform over the workgroup)
+        sq += __shfl_xor(sq, 8, 64);
+        sq += __shfl_xor(sq, 4, 64);
+        sq += __shfl_xor(sq, 2, 64);
+        sq += __shfl_xor(sq, 1, 64);
+        if (on && (rl & 15) == 0 && n < N) fz.sumsq_out[(int64_t)b * parts_out + (n >> 4)] = sq;
       }
     }
   } else if (MODE == 1) {
@@ -571,9 +750,10 @@ GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode, bool may_split 
 // bytes of the arrival counters in front of the partial sums: one per 16 rows covers every configuration
 int64_t gemv_counter_bytes(int64_t N) { return ((N + 15) / 16 * (int64_t)sizeof(int32_t) + 255) / 256 * 256; }
 
-template <int MODE>
+template <int MODE, bool NORM = false>
 int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart* part, int64_t B, int64_t N,
-                int64_t K, GemvCfg cfg, hipStream_t s, unsigned* n_wg_out, bool f16, void* workspace = nullptr) {
+                int64_t K, GemvCfg cfg, hipStream_t s, unsigned* n_wg_out, bool f16, void* workspace = nullptr,
+                GemvFuse fz = GemvFuse{nullptr, nullptr, 0.f, nullptr, nullptr}) {
   const int R = cfg.R;
   const int64_t rows_per_wg = (MODE == 1) ? 8 * R : 16 * R;
   const int64_t span = (MODE == 1) ? N / 2 : N;
@@ -590,11 +770,13 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   int32_t* karrived = static_cast<int32_t*>(workspace);
   float* kpart = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + gemv_counter_bytes(N)) : nullptr;
   const int64_t k_slice = K / S;
+// two operand sets wherever the registers hold them (8 waves: 256 per lane)
+#define GV_PP(RR, NNB) (MODE != 2)
 #define GV_LAUNCH_T(RR, NNB, GG, DD, FF)                                                                        \
-  hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD, (RR >= 8 ? 4 : 8), FF>), dim3(n_wg, S),                \
+  hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD, (RR >= 8 ? 4 : 8), FF, NORM, GV_PP(RR, NNB)>), dim3(n_wg, S), \
                      dim3((RR >= 8 ? 4 : 8) * MTP_WAVE), 0, s,                                                  \
                      (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part, (int)B, \
-                     N, k_slice, rot_mul, K, kpart, karrived, flags)
+                     N, k_slice, rot_mul, K, kpart, karrived, flags, fz)
 #define GV_LAUNCH(RR, NNB, GG, DD)                 \
   do {                                             \
     if (f16) GV_LAUNCH_T(RR, NNB, GG, DD, true);   \
@@ -602,18 +784,20 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   } while (0)
 #define GV_BY_DEPTH(RR, NNB)                                                   \
   do {                                                                         \
-    if (K % 64 != 0) GV_LAUNCH(RR, NNB, true, 1);                              \
-    else if (S > 1) GV_LAUNCH(RR, NNB, false, 1);                              \
+    if (K % 64 != 0) {                                                         \
+      if constexpr (!NORM) GV_LAUNCH(RR, NNB, true, 1);                        \
+    } else if (S > 1) GV_LAUNCH(RR, NNB, false, 1);                            \
     else if (RR * 4 <= 4 && cfg.D == 4) GV_LAUNCH(RR, NNB, false, (RR * 4 <= 4 ? 4 : 1)); \
     else if (RR * 2 <= 4 && cfg.D == 2) GV_LAUNCH(RR, NNB, false, (RR * 2 <= 4 ? 2 : 1)); \
     else GV_LAUNCH(RR, NNB, false, 1);                                         \
   } while (0)
   if (NB == 1) {
-    if (R == 8) GV_BY_DEPTH(8, 1);
-    else if (R == 4) GV_BY_DEPTH(4, 1);
+    if (R == 8) {
+      if constexpr (!NORM) GV_BY_DEPTH(8, 1);   // 4 waves: batches above 16 only
+    } else if (R == 4) GV_BY_DEPTH(4, 1);
     else if (R == 2) GV_BY_DEPTH(2, 1);
     else if constexpr (MODE != 1) GV_BY_DEPTH(1, 1);
-  } else {
+  } else if constexpr (!NORM) {
     if (R == 8) GV_BY_DEPTH(8, 2);
     else if (R == 4) GV_BY_DEPTH(4, 2);
     else if (R == 2) GV_BY_DEPTH(2, 2);
@@ -622,6 +806,7 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
 #undef GV_BY_DEPTH
 #undef GV_LAUNCH
 #undef GV_LAUNCH_T
+#undef GV_PP
   MTP_CHECK_LAUNCH("gemv");
   return MTP_OK;
 }
@@ -651,17 +836,19 @@ int pick_mixed_groups(int64_t B, int64_t N, int64_t K) {
   return best_eff >= 0.9 ? best : 0;   // MODE 1 with R = 4 reaches 0.875 on the usual shapes
 }
 
+template <bool NORM = false>
 int launch_gemv_mixed(const void* x, const void* w, const void* bias, void* y, int64_t B, int64_t N, int64_t K, int R,
-                      hipStream_t s, bool f16) {
+                      hipStream_t s, bool f16, GemvFuse fz = GemvFuse{nullptr, nullptr, 0.f, nullptr, nullptr}) {
   const int64_t half = N / 2;
   const unsigned n_wg = (unsigned)((half + 8 * R - 1) / (8 * R));
   int rot_mul = 1;
   if (const char* e = getenv("MTP_GEMV_ROT")) rot_mul = atoi(e);
   if (rot_mul < 0) rot_mul = 0;
 #define GVM_T(RR, FF)                                                                                              \
-  hipLaunchKernelGGL((gemv_kernel<RR, 1, 3, false, 1, GV_MAX_WAVES, FF>), dim3(n_wg), dim3(GV_MAX_WAVES * MTP_WAVE), 0, \
-                     s, (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y,              \
-                     (ArgPart*)nullptr, (int)B, N, K, rot_mul, K, (float*)nullptr, (int32_t*)nullptr, 0)
+  hipLaunchKernelGGL((gemv_kernel<RR, 1, 3, false, 1, GV_MAX_WAVES, FF, NORM, (RR <= 6)>), dim3(n_wg),                \
+                     dim3(GV_MAX_WAVES * MTP_WAVE), 0, s, (const uint16_t*)x, (const uint16_t*)w,                 \
+                     (const uint16_t*)bias, (uint16_t*)y, (ArgPart*)nullptr, (int)B, N, K, rot_mul, K,            \
+                     (float*)nullptr, (int32_t*)nullptr, 0, fz)
 #define GVM(RR)                  \
   case RR:                       \
     if (f16) GVM_T(RR, true);    \
@@ -681,6 +868,14 @@ int launch_gemv_mixed(const void* x, const void* w, const void* bias, void* y, i
 #undef GVM_T
   MTP_CHECK_LAUNCH("gemv");
   return MTP_OK;
+}
+
+// the norm prologue keeps RMSNorm(X) in LDS (8 rows of 4096 + 32 elements) and every thread of the 512 holds
+// at most 8 sixteen-byte pieces of X on the way there
+bool gemv_norm_fits(int64_t B, int64_t K) {
+  if (B < 1 || K < 512 || K % 512 != 0 || K > 8192) return false;   // 8192 / 16 partial sums: 8 loads of 16 lanes
+  const int64_t per_thread = (K / 8 + 511) / 512;
+  return per_thread * B <= 8 && B * (K + 32) <= 8 * (4096 + 32);
 }
 
 int check_gemv_args(const char* what, const void* x, const void* w, int64_t B, int64_t N, int64_t K, int dtype) {
@@ -706,9 +901,9 @@ extern "C" int64_t mtp_gemv_workspace_bytes(int64_t B, int64_t N, int64_t K, int
   return gemv_counter_bytes(N) + (int64_t)c.S * B * rows * (int64_t)sizeof(float);
 }
 
-extern "C" int mtp_gemv_ws(const void* x, const void* w, const void* bias, void* y, void* workspace,
-                           int64_t workspace_bytes, int64_t B, int64_t N, int64_t K, int epilogue, int dtype,
-                           void* stream) {
+namespace {
+int gemv_dispatch(const void* x, const void* w, const void* bias, void* y, void* workspace, int64_t workspace_bytes,
+                  int64_t B, int64_t N, int64_t K, int epilogue, int dtype, void* stream, GemvFuse fz) {
   int rc = check_gemv_args("gemv", x, w, B, N, K, dtype);
   const bool f16 = dtype == MTP_F16;
   if (rc) return rc;
@@ -718,17 +913,58 @@ extern "C" int mtp_gemv_ws(const void* x, const void* w, const void* bias, void*
   MTP_REQUIRE(epilogue != MTP_EPI_BIAS || bias, MTP_EINVAL, "gemv: MTP_EPI_BIAS without bias");
   hipStream_t s = (hipStream_t)stream;
   const int mode = epilogue == MTP_EPI_SWIGLU ? 1 : 0;
-  // without a workspace (or with one too small for the slices) every workgroup walks all of k
-  const int64_t need = workspace ? mtp_gemv_workspace_bytes(B, N, K, epilogue) : 0;
+  const bool norm = fz.norm_w != nullptr;
+  // without a workspace (or with one too small for the slices) every workgroup walks all of k; so does the
+  // norm prologue, whose row statistics cover all of k
+  const int64_t need = workspace && !norm ? mtp_gemv_workspace_bytes(B, N, K, epilogue) : 0;
   const bool split = need > 0 && workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0;
   const GemvCfg cfg = pick_gemv_cfg(B, N, K, mode, split);
   if (mode == 1) {
     MTP_REQUIRE(N % 2 == 0, MTP_EINVAL, "gemv: SwiGLU needs an even N, got %lld", (long long)N);
-    if (const int mixed = pick_mixed_groups(B, N, K)) return launch_gemv_mixed(x, w, bias, y, B, N, K, mixed, s, f16);
-    return launch_gemv<1>(x, w, bias, y, nullptr, B, N, K, cfg, s, nullptr, f16, split ? workspace : nullptr);
+    if (const int mixed = pick_mixed_groups(B, N, K))
+      return norm ? launch_gemv_mixed<true>(x, w, bias, y, B, N, K, mixed, s, f16, fz)
+                  : launch_gemv_mixed<false>(x, w, bias, y, B, N, K, mixed, s, f16, fz);
+    if (norm) return launch_gemv<1, true>(x, w, bias, y, nullptr, B, N, K, cfg, s, nullptr, f16, nullptr, fz);
+    return launch_gemv<1>(x, w, bias, y, nullptr, B, N, K, cfg, s, nullptr, f16, split ? workspace : nullptr, fz);
   }
-  return launch_gemv<0>(x, w, epilogue == MTP_EPI_NONE ? nullptr : bias, y, nullptr, B, N, K, cfg, s, nullptr, f16,
-                        split ? workspace : nullptr);
+  const void* b0 = epilogue == MTP_EPI_NONE ? nullptr : bias;
+  if (norm) return launch_gemv<0, true>(x, w, b0, y, nullptr, B, N, K, cfg, s, nullptr, f16, nullptr, fz);
+  return launch_gemv<0>(x, w, b0, y, nullptr, B, N, K, cfg, s, nullptr, f16, split ? workspace : nullptr, fz);
+}
+}  // namespace
+
+extern "C" int mtp_gemv_ws(const void* x, const void* w, const void* bias, void* y, void* workspace,
+                           int64_t workspace_bytes, int64_t B, int64_t N, int64_t K, int epilogue, int dtype,
+                           void* stream) {
+  return gemv_dispatch(x, w, bias, y, workspace, workspace_bytes, B, N, K, epilogue, dtype, stream,
+                       GemvFuse{nullptr, nullptr, 0.f, nullptr, nullptr});
+}
+
+extern "C" int mtp_gemv_norm_fits(int64_t B, int64_t K) { return gemv_norm_fits(B, K) ? 1 : 0; }
+
+extern "C" int mtp_gemv_fused(const void* x, const void* w, const void* bias, void* y, const void* norm_weight,
+                              const float* sumsq_in, float eps, const void* residual, float* sumsq_out,
+                              void* workspace, int64_t workspace_bytes, int64_t B, int64_t N, int64_t K, int epilogue,
+                              int dtype, void* stream) {
+  if (norm_weight || sumsq_in) {
+    MTP_REQUIRE(norm_weight && sumsq_in, MTP_EINVAL, "gemv_fused: the norm prologue needs its weight and the sums of squares");
+    // every wave of a workgroup walks the same number of 64-element pairs, and a row's partial sums (one per 16
+    // elements) are read 16 bytes at a time
+    MTP_REQUIRE(K % 512 == 0, MTP_EUNSUPPORTED, "gemv_fused: the norm prologue needs K %% 512 == 0, got %lld", (long long)K);
+    MTP_REQUIRE(gemv_norm_fits(B, K), MTP_EUNSUPPORTED,
+                "gemv_fused: the norm prologue holds B K <= 8 x 4096 elements, K <= 8192, got B=%lld K=%lld (mtp_gemv_norm_fits)",
+                (long long)B, (long long)K);
+    MTP_REQUIRE(((reinterpret_cast<uintptr_t>(norm_weight) | reinterpret_cast<uintptr_t>(sumsq_in)) & 15) == 0,
+                MTP_EUNSUPPORTED, "gemv_fused: norm_weight and sumsq_in must be 16-byte aligned");
+    MTP_REQUIRE(eps >= 0.f, MTP_EINVAL, "gemv_fused: eps %g", (double)eps);
+  }
+  if (residual || sumsq_out) {
+    MTP_REQUIRE(epilogue == MTP_EPI_NONE || epilogue == MTP_EPI_BIAS, MTP_EINVAL,
+                "gemv_fused: residual / sumsq_out go with plain stores, not epilogue %d", epilogue);
+    MTP_REQUIRE((reinterpret_cast<uintptr_t>(sumsq_out) & 3) == 0, MTP_EINVAL, "gemv_fused: sumsq_out not 4-byte aligned");
+  }
+  return gemv_dispatch(x, w, bias, y, workspace, workspace_bytes, B, N, K, epilogue, dtype, stream,
+                       GemvFuse{(const uint16_t*)norm_weight, sumsq_in, eps, (const uint16_t*)residual, sumsq_out});
 }
 
 extern "C" int mtp_gemv(const void* x, const void* w, const void* bias, void* y, int64_t B, int64_t N, int64_t K,

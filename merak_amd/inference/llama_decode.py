@@ -67,11 +67,16 @@ class LlamaDecoder:
     def __init__(self, embed: torch.Tensor, blocks: List[LlamaBlockWeights], final_norm: torch.Tensor,
                  lm_head: torch.Tensor, n_q_heads: int, n_kv_heads: int, head_dim: int = 128, eps: float = 1e-5,
                  rope_theta: float = 10000.0, rope_scaling: Optional[dict] = None, max_len: int = 4096,
-                 batch: int = 1):
+                 batch: int = 1, fused: Optional[bool] = None):
         dev, dt = lm_head.device, lm_head.dtype
         self.embed, self.blocks, self.final_norm, self.lm_head = embed, blocks, final_norm, lm_head
         self.n_q, self.n_kv, self.head_dim, self.eps = n_q_heads, n_kv_heads, head_dim, eps
         self.max_len, self.batch = max_len, batch
+        # norms and residual adds inside the linears: the norm prologue keeps the batch's normalised rows in LDS
+        can_fuse = ops.gemv_norm_fits(batch, embed.shape[1])
+        if fused and not can_fuse:
+            raise ValueError(f"fused=True needs batch x hidden <= 8 x 4096 and hidden % 512 == 0, got {batch} x {embed.shape[1]}")
+        self.fused = can_fuse if fused is None else bool(fused)
         self.cos, self.sin = rope_tables(head_dim, max_len, rope_theta, rope_scaling, dtype=dt, device=dev)
         self.k_cache = [torch.zeros((batch, n_kv_heads, max_len, head_dim), dtype=dt, device=dev) for _ in blocks]
         self.v_cache = [torch.zeros((batch, n_kv_heads, max_len, head_dim), dtype=dt, device=dev) for _ in blocks]
@@ -90,7 +95,7 @@ class LlamaDecoder:
         self.gemv_ws = max(need, key=lambda t: t.numel()) if need else None
 
     @classmethod
-    def from_hf(cls, model, max_len: int = 4096, batch: int = 1):
+    def from_hf(cls, model, max_len: int = 4096, batch: int = 1, fused: Optional[bool] = None):
         """From a ``transformers`` ``LlamaForCausalLM`` (weights are concatenated once, not shared)."""
         cfg = model.config
         blocks = []
@@ -108,13 +113,15 @@ class LlamaDecoder:
         head_dim = getattr(cfg, "head_dim", None) or cfg.hidden_size // cfg.num_attention_heads
         return cls(model.model.embed_tokens.weight.data, blocks, model.model.norm.weight.data,
                    model.lm_head.weight.data, cfg.num_attention_heads, cfg.num_key_value_heads, head_dim,
-                   cfg.rms_norm_eps, theta, scaling, max_len, batch)
+                   cfg.rms_norm_eps, theta, scaling, max_len, batch, fused)
 
     def reset(self):
         self.lens.zero_()
         self.host_len_bound = 0
 
     def _hidden(self, tokens: torch.Tensor, len_bound: int) -> torch.Tensor:
+        if self.fused:
+            return self._hidden_fused(tokens, len_bound)
         positions = self.lens             # tokens cached so far = position of the new one
         x = ops.embedding_gather(tokens, self.embed, 0, self.embed.shape[0])
         residual = None
@@ -130,6 +137,27 @@ class LlamaDecoder:
             x = ops.gemv(act, w.down, workspace=self.gemv_ws)
         self.lens += 1
         return ops.rmsnorm(x, self.final_norm, self.eps, residual)
+
+    def _hidden_fused(self, tokens: torch.Tensor, len_bound: int) -> torch.Tensor:
+        """Five launches per block: the two RMSNorms ride in the QKV and gate/up products (the o and down products
+        hand them the sums of squares of the residual stream they write), the residual adds in the o and down
+        products.  The rounding steps are those of the seven-launch form."""
+        positions = self.lens
+        x = ops.embedding_gather(tokens, self.embed, 0, self.embed.shape[0])      # the residual stream
+        B = x.shape[0]
+        ss = None
+        for w, kc, vc in zip(self.blocks, self.k_cache, self.v_cache):
+            if ss is None:      # first block: the stream comes from the embedding, nobody has summed its squares
+                qkv = ops.gemv(ops.rmsnorm(x, w.input_norm, self.eps), w.qkv, workspace=self.gemv_ws)
+            else:
+                qkv = ops.gemv_fused(x, w.qkv, norm_weight=w.input_norm, sumsq_in=ss, eps=self.eps)
+            a = ops.attn_decode_append(qkv, self.cos, self.sin, positions, kc, vc, self.n_q, len_bound=len_bound,
+                                       workspace=self.attn_ws)
+            x, ss = ops.gemv_fused(a.view(B, -1), w.o, residual=x, want_sumsq=True, workspace=self.gemv_ws)
+            act = ops.gemv_fused(x, w.gate_up, None, ops.EPI_SWIGLU, norm_weight=w.post_norm, sumsq_in=ss, eps=self.eps)
+            x, ss = ops.gemv_fused(act, w.down, residual=x, want_sumsq=True, workspace=self.gemv_ws)
+        self.lens += 1
+        return ops.rmsnorm(x, self.final_norm, self.eps)
 
     def capture(self):
         """Records one step (all blocks, final norm, LM head with argmax) into a HIP graph; ``hidden`` / ``logits``

@@ -296,6 +296,48 @@ def gemv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     return y
 
 
+def gemv_norm_fits(B: int, K: int) -> bool:
+    """Whether ``gemv_fused`` can take the RMSNorm of a [B, K] input inside the product (B K <= 8 x 4096, K % 512 == 0, K <= 8192)."""
+    return bool(_lib.lib().mtp_gemv_norm_fits(B, K))
+
+
+def gemv_fused(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE,
+               norm_weight: Optional[torch.Tensor] = None, sumsq_in: Optional[torch.Tensor] = None, eps: float = 1e-5,
+               residual: Optional[torch.Tensor] = None, want_sumsq: bool = False,
+               workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
+    """``gemv`` with a decoder block's surroundings folded in.
+
+    ``norm_weight`` + ``sumsq_in`` (fp32 [B, K/16]): the product is taken with ``RMSNorm(x)``;
+    ``residual`` ([B, N]): ``y = dtype(dtype(x W^T + bias) + residual)`` (``out`` may be ``residual``);
+    ``want_sumsq``: also returns fp32 [B, ceil(N/16)] sums of squares of ``y``, the next norm's ``sumsq_in``.
+    Returns ``y`` or ``(y, sumsq)``."""
+    dev = _require_gpu(x, w, bias, workspace, norm_weight, sumsq_in, residual, out)
+    dt = _decode_dtype("gemv_fused", x, w, bias)
+    B, K = x.shape
+    N = w.shape[0]
+    x, w = _contig(x), _contig(w)
+    n_out = N // 2 if epilogue == EPI_SWIGLU else N
+    if norm_weight is not None:
+        if sumsq_in is None or sumsq_in.dtype != torch.float32 or tuple(sumsq_in.shape) != (B, K // 16) \
+                or not sumsq_in.is_contiguous():
+            raise ValueError(f"gemv_fused: sumsq_in must be contiguous fp32 [{B}, {K // 16}]")
+        if norm_weight.dtype != dt or norm_weight.numel() != K or not norm_weight.is_contiguous():
+            raise ValueError(f"gemv_fused: norm_weight must be contiguous {dt} [{K}]")
+    if residual is not None and (residual.dtype != dt or tuple(residual.shape) != (B, n_out) or not residual.is_contiguous()):
+        raise ValueError(f"gemv_fused: residual must be contiguous {dt} [{B}, {n_out}]")
+    if out is None:
+        out = torch.empty((B, n_out), dtype=dt, device=dev)
+    elif out.dtype != dt or tuple(out.shape) != (B, n_out) or not out.is_contiguous():
+        raise ValueError(f"gemv_fused: out must be contiguous {dt} [{B}, {n_out}]")
+    sumsq = torch.empty((B, (N + 15) // 16), dtype=torch.float32, device=dev) if want_sumsq else None
+    wbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_gemv_fused(_p(x), _p(w), _p(bias), _p(out), _p(norm_weight), _p(sumsq_in), float(eps),
+                                             _p(residual), _p(sumsq), _p(workspace), wbytes, B, N, K, epilogue,
+                                             _DTYPES[dt], _stream(dev)), "mtp_gemv_fused")
+    return (out, sumsq) if want_sumsq else out
+
+
 def gemv_argmax(x: torch.Tensor, w: torch.Tensor, workspace: Optional[torch.Tensor] = None):
     """-> (idx int64 [B], maxval fp32 [B]) without materialising the logits."""
     dev = _require_gpu(x, w, workspace)

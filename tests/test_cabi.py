@@ -26,7 +26,7 @@ def test_header_symbols_are_exported_and_bound():
 
 def test_loader_and_versions():
     lib = _lib.lib()
-    assert lib.mtp_abi_version() == _lib.ABI_VERSION == 4
+    assert lib.mtp_abi_version() == _lib.ABI_VERSION == 5
     hdr = open(os.path.join(ROOT, "include", "merak_tp_gfx950.h")).read()
     assert f"#define MTP_ABI_VERSION {_lib.ABI_VERSION}" in hdr
     for name, val in (("MTP_F32", _lib.MTP_F32), ("MTP_BF16", _lib.MTP_BF16), ("MTP_EPI_NONE", _lib.EPI_NONE),
@@ -47,6 +47,11 @@ def test_argument_errors_are_reported_without_a_device():
     assert lib.mtp_gemv(None, None, None, None, 4, 8, 8, 0, 0, None) == -2          # fp32 is not a decode dtype
     assert b"dtype 0" in lib.mtp_last_error()
     assert lib.mtp_stream_copy(None, None, 24, None) == -1
+    # fused decode GEMV: a norm weight without the sums of squares; K not a multiple of 512; residual with SwiGLU
+    assert lib.mtp_gemv_fused(None, None, None, None, 16, None, 1e-5, None, None, None, 0, 1, 64, 512, 0, 1, None) == -1
+    assert lib.mtp_gemv_fused(None, None, None, None, 16, 16, 1e-5, None, None, None, 0, 1, 64, 576, 0, 1, None) == -2
+    assert b"512" in lib.mtp_last_error()
+    assert lib.mtp_gemv_fused(None, None, None, None, None, None, 0.0, 16, None, None, 0, 1, 64, 512, 3, 1, None) == -1
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -222,7 +222,8 @@ def _tiny_model(seed):
     return cfg, model
 
 
-def test_llama_decoder_matches_full_sequence_forward(gpu):
+@pytest.mark.parametrize("fused", [False, True])
+def test_llama_decoder_matches_full_sequence_forward(gpu, fused):
     """Token by token with the cache on the GPU == what the generation loop computes: the full-sequence forward
     of the library model (fp32, CPU, same bf16-representable weights), row context_length-1 (:223)."""
     cfg, model = _tiny_model(7)
@@ -230,7 +231,8 @@ def test_llama_decoder_matches_full_sequence_forward(gpu):
     ids = torch.randint(0, cfg.vocab_size, (B, T), generator=gen(7))
     with torch.no_grad():
         full = model(input_ids=ids).logits                              # [B, T, V] fp32
-    dec = LlamaDecoder.from_hf(model.bfloat16().to(gpu), max_len=64, batch=B)
+    dec = LlamaDecoder.from_hf(model.bfloat16().to(gpu), max_len=64, batch=B, fused=fused)
+    assert dec.fused == fused
     worst = 0.0
     for t in range(T):
         logits = dec.logits(ids[:, t].to(gpu))
@@ -292,7 +294,8 @@ def test_negative_rotation_knobs_are_clamped(gpu, monkeypatch):
     assert rel(ops.attn_decode(q, kc, vc, dl), ref) < TOL_BF16
 
 
-def test_llama_decoder_graph_replay_matches_eager(gpu):
+@pytest.mark.parametrize("fused", [False, True])
+def test_llama_decoder_graph_replay_matches_eager(gpu, fused):
     """A step recorded into a HIP graph, replayed for every position with eager work and synchronisations in
     between, gives what the eager launches give (the split count of the attention differs, so equal to
     rounding), on every replay."""
@@ -300,8 +303,8 @@ def test_llama_decoder_graph_replay_matches_eager(gpu):
     B, T = 2, 12
     ids = torch.randint(0, cfg.vocab_size, (B, T), generator=gen(9)).to(gpu)
     model = model.bfloat16().to(gpu)
-    eager = LlamaDecoder.from_hf(model, max_len=64, batch=B)
-    graphed = LlamaDecoder.from_hf(model, max_len=64, batch=B)
+    eager = LlamaDecoder.from_hf(model, max_len=64, batch=B, fused=fused)
+    graphed = LlamaDecoder.from_hf(model, max_len=64, batch=B, fused=fused)
     for t in range(3):                                  # a prefix before the capture: the graph starts mid-sequence
         eager.logits(ids[:, t])
         graphed.logits(ids[:, t])
@@ -323,6 +326,143 @@ def test_llama_decoder_graph_replay_matches_eager(gpu):
     top2 = le.topk(2, dim=-1).values
     clear = (top2[:, 0] - top2[:, 1]) > 1e-2 * top2[:, 0].abs()
     assert tok_g.shape == (B,) and torch.equal(tok_g[clear], le.argmax(-1)[clear])
+
+
+def _sumsq16(x):
+    """fp32 [B, K/16]: sums of squares per 16 elements, what the producing linear hands to the norm prologue"""
+    return x.float().pow(2).view(x.shape[0], -1, 16).sum(-1).contiguous()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,N,K", [(1, 4096, 4096), (5, 4096, 14336), (16, 1024, 512), (32, 4096, 14336), (32, 6144, 1024),
+                                   (3, 1000, 520)])
+def test_gemv_residual_epilogue(gpu, dtype, B, N, K):
+    """y = dtype(dtype(x W^T) + residual), bit for bit what the plain product followed by the tensor add gives,
+    and the sums of squares of y per 16 rows (also through the k-sliced form, which B = 32 x 14336 takes)."""
+    g = gen(60)
+    x = torch.randn(B, K, generator=g).to(dtype).to(gpu)
+    w = (torch.randn(N, K, generator=g) * 0.03).to(dtype).to(gpu)
+    res = torch.randn(B, N, generator=g).to(dtype).to(gpu)
+    ws = ops.gemv_workspace(B, N, K, ops.EPI_NONE, gpu)
+    plain = ops.gemv(x, w, workspace=ws)
+    y, ss = ops.gemv_fused(x, w, residual=res, want_sumsq=True, workspace=ws)
+    assert torch.equal(y, plain + res)
+    pad = (-N) % 16
+    ref_ss = torch.nn.functional.pad(y.float().pow(2), (0, pad)).view(B, -1, 16).sum(-1)
+    assert ss.shape == (B, (N + 15) // 16) and torch.allclose(ss, ref_ss, rtol=1e-5, atol=1e-30)
+    y2 = res.clone()                                     # in place on the residual stream
+    ops.gemv_fused(x, w, residual=y2, out=y2, workspace=ws)
+    assert torch.equal(y2, y)
+    assert torch.equal(ops.gemv_fused(x, w, workspace=ws), plain)            # nothing fused: the plain product
+    y3, ss3 = ops.gemv_fused(x, w, want_sumsq=True, workspace=ws)          # sums of squares without a residual
+    assert torch.equal(y3, plain) and torch.allclose(
+        ss3, torch.nn.functional.pad(plain.float().pow(2), (0, pad)).view(B, -1, 16).sum(-1), rtol=1e-5, atol=1e-30)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,N,K,epi", [(1, 6144, 4096, "none"), (8, 6144, 4096, "none"), (5, 4096, 4096, "none"),
+                                       (1, 28672, 4096, "swiglu"), (8, 28672, 4096, "swiglu"), (3, 28672, 4096, "swiglu"),
+                                       (4, 8192, 512, "swiglu"), (3, 2048, 512, "swiglu"), (8, 2048, 1024, "swiglu"),
+                                       (2, 1280, 8192, "none"), (4, 1280, 8192, "none"), (4, 512, 5120, "none"),
+                                       (8, 256, 1024, "none"), (1, 1000, 512, "none")])
+def test_gemv_norm_prologue(gpu, dtype, B, N, K, epi):
+    """The product with RMSNorm(x) taken inside the linear against (a) the stand-alone norm kernel followed by
+    the plain product and (b) the oracle in fp32.  The two GPU forms add the squares in different orders, so a
+    row's scale may differ in its last bit and a few normalised elements by one unit of the tensor dtype."""
+    g = gen(61)
+    E = ops.EPI_SWIGLU if epi == "swiglu" else ops.EPI_NONE
+    x = (torch.randn(B, K, generator=g) * 2).to(dtype)
+    nw = (torch.rand(K, generator=g) + 0.5).to(dtype)
+    w = (torch.randn(N, K, generator=g) * 0.03).to(dtype)
+    xg, nwg, wg = x.to(gpu), nw.to(gpu), w.to(gpu)
+    fused = ops.gemv_fused(xg, wg, None, E, norm_weight=nwg, sumsq_in=_sumsq16(xg), eps=1e-5)
+    two = ops.gemv(ops.rmsnorm(xg, nwg, 1e-5), wg, None, E)
+    tol = TOL_BF16 if dtype == torch.bfloat16 else 2e-3
+    assert fused.shape == two.shape and rel(fused, two) < tol / 4
+    hn = R.rms_norm(x.float(), nw.float(), 1e-5)[0]
+    hn = hn.to(dtype).float()                                   # the normalised row as the tensor dtype holds it
+    ref = torch.nn.functional.linear(hn, w.float())
+    if epi == "swiglu":
+        gate, up = ref[:, :N // 2].to(dtype).float(), ref[:, N // 2:].to(dtype).float()
+        ref = torch.nn.functional.silu(gate) * up
+    assert rel(fused, ref) < tol
+
+
+@pytest.mark.parametrize("groups", [1, 2, 3, 4, 5, 6, 7])
+def test_gemv_norm_prologue_every_mixed_group_count(gpu, groups, monkeypatch):
+    monkeypatch.setenv("MTP_GEMV_MIX", str(groups))
+    g = gen(62)
+    B, N, K = 6, 2 * 1288, 1024
+    x = torch.randn(B, K, generator=g).bfloat16().to(gpu)
+    nw = (torch.rand(K, generator=g) + 0.5).bfloat16().to(gpu)
+    w = (torch.randn(N, K, generator=g) * 0.03).bfloat16().to(gpu)
+    fused = ops.gemv_fused(x, w, None, ops.EPI_SWIGLU, norm_weight=nw, sumsq_in=_sumsq16(x), eps=1e-6)
+    two = ops.gemv(ops.rmsnorm(x, nw, 1e-6), w, None, ops.EPI_SWIGLU)
+    assert rel(fused, two) < TOL_BF16 / 4
+    plain = ops.gemv(x, w, None, ops.EPI_SWIGLU)                # the two-set main loop without the norm
+    monkeypatch.setenv("MTP_GEMV_MIX", "0")
+    assert rel(plain, ops.gemv(x, w, None, ops.EPI_SWIGLU)) < TOL_BF16 / 4
+
+
+def test_gemv_fused_chain_is_a_block(gpu):
+    """o product (+ residual, sums of squares) -> gate/up product with the norm inside -> down product
+    (+ residual): the second half of a Llama-3-8B block against the oracle, at B = 1, 8 and 32."""
+    g = gen(63)
+    H, I = 4096, 14336
+    wo = (torch.randn(H, H, generator=g) * 0.02).bfloat16()
+    wgu = (torch.randn(2 * I, H, generator=g) * 0.02).bfloat16()
+    wd = (torch.randn(H, I, generator=g) * 0.02).bfloat16()
+    nw = (torch.rand(H, generator=g) + 0.5).bfloat16()
+    G = [t.to(gpu) for t in (wo, wgu, wd, nw)]
+    for B in (1, 8, 32):
+        a = torch.randn(B, H, generator=g).bfloat16()
+        res = torch.randn(B, H, generator=g).bfloat16()
+        ws = ops.gemv_workspace(B, H, I, ops.EPI_NONE, gpu)
+        r1, ss = ops.gemv_fused(a.to(gpu), G[0], residual=res.to(gpu), want_sumsq=True, workspace=ws)
+        assert ops.gemv_norm_fits(B, H) == (B <= 8)
+        if B <= 8:
+            act = ops.gemv_fused(r1, G[1], None, ops.EPI_SWIGLU, norm_weight=G[3], sumsq_in=ss, eps=1e-5)
+        else:       # more rows than the norm prologue holds: the stand-alone norm in between
+            act = ops.gemv(ops.rmsnorm(r1, G[3], 1e-5), G[1], None, ops.EPI_SWIGLU)
+        r2 = ops.gemv_fused(act, G[2], residual=r1, workspace=ws)
+        # oracle, rounding to bf16 where the tensors of the model are bf16
+        bf = lambda t: t.bfloat16().float()
+        o = bf(torch.nn.functional.linear(a.float(), wo.float()))
+        ref_r1 = bf(o + res.float())
+        hn = bf(R.rms_norm(ref_r1, nw.float(), 1e-5)[0])
+        gu = bf(torch.nn.functional.linear(hn, wgu.float()))
+        ref_act = bf(torch.nn.functional.silu(gu[:, :I]) * gu[:, I:])
+        ref_r2 = bf(bf(torch.nn.functional.linear(ref_act, wd.float())) + ref_r1)
+        assert rel(r1, ref_r1) < TOL_BF16 and rel(act, ref_act) < TOL_BF16 and rel(r2, ref_r2) < TOL_BF16, B
+
+
+def test_gemv_fused_rejects_bad_arguments(gpu):
+    x = torch.zeros(2, 1024, dtype=torch.bfloat16, device=gpu)
+    w = torch.zeros(64, 1024, dtype=torch.bfloat16, device=gpu)
+    nw = torch.ones(1024, dtype=torch.bfloat16, device=gpu)
+    ss = _sumsq16(x)
+    with pytest.raises(ValueError, match="sumsq_in"):
+        ops.gemv_fused(x, w, norm_weight=nw)                                        # the norm needs the sums
+    with pytest.raises(ValueError, match="sumsq_in"):
+        ops.gemv_fused(x, w, norm_weight=nw, sumsq_in=ss[:, :-1].contiguous())
+    with pytest.raises(ValueError, match="norm_weight"):
+        ops.gemv_fused(x, w, norm_weight=nw[:-8].contiguous(), sumsq_in=ss)
+    with pytest.raises(RuntimeError, match="512"):                                  # K = 576: not a multiple of 512
+        ops.gemv_fused(x[:, :576].contiguous(), w[:, :576].contiguous(), norm_weight=nw[:576].contiguous(),
+                       sumsq_in=ss[:, :36].contiguous())
+    with pytest.raises(RuntimeError, match="plain stores"):                         # residual with SwiGLU
+        ops.gemv_fused(x, w, None, ops.EPI_SWIGLU, residual=torch.zeros(2, 32, dtype=torch.bfloat16, device=gpu))
+    with pytest.raises(ValueError, match="residual"):
+        ops.gemv_fused(x, w, residual=torch.zeros(2, 63, dtype=torch.bfloat16, device=gpu))
+    with pytest.raises(RuntimeError, match="8 x 4096"):                             # 9 rows do not fit
+        x9 = torch.zeros(9, 1024, dtype=torch.bfloat16, device=gpu)
+        ops.gemv_fused(x9, w, norm_weight=nw, sumsq_in=_sumsq16(x9))
+    assert ops.gemv_norm_fits(8, 4096) and ops.gemv_norm_fits(4, 8192) and not ops.gemv_norm_fits(2, 16384)
+    assert not ops.gemv_norm_fits(9, 512) and not ops.gemv_norm_fits(5, 8192) and not ops.gemv_norm_fits(1, 576)
+    with pytest.raises(ValueError, match="fused=True"):
+        LlamaDecoder(torch.zeros(10, 640, dtype=torch.bfloat16, device=gpu), [], nw, w, 4, 2, fused=True)
+    with pytest.raises(ValueError, match="fused=True"):
+        LlamaDecoder(torch.zeros(10, 1024, dtype=torch.bfloat16, device=gpu), [], nw, w, 4, 2, batch=16, fused=True)
 
 
 def test_attn_decode_seeded_sweep(gpu):

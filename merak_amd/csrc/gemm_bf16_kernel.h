@@ -34,6 +34,9 @@
 
 namespace {
 
+#ifndef MTP_GEMM_VSTAGE
+#define MTP_GEMM_VSTAGE 1
+#endif
 constexpr int BK = 32;      // k-tile depth
 constexpr int NSTAGE = 4;   // LDS ring: 4 x (16 KiB A + 16 KiB B) at 256x256
 constexpr int KSTEPS = BK / 16;  // MFMA k16 steps per k-tile
@@ -109,6 +112,22 @@ __device__ __forceinline__ void dma16(rsrc_t rsrc, uint32_t lds_addr, uint32_t v
                :
                : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff));
 }
+// Register-staged loads, also inline assembly so that their order against the DMA-style waits stays in this
+// file's hands: 64 lanes x 16 bytes from the buffer into four VGPRs ...
+__device__ __forceinline__ u32x4_t load16_to_vgpr(rsrc_t rsrc, uint32_t voff, uint32_t soff) {
+  u32x4_t v;
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(v) : "v"(voff), "s"(rsrc), "s"(soff));
+  return v;
+}
+// ... and, once at most PENDING younger loads are outstanding, from there to LDS
+template <int PENDING, int OFFSET>
+__device__ __forceinline__ void wait_and_write16(uint32_t lds_addr, u32x4_t v) {
+  static_assert(OFFSET >= 0 && OFFSET < 65536 && PENDING >= 0 && PENDING < 64, "ds_write offset / vmcnt range");
+  asm volatile("s_waitcnt vmcnt(%2)\n\tds_write_b128 %0, %1 offset:%3"
+               :
+               : "v"(lds_addr), "v"(v), "n"(PENDING), "n"(OFFSET)
+               : "memory");
+}
 __device__ __forceinline__ uint32_t lds_addr_of(const void* p) {
   return (uint32_t)(uintptr_t)(const void __attribute__((address_space(3)))*)p;
 }
@@ -183,8 +202,14 @@ struct RowOperand {
   // DMA instructions per wave per k-tile (16 rows each); instructions whose rows all lie past ROWS are skipped
   static constexpr int NINSTR = (ROWS / 16 + NW - 1) / NW;
   static constexpr int NREADS = 1;               // LDS reads per fragment
+  // Register-staged path (forward kernels): two k-tiles at a time, so that a load instruction covers whole
+  // 128-byte lines: 8 rows x 128 bytes, lane l -> row l/8, 16-byte piece l%8 (pieces 0-3 belong to the even
+  // k-tile of the pair, 4-7 to the odd one).  NPAIR such instructions per wave and pair of k-tiles.
+  static constexpr int NPAIR = (ROWS / 8 + NW - 1) / NW;
   rsrc_t rsrc;
   uint32_t voff[NINSTR];
+  uint32_t pvoff[NPAIR];   // global byte offsets of the paired loads (0x80000000: no such row)
+  uint32_t pwoff;          // LDS byte offset (inside the operand's part of the even stage) of paired instruction 0
   uint32_t fo[KSTEPS];
   int chunk, K;
 
@@ -208,7 +233,23 @@ struct RowOperand {
     const int row = wave_row0 + (lane & 31), h = lane >> 5;
 #pragma unroll
     for (int kk = 0; kk < KSTEPS; kk++) fo[kk] = (uint32_t)(row * 64 + ((((2 * kk + h) ^ (row >> 2)) & 3) << 4));
+    // paired loads: instruction j of this wave covers tile rows 8 (wave + NW j) .. + 7
+    const int prow = lane >> 3, c8 = lane & 7;
+#pragma unroll
+    for (int j = 0; j < NPAIR; j++) {
+      const int r = (wave + NW * j) * 8 + prow;
+      const int64_t gr = r < ROWS ? rowmap(r) : -1;
+      pvoff[j] = (gr < 0 || gr >= nrows - row0) ? 0x80000000u : (uint32_t)((gr * ld + c8 * 8) * 2);
+    }
+    // where the lane's 16 bytes go: stage of the even or odd k-tile, row r, piece (c8 & 3) swizzled like the
+    // DMA path does; (r >> 2) & 3 = (2 wave + lane / 32) & 3 for every j (8 NW j is a multiple of 4)
+    {
+      const int r0 = wave * 8 + prow;
+      pwoff = (uint32_t)(r0 * 64 + ((((c8 & 3) ^ (r0 >> 2)) & 3) << 4));
+    }
   }
+  // odd k-tile of the pair: the lane's piece goes one stage further
+  __device__ __forceinline__ bool pair_odd(int lane) const { return (lane & 4) != 0; }
   // Per k-tile state of the DMA.  INSIDE: the caller knows the k-tile lies completely below K (no tail
   // masking needed).
   struct Prep {
@@ -234,6 +275,7 @@ struct ColOperand {
   static constexpr int BYTES = BK * LROWS * 2;
   static constexpr int NINSTR = BYTES / 1024 / NW;
   static constexpr int NREADS = 2;
+  static constexpr int NPAIR = 0;   // no register-staged form: a DMA instruction already covers whole lines
   const char* base;    // &mem[0][row0]
   int64_t total;       // bytes from base to the end of the matrix
   int64_t ktile_bytes; // BK * ld * 2
@@ -352,6 +394,12 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
     for (int j = 0; j < AOp::NINSTR; j++) opA.voff[j] = 0x80000000u;
 #pragma unroll
     for (int j = 0; j < BOp::NINSTR; j++) opB.voff[j] = 0x80000000u;
+    if constexpr (ALAY == LAY_ROW && BLAY == LAY_ROW) {
+#pragma unroll
+      for (int j = 0; j < AOp::NPAIR; j++) opA.pvoff[j] = 0x80000000u;
+#pragma unroll
+      for (int j = 0; j < BOp::NPAIR; j++) opB.pvoff[j] = 0x80000000u;
+    }
   }
 
   constexpr int NDMA = AOp::NINSTR + BOp::NINSTR;  // DMA instructions per wave per k-tile
@@ -440,6 +488,94 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   constexpr int PRE = NMF * 3 / 8, REST = NMF - PRE;
   // MFMA index (0 .. TILE_MF-1) after which the d-th DMA instruction is issued
   auto dma_slot = [](int d) constexpr { return d * TILE_MF / NDMA + 1; };
+  // VSTAGE (row operands on both sides: the forward product).  A k-tile of a row operand is 64 bytes per row,
+  // half a cache line; fetched one k-tile at a time every line is requested twice from the L2.  Here the k-tiles
+  // travel in pairs: one load instruction covers 8 rows x 128 bytes (both k-tiles of the pair), lands in
+  // registers and is written to the two LDS stages two k-tiles later — the prefetch distance of the DMA ring,
+  // with whole lines per request and one barrier per pair of k-tiles.  During the even tile kt of a pair the
+  // registers (pair kt+2, kt+3) are written to the stages the barrier behind tile kt-1 released and are
+  // refilled with pair kt+4, kt+5, one instruction of each kind every second MFMA.
+  constexpr bool VSTAGE = MTP_GEMM_VSTAGE && ALAY == LAY_ROW && BLAY == LAY_ROW && NSTAGE == 4 && KSTEPS == 2;
+  constexpr int NPA = VSTAGE ? AOp::NPAIR : 0, NPB = VSTAGE ? BOp::NPAIR : 0, NPL = NPA + NPB;
+  u32x4_t st[NPL > 0 ? NPL : 1];
+  [[maybe_unused]] uint32_t wlane_a = 0, wlane_b = 0;
+  if constexpr (VSTAGE) {
+    wlane_a = opA.pwoff + (opA.pair_odd(lane) ? STAGE_BYTES : 0);
+    wlane_b = opB.pwoff + (opB.pair_odd(lane) ? STAGE_BYTES : 0);
+  }
+  // q-th paired instruction of a pair: A and B alternate while both have instructions left
+  auto pair_sel = [](int q, int na, int nb, bool& is_a, int& jj) constexpr {
+    const int nmin = na < nb ? na : nb;
+    if (q < 2 * nmin) {
+      is_a = (q & 1) == 0;
+      jj = q >> 1;
+    } else {
+      is_a = na > nb;
+      jj = q - nmin;
+    }
+  };
+  auto pair_load = [&](int kt_even, auto q_tag) {
+    if constexpr (VSTAGE) {
+      constexpr int q = decltype(q_tag)::value;
+      bool is_a = true;
+      int jj = 0;
+      pair_sel(q, NPA, NPB, is_a, jj);
+      const uint32_t soff = (uint32_t)(kt_even * BK * 2);
+      st[q] = is_a ? load16_to_vgpr(opA.rsrc, opA.pvoff[jj], soff) : load16_to_vgpr(opB.rsrc, opB.pvoff[jj], soff);
+    }
+  };
+  auto pair_write = [&](int kt_even, auto q_tag, auto pending_tag) {
+    if constexpr (VSTAGE) {
+      constexpr int q = decltype(q_tag)::value;
+      constexpr int PENDING = decltype(pending_tag)::value;
+      constexpr bool is_a = q < 2 * (NPA < NPB ? NPA : NPB) ? (q & 1) == 0 : (NPA > NPB);
+      constexpr int jj = q < 2 * (NPA < NPB ? NPA : NPB) ? (q >> 1) : q - (NPA < NPB ? NPA : NPB);
+      const uint32_t base = lds0 + (uint32_t)((kt_even % NSTAGE) * STAGE_BYTES) + (is_a ? 0u : (uint32_t)AOp::BYTES);
+      wait_and_write16<PENDING, jj * NW * 8 * 64>(base + (is_a ? wlane_a : wlane_b), st[q]);
+    }
+  };
+  auto ktile_v = [&](int kt, auto odd_tag, auto loads_tag) {
+    constexpr bool ODD = decltype(odd_tag)::value, LOADS = decltype(loads_tag)::value;
+    const int stage = kt % NSTAGE, nxt = (kt + 1) % NSTAGE;
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<KSTEPS>([&](auto s_tag) {
+      constexpr int s = decltype(s_tag)::value;
+      constexpr bool last = s == KSTEPS - 1;
+      static_for<NMF>([&](auto t_tag) {
+        constexpr int t = decltype(t_tag)::value;
+        constexpr int g = s * NMF + t;  // MFMA index inside the tile
+        if constexpr (ODD && last && t == PRE) {
+          // one barrier per pair: every wave's writes of the pair behind this one are in LDS, and everyone is
+          // done reading the two stages the next even tile writes to
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          __syncthreads();
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        mfma_one(s & 1, t_tag);
+        if constexpr (!ODD) {
+          static_for<(NPL > 0 ? NPL : 1)>([&](auto q_tag) {
+            constexpr int q = decltype(q_tag)::value;
+            if constexpr (NPL > 0 && q * TILE_MF / (NPL > 0 ? NPL : 1) + 1 == g + 1) {
+              pair_write(kt + 2, q_tag, std::integral_constant<int, LOADS ? NPL - 1 : NPL - 1 - q>{});
+              if constexpr (LOADS) pair_load(kt + 4, q_tag);
+            }
+          });
+        }
+        if constexpr (!last) {
+          static_for<(t + 1) * NFR / NMF - t * NFR / NMF>([&](auto e) {
+            read_one(stage, s + 1, (s + 1) & 1, std::integral_constant<int, t * NFR / NMF + decltype(e)::value>{});
+          });
+        } else if constexpr (t >= PRE) {
+          constexpr int r = t - PRE;
+          static_for<(r + 1) * NFR / REST - r * NFR / REST>([&](auto e) {
+            read_one(nxt, 0, (s + 1) & 1, std::integral_constant<int, r * NFR / REST + decltype(e)::value>{});
+          });
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
+  };
+  constexpr int AHEAD = VSTAGE ? 2 : NSTAGE - 1;   // the DMA tiles (tail, short k) request tile kt + AHEAD
   auto ktile = [&](int kt, auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
     const int stage = kt % NSTAGE, nxt = (kt + 1) % NSTAGE;
@@ -486,14 +622,14 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
         });
       });
     } else {
-      if (kt + NSTAGE - 1 < KT) issue_loads(kt + NSTAGE - 1);
+      if (kt + AHEAD < KT) issue_loads(kt + AHEAD);
       static_for<KSTEPS - 1>([&](auto s_tag) {
         constexpr int s = decltype(s_tag)::value;
         read_frags(stage, s + 1, (s + 1) & 1);
         mfmas(s & 1);
       });
       // wait for everything but (at most) the tile just requested
-      if (kt + NSTAGE - 1 < KT)
+      if (kt + AHEAD < KT)
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(NSTAGE >= 3 ? NDMA : 0));
       else
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
@@ -504,15 +640,39 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   };
   static_assert(KSTEPS % 2 == 0, "slot parity assumes an even number of k16 steps per tile");
 
-#pragma unroll
-  for (int t = 0; t < NSTAGE - 1; t++)
-    if (t < KT) issue_loads(t);
-  __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-  __syncthreads();
-  read_frags(0, 0, 0);
   int kt = 0;
   const int KT_inside = p.K / BK;  // k-tiles that lie completely below K
-  for (; kt + NSTAGE - 1 < KT_inside; kt++) ktile(kt, std::true_type{});
+  bool staged = false;
+  if constexpr (VSTAGE) {
+    if (KT_inside >= 6) {
+      staged = true;
+      // pair (0, 1) through the registers into stages 0 and 1, pair (2, 3) requested
+      static_for<NPL>([&](auto q) { pair_load(0, q); });
+      static_for<NPL>([&](auto q) { pair_write(0, q, std::integral_constant<int, NPL - 1 - decltype(q)::value>{}); });
+      static_for<NPL>([&](auto q) { pair_load(2, q); });
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __syncthreads();
+      read_frags(0, 0, 0);
+      for (; kt + 5 < KT_inside; kt += 2) {
+        ktile_v(kt, std::false_type{}, std::true_type{});
+        ktile_v(kt + 1, std::true_type{}, std::true_type{});
+      }
+      // the pair still in registers goes to LDS, nothing new is requested; the DMA tiles take over behind it
+      ktile_v(kt, std::false_type{}, std::false_type{});
+      ktile_v(kt + 1, std::true_type{}, std::false_type{});
+      kt += 2;
+    }
+  }
+  if (!staged) {
+#pragma unroll
+    for (int t = 0; t < AHEAD; t++)
+      if (t < KT) issue_loads(t);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    __syncthreads();
+    read_frags(0, 0, 0);
+    if constexpr (!VSTAGE)
+      for (; kt + NSTAGE - 1 < KT_inside; kt++) ktile(kt, std::true_type{});
+  }
   for (; kt < KT; kt++) ktile(kt, std::false_type{});
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
   __syncthreads();  // the epilogue reuses the tile buffers

@@ -37,6 +37,12 @@ namespace {
 #ifndef MTP_GEMM_VSTAGE
 #define MTP_GEMM_VSTAGE 1
 #endif
+#ifndef MTP_STAGE_SKEW
+#define MTP_STAGE_SKEW 1
+#endif
+#ifndef MTP_VSTAGE_SPREAD
+#define MTP_VSTAGE_SPREAD 1
+#endif
 constexpr int BK = 32;      // k-tile depth
 constexpr int NSTAGE = 4;   // LDS ring: 4 x (16 KiB A + 16 KiB B) at 256x256
 constexpr int KSTEPS = BK / 16;  // MFMA k16 steps per k-tile
@@ -348,7 +354,12 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   using BOp = typename OperandOf<BLAY, BN, NW>::type;
   constexpr int STAGE_BYTES = AOp::BYTES + BOp::BYTES;
   static_assert(NSTAGE * STAGE_BYTES <= 128 * 1024, "LDS ring too large");
-  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE_BYTES];
+  // Stages sit STAGE_SKEW bytes further apart than their size.  A register-staged write instruction puts the two
+  // 64-byte halves of a row into neighbouring stages; with the stages a multiple of 256 bytes apart the two
+  // halves fall on the same banks (two-way conflict on every write), 64 bytes of skew puts them side by side.
+  constexpr int STAGE_SKEW = (MTP_GEMM_VSTAGE && MTP_STAGE_SKEW && ALAY == LAY_ROW && BLAY == LAY_ROW) ? 64 : 0;
+  constexpr int STAGE_STRIDE = STAGE_BYTES + STAGE_SKEW;
+  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE_STRIDE];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -406,7 +417,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr_of(lds));
   // d-th DMA instruction of a k-tile whose per-tile state (pa, pb) has been prepared; A and B alternate
   auto issue_one = [&](const typename AOp::Prep& pa, const typename BOp::Prep& pb, int stage, int d) {
-    const uint32_t la = lds0 + stage * STAGE_BYTES;
+    const uint32_t la = lds0 + stage * STAGE_STRIDE;
     // A and B alternate while both have instructions left
     constexpr int NMIN = AOp::NINSTR < BOp::NINSTR ? AOp::NINSTR : BOp::NINSTR;
     if (d < 2 * NMIN) {
@@ -444,7 +455,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   constexpr int NMF = TI * TJ;   // MFMAs per k16 step
   auto read_one = [&](int stage, int kk, int slot, auto u_tag) {  // u-th fragment in A0 B0 A1 B1 ... order
     constexpr int u = decltype(u_tag)::value;
-    const char* la = lds + stage * STAGE_BYTES;
+    const char* la = lds + stage * STAGE_STRIDE;
     // with TI == TJ the order alternates; otherwise the longer side's leftovers come last
     constexpr int d = u < 2 * (TI < TJ ? TI : TJ) ? u / 2 : u - (TI < TJ ? TI : TJ);
     constexpr bool is_a = u < 2 * (TI < TJ ? TI : TJ) ? (u % 2 == 0) : (TI > TJ);
@@ -500,8 +511,8 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   u32x4_t st[NPL > 0 ? NPL : 1];
   [[maybe_unused]] uint32_t wlane_a = 0, wlane_b = 0;
   if constexpr (VSTAGE) {
-    wlane_a = opA.pwoff + (opA.pair_odd(lane) ? STAGE_BYTES : 0);
-    wlane_b = opB.pwoff + (opB.pair_odd(lane) ? STAGE_BYTES : 0);
+    wlane_a = opA.pwoff + (opA.pair_odd(lane) ? STAGE_STRIDE : 0);
+    wlane_b = opB.pwoff + (opB.pair_odd(lane) ? STAGE_STRIDE : 0);
   }
   // q-th paired instruction of a pair: A and B alternate while both have instructions left
   auto pair_sel = [](int q, int na, int nb, bool& is_a, int& jj) constexpr {
@@ -530,7 +541,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
       constexpr int PENDING = decltype(pending_tag)::value;
       constexpr bool is_a = q < 2 * (NPA < NPB ? NPA : NPB) ? (q & 1) == 0 : (NPA > NPB);
       constexpr int jj = q < 2 * (NPA < NPB ? NPA : NPB) ? (q >> 1) : q - (NPA < NPB ? NPA : NPB);
-      const uint32_t base = lds0 + (uint32_t)((kt_even % NSTAGE) * STAGE_BYTES) + (is_a ? 0u : (uint32_t)AOp::BYTES);
+      const uint32_t base = lds0 + (uint32_t)((kt_even % NSTAGE) * STAGE_STRIDE) + (is_a ? 0u : (uint32_t)AOp::BYTES);
       wait_and_write16<PENDING, jj * NW * 8 * 64>(base + (is_a ? wlane_a : wlane_b), st[q]);
     }
   };
@@ -552,12 +563,16 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
           __builtin_amdgcn_sched_barrier(0);
         }
         mfma_one(s & 1, t_tag);
-        if constexpr (!ODD) {
+        {
+          // the pair's instructions are spread over the MFMAs of both tiles up to the barrier
+          constexpr int SPAN = MTP_VSTAGE_SPREAD ? TILE_MF + (KSTEPS - 1) * NMF + PRE - 2 : TILE_MF;
+          constexpr int gp = (ODD ? TILE_MF : 0) + g;   // MFMA index inside the pair
+          const int kb = ODD ? kt - 1 : kt;             // the pair's even tile
           static_for<(NPL > 0 ? NPL : 1)>([&](auto q_tag) {
             constexpr int q = decltype(q_tag)::value;
-            if constexpr (NPL > 0 && q * TILE_MF / (NPL > 0 ? NPL : 1) + 1 == g + 1) {
-              pair_write(kt + 2, q_tag, std::integral_constant<int, LOADS ? NPL - 1 : NPL - 1 - q>{});
-              if constexpr (LOADS) pair_load(kt + 4, q_tag);
+            if constexpr (NPL > 0 && q * SPAN / (NPL > 0 ? NPL : 1) + 1 == gp + 1) {
+              pair_write(kb + 2, q_tag, std::integral_constant<int, LOADS ? NPL - 1 : NPL - 1 - q>{});
+              if constexpr (LOADS) pair_load(kb + 4, q_tag);
             }
           });
         }

@@ -41,7 +41,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM bytes per launch of the largest GEMMs, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file
 # scaled by a 1 GiB copy kernel (x2.000 / x1.000): profiles/hbm_traffic_fetch_write_size.txt
-HBM_TRAFFIC_BYTES = {"gate_up.fwd": 1.805e9, "gate_up.wgrad": 1.645e9, "down.dgrad": 0.889e9}
+HBM_TRAFFIC_BYTES = {"gate_up.fwd": 1.763e9, "gate_up.wgrad": 1.645e9, "down.dgrad": 0.889e9}
 
 LLAMA8B = [  # (name, K, N, epilogue)
     ("qkv", 4096, 6144, "none"),

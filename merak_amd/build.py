@@ -27,7 +27,7 @@ SOURCES = [
     "embedding.hip",
     "gemv.hip",
     "elementwise.hip", "sampling.hip",
-    "gemm_bf16_fwd.hip",
+    "gemm_bf16_fwd.hip", "gemm_f16_fwd.hip",
     "gemm_bf16_dgrad.hip",
     "gemm_bf16_wgrad.hip",
     "gemm_generic.hip", "gemm_f32.hip", "decode_attn.hip",

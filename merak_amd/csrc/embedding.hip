@@ -30,6 +30,36 @@ __global__ __launch_bounds__(256) void embedding_gather_kernel(const int64_t* __
   }
 }
 
+// Rows of at least 256 pieces: one workgroup per row (grid-stride over rows), the id read once per row, up to four
+// pieces per lane requested before the first is stored; no division per piece.
+template <typename V>
+__global__ __launch_bounds__(256) void embedding_gather_rows_kernel(const int64_t* __restrict__ ids,
+                                                                    const V* __restrict__ table, V* __restrict__ out,
+                                                                    int64_t n_ids, int vec_per_row, int64_t vocab_start,
+                                                                    int64_t vocab_end, int32_t* __restrict__ oob_count) {
+  for (int64_t r = blockIdx.x; r < n_ids; r += gridDim.x) {
+    const int64_t id = ids[r];
+    const bool ok = id >= vocab_start && id < vocab_end;
+    const V* src = table + (ok ? id - vocab_start : 0) * (int64_t)vec_per_row;
+    V* dst = out + r * (int64_t)vec_per_row;
+    for (int c0 = threadIdx.x; c0 < vec_per_row; c0 += 4 * 256) {
+      V v[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int c = c0 + 256 * u;
+        v[u] = V{};
+        if (ok && c < vec_per_row) v[u] = src[c];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int c = c0 + 256 * u;
+        if (c < vec_per_row) dst[c] = v[u];
+      }
+    }
+    if (!ok && threadIdx.x == 0 && oob_count) atomicAdd(oob_count, 1);
+  }
+}
+
 // ---- dense gradient of the lookup ---------------------------------------------
 // dtable[id - start, :] += sum of dout[i, :] over the tokens i with ids[i] == id, added in ascending i with
 // fp32 accumulation: the result does not depend on scheduling (no atomics on the gradient).
@@ -99,6 +129,13 @@ template <typename V>
 int launch_gather(const int64_t* ids, const void* table, void* out, int64_t n_ids, int64_t row_bytes,
                   int64_t vocab_start, int64_t vocab_end, int32_t* oob, hipStream_t s) {
   const int64_t vpr = row_bytes / (int64_t)sizeof(V);
+  if (vpr >= 256 && vpr < (1ll << 30)) {
+    const int64_t rows = n_ids < 256 * 256 ? n_ids : 256 * 256;
+    hipLaunchKernelGGL(embedding_gather_rows_kernel<V>, dim3((unsigned)rows), dim3(256), 0, s, ids, (const V*)table,
+                       (V*)out, n_ids, (int)vpr, vocab_start, vocab_end, oob);
+    MTP_CHECK_LAUNCH("embedding_gather");
+    return MTP_OK;
+  }
   const int64_t total = n_ids * vpr;
   int64_t blocks = (total + 255) / 256;
   if (blocks > 256 * 64) blocks = 256 * 64;

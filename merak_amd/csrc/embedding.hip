@@ -73,14 +73,35 @@ struct TokenLink {
   int32_t leader;  // 1: first token of its id (and the id is in range)
 };
 
+// Most ids of a batch occur once.  A table of counters, several per token and indexed by the id modulo its size,
+// tells which tokens may have company: a token alone in its bucket is a leader without a chain and skips the
+// comparison with all the others.  (Sharing a bucket with another id only costs the comparison.)
+__global__ __launch_bounds__(256) void embedding_bucket_zero_kernel(int32_t* __restrict__ bucket, int n_bucket) {
+  const int b = blockIdx.x * 256 + threadIdx.x;
+  if (b < n_bucket) bucket[b] = 0;
+}
+__global__ __launch_bounds__(256) void embedding_bucket_count_kernel(const int64_t* __restrict__ ids,
+                                                                     int32_t* __restrict__ bucket, int n_bucket,
+                                                                     int n_ids, int64_t vocab_start, int64_t vocab_end) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n_ids) return;
+  const int64_t id = ids[i];
+  if (id >= vocab_start && id < vocab_end) atomicAdd(bucket + (int)((id - vocab_start) & (n_bucket - 1)), 1);
+}
+
 __global__ __launch_bounds__(256) void embedding_link_kernel(const int64_t* __restrict__ ids,
                                                              TokenLink* __restrict__ link, int n_ids,
-                                                             int64_t vocab_start, int64_t vocab_end) {
+                                                             int64_t vocab_start, int64_t vocab_end,
+                                                             const int32_t* __restrict__ bucket, int n_bucket) {
   const int i = blockIdx.x;
   const int tid = threadIdx.x;
   const int64_t id = ids[i];
   if (id < vocab_start || id >= vocab_end) {
     if (tid == 0) link[i] = TokenLink{-1, 0};
+    return;
+  }
+  if (bucket[(int)((id - vocab_start) & (n_bucket - 1))] == 1) {   // the only token of its bucket
+    if (tid == 0) link[i] = TokenLink{-1, 1};
     return;
   }
   int dup = 0;
@@ -125,6 +146,33 @@ __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t* __res
   for (int e = 0; e < nc; e++) elem_set(dst + e, elem_f32(dst[e]) + acc[e]);
 }
 
+// The same walk with 8 columns per lane (16-byte loads of 16-bit gradients), for dim % 8 == 0 and 32-byte aligned
+// tensors: half the workgroups, twice the bytes per request.
+template <typename T, int N> struct alignas(sizeof(T) * N) Pack {
+  T v[N];
+};
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void embedding_bwd_vec_kernel(const int64_t* __restrict__ ids,
+                                                                const T* __restrict__ dout, TO* __restrict__ dtable,
+                                                                const TokenLink* __restrict__ link, int64_t dim,
+                                                                int64_t vocab_start) {
+  const int i = blockIdx.x;
+  if (!link[i].leader) return;
+  const int64_t c0 = ((int64_t)blockIdx.y * 256 + threadIdx.x) * 8;
+  if (c0 >= dim) return;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int j = i; j >= 0; j = link[j].next) {
+    const Pack<T, 8> p = *reinterpret_cast<const Pack<T, 8>*>(dout + (int64_t)j * dim + c0);
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[e] += elem_f32(p.v[e]);
+  }
+  Pack<TO, 8>* dst = reinterpret_cast<Pack<TO, 8>*>(dtable + (ids[i] - vocab_start) * dim + c0);
+  Pack<TO, 8> t = *dst;
+#pragma unroll
+  for (int e = 0; e < 8; e++) elem_set(&t.v[e], elem_f32(t.v[e]) + acc[e]);
+  *dst = t;
+}
+
 template <typename V>
 int launch_gather(const int64_t* ids, const void* table, void* out, int64_t n_ids, int64_t row_bytes,
                   int64_t vocab_start, int64_t vocab_end, int32_t* oob, hipStream_t s) {
@@ -165,8 +213,17 @@ extern "C" int mtp_embedding_gather(const int64_t* ids, const void* table, void*
   return launch_gather<uint8_t>(ids, table, out, n_ids, row_bytes, vocab_start, vocab_end, oob_count, s);
 }
 
+namespace {
+// counters per batch: the power of two at or above 8 per token, between 1024 and 2^24
+int64_t embedding_buckets(int64_t n_ids) {
+  int64_t nb = 1024;
+  while (nb < 8 * n_ids && nb < (1ll << 24)) nb <<= 1;
+  return nb;
+}
+}  // namespace
+
 extern "C" int64_t mtp_embedding_bwd_workspace_bytes(int64_t n_ids) {
-  return n_ids > 0 ? n_ids * (int64_t)sizeof(TokenLink) : 0;
+  return n_ids > 0 ? n_ids * (int64_t)sizeof(TokenLink) + embedding_buckets(n_ids) * (int64_t)sizeof(int32_t) : 0;
 }
 
 extern "C" int mtp_embedding_bwd(const int64_t* ids, const void* dout, void* dtable, void* workspace,
@@ -189,28 +246,43 @@ extern "C" int mtp_embedding_bwd(const int64_t* ids, const void* dout, void* dta
   MTP_REQUIRE(chunks <= 65535, MTP_EUNSUPPORTED, "embedding_bwd: dim=%lld too large", (long long)dim);
   hipStream_t s = (hipStream_t)stream;
   TokenLink* link = (TokenLink*)workspace;
+  int32_t* bucket = reinterpret_cast<int32_t*>(link + n_ids);
+  const int n_bucket = (int)embedding_buckets(n_ids);
+  hipLaunchKernelGGL(embedding_bucket_zero_kernel, dim3((unsigned)((n_bucket + 255) / 256)), dim3(256), 0, s, bucket,
+                     n_bucket);
+  hipLaunchKernelGGL(embedding_bucket_count_kernel, dim3((unsigned)((n_ids + 255) / 256)), dim3(256), 0, s, ids, bucket,
+                     n_bucket, (int)n_ids, vocab_start, vocab_end);
   hipLaunchKernelGGL(embedding_link_kernel, dim3((unsigned)n_ids), dim3(256), 0, s, ids, link, (int)n_ids,
-                     vocab_start, vocab_end);
+                     vocab_start, vocab_end, bucket, n_bucket);
   MTP_CHECK_LAUNCH("embedding_link");
-  const dim3 grid((unsigned)n_ids, (unsigned)chunks), block(256);
+  const dim3 block(256);
+  const bool vec = dim % 8 == 0 &&
+                   ((reinterpret_cast<uintptr_t>(dout) | reinterpret_cast<uintptr_t>(dtable)) & 31) == 0;
+  const dim3 grid((unsigned)n_ids, (unsigned)(vec ? (dim + 2047) / 2048 : chunks));
+#define MTP_EMB_BWD(T, TO)                                                                                         \
+  do {                                                                                                             \
+    if (vec)                                                                                                       \
+      hipLaunchKernelGGL((embedding_bwd_vec_kernel<T, TO>), grid, block, 0, s, ids, (const T*)dout, (TO*)dtable,   \
+                         link, dim, vocab_start);                                                                  \
+    else                                                                                                           \
+      hipLaunchKernelGGL((embedding_bwd_kernel<T, TO>), grid, block, 0, s, ids, (const T*)dout, (TO*)dtable, link, \
+                         dim, vocab_start);                                                                        \
+  } while (0)
   if (dtype == MTP_F32 && dtable_dtype == MTP_F32)
-    hipLaunchKernelGGL((embedding_bwd_kernel<float, float>), grid, block, 0, s, ids, (const float*)dout,
-                       (float*)dtable, link, dim, vocab_start);
+    MTP_EMB_BWD(float, float);
   else if (dtype == MTP_BF16 && dtable_dtype == MTP_F32)
-    hipLaunchKernelGGL((embedding_bwd_kernel<uint16_t, float>), grid, block, 0, s, ids, (const uint16_t*)dout,
-                       (float*)dtable, link, dim, vocab_start);
+    MTP_EMB_BWD(uint16_t, float);
   else if (dtype == MTP_BF16 && dtable_dtype == MTP_BF16)
-    hipLaunchKernelGGL((embedding_bwd_kernel<uint16_t, uint16_t>), grid, block, 0, s, ids, (const uint16_t*)dout,
-                       (uint16_t*)dtable, link, dim, vocab_start);
+    MTP_EMB_BWD(uint16_t, uint16_t);
   else if (dtype == MTP_F16 && dtable_dtype == MTP_F32)
-    hipLaunchKernelGGL((embedding_bwd_kernel<f16s, float>), grid, block, 0, s, ids, (const f16s*)dout, (float*)dtable,
-                       link, dim, vocab_start);
+    MTP_EMB_BWD(f16s, float);
   else if (dtype == MTP_F16 && dtable_dtype == MTP_F16)
-    hipLaunchKernelGGL((embedding_bwd_kernel<f16s, f16s>), grid, block, 0, s, ids, (const f16s*)dout, (f16s*)dtable,
-                       link, dim, vocab_start);
+    MTP_EMB_BWD(f16s, f16s);
   else
     MTP_REQUIRE(false, MTP_EUNSUPPORTED, "embedding_bwd: the table gradient is fp32 or of the dtype of dout (%d -> %d)",
                 dtype, dtable_dtype);
+#undef MTP_EMB_BWD
   MTP_CHECK_LAUNCH("embedding_bwd");
   return MTP_OK;
 }
+

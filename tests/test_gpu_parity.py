@@ -416,6 +416,9 @@ def _lin_inputs(m, n, k, dtype, seed, bias=True):
     (torch.bfloat16, 300, 520, 136), (torch.bfloat16, 64, 50, 27), (torch.bfloat16, 1, 8, 8),
     (torch.float32, 100, 77, 33), (torch.float32, 1, 1, 1), (torch.bfloat16, 257, 255, 72),
     (torch.float32, 300, 520, 136), (torch.float32, 129, 132, 20), (torch.float32, 64, 8, 4), (torch.float32, 3, 260, 4100),
+    # k long enough for the forward kernel's register-staged pairs of k-tiles, with ragged m, n and end of k
+    (torch.bfloat16, 300, 520, 1000), (torch.bfloat16, 257, 255, 456), (torch.bfloat16, 129, 1000, 200),
+    (torch.bfloat16, 1000, 264, 232), (torch.bfloat16, 31, 700, 192), (torch.float16, 300, 520, 1000),
 ])
 def test_linear_fwd_bwd_vs_oracle(gpu, dtype, m, n, k):
     tol = TOL_F32 if dtype == torch.float32 else TOL_BF16
@@ -453,7 +456,9 @@ def test_bias_gelu_epilogue(gpu, dtype, m, n, k):
 
 @pytest.mark.parametrize("dtype,m,n,k", [(torch.bfloat16, 512, 2 * 14336, 4096), (torch.bfloat16, 512, 2 * 3584, 8192),
                                           (torch.bfloat16, 130, 2 * 100, 72), (torch.float32, 65, 2 * 24, 40),
-                                          (torch.bfloat16, 40, 2 * 13, 16)])
+                                          (torch.bfloat16, 40, 2 * 13, 16),
+                                          # ragged halves and end of k behind the staged pairs of k-tiles
+                                          (torch.bfloat16, 130, 2 * 300, 1000), (torch.bfloat16, 257, 2 * 136, 264)])
 def test_swiglu_epilogue(gpu, dtype, m, n, k):
     tol = TOL_F32 if dtype == torch.float32 else TOL_BF16
     x, w, _, _ = _lin_inputs(m, n, k, dtype, 50, bias=False)

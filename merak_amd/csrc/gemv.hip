@@ -908,6 +908,7 @@ int gemv_dispatch(const void* x, const void* w, const void* bias, void* y, void*
   const bool f16 = dtype == MTP_F16;
   if (rc) return rc;
   MTP_REQUIRE(y, MTP_EINVAL, "gemv: null output");
+  MTP_REQUIRE(y != x, MTP_EINVAL, "gemv: the output must not be the input (every workgroup reads all of X)");
   MTP_REQUIRE(epilogue == MTP_EPI_NONE || epilogue == MTP_EPI_BIAS || epilogue == MTP_EPI_SWIGLU, MTP_EINVAL,
               "gemv: epilogue %d not supported", epilogue);
   MTP_REQUIRE(epilogue != MTP_EPI_BIAS || bias, MTP_EINVAL, "gemv: MTP_EPI_BIAS without bias");

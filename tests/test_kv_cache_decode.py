@@ -454,6 +454,9 @@ def test_gemv_fused_rejects_bad_arguments(gpu):
         ops.gemv_fused(x, w, None, ops.EPI_SWIGLU, residual=torch.zeros(2, 32, dtype=torch.bfloat16, device=gpu))
     with pytest.raises(ValueError, match="residual"):
         ops.gemv_fused(x, w, residual=torch.zeros(2, 63, dtype=torch.bfloat16, device=gpu))
+    sq = torch.zeros(2, 1024, dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(RuntimeError, match="must not be the input"):                # in place on the input
+        ops.gemv_fused(sq, torch.zeros(1024, 1024, dtype=torch.bfloat16, device=gpu), out=sq)
     with pytest.raises(RuntimeError, match="8 x 4096"):                             # 9 rows do not fit
         x9 = torch.zeros(9, 1024, dtype=torch.bfloat16, device=gpu)
         ops.gemv_fused(x9, w, norm_weight=nw, sumsq_in=_sumsq16(x9))

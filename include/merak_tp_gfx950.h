@@ -198,7 +198,8 @@ int mtp_vocab_ce_rescale(void* grad, const float* grad_rows, float assumed,
  * ------------------------------------------------------------------------ */
 
 /* Y[B,N] = X[B,K] W[N,K]^T (+bias) ; epilogue NONE, BIAS or SWIGLU
- * (SWIGLU: y is [B,N/2] = silu(gate)*up with W = [gate rows | up rows]). */
+ * (SWIGLU: y is [B,N/2] = silu(gate)*up with W = [gate rows | up rows]).
+ * y must not be x (every workgroup reads all of X). */
 int mtp_gemv(const void* x, const void* w, const void* bias, void* y,
              int64_t B, int64_t N, int64_t K, int epilogue, int dtype, void* stream);
 

@@ -211,9 +211,8 @@ class _LMHeadCrossEntropy(torch.autograd.Function):
                                "sum of the losses); weight the positions through the unfused layers instead")
         ratio = float(first) / ctx.assumed_grad
         if ratio != 1.0:
-            for t in (dh, dw, db):
-                if t is not None:
-                    t.mul_(ratio)
+            # out of place: the saved gradients stay valid for a second backward over a retained graph
+            dh, dw, db = (None if t is None else t * ratio for t in (dh, dw, db))
         return (dh.view(*ctx.lead, dh.shape[-1]) if dh is not None else None), dw, db, None, None, None
 
 

@@ -66,12 +66,18 @@ def linear_fwd(x2d: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
                want_pre: bool = True) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
     """(y, act) = epilogue(x2d @ w.T + bias).  x2d [M,K], w [N,K] contiguous, same dtype."""
     dev = _require_gpu(x2d, w, bias)
+    if x2d.dim() != 2 or w.dim() != 2:
+        raise ValueError(f"linear_fwd: x must be [M, K] and weight [N, K], got {tuple(x2d.shape)} and {tuple(w.shape)}")
     M, K = x2d.shape
     N, K2 = w.shape
     if K != K2:
         raise ValueError(f"linear_fwd: x is [*, {K}] but weight is [{N}, {K2}]")
     if w.dtype != x2d.dtype or (bias is not None and bias.dtype != x2d.dtype):
         raise TypeError("linear_fwd: x, weight and bias must share one dtype")
+    if bias is not None and (bias.numel() != N or not bias.is_contiguous()):
+        raise ValueError(f"linear_fwd: bias must be a contiguous [{N}] tensor, got {tuple(bias.shape)}")
+    if epilogue == EPI_SWIGLU and N % 2:
+        raise ValueError(f"linear_fwd: SwiGLU needs an even number of weight rows, got {N}")
     x2d, w = _contig(x2d), _contig(w)
     has_act = epilogue in (EPI_BIAS_GELU, EPI_SWIGLU, EPI_GELU)
     y = torch.empty((M, N), dtype=x2d.dtype, device=dev) if (want_pre or not has_act) else None
@@ -93,6 +99,8 @@ def linear_fwd(x2d: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
 
 def linear_dgrad(dy2d: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     dev = _require_gpu(dy2d, w)
+    if dy2d.dim() != 2 or w.dim() != 2:
+        raise ValueError(f"linear_dgrad: dy must be [M, N] and weight [N, K], got {tuple(dy2d.shape)} and {tuple(w.shape)}")
     M, N = dy2d.shape
     N2, K = w.shape
     if N != N2 or dy2d.dtype != w.dtype:
@@ -109,6 +117,8 @@ def linear_wgrad(dy2d: torch.Tensor, x2d: torch.Tensor, want_db: bool, out_dtype
                  dw: Optional[torch.Tensor] = None, db: Optional[torch.Tensor] = None,
                  accumulate: bool = False) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     dev = _require_gpu(dy2d, x2d, dw, db)
+    if dy2d.dim() != 2 or x2d.dim() != 2:
+        raise ValueError(f"linear_wgrad: dy must be [M, N] and x [M, K], got {tuple(dy2d.shape)} and {tuple(x2d.shape)}")
     M, N = dy2d.shape
     M2, K = x2d.shape
     if M != M2 or dy2d.dtype != x2d.dtype:
@@ -125,6 +135,8 @@ def linear_wgrad(dy2d: torch.Tensor, x2d: torch.Tensor, want_db: bool, out_dtype
         db = torch.empty((N,), dtype=out_dtype, device=dev)
     if dw.shape != (N, K) or not dw.is_contiguous() or dw.dtype != out_dtype:
         raise ValueError("linear_wgrad: dw must be a contiguous [N,K] tensor of the output dtype")
+    if want_db and (db.numel() != N or not db.is_contiguous() or db.dtype != out_dtype):
+        raise ValueError("linear_wgrad: db must be a contiguous [N] tensor of the output dtype")
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().mtp_linear_wgrad(_p(dy2d), _p(x2d), _p(dw), _p(db) if want_db else None, M, N, K,
                                                _dt(dy2d), _DTYPES[out_dtype], int(accumulate), _stream(dev)),
@@ -134,7 +146,11 @@ def linear_wgrad(dy2d: torch.Tensor, x2d: torch.Tensor, want_db: bool, out_dtype
 
 def activation_bwd(dact: torch.Tensor, y: torch.Tensor, epilogue: int) -> torch.Tensor:
     dev = _require_gpu(dact, y)
+    if y.dim() != 2 or dact.dim() != 2 or dact.dtype != y.dtype:
+        raise ValueError("activation_bwd: dact and y must be 2-D tensors of one dtype")
     M, N = y.shape
+    if tuple(dact.shape) != (M, N // 2 if epilogue == EPI_SWIGLU else N):
+        raise ValueError(f"activation_bwd: dact {tuple(dact.shape)} does not match y {tuple(y.shape)} for epilogue {epilogue}")
     dact, y = _contig(dact), _contig(y)
     dy = torch.empty_like(y)
     with torch.cuda.device(dev):
@@ -174,6 +190,10 @@ def embedding_bwd(ids: torch.Tensor, dout: torch.Tensor, rows: int, vocab_start:
     d2 = _contig(dout).view(-1, dim)
     if flat.dtype != torch.int64:
         raise TypeError(f"embedding ids must be int64, got {flat.dtype}")
+    if d2.shape[0] != flat.numel():
+        raise ValueError(f"embedding_bwd: {d2.shape[0]} gradient rows for {flat.numel()} ids")
+    if rows != vocab_end - vocab_start:
+        raise ValueError("embedding_bwd: table rows do not match the vocab range")
     if out is None:
         out = torch.zeros((rows, dim), dtype=dtype or d2.dtype, device=dev)
     elif tuple(out.shape) != (rows, dim) or not out.is_contiguous():
@@ -212,9 +232,20 @@ def vocab_ce_bwd_(logits2d: torch.Tensor, target1d: torch.Tensor, row_max: Optio
 
     row_max = row_sumexp = None: logits2d already holds the softmax."""
     dev = _require_gpu(logits2d, target1d, row_max, row_sumexp, grad_out)
+    if target1d.dtype != torch.int64:
+        raise TypeError(f"cross-entropy targets must be int64, got {target1d.dtype}")
+    if not logits2d.is_contiguous():
+        raise ValueError("vocab_parallel_cross_entropy needs contiguous logits")
     n, v = logits2d.shape
+    if target1d.numel() != n:
+        raise ValueError(f"target has {target1d.numel()} entries for {n} logits rows")
+    for name, t in (("row_max", row_max), ("row_sumexp", row_sumexp)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != n or not t.is_contiguous()):
+            raise ValueError(f"vocab_ce_bwd_: {name} must be contiguous fp32 [{n}]")
     if grad_out is not None:
         grad_out = _contig(grad_out.to(torch.float32))
+        if grad_out.numel() != n:
+            raise ValueError(f"grad_out has {grad_out.numel()} entries for {n} logits rows")
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().mtp_vocab_ce_bwd(_p(logits2d), _p(_contig(target1d)), _p(row_max), _p(row_sumexp),
                                                _p(grad_out), n, v, vocab_start, _dt(logits2d), _stream(dev)),
@@ -281,12 +312,19 @@ def _decode_dtype(what: str, *ts: torch.Tensor) -> torch.dtype:
     return dt
 
 
+def _gemv_shapes(what: str, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]):
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise ValueError(f"{what}: x must be [B, K] and weight [N, K], got {tuple(x.shape)} and {tuple(w.shape)}")
+    if bias is not None and (bias.numel() != w.shape[0] or not bias.is_contiguous()):
+        raise ValueError(f"{what}: bias must be a contiguous [{w.shape[0]}] tensor, got {tuple(bias.shape)}")
+    return x.shape[0], w.shape[0], x.shape[1]
+
+
 def gemv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE,
          workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     dev = _require_gpu(x, w, bias, workspace)
     dt = _decode_dtype("gemv", x, w, bias)
-    B, K = x.shape
-    N = w.shape[0]
+    B, N, K = _gemv_shapes("gemv", x, w, bias)
     x, w = _contig(x), _contig(w)
     y = torch.empty((B, N // 2 if epilogue == EPI_SWIGLU else N), dtype=dt, device=dev)
     wbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
@@ -313,8 +351,7 @@ def gemv_fused(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = 
     Returns ``y`` or ``(y, sumsq)``."""
     dev = _require_gpu(x, w, bias, workspace, norm_weight, sumsq_in, residual, out)
     dt = _decode_dtype("gemv_fused", x, w, bias)
-    B, K = x.shape
-    N = w.shape[0]
+    B, N, K = _gemv_shapes("gemv_fused", x, w, bias)
     x, w = _contig(x), _contig(w)
     n_out = N // 2 if epilogue == EPI_SWIGLU else N
     if norm_weight is not None:
@@ -342,8 +379,7 @@ def gemv_argmax(x: torch.Tensor, w: torch.Tensor, workspace: Optional[torch.Tens
     """-> (idx int64 [B], maxval fp32 [B]) without materialising the logits."""
     dev = _require_gpu(x, w, workspace)
     dt = _decode_dtype("gemv_argmax", x, w)
-    B, K = x.shape
-    N = w.shape[0]
+    B, N, K = _gemv_shapes("gemv_argmax", x, w, None)
     x, w = _contig(x), _contig(w)
     need = _lib.lib().mtp_gemv_argmax_workspace_bytes(B, N, K)
     if workspace is None:
@@ -351,7 +387,8 @@ def gemv_argmax(x: torch.Tensor, w: torch.Tensor, workspace: Optional[torch.Tens
     idx = torch.empty((B,), dtype=torch.int64, device=dev)
     val = torch.empty((B,), dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().mtp_gemv_argmax(_p(x), _p(w), _p(idx), _p(val), _p(workspace), workspace.numel(), B, N, K,
+        _lib.check(_lib.lib().mtp_gemv_argmax(_p(x), _p(w), _p(idx), _p(val), _p(workspace),
+                                              workspace.numel() * workspace.element_size(), B, N, K,
                                               _DTYPES[dt], _stream(dev)), "mtp_gemv_argmax")
     return idx, val
 

@@ -311,7 +311,10 @@ def test_lm_head_cross_entropy_chunked(gpu, dtype, n, k, v, chunk, has_bias):
     hg2 = h.to(gpu).requires_grad_(True)
     head.weight.grad = None
     l2 = mpu.lm_head_cross_entropy(hg2, head, t.to(gpu), chunk_rows=chunk)
-    (5.0 * l2.sum()).backward()
+    (5.0 * l2.sum()).backward(retain_graph=True)
+    assert rel(hg2.grad, hr.grad * (5.0 * n / 3.0)) < tol
+    hg2.grad = None
+    (5.0 * l2.sum()).backward()                    # a second pass over the retained graph scales once, not twice
     assert rel(hg2.grad, hr.grad * (5.0 * n / 3.0)) < tol
     with pytest.raises(RuntimeError, match="one upstream gradient"):
         l3 = mpu.lm_head_cross_entropy(h.to(gpu).requires_grad_(True), head, t.to(gpu), chunk_rows=chunk)
@@ -965,3 +968,37 @@ def test_gemv_swiglu_seeded_sweep(gpu):
         pre = F.linear(x.float(), w.float()).bfloat16().float()
         y = ops.gemv(x.to(gpu), w.to(gpu), None, ops.EPI_SWIGLU)
         assert rel(y, R.swiglu(pre)) < TOL_BF16, (case, b, half, k)
+
+
+def test_wrappers_reject_mismatched_shapes_before_any_launch(gpu):
+    """Pointers carry no shape: the tensor-level wrappers are where a mismatch must stop."""
+    bf = dict(device=gpu, dtype=torch.bfloat16)
+    x, w = torch.zeros(4, 64, **bf), torch.zeros(32, 64, **bf)
+    with pytest.raises(ValueError, match="bias"):
+        ops.linear_fwd(x, w, torch.zeros(31, **bf), ops.EPI_BIAS)
+    with pytest.raises(ValueError, match="even"):
+        ops.linear_fwd(x, torch.zeros(31, 64, **bf), None, ops.EPI_SWIGLU)
+    with pytest.raises(ValueError):
+        ops.linear_fwd(x.view(2, 2, 64), w, None)
+    with pytest.raises(ValueError, match="db"):
+        ops.linear_wgrad(torch.zeros(4, 32, **bf), x, True, dw=torch.zeros(32, 64, **bf), db=torch.zeros(8, **bf))
+    with pytest.raises(ValueError, match="dact"):
+        ops.activation_bwd(torch.zeros(4, 32, **bf), torch.zeros(4, 32, **bf), ops.EPI_SWIGLU)
+    ids = torch.zeros(6, dtype=torch.int64, device=gpu)
+    with pytest.raises(ValueError, match="gradient rows"):
+        ops.embedding_bwd(ids, torch.zeros(5, 16, **bf), 10, 0, 10)
+    with pytest.raises(ValueError, match="vocab range"):
+        ops.embedding_bwd(ids, torch.zeros(6, 16, **bf), 12, 0, 10)
+    with pytest.raises(ValueError, match=r"\[B, K\]"):
+        ops.gemv(torch.zeros(2, 32, **bf), w)
+    with pytest.raises(ValueError, match="bias"):
+        ops.gemv(torch.zeros(2, 64, **bf), w, torch.zeros(16, **bf), ops.EPI_BIAS)
+    with pytest.raises(ValueError, match=r"\[B, K\]"):
+        ops.gemv_argmax(torch.zeros(2, 128, **bf), w)
+    lg, t = torch.zeros(4, 8, device=gpu), torch.zeros(4, dtype=torch.int64, device=gpu)
+    with pytest.raises(ValueError, match="row_max"):
+        ops.vocab_ce_bwd_(lg, t, torch.zeros(3, device=gpu), torch.zeros(4, device=gpu), None, 0)
+    with pytest.raises(ValueError, match="grad_out"):
+        ops.vocab_ce_bwd_(lg, t, None, None, torch.zeros(5, device=gpu), 0)
+    with pytest.raises(TypeError):
+        ops.vocab_ce_bwd_(lg, t.int(), None, None, None, 0)

@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ d
     }
 #pragma unroll
     for (int e = 0; e < EPV; e++) {
-      const float s = 1.0f / (1.0f + __expf(-g[e]));  // sigmoid(gate)
+      const float s = sigmoid_f(g[e]);
       const float silu = g[e] * s;
       rg[e] = d[e] * u[e] * (s + silu * (1.0f - s));
       ru[e] = d[e] * silu;

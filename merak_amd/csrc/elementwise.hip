@@ -70,42 +70,62 @@ __global__ __launch_bounds__(256) void gelu_bwd_kernel(const T* __restrict__ dac
 
 // y = [gate | up] of width N = 2H per row; dact has width H.
 //   dgate = dact * up * silu'(gate),  dup = dact * silu(gate)
-// VEC: rows are 16-byte aligned and H % EPV == 0
+// VEC: rows are 16-byte aligned and H % EPV == 0.
+// blockIdx.x picks 256 vectors of a row, blockIdx.y the rows (stride gridDim.y): no index arithmetic beyond
+// additions, and two rows per step so that six loads per thread are on their way before the first is used.
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ dact, const T* __restrict__ y,
                                                          T* __restrict__ dy, int64_t M, int64_t H) {
   constexpr int EPV = VEC ? Io<T>::EPV : 1;
-  const int64_t hv = H / EPV;
-  const int64_t total = M * hv;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int64_t m = i / hv, c = (i - m * hv) * EPV;
+  const int64_t c = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * EPV;   // first column of this thread
+  if (c >= H) return;
+  struct Row {
+    float g[EPV], u[EPV], d[EPV];
+  };
+  auto load = [&](int64_t m, Row& r) {
     const T* pg = y + m * 2 * H + c;
-    const T* pu = pg + H;
-    const T* pd = dact + m * H + c;
-    T* og = dy + m * 2 * H + c;
-    T* ou = og + H;
-    float g[EPV], u[EPV], d[EPV], rg[EPV], ru[EPV];
     if constexpr (VEC) {
-      Io<T>::unpack(*reinterpret_cast<const u32x4_t*>(pg), g);
-      Io<T>::unpack(*reinterpret_cast<const u32x4_t*>(pu), u);
-      Io<T>::unpack(*reinterpret_cast<const u32x4_t*>(pd), d);
+      // read once, by this kernel only: streaming loads
+      const u32x4_t vg = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(pg));
+      const u32x4_t vu = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(pg + H));
+      const u32x4_t vd = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(dact + m * H + c));
+      Io<T>::unpack(vg, r.g);
+      Io<T>::unpack(vu, r.u);
+      Io<T>::unpack(vd, r.d);
     } else {
-      g[0] = Io<T>::ld(pg); u[0] = Io<T>::ld(pu); d[0] = Io<T>::ld(pd);
+      r.g[0] = Io<T>::ld(pg); r.u[0] = Io<T>::ld(pg + H); r.d[0] = Io<T>::ld(dact + m * H + c);
     }
+  };
+  auto finish = [&](int64_t m, const Row& r) {
+    float rg[EPV], ru[EPV];
 #pragma unroll
     for (int e = 0; e < EPV; e++) {
-      const float s = sigmoid_f(g[e]);
-      const float silu = g[e] * s;
-      rg[e] = d[e] * u[e] * (s + silu * (1.0f - s));
-      ru[e] = d[e] * silu;
+      const float s = sigmoid_f(r.g[e]);
+      const float silu = r.g[e] * s;
+      rg[e] = r.d[e] * r.u[e] * (s + silu * (1.0f - s));
+      ru[e] = r.d[e] * silu;
     }
+    T* og = dy + m * 2 * H + c;
     if constexpr (VEC) {
       *reinterpret_cast<u32x4_t*>(og) = Io<T>::pack(rg);
-      *reinterpret_cast<u32x4_t*>(ou) = Io<T>::pack(ru);
+      *reinterpret_cast<u32x4_t*>(og + H) = Io<T>::pack(ru);
     } else {
-      Io<T>::st(og, rg[0]); Io<T>::st(ou, ru[0]);
+      Io<T>::st(og, rg[0]); Io<T>::st(og + H, ru[0]);
     }
+  };
+  const int64_t step = gridDim.y;
+  int64_t m = blockIdx.y;
+  for (; m + step < M; m += 2 * step) {
+    Row r0, r1;
+    load(m, r0);
+    load(m + step, r1);
+    finish(m, r0);
+    finish(m + step, r1);
+  }
+  if (m < M) {
+    Row r0;
+    load(m, r0);
+    finish(m, r0);
   }
 }
 
@@ -208,28 +228,26 @@ extern "C" int mtp_activation_bwd(const void* dact, const void* y, void* dy, int
     const int64_t H = N / 2;
     const int epv = dtype == MTP_F32 ? 4 : 8;
     const bool vec = (al & 15) == 0 && H % epv == 0;
-    if (dtype == MTP_F32) {
-      if (vec)
-        hipLaunchKernelGGL((swiglu_bwd_kernel<float, true>), dim3(grid_for(M * H / 4)), dim3(256), 0, s,
-                           (const float*)dact, (const float*)y, (float*)dy, M, H);
-      else
-        hipLaunchKernelGGL((swiglu_bwd_kernel<float, false>), dim3(grid_for(M * H)), dim3(256), 0, s,
-                           (const float*)dact, (const float*)y, (float*)dy, M, H);
-    } else if (dtype == MTP_F16) {
-      if (vec)
-        hipLaunchKernelGGL((swiglu_bwd_kernel<f16s, true>), dim3(grid_for(M * H / 8)), dim3(256), 0, s,
-                           (const f16s*)dact, (const f16s*)y, (f16s*)dy, M, H);
-      else
-        hipLaunchKernelGGL((swiglu_bwd_kernel<f16s, false>), dim3(grid_for(M * H)), dim3(256), 0, s,
-                           (const f16s*)dact, (const f16s*)y, (f16s*)dy, M, H);
-    } else {
-      if (vec)
-        hipLaunchKernelGGL((swiglu_bwd_kernel<uint16_t, true>), dim3(grid_for(M * H / 8)), dim3(256), 0, s,
-                           (const uint16_t*)dact, (const uint16_t*)y, (uint16_t*)dy, M, H);
-      else
-        hipLaunchKernelGGL((swiglu_bwd_kernel<uint16_t, false>), dim3(grid_for(M * H)), dim3(256), 0, s,
-                           (const uint16_t*)dact, (const uint16_t*)y, (uint16_t*)dy, M, H);
-    }
+    // columns in blocks of 256 threads; rows spread over about 16 workgroups per CU
+    const int64_t col_blocks = ((vec ? H / epv : H) + 255) / 256;
+    MTP_REQUIRE(col_blocks < (1ll << 31), MTP_EINVAL, "activation_bwd: rows too long");
+    int64_t row_groups = (4096 + col_blocks - 1) / col_blocks;
+    if (row_groups > M) row_groups = M;
+    if (row_groups > 65535) row_groups = 65535;
+    const dim3 grid((unsigned)col_blocks, (unsigned)row_groups);
+#define MTP_SWIGLU_BWD(T)                                                                                          \
+  do {                                                                                                             \
+    if (vec)                                                                                                       \
+      hipLaunchKernelGGL((swiglu_bwd_kernel<T, true>), grid, dim3(256), 0, s, (const T*)dact, (const T*)y, (T*)dy, \
+                         M, H);                                                                                    \
+    else                                                                                                           \
+      hipLaunchKernelGGL((swiglu_bwd_kernel<T, false>), grid, dim3(256), 0, s, (const T*)dact, (const T*)y,        \
+                         (T*)dy, M, H);                                                                            \
+  } while (0)
+    if (dtype == MTP_F32) MTP_SWIGLU_BWD(float);
+    else if (dtype == MTP_F16) MTP_SWIGLU_BWD(f16s);
+    else MTP_SWIGLU_BWD(uint16_t);
+#undef MTP_SWIGLU_BWD
   } else {
     MTP_REQUIRE(false, MTP_EINVAL, "activation_bwd: epilogue %d has no activation", epilogue);
   }

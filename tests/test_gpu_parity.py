@@ -474,6 +474,17 @@ def test_swiglu_epilogue(gpu, dtype, m, n, k):
     assert rel(d, R.swiglu_backward(dact.float(), y.float().cpu())) < tol
 
 
+@pytest.mark.parametrize("dtype,m,h", [(torch.bfloat16, 1, 8), (torch.bfloat16, 3, 4096), (torch.float32, 5001, 24),
+                                       (torch.bfloat16, 9000, 40), (torch.float16, 777, 2056), (torch.bfloat16, 300, 7)])
+def test_swiglu_backward_row_and_column_split(gpu, dtype, m, h):
+    """One row, more rows than row groups (several steps and an odd one left), rows wider than one column
+    block, unaligned rows."""
+    y = torch.randn(m, 2 * h, generator=gen(58)).to(dtype)
+    dact = torch.randn(m, h, generator=gen(59)).to(dtype)
+    d = ops.activation_bwd(dact.to(gpu), y.to(gpu), ops.EPI_SWIGLU)
+    assert rel(d, R.swiglu_backward(dact.float(), y.float())) < (TOL_F32 if dtype == torch.float32 else TOL_BF16)
+
+
 def test_gpt2_small_fp32_full_size(gpu):
     """Config 1 in full: Column 768->3072 bias+GeLU, Row 3072->768 bias, 8x1024 tokens, fp32, via the modules."""
     set_args(use_cpu_initialization=True, params_dtype=torch.float32)

@@ -596,21 +596,31 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   }
 }
 
-// One workgroup per batch row folds that row's per-workgroup partials.
-__global__ __launch_bounds__(256) void argmax_finish_kernel(const ArgPart* __restrict__ part, int n_part, int B,
-                                                            int64_t* __restrict__ idx, float* __restrict__ maxval) {
+// One workgroup per batch row folds that row's per-workgroup partials.  The kernel is a chain of memory
+// latencies (its input was written a moment ago by other CUs), so every thread asks for eight partials
+// before it looks at the first: 256 threads cover 2048 partials per round trip.
+constexpr int AF_THREADS = 256, AF_WAVES = AF_THREADS / MTP_WAVE, AF_DEPTH = 8;
+__global__ __launch_bounds__(AF_THREADS) void argmax_finish_kernel(const ArgPart* __restrict__ part, int n_part, int B,
+                                                                   int64_t* __restrict__ idx, float* __restrict__ maxval) {
   const int b = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   float bv = 0.f;
   int64_t bi = INT64_MAX;
   bool have = false;
-  for (int p = threadIdx.x; p < n_part; p += 256) {
-    const ArgPart a = part[(int64_t)p * B + b];
-    if (!have || arg_better(a.v, a.i, bv, bi)) {
-      bv = a.v;
-      bi = a.i;
-      have = true;
+  for (int p0 = threadIdx.x; p0 < n_part; p0 += AF_THREADS * AF_DEPTH) {
+    ArgPart a[AF_DEPTH];
+#pragma unroll
+    for (int u = 0; u < AF_DEPTH; u++) {
+      const int p = p0 + u * AF_THREADS;
+      a[u] = part[(int64_t)(p < n_part ? p : p0) * B + b];   // past the end: the first one again (changes nothing)
     }
+#pragma unroll
+    for (int u = 0; u < AF_DEPTH; u++)
+      if (!have || arg_better(a[u].v, a[u].i, bv, bi)) {
+        bv = a[u].v;
+        bi = a[u].i;
+        have = true;
+      }
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
@@ -623,9 +633,9 @@ __global__ __launch_bounds__(256) void argmax_finish_kernel(const ArgPart* __res
       have = true;
     }
   }
-  __shared__ float sv[4];
-  __shared__ int64_t si[4];
-  __shared__ int sh[4];
+  __shared__ float sv[AF_WAVES];
+  __shared__ int64_t si[AF_WAVES];
+  __shared__ int sh[AF_WAVES];
   if (lane == 0) {
     sv[wave] = bv;
     si[wave] = bi;
@@ -633,7 +643,7 @@ __global__ __launch_bounds__(256) void argmax_finish_kernel(const ArgPart* __res
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int wv = 1; wv < 4; wv++)
+    for (int wv = 1; wv < AF_WAVES; wv++)
       if (sh[wv] && (!have || arg_better(sv[wv], si[wv], bv, bi))) {
         bv = sv[wv];
         bi = si[wv];
@@ -994,7 +1004,7 @@ extern "C" int mtp_gemv_argmax(const void* x, const void* w, int64_t* idx, float
   rc = launch_gemv<2>(x, w, nullptr, nullptr, (ArgPart*)workspace, B, N, K, pick_gemv_cfg(B, N, K, 2), s, &n_wg,
                       dtype == MTP_F16);
   if (rc) return rc;
-  hipLaunchKernelGGL(argmax_finish_kernel, dim3((unsigned)B), dim3(256), 0, s, (const ArgPart*)workspace, (int)n_wg, (int)B,
+  hipLaunchKernelGGL(argmax_finish_kernel, dim3((unsigned)B), dim3(AF_THREADS), 0, s, (const ArgPart*)workspace, (int)n_wg, (int)B,
                      idx, maxval);
   MTP_CHECK_LAUNCH("argmax_finish");
   return MTP_OK;

@@ -29,6 +29,15 @@ are closed forms, library routines and brute force:
   sample_tail             numpy.searchsorted on the cumulative distribution; draw frequencies over 40000
                           uniforms against the probabilities (torch.multinomial's own random stream cannot be
                           reproduced, so the draw takes the uniforms as an argument)
+  decode_step             reduces to the plain linears, swiglu and greedy_argmax above on the same inputs
+  rms_norm                transformers' LlamaRMSNorm module; constant rows (closed form 3 / sqrt(9 + eps))
+  rope_tables, apply_rope transformers' LlamaRotaryEmbedding + apply_rotary_pos_emb; position 0 is the identity
+    (rotate_half)
+  attn_decode             torch's scaled_dot_product_attention over the valid prefix with the kv heads repeated
+                          per group; a single cached token returns its value; entries past the valid length
+                          (junk, NaN) do not change the result
+  llama_block_step        token by token through the cache == the full-sequence forward of a random-weight
+                          transformers LlamaForCausalLM (the row the reference slices out of it)
 
 The third-party arithmetic under all of this is PyTorch (the reference pins
 torch>=2.0.0, setup.py:46) and, for the activations, transformers

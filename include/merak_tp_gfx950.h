@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTP_ABI_VERSION 5
+#define MTP_ABI_VERSION 6
 
 /* element types.  MTP_F16 is IEEE half, what the reference's --fp16 sets as
  * params_dtype (Merak/merak_args/args.py:584-585). */
@@ -349,6 +349,12 @@ int mtp_attn_decode_append(const void* qkv, const void* cos_table, const void* s
 /* ------------------------------------------------------------------------
  * Measurement helpers (used by bench.py to state what this GPU can do).
  * ------------------------------------------------------------------------ */
+/* The library reads its MTP_* tuning variables (tile and slice choices that
+ * select among kernels computing the same result) from the environment once,
+ * at their first use; no launch calls getenv.  This re-reads all of them, for
+ * a process that changes its environment between measurements or tests.  Must
+ * not run concurrently with launches.  No counterpart in the reference. */
+void mtp_reload_tuning(void);
 /* dst[0:bytes] = src[0:bytes] with 16-byte accesses; bytes % 16 == 0. */
 int mtp_stream_copy(const void* src, void* dst, int64_t bytes, void* stream);
 /* Register-resident bf16 MFMA loop: iters x 32x32x16 MFMAs per wave on

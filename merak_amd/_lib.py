@@ -19,7 +19,7 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmerak_tp_gfx950.so"
 
 MTP_F32, MTP_BF16, MTP_F16 = 0, 1, 2
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_SWIGLU, EPI_GELU = 0, 1, 2, 3, 4
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _i64, _int, _vp = C.c_int64, C.c_int, C.c_void_p
 
@@ -57,6 +57,7 @@ SIGNATURES = {
     "mtp_attn_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _int, _i64, _i64, C.c_float, _int, _vp]),
     "mtp_attn_decode_append": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _int, _i64, _i64, _i64,
                                       C.c_float, _int, _vp]),
+    "mtp_reload_tuning": (None, []),
     "mtp_stream_copy": (_int, [_vp, _vp, _i64, _vp]),
     "mtp_mfma_peak": (_int, [_vp, _i64, _i64, _int, _vp]),
 }

@@ -15,6 +15,45 @@ void mtp_set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
+// ---- tuning variables: read once, re-read on request ----------------------------------------------------
+#include <atomic>
+#include <mutex>
+#include <stdlib.h>
+namespace {
+std::mutex g_tune_mu;
+MtpTune* g_tune_head = nullptr;
+void tune_read(MtpTune* t) {
+  const char* e = getenv(t->name);
+  if (e && *e) {
+    t->value = atoi(e);
+    __atomic_store_n(&t->state, 2, __ATOMIC_RELEASE);
+  } else {
+    __atomic_store_n(&t->state, 1, __ATOMIC_RELEASE);
+  }
+}
+}  // namespace
+
+MtpTune::MtpTune(const char* n) : name(n), value(0), state(0), next(nullptr) {
+  std::lock_guard<std::mutex> lk(g_tune_mu);
+  next = g_tune_head;
+  g_tune_head = this;
+}
+bool MtpTune::is_set() {
+  int st = __atomic_load_n(&state, __ATOMIC_ACQUIRE);
+  if (st == 0) {
+    std::lock_guard<std::mutex> lk(g_tune_mu);
+    if (state == 0) tune_read(this);
+    st = state;
+  }
+  return st == 2;
+}
+int MtpTune::get(int dflt) { return is_set() ? value : dflt; }
+
+extern "C" void mtp_reload_tuning(void) {
+  std::lock_guard<std::mutex> lk(g_tune_mu);
+  for (MtpTune* t = g_tune_head; t; t = t->next) tune_read(t);
+}
+
 extern "C" int mtp_abi_version(void) { return MTP_ABI_VERSION; }
 
 extern "C" const char* mtp_last_error(void) { return g_err; }

@@ -622,10 +622,8 @@ __global__ __launch_bounds__(64) void rope_append_kernel(const uint16_t* __restr
 }
 
 int pick_splits(int64_t B, int n_kv, int64_t len_bound) {
-  if (const char* e = getenv("MTP_ATTN_SPLITS")) {
-    const int v = atoi(e);
-    if (v >= 1) return v;
-  }
+  static MtpTune tune_splits("MTP_ATTN_SPLITS");
+  if (tune_splits.get(0) >= 1) return tune_splits.get(0);
   const int64_t tiles = (len_bound + AD_TILE - 1) / AD_TILE;
   const int64_t by_len = (tiles + 2 * AD_MAX_WAVES - 1) / (2 * AD_MAX_WAVES);   // at least two tiles per wave
   // about one workgroup per CU: a workgroup's start-up and its merge are paid once per split
@@ -682,14 +680,13 @@ int launch_attn(bool append, AttnArgs a, const char* what, void* workspace, int6
   a.group = group;
   a.max_len = max_len;
   a.splits = splits;
-  a.rot_mul = 1;
-  if (const char* e = getenv("MTP_ATTN_ROT")) a.rot_mul = atoi(e);
+  static MtpTune tune_rot("MTP_ATTN_ROT"), tune_cfg("MTP_ATTN_CFG");
+  a.rot_mul = tune_rot.get(1);
   if (a.rot_mul < 0) a.rot_mul = 0;   // taken modulo the tile count: must not go negative
   a.scale_log2e = scale * 1.4426950408889634f;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(splits, n_kv_heads, (unsigned)B);
-  int cfg = 0;
-  if (const char* e = getenv("MTP_ATTN_CFG")) cfg = atoi(e);
+  const int cfg = tune_cfg.get(0);
   const bool f16 = dtype == MTP_F16;
 #define MTP_ATTN_LAUNCH(W, R, NT)                                                                        \
   do {                                                                                                   \

@@ -60,9 +60,17 @@ struct GemmArgs {
   int64_t lda, ldb, ldc, ldc2;
   int accumulate;      // C += result
   int half;            // SwiGLU: number of gate columns (N/2)
-  int debug;           // measurement only (MTP_GEMM_DEBUG): 1 = every tile loads tile (0,0), 2 = no epilogue
+#ifdef MTP_MEASURE
+  int debug;           // measurement builds only (MTP_GEMM_DEBUG): 1 = every tile loads tile (0,0), 2 = no epilogue
                        // stores, 4 = every DMA reads out of range (no memory traffic).  Results are wrong with any bit set.
+#endif
 };
+// The measurement switches exist only in builds made with -DMTP_MEASURE; the shipped library has none of them.
+#ifdef MTP_MEASURE
+#define MTP_DBG(p, bits) (((p).debug & (bits)) != 0)
+#else
+#define MTP_DBG(p, bits) false
+#endif
 
 enum : int { OUT_BF16 = 0, OUT_F32 = 1 };
 // Plain product that also sums the rows of its A operand along k: with A = dY^T (the wgrad product) those sums
@@ -340,6 +348,634 @@ struct ColOperand {
 template <int LAY, int ROWS, int NW> struct OperandOf { using type = RowOperand<ROWS, NW>; };
 template <int ROWS, int NW> struct OperandOf<LAY_COL, ROWS, NW> { using type = ColOperand<ROWS, NW>; };
 
+// ---------------------------------------------------------------------------
+// Epilogue, shared by the two main loops.  acc[i][j] is the 32x32 block (i, j) of the wave's part of the tile;
+// which rows and columns of the tile that is depends on the main loop:
+//   QMAP = false: the wave owns a contiguous (BM/2) x (BN/WGN) rectangle: block row i starts at tile row
+//                 wm*BM/2 + 32 i, block column j at tile column wn*BN/WGN + 32 j;
+//   QMAP = true:  the tile's rows (columns) form two halves, and a wave owns HI (HJ) blocks of each half:
+//                 block row i starts at tile row (i/HI)*BM/2 + wm*32*HI + 32 (i%HI), columns likewise.
+// With SwiGLU both forms put the gate columns into blocks j < TJ/2 and the matching up columns into the others.
+// ---------------------------------------------------------------------------
+template <int BM, int BN, int EPI, int OUT, int NW, bool F16, bool QMAP, int LDS_BYTES, int TI, int TJ>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16_t (&acc)[TI][TJ], float (&rsum)[TI], char* lds,
+                                              int m0, int n0, int tn, int wave, int lane) {
+  using X = X16<F16>;
+  constexpr int WGM = 2, WGN = NW / 2;
+  constexpr int HI = TI / 2, HJ = TJ / 2;
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int lh = lane >> 5, l32 = lane & 31;
+  // first tile row of the wave's block row i
+  auto blk_row = [&](int i) -> int {
+    if (QMAP) return (i / HI) * (BM / 2) + wm * (32 * HI) + (i % HI) * 32;
+    return wm * (BM / WGM) + 32 * i;
+  };
+
+  if constexpr (EPI == EPI_ROWSUM) {
+
+    if (tn == 0 && wn == 0) {
+#pragma unroll
+      for (int i = 0; i < TI; i++) {
+        const float t = rsum[i] + __shfl_xor(rsum[i], 32, 64);  // the two k halves of a row
+        const int row = m0 + blk_row(i) + l32;
+        if (lh == 0 && row < p.M) {
+          if (OUT == OUT_F32) {
+            float* q = (float*)p.rowsum + row;
+            *q = p.accumulate ? *q + t : t;
+          } else {
+            uint16_t* q = (uint16_t*)p.rowsum + row;
+            *q = X::to_bits(p.accumulate ? X::from_bits(*q) + t : t);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- epilogue ----------------------------------------------------------------
+  // acc[i][j][r]: row m = m0 + wm*BM/2 + 32i + l32, column block j, n_local = 8*(r/4) + 4*lh + r%4.
+  // Stage 32 rows x (BN/2) columns per wave through LDS, then 16-byte row-contiguous stores.
+  constexpr int WN = BN / WGN;                     // columns per wave
+  constexpr int ESZ = (OUT == OUT_F32) ? 4 : 2;
+  constexpr int PITCH = WN * ESZ + 16;             // bytes per staged row (+16: spread rows over banks)
+  static_assert(NW * 32 * PITCH <= LDS_BYTES, "epilogue staging exceeds the tile buffers");
+  char* stage = lds + wave * (32 * PITCH);
+
+  // global column of the first element of block j for this wave (main output C)
+  auto col_of_block = [&](int j) -> int {
+    if (EPI == MTP_EPI_SWIGLU) {
+      const int hj = TJ / 2;
+      return (j < hj ? 0 : p.half) + n0 + wn * (WN / 2) + (j % hj) * 32;
+    }
+    if (QMAP) return n0 + (j / HJ) * (BN / 2) + wn * (32 * HJ) + (j % HJ) * 32;
+    return n0 + wn * WN + j * 32;
+  };
+  // first column past the valid range of block j: SwiGLU gate blocks end at `half` (the columns after it
+  // are the up matrix, owned by other blocks)
+  auto lim_of_block = [&](int j) -> int {
+    if (EPI == MTP_EPI_SWIGLU) return j < TJ / 2 ? p.half : p.N;
+    return p.N;
+  };
+
+  // The whole tile lies inside the matrix: the epilogue needs no bounds checks.
+  const bool tile_inside = m0 + BM <= p.M && (EPI == MTP_EPI_SWIGLU ? n0 + BN / 2 <= p.half : n0 + BN <= p.N);
+
+  auto flush = [&](int i, void* out, int64_t ld, auto nblk_tag, auto colfn, auto limfn, auto f32_tag, bool accumulate) {
+    constexpr int nblk = decltype(nblk_tag)::value;
+    constexpr bool f32out = decltype(f32_tag)::value;
+    {
+      // Fast path: 16-byte aligned rows of a tile that is completely inside: lane l owns chunk l % CPR of
+      // rows l / CPR, l / CPR + 64 / CPR, ...; one address computation, then constant strides.
+      constexpr int esz_c = f32out ? 4 : 2;
+      constexpr int CPR = nblk * 32 * esz_c / 16;                            // 16-byte chunks per staged row
+      constexpr int CPRP = CPR <= 4 ? 4 : CPR <= 8 ? 8 : CPR <= 16 ? 16 : 32;  // lanes per row (power of two)
+      constexpr int RPI = 64 / CPRP, ITERS = 32 / RPI;
+      const int r0 = lane / CPRP, cc = lane % CPRP;
+      const int e0 = cc * (16 / esz_c);
+      const int col = colfn(e0 >> 5) + (e0 & 31);
+      char* gp = (char*)out + ((int64_t)(m0 + blk_row(i) + r0) * ld + col) * esz_c;
+      const bool aligned = ((reinterpret_cast<uintptr_t>(out) | (uintptr_t)(ld * esz_c)) & 15) == 0;
+      if (tile_inside && aligned) {
+        if (CPRP != CPR && cc >= CPR) return;
+        const char* sp = stage + r0 * PITCH + cc * 16;
+        const int64_t gstride = (int64_t)RPI * ld * esz_c;
+#pragma unroll
+        for (int it = 0; it < ITERS; it++) {
+          u32x4_t v = *reinterpret_cast<const u32x4_t*>(sp + it * RPI * PITCH);
+          u32x4_t* q = reinterpret_cast<u32x4_t*>(gp + it * gstride);
+          if (accumulate) {
+            const u32x4_t o = *q;
+            if (f32out) {
+              v.x = __float_as_uint(__uint_as_float(v.x) + __uint_as_float(o.x));
+              v.y = __float_as_uint(__uint_as_float(v.y) + __uint_as_float(o.y));
+              v.z = __float_as_uint(__uint_as_float(v.z) + __uint_as_float(o.z));
+              v.w = __float_as_uint(__uint_as_float(v.w) + __uint_as_float(o.w));
+            } else {
+              v.x = X::pack2(X::lo(v.x) + X::lo(o.x), X::hi(v.x) + X::hi(o.x));
+              v.y = X::pack2(X::lo(v.y) + X::lo(o.y), X::hi(v.y) + X::hi(o.y));
+              v.z = X::pack2(X::lo(v.z) + X::lo(o.z), X::hi(v.z) + X::hi(o.z));
+              v.w = X::pack2(X::lo(v.w) + X::lo(o.w), X::hi(v.w) + X::hi(o.w));
+            }
+          }
+          __builtin_nontemporal_store(v, q);  // written once, read by a later kernel: keep it out of the way of A/B in L2
+        }
+        return;
+      }
+    }
+    // 16-byte chunks of the staged 32 x (nblk*32) block
+    const int esz = f32out ? 4 : 2;
+    const int chunks_per_row = nblk * 32 * esz / 16;
+    const int epc = 16 / esz;  // elements per chunk
+    const int total = 32 * chunks_per_row;
+    const int mrow0 = m0 + blk_row(i);
+    for (int c = lane; c < total; c += 64) {
+      const int r = c / chunks_per_row, cc = c - r * chunks_per_row;
+      const int e0 = cc * epc;           // element offset inside the staged row
+      const int j = e0 >> 5;
+      const int col = colfn(j) + (e0 & 31);
+      const int col_limit = limfn(j);
+      const int row = mrow0 + r;
+      if (row < p.M && col < col_limit) {
+        u32x4_t v = *reinterpret_cast<const u32x4_t*>(stage + r * PITCH + cc * 16);
+        char* gp = (char*)out + ((int64_t)row * ld + col) * esz;
+        if (col + epc <= col_limit && ((reinterpret_cast<uintptr_t>(gp) & 15) == 0)) {
+          if (accumulate) {
+            u32x4_t o = *reinterpret_cast<const u32x4_t*>(gp);
+            if (f32out) {
+              v.x = __float_as_uint(__uint_as_float(v.x) + __uint_as_float(o.x));
+              v.y = __float_as_uint(__uint_as_float(v.y) + __uint_as_float(o.y));
+              v.z = __float_as_uint(__uint_as_float(v.z) + __uint_as_float(o.z));
+              v.w = __float_as_uint(__uint_as_float(v.w) + __uint_as_float(o.w));
+            } else {
+              v.x = X::pack2(X::lo(v.x) + X::lo(o.x), X::hi(v.x) + X::hi(o.x));
+              v.y = X::pack2(X::lo(v.y) + X::lo(o.y), X::hi(v.y) + X::hi(o.y));
+              v.z = X::pack2(X::lo(v.z) + X::lo(o.z), X::hi(v.z) + X::hi(o.z));
+              v.w = X::pack2(X::lo(v.w) + X::lo(o.w), X::hi(v.w) + X::hi(o.w));
+            }
+          }
+          *reinterpret_cast<u32x4_t*>(gp) = v;
+        } else {
+          // ragged right edge or unaligned row: element by element
+          const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+          for (int e = 0; e < epc && col + e < col_limit; e++) {
+            if (f32out) {
+              float* q = reinterpret_cast<float*>(gp) + e;
+              const float nv = __uint_as_float(w4[e]);
+              *q = accumulate ? *q + nv : nv;
+            } else {
+              uint16_t* q = reinterpret_cast<uint16_t*>(gp) + e;
+              const uint32_t pr = w4[e >> 1];
+              const float nv = (e & 1) ? X::hi(pr) : X::lo(pr);
+              *q = X::to_bits(accumulate ? X::from_bits(*q) + nv : nv);
+            }
+          }
+        }
+      }
+    }
+  };
+
+#pragma unroll
+  for (int i = 0; i < TI; i++) {
+    // -- pre-activation (or plain) output: add bias, round, stage
+    float pre[TJ][16];
+#pragma unroll
+    for (int j = 0; j < TJ; j++) {
+      const int cb = col_of_block(j);
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        float b4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (EPI == MTP_EPI_BIAS || EPI == MTP_EPI_BIAS_GELU || (EPI == MTP_EPI_SWIGLU)) {
+          if (p.bias) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const int col = cb + 8 * g + 4 * lh + e;
+              b4[e] = col < lim_of_block(j) ? X::from_bits(p.bias[col]) : 0.f;
+            }
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) pre[j][4 * g + e] = acc[i][j][4 * g + e] + b4[e];
+      }
+    }
+    if (OUT == OUT_F32) {
+      if (p.C) {
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            f32x4_t v = {pre[j][4 * g], pre[j][4 * g + 1], pre[j][4 * g + 2], pre[j][4 * g + 3]};
+            *reinterpret_cast<f32x4_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 4) = v;
+          }
+        wave_lds_sync();
+        flush(i, p.C, p.ldc, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::true_type{}, p.accumulate != 0);
+        wave_lds_sync();
+      }
+    } else {
+      // round to bf16 once (one v_cvt_pk_bf16_f32 per pair); an activation sees the rounded value, as
+      // the unfused layers would
+      uint32_t pk[TJ][8];
+#pragma unroll
+      for (int j = 0; j < TJ; j++)
+#pragma unroll
+        for (int q = 0; q < 8; q++) pk[j][q] = X::pack2(pre[j][2 * q], pre[j][2 * q + 1]);
+      if (p.C) {
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            u32x2_t v = {pk[j][2 * g], pk[j][2 * g + 1]};
+            *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
+          }
+        wave_lds_sync();
+        flush(i, p.C, p.ldc, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::false_type{}, p.accumulate != 0);
+        wave_lds_sync();
+      }
+      if (EPI != MTP_EPI_NONE && EPI != MTP_EPI_BIAS && EPI != EPI_ROWSUM) {
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+#pragma unroll
+          for (int q = 0; q < 8; q++) {
+            pre[j][2 * q] = X::lo(pk[j][q]);
+            pre[j][2 * q + 1] = X::hi(pk[j][q]);
+          }
+      }
+      if constexpr (EPI == MTP_EPI_BIAS_GELU || EPI == MTP_EPI_GELU) {
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            u32x2_t v = {X::pack2(gelu_new_f(pre[j][4 * g]), gelu_new_f(pre[j][4 * g + 1])),
+                         X::pack2(gelu_new_f(pre[j][4 * g + 2]), gelu_new_f(pre[j][4 * g + 3]))};
+            *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
+          }
+        wave_lds_sync();
+        flush(i, p.C2, p.ldc2, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::false_type{}, false);
+        wave_lds_sync();
+      }
+      if constexpr (EPI == MTP_EPI_SWIGLU) {
+        constexpr int HJ = TJ / 2;
+#pragma unroll
+        for (int j = 0; j < HJ; j++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            float a4[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) a4[e] = silu_f(pre[j][4 * g + e]) * pre[j + HJ][4 * g + e];
+            u32x2_t v = {X::pack2(a4[0], a4[1]), X::pack2(a4[2], a4[3])};
+            *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
+          }
+        wave_lds_sync();
+        auto act_col = [&](int j) -> int { return n0 + wn * (WN / 2) + j * 32; };
+        auto act_lim = [&](int) -> int { return p.half; };
+        flush(i, p.C2, p.ldc2, std::integral_constant<int, HJ>{}, act_col, act_lim, std::false_type{}, false);
+        wave_lds_sync();
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The 64-deep main loop ("Q" configurations of the 256x256 tile).
+//
+// A k-tile is 64 deep, so that the slice of a K-contiguous row is one whole 128-byte line and one DMA
+// instruction requests 8 whole lines.  LDS holds two k-tiles (2 x 64 KiB); each operand's tile is split by rows
+// into two units of 128 rows (16 KiB), and a wave owns HI (HJ) 32-row blocks of either unit, so its part of the
+// tile is four quadrants Q(I,J) = unit I of A x unit J of B.  A wave keeps the fragments of all four units of
+// the current k-tile in registers (one register set per unit) and works through the quadrants, 4 k16 steps
+// each, in an order in which consecutive quadrants share a unit:
+//
+//   even tile t:  Q00  Q01 | Q11  Q10        reads meanwhile:  B1[t]  A1[t]   | A0[t+1]  B1[t+1]
+//   odd  tile t:  Q01  Q00 | Q10  Q11                          B0[t]  A1[t]   | A0[t+1]  B0[t+1]
+//
+// (every register set is refilled during the phase after its last use).  A unit of LDS is free as soon as every
+// wave has copied it to registers, long before the MFMAs that use the copy are done: one barrier per half
+// k-tile (the "|") hands the two units read since the previous barrier to the DMA, which refills them with
+// the tile after next while the following half tile is multiplied.  A unit is requested three half tiles
+// (about 1.5 k-tiles of 64) before it is read; s_waitcnt vmcnt(n) in front of the barrier asks for exactly
+// the two units the next half tile reads.  The requests of tiles past the end of k are still issued, with
+// every lane out of range (zero fill, no memory traffic), so that the counting never changes.
+// ---------------------------------------------------------------------------
+constexpr int QBK = 64;    // k-tile depth
+constexpr int QKS = 4;     // k16 steps per k-tile
+
+// K-contiguous operand: LDS unit = 128 rows x 128 bytes; the 16-byte chunk c of row r sits at position
+// c ^ ((r >> 1) & 7): 16 consecutive rows read at one k cover all 64 banks.  One DMA instruction fills 8 rows
+// (lane l -> row l/8, position l%8, fetching chunk (l%8) ^ swizzle of its row: the 8 lanes of a row still ask
+// for one whole line).  Fragment = one ds_read_b128.
+template <int NW, int WG>
+struct RowOperandQ {
+  static constexpr int UROWS = 128;                  // rows per unit
+  static constexpr int UBYTES = UROWS * QBK * 2;     // 16 KiB
+  static constexpr int BYTES = 2 * UBYTES;           // per k-tile buffer
+  static constexpr int H = UROWS / (32 * WG);        // 32-row blocks per wave and unit
+  static constexpr int NU = UROWS / 8 / NW;          // DMA instructions per wave and unit
+  static_assert(H >= 1 && NU >= 1, "wave grid too fine for the unit");
+  rsrc_t rsrc;
+  uint32_t voff[2][NU];
+  uint32_t fo[QKS];
+  int gchunk, K;
+
+  // rowmap(r): global row (relative to row0) of tile row r (unit r / 128), or a negative value for "no such row";
+  // wsub: the wave's index along this operand's dimension
+  template <typename RowMap>
+  __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int row0, int nrows, int K_, int lane,
+                                       int wave, int wsub, RowMap rowmap) {
+    K = K_;
+    rsrc = make_rsrc(base + (int64_t)row0 * ld, (int64_t)(nrows - row0) * ld * 2);
+    // tile row of lane l in instruction q = wave + NW j of unit u: 128 u + 8 q + l/8; its swizzle (row >> 1) & 7
+    // = (4 wave + l/16) & 7 whatever j and u are (8 NW j and 128 u are multiples of 16 rows)
+    gchunk = (lane & 7) ^ ((4 * wave + (lane >> 4)) & 7);
+#pragma unroll
+    for (int u = 0; u < 2; u++)
+#pragma unroll
+      for (int j = 0; j < NU; j++) {
+        const int r = u * UROWS + (wave + NW * j) * 8 + (lane >> 3);
+        const int64_t gr = rowmap(r);
+        voff[u][j] = (gr < 0 || gr >= nrows - row0) ? 0x80000000u : (uint32_t)((gr * ld + gchunk * 8) * 2);
+      }
+    // fragment of block b at step kk: row 32 H wsub + 32 b + l32 of the unit, chunk 2 kk + l/32
+    const int l32 = lane & 31, h = lane >> 5;
+#pragma unroll
+    for (int kk = 0; kk < QKS; kk++)
+      fo[kk] = (uint32_t)((wsub * 32 * H + l32) * 128 + ((((2 * kk + h) ^ (l32 >> 1)) & 7) << 4));
+  }
+  struct Prep {
+    uint32_t soff;
+    bool dead;
+  };
+  __device__ __forceinline__ Prep prep(int kt) const {
+    return Prep{(uint32_t)(kt * QBK * 2), kt * QBK + gchunk * 8 >= K};  // chunk at or past the end of k: zero fill
+  }
+  // j-th DMA instruction of this wave for unit u; unit_lds = LDS byte address of the unit
+  __device__ __forceinline__ void issue(const Prep& pp, uint32_t unit_lds, int wave, int u, int j) const {
+    dma16(rsrc, unit_lds + (wave + NW * j) * 1024, pp.dead ? 0x80000000u : voff[u][j], pp.soff);
+  }
+  __device__ __forceinline__ bf16x8_t frag(const char* unit, int b, int kk) const {
+    return *reinterpret_cast<const bf16x8_t*>(unit + b * (32 * 128) + fo[kk]);
+  }
+};
+
+// Transposed operand (memory [K, rows], rows contiguous): LDS unit = 64 k-rows x 128 rows, 256 bytes per k-row;
+// chunk c of k-row k sits at position c ^ ((k & 3) << 2).  One DMA instruction fills 4 k-rows (lane l -> k-row
+// l/16, position l%16).  Fragment = two ds_read_b64_tr_b16, addressed as in ColOperand.
+template <int NW, int WG>
+struct ColOperandQ {
+  static constexpr int UROWS = 128;
+  static constexpr int UBYTES = QBK * UROWS * 2;
+  static constexpr int BYTES = 2 * UBYTES;
+  static constexpr int H = UROWS / (32 * WG);
+  static constexpr int NU = QBK / 4 / NW;
+  static_assert(H >= 1 && NU >= 1, "wave grid too fine for the unit");
+  const char* base;     // &mem[0][row0]
+  int64_t total;        // bytes from base to the end of the matrix
+  int64_t ktile_bytes;  // QBK * ld * 2
+  uint32_t voff[2][NU];
+  uint32_t lane_base;
+  uint32_t moff[H];
+
+  __device__ __forceinline__ void init(const uint16_t* mem, int64_t ld, int row0, int K_, int lane, int wave, int wsub) {
+    base = reinterpret_cast<const char*>(mem + row0);
+    total = ((int64_t)K_ * ld - row0) * 2;
+    ktile_bytes = (int64_t)QBK * ld * 2;
+    const int ksub = lane >> 4;                        // k-row inside the instruction = k & 3
+    const int c = (lane & 15) ^ (ksub << 2);           // chunk of the unit's 128 rows this lane fetches
+#pragma unroll
+    for (int u = 0; u < 2; u++)
+#pragma unroll
+      for (int j = 0; j < NU; j++) {
+        const int krow = 4 * (wave + NW * j) + ksub;
+        voff[u][j] = (uint32_t)(((int64_t)krow * ld + u * UROWS + c * 8) * 2);
+      }
+    // lane (group G = l/16, i = l%16) addresses k-row 8 (G/2) + i/4 (+16 kk, +4 for the second read) and
+    // elements 16 (G%2) + 4 (i%4) .. +3 of the block
+    const int G = lane >> 4, i = lane & 15, kq = i >> 2;
+    lane_base = (uint32_t)((8 * (G >> 1) + kq) * (UROWS * 2) + 8 * (i & 1));
+#pragma unroll
+    for (int b = 0; b < H; b++) {
+      const int c2 = (wsub * 32 * H + 32 * b) / 8 + 2 * (G & 1) + ((i & 3) >> 1);
+      moff[b] = (uint32_t)((c2 ^ (kq << 2)) * 16);
+    }
+  }
+  struct Prep {
+    rsrc_t r;
+  };
+  __device__ __forceinline__ Prep prep(int kt) const {
+    // the whole address goes through the range check: k-rows past K read as zero
+    return Prep{make_rsrc(base + kt * ktile_bytes, total - kt * ktile_bytes)};
+  }
+  __device__ __forceinline__ void issue(const Prep& pp, uint32_t unit_lds, int wave, int u, int j) const {
+    dma16(pp.r, unit_lds + (wave + NW * j) * 1024, voff[u][j], 0);
+  }
+  __device__ __forceinline__ bf16x8_t frag(const char* unit, int b, int kk) const {
+    const char* a = unit + lane_base + moff[b] + kk * (16 * UROWS * 2);
+    const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+        (bf16x4_t __attribute__((address_space(3)))*)(a));
+    const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+        (bf16x4_t __attribute__((address_space(3)))*)(a + 4 * UROWS * 2));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  }
+};
+
+template <int LAY, int NW, int WG> struct QOperandOf { using type = RowOperandQ<NW, WG>; };
+template <int NW, int WG> struct QOperandOf<LAY_COL, NW, WG> { using type = ColOperandQ<NW, WG>; };
+
+// compile-time list of ints, read by index
+template <int... V>
+struct IntList {
+  static constexpr int v[sizeof...(V)] = {V...};
+};
+
+template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16>
+__device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
+  using X = X16<F16>;
+  constexpr int BM = 256, BN = 256;
+  static_assert(EPI != MTP_EPI_SWIGLU || BLAY == LAY_ROW, "the SwiGLU row interleave is a forward (row B) feature");
+  static_assert(NW == 4 || NW == 8, "4 waves (2x2) or 8 waves (2x4) per workgroup");
+  constexpr int WGM = 2, WGN = NW / 2;
+  constexpr int TI = BM / (32 * WGM), TJ = BN / (32 * WGN);
+  using AOp = typename QOperandOf<ALAY, NW, WGM>::type;
+  using BOp = typename QOperandOf<BLAY, NW, WGN>::type;
+  constexpr int HI = AOp::H, HJ = BOp::H;
+  static_assert(2 * HI == TI && 2 * HJ == TJ, "two units per operand");
+  constexpr int QBUF = AOp::BYTES + BOp::BYTES;   // one k-tile of both operands: 64 KiB
+  constexpr int LDS_BYTES = 2 * QBUF;
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+
+  const int tiles_m = (p.M + BM - 1) / BM;
+  const int n_span = (EPI == MTP_EPI_SWIGLU) ? p.half : p.N;  // SwiGLU tiles cover BN/2 gate + BN/2 up columns
+  constexpr int BN_SPAN = (EPI == MTP_EPI_SWIGLU) ? BN / 2 : BN;
+  const int tiles_n = (n_span + BN_SPAN - 1) / BN_SPAN;
+  int tm, tn;
+  tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM;
+  const int n0 = tn * BN_SPAN;
+  const int lm0 = MTP_DBG(p, 1) ? 0 : MTP_DBG(p, 8) ? (tm & 1) * BM : m0;
+  const int ln0 = MTP_DBG(p, 9) ? 0 : n0;
+
+  AOp opA;
+  BOp opB;
+  if constexpr (ALAY == LAY_ROW)
+    opA.init(p.A, p.lda, lm0, p.M, p.K, lane, wave, wm, [](int r) -> int64_t { return r; });
+  else
+    opA.init(p.A, p.lda, lm0, p.K, lane, wave, wm);
+  if constexpr (BLAY == LAY_ROW) {
+    // SwiGLU: unit 0 of the B tile holds BN/2 gate rows, unit 1 the matching up rows
+    opB.init(p.B, p.ldb, ln0, p.N, p.K, lane, wave, wn, [&](int r) -> int64_t {
+      if (EPI == MTP_EPI_SWIGLU) {
+        if (r < BN / 2) return ln0 + r >= p.half ? -1 : r;   // gate rows at or past `half` belong to the up matrix
+        return (int64_t)p.half + (r - BN / 2);
+      }
+      return r;
+    });
+  } else {
+    opB.init(p.B, p.ldb, ln0, p.K, lane, wave, wn);
+  }
+#ifdef MTP_MEASURE
+  if (MTP_DBG(p, 4)) {  // measurement: every DMA reads out of range (zero fill, no memory traffic)
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+#pragma unroll
+      for (int j = 0; j < AOp::NU; j++) opA.voff[u][j] = 0x80000000u;
+#pragma unroll
+      for (int j = 0; j < BOp::NU; j++) opB.voff[u][j] = 0x80000000u;
+    }
+  }
+#endif
+
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr_of(lds));
+  // byte offsets of the units inside lds
+  auto unit_a = [](int buf, int u) constexpr { return buf * QBUF + u * AOp::UBYTES; };
+  auto unit_b = [](int buf, int u) constexpr { return buf * QBUF + AOp::BYTES + u * BOp::UBYTES; };
+
+  f32x16_t acc[TI][TJ];
+#pragma unroll
+  for (int i = 0; i < TI; i++)
+#pragma unroll
+    for (int j = 0; j < TJ; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+  float rsum[TI];
+#pragma unroll
+  for (int i = 0; i < TI; i++) rsum[i] = 0.f;
+
+  // register sets: fragments of A unit u / B unit u of the current (or next) k-tile
+  bf16x8_t ra[2][HI][QKS], rb[2][HJ][QKS];
+
+  constexpr int PH = HI * HJ * QKS;          // MFMAs per phase (one quadrant)
+  constexpr int HT = 2 * PH;                 // MFMAs per half tile
+  constexpr int NDH = AOp::NU + BOp::NU;     // DMA instructions per wave and half tile (one unit of A, one of B)
+  static_assert(AOp::NU == BOp::NU, "the units of A and B take the same number of DMA instructions");
+  constexpr int BPOST = PH >= 16 ? 4 : 2;    // MFMAs of a half tile issued behind its barrier
+  constexpr int BARRIER_AT = HT - BPOST;
+  // the d-th DMA instruction of a half tile is issued behind MFMA number d HT / NDH + 1 of the half tile
+  constexpr int NAFTER = [&]() constexpr {   // DMA instructions of a half tile issued behind its barrier
+    int n = 0;
+    for (int d = 0; d < NDH; d++) n += (d * HT / NDH + 1) >= BARRIER_AT ? 1 : 0;
+    return n;
+  }();
+  // At a barrier the two units the next half tile reads must have landed: they were requested three half tiles
+  // ago, and behind them came one whole half tile of requests and this half tile's up to the barrier.
+  constexpr int VM_AT_BARRIER = 2 * NDH - NAFTER;
+  static_assert(VM_AT_BARRIER < 64, "vmcnt range");
+
+  // m-th MFMA of a phase on the register sets (MA, MB): k16 step m / (HI HJ), blocks walked in a snake
+  auto mfma_q = [&](auto ma_tag, auto mb_tag, auto m_tag) {
+    constexpr int MA = decltype(ma_tag)::value, MB = decltype(mb_tag)::value, m = decltype(m_tag)::value;
+    constexpr int kk = m / (HI * HJ), w = m % (HI * HJ);
+    constexpr int i = w / HJ, j = (i & 1) ? HJ - 1 - w % HJ : w % HJ;
+    acc[MA * HI + i][MB * HJ + j] = X::mfma32(rb[MB][j][kk], ra[MA][i][kk], acc[MA * HI + i][MB * HJ + j]);
+    if constexpr (EPI == EPI_ROWSUM && MB == 0 && j == 0) rsum[MA * HI + i] = X::sum8(ra[MA][i][kk], rsum[MA * HI + i]);
+  };
+  // f-th fragment read of a phase that refills register set U of A (IS_A) or B from buffer BUF; fragments in the
+  // order they are used: step 0 of every block, step 1, ...
+  auto read_q = [&](auto isa_tag, auto u_tag, auto buf_tag, auto f_tag) {
+    constexpr bool IS_A = decltype(isa_tag)::value != 0;
+    constexpr int U = decltype(u_tag)::value, BUF = decltype(buf_tag)::value, f = decltype(f_tag)::value;
+    if constexpr (IS_A) {
+      constexpr int kk = f / HI, b = f % HI;
+      ra[U][b][kk] = opA.frag(lds + unit_a(BUF, U), b, kk);
+    } else {
+      constexpr int kk = f / HJ, b = f % HJ;
+      rb[U][b][kk] = opB.frag(lds + unit_b(BUF, U), b, kk);
+    }
+  };
+  // d-th DMA instruction of the group (A unit UA, B unit UB, buffer BUF): A and B alternate
+  auto dma_q = [&](const typename AOp::Prep& pa, const typename BOp::Prep& pb, auto ua_tag, auto ub_tag, auto buf_tag,
+                   auto d_tag) {
+    constexpr int UA = decltype(ua_tag)::value, UB = decltype(ub_tag)::value, BUF = decltype(buf_tag)::value;
+    constexpr int d = decltype(d_tag)::value;
+    if constexpr ((d & 1) == 0)
+      opA.issue(pa, lds0 + unit_a(BUF, UA), wave, UA, d >> 1);
+    else
+      opB.issue(pb, lds0 + unit_b(BUF, UB), wave, UB, d >> 1);
+  };
+  auto dma_group = [&](int kt, auto ua_tag, auto ub_tag, auto buf_tag) {
+    const auto pa = opA.prep(kt);
+    const auto pb = opB.prep(kt);
+    static_for<NDH>([&](auto d) { dma_q(pa, pb, ua_tag, ub_tag, buf_tag, d); });
+  };
+
+  // One half tile.  D = IntList<MA0, MB0, MA1, MB1,  R0A, R0U, R0BUF,  R1A, R1U, R1BUF,  DUA, DUB, DBUF>:
+  // phase 0 multiplies register sets (MA0, MB0) while set R0U of A (R0A = 1) or B is refilled from buffer R0BUF,
+  // phase 1 likewise; the DMA group (A unit DUA, B unit DUB) of k-tile kt_dma goes to buffer DBUF.
+  // The fragment reads of a phase sit behind its first MFMAs, so that every read of the half tile has been
+  // issued well before the barrier (which hands the units over) and has about half a phase to land.
+  auto half_tile = [&](int kt_dma, auto desc) {
+    using D = decltype(desc);
+    const auto pa = opA.prep(kt_dma);
+    const auto pb = opB.prep(kt_dma);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<HT>([&](auto g_tag) {
+      constexpr int g = decltype(g_tag)::value;
+      constexpr int ph = g / PH, m = g % PH;
+      constexpr int MA = D::v[ph ? 2 : 0], MB = D::v[ph ? 3 : 1];
+      constexpr int RA = D::v[ph ? 7 : 4], RU = D::v[ph ? 8 : 5], RBUF = D::v[ph ? 9 : 6];
+      constexpr int NR = (RA ? HI : HJ) * QKS;     // fragment reads of this phase
+      constexpr int RSPAN = PH / 2;                // spread over the first half of the phase
+      if constexpr (g == BARRIER_AT) {
+        // own reads of this half tile done, own requests for the next half tile's units landed ...
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(VM_AT_BARRIER) : "memory");
+        __syncthreads();  // ... for every wave
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mfma_q(std::integral_constant<int, MA>{}, std::integral_constant<int, MB>{}, std::integral_constant<int, m>{});
+      static_for<NDH>([&](auto d_tag) {
+        constexpr int d = decltype(d_tag)::value;
+        if constexpr (d * HT / NDH + 1 == g + 1)
+          dma_q(pa, pb, std::integral_constant<int, D::v[10]>{}, std::integral_constant<int, D::v[11]>{},
+                std::integral_constant<int, D::v[12]>{}, d_tag);
+      });
+      if constexpr (m < RSPAN) {
+        static_for<(m + 1) * NR / RSPAN - m * NR / RSPAN>([&](auto e) {
+          read_q(std::integral_constant<int, RA>{}, std::integral_constant<int, RU>{},
+                 std::integral_constant<int, RBUF>{}, std::integral_constant<int, m * NR / RSPAN + decltype(e)::value>{});
+        });
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  //                       MA0 MB0 MA1 MB1   R0: A  U BUF   R1: A  U BUF   DMA: UA UB BUF
+  using EvenH0 = IntList<0, 0, 0, 1, /**/ 0, 1, 0, /**/ 1, 1, 0, /**/ 0, 0, 0>;  // Q00 Q01; reads B1[t] A1[t]
+  using EvenH1 = IntList<1, 1, 1, 0, /**/ 1, 0, 1, /**/ 0, 1, 1, /**/ 1, 1, 0>;  // Q11 Q10; reads A0[t+1] B1[t+1]
+  using OddH0 = IntList<0, 1, 0, 0, /**/ 0, 0, 1, /**/ 1, 1, 1, /**/ 0, 1, 1>;   // Q01 Q00; reads B0[t] A1[t]
+  using OddH1 = IntList<1, 0, 1, 1, /**/ 1, 0, 0, /**/ 0, 0, 0, /**/ 1, 0, 1>;   // Q10 Q11; reads A0[t+1] B0[t+1]
+
+  const int KT = (p.K + QBK - 1) / QBK;
+  {
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    // the four request groups in front of the loop, in the order the loop would have issued them
+    dma_group(0, I0{}, I0{}, I0{});   // A0[0] B0[0]
+    dma_group(0, I1{}, I1{}, I0{});   // A1[0] B1[0]
+    dma_group(1, I0{}, I1{}, I1{});   // A0[1] B1[1]
+    dma_group(1, I1{}, I0{}, I1{});   // A1[1] B0[1]
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NDH) : "memory");   // all of k-tile 0
+    __syncthreads();
+    static_for<HI * QKS>([&](auto f) { read_q(I1{}, I0{}, I0{}, f); });
+    static_for<HJ * QKS>([&](auto f) { read_q(I0{}, I0{}, I0{}, f); });
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();   // everyone holds A0[0], B0[0]: the loop's first requests may overwrite them
+  }
+  int kt = 0;
+  for (; kt + 1 < KT; kt += 2) {
+    half_tile(kt + 2, EvenH0{});
+    half_tile(kt + 2, EvenH1{});
+    half_tile(kt + 3, OddH0{});
+    half_tile(kt + 3, OddH1{});
+  }
+  if (kt < KT) {
+    half_tile(kt + 2, EvenH0{});
+    half_tile(kt + 2, EvenH1{});
+  }
+  __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+  __syncthreads();  // the epilogue reuses the tile buffers
+  if (MTP_DBG(p, 2)) return;
+  gemm_epilogue<BM, BN, EPI, OUT, NW, F16, true, LDS_BYTES>(p, acc, rsum, lds, m0, n0, tn, wave, lane);
+}
+
 // The body lives in a __device__ function: it uses inline assembly operands that the host pass over a
 // __global__ function would trip on.
 template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16>
@@ -375,8 +1011,8 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   const int m0 = tm * BM;
   const int n0 = tn * BN_SPAN;
   // load origins (debug 1: all tiles load tile (0,0); debug 8: two A tiles, one B tile: a cache-resident set)
-  const int lm0 = (p.debug & 1) ? 0 : (p.debug & 8) ? (tm & 1) * BM : m0;
-  const int ln0 = (p.debug & 9) ? 0 : n0;
+  const int lm0 = MTP_DBG(p, 1) ? 0 : MTP_DBG(p, 8) ? (tm & 1) * BM : m0;
+  const int ln0 = MTP_DBG(p, 9) ? 0 : n0;
 
   AOp opA;
   BOp opB;
@@ -400,7 +1036,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   } else {
     opB.init(p.B, p.ldb, ln0, p.K, lane, wave, wn * (BN / WGN));
   }
-  if (p.debug & 4) {  // measurement: every DMA reads out of range (zero fill, no memory traffic)
+  if (MTP_DBG(p, 4)) {  // measurement: every DMA reads out of range (zero fill, no memory traffic)
 #pragma unroll
     for (int j = 0; j < AOp::NINSTR; j++) opA.voff[j] = 0x80000000u;
 #pragma unroll
@@ -691,252 +1327,20 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   for (; kt < KT; kt++) ktile(kt, std::false_type{});
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
   __syncthreads();  // the epilogue reuses the tile buffers
-  if (p.debug & 2) return;
+  if (MTP_DBG(p, 2)) return;
 
-  if constexpr (EPI == EPI_ROWSUM) {
-    static_assert(NMF >= TI, "every A fragment of a step must meet an MFMA");
-    if (tn == 0 && wn == 0) {
-#pragma unroll
-      for (int i = 0; i < TI; i++) {
-        const float t = rsum[i] + __shfl_xor(rsum[i], 32, 64);  // the two k halves of a row
-        const int row = m0 + wm * (BM / WGM) + 32 * i + l32;
-        if (lh == 0 && row < p.M) {
-          if (OUT == OUT_F32) {
-            float* q = (float*)p.rowsum + row;
-            *q = p.accumulate ? *q + t : t;
-          } else {
-            uint16_t* q = (uint16_t*)p.rowsum + row;
-            *q = X::to_bits(p.accumulate ? X::from_bits(*q) + t : t);
-          }
-        }
-      }
-    }
-  }
-
-  // ---- epilogue ----------------------------------------------------------------
-  // acc[i][j][r]: row m = m0 + wm*BM/2 + 32i + l32, column block j, n_local = 8*(r/4) + 4*lh + r%4.
-  // Stage 32 rows x (BN/2) columns per wave through LDS, then 16-byte row-contiguous stores.
-  constexpr int WN = BN / WGN;                     // columns per wave
-  constexpr int ESZ = (OUT == OUT_F32) ? 4 : 2;
-  constexpr int PITCH = WN * ESZ + 16;             // bytes per staged row (+16: spread rows over banks)
-  static_assert(NW * 32 * PITCH <= NSTAGE * STAGE_BYTES, "epilogue staging exceeds the tile buffers");
-  char* stage = lds + wave * (32 * PITCH);
-
-  // global column of the first element of block j for this wave (main output C)
-  auto col_of_block = [&](int j) -> int {
-    if (EPI == MTP_EPI_SWIGLU) {
-      const int hj = TJ / 2;
-      return (j < hj ? 0 : p.half) + n0 + wn * (WN / 2) + (j % hj) * 32;
-    }
-    return n0 + wn * WN + j * 32;
-  };
-  // first column past the valid range of block j: SwiGLU gate blocks end at `half` (the columns after it
-  // are the up matrix, owned by other blocks)
-  auto lim_of_block = [&](int j) -> int {
-    if (EPI == MTP_EPI_SWIGLU) return j < TJ / 2 ? p.half : p.N;
-    return p.N;
-  };
-
-  // The whole tile lies inside the matrix: the epilogue needs no bounds checks.
-  const bool tile_inside = m0 + BM <= p.M && (EPI == MTP_EPI_SWIGLU ? n0 + BN / 2 <= p.half : n0 + BN <= p.N);
-
-  auto flush = [&](int i, void* out, int64_t ld, auto nblk_tag, auto colfn, auto limfn, auto f32_tag, bool accumulate) {
-    constexpr int nblk = decltype(nblk_tag)::value;
-    constexpr bool f32out = decltype(f32_tag)::value;
-    {
-      // Fast path: 16-byte aligned rows of a tile that is completely inside: lane l owns chunk l % CPR of
-      // rows l / CPR, l / CPR + 64 / CPR, ...; one address computation, then constant strides.
-      constexpr int esz_c = f32out ? 4 : 2;
-      constexpr int CPR = nblk * 32 * esz_c / 16;                            // 16-byte chunks per staged row
-      constexpr int CPRP = CPR <= 4 ? 4 : CPR <= 8 ? 8 : CPR <= 16 ? 16 : 32;  // lanes per row (power of two)
-      constexpr int RPI = 64 / CPRP, ITERS = 32 / RPI;
-      const int r0 = lane / CPRP, cc = lane % CPRP;
-      const int e0 = cc * (16 / esz_c);
-      const int col = colfn(e0 >> 5) + (e0 & 31);
-      char* gp = (char*)out + ((int64_t)(m0 + wm * (BM / WGM) + 32 * i + r0) * ld + col) * esz_c;
-      const bool aligned = ((reinterpret_cast<uintptr_t>(out) | (uintptr_t)(ld * esz_c)) & 15) == 0;
-      if (tile_inside && aligned) {
-        if (CPRP != CPR && cc >= CPR) return;
-        const char* sp = stage + r0 * PITCH + cc * 16;
-        const int64_t gstride = (int64_t)RPI * ld * esz_c;
-#pragma unroll
-        for (int it = 0; it < ITERS; it++) {
-          u32x4_t v = *reinterpret_cast<const u32x4_t*>(sp + it * RPI * PITCH);
-          u32x4_t* q = reinterpret_cast<u32x4_t*>(gp + it * gstride);
-          if (accumulate) {
-            const u32x4_t o = *q;
-            if (f32out) {
-              v.x = __float_as_uint(__uint_as_float(v.x) + __uint_as_float(o.x));
-              v.y = __float_as_uint(__uint_as_float(v.y) + __uint_as_float(o.y));
-              v.z = __float_as_uint(__uint_as_float(v.z) + __uint_as_float(o.z));
-              v.w = __float_as_uint(__uint_as_float(v.w) + __uint_as_float(o.w));
-            } else {
-              v.x = X::pack2(X::lo(v.x) + X::lo(o.x), X::hi(v.x) + X::hi(o.x));
-              v.y = X::pack2(X::lo(v.y) + X::lo(o.y), X::hi(v.y) + X::hi(o.y));
-              v.z = X::pack2(X::lo(v.z) + X::lo(o.z), X::hi(v.z) + X::hi(o.z));
-              v.w = X::pack2(X::lo(v.w) + X::lo(o.w), X::hi(v.w) + X::hi(o.w));
-            }
-          }
-          __builtin_nontemporal_store(v, q);  // written once, read by a later kernel: keep it out of the way of A/B in L2
-        }
-        return;
-      }
-    }
-    // 16-byte chunks of the staged 32 x (nblk*32) block
-    const int esz = f32out ? 4 : 2;
-    const int chunks_per_row = nblk * 32 * esz / 16;
-    const int epc = 16 / esz;  // elements per chunk
-    const int total = 32 * chunks_per_row;
-    const int mrow0 = m0 + wm * (BM / WGM) + 32 * i;
-    for (int c = lane; c < total; c += 64) {
-      const int r = c / chunks_per_row, cc = c - r * chunks_per_row;
-      const int e0 = cc * epc;           // element offset inside the staged row
-      const int j = e0 >> 5;
-      const int col = colfn(j) + (e0 & 31);
-      const int col_limit = limfn(j);
-      const int row = mrow0 + r;
-      if (row < p.M && col < col_limit) {
-        u32x4_t v = *reinterpret_cast<const u32x4_t*>(stage + r * PITCH + cc * 16);
-        char* gp = (char*)out + ((int64_t)row * ld + col) * esz;
-        if (col + epc <= col_limit && ((reinterpret_cast<uintptr_t>(gp) & 15) == 0)) {
-          if (accumulate) {
-            u32x4_t o = *reinterpret_cast<const u32x4_t*>(gp);
-            if (f32out) {
-              v.x = __float_as_uint(__uint_as_float(v.x) + __uint_as_float(o.x));
-              v.y = __float_as_uint(__uint_as_float(v.y) + __uint_as_float(o.y));
-              v.z = __float_as_uint(__uint_as_float(v.z) + __uint_as_float(o.z));
-              v.w = __float_as_uint(__uint_as_float(v.w) + __uint_as_float(o.w));
-            } else {
-              v.x = X::pack2(X::lo(v.x) + X::lo(o.x), X::hi(v.x) + X::hi(o.x));
-              v.y = X::pack2(X::lo(v.y) + X::lo(o.y), X::hi(v.y) + X::hi(o.y));
-              v.z = X::pack2(X::lo(v.z) + X::lo(o.z), X::hi(v.z) + X::hi(o.z));
-              v.w = X::pack2(X::lo(v.w) + X::lo(o.w), X::hi(v.w) + X::hi(o.w));
-            }
-          }
-          *reinterpret_cast<u32x4_t*>(gp) = v;
-        } else {
-          // ragged right edge or unaligned row: element by element
-          const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
-          for (int e = 0; e < epc && col + e < col_limit; e++) {
-            if (f32out) {
-              float* q = reinterpret_cast<float*>(gp) + e;
-              const float nv = __uint_as_float(w4[e]);
-              *q = accumulate ? *q + nv : nv;
-            } else {
-              uint16_t* q = reinterpret_cast<uint16_t*>(gp) + e;
-              const uint32_t pr = w4[e >> 1];
-              const float nv = (e & 1) ? X::hi(pr) : X::lo(pr);
-              *q = X::to_bits(accumulate ? X::from_bits(*q) + nv : nv);
-            }
-          }
-        }
-      }
-    }
-  };
-
-#pragma unroll
-  for (int i = 0; i < TI; i++) {
-    // -- pre-activation (or plain) output: add bias, round, stage
-    float pre[TJ][16];
-#pragma unroll
-    for (int j = 0; j < TJ; j++) {
-      const int cb = col_of_block(j);
-#pragma unroll
-      for (int g = 0; g < 4; g++) {
-        float b4[4] = {0.f, 0.f, 0.f, 0.f};
-        if (EPI == MTP_EPI_BIAS || EPI == MTP_EPI_BIAS_GELU || (EPI == MTP_EPI_SWIGLU)) {
-          if (p.bias) {
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              const int col = cb + 8 * g + 4 * lh + e;
-              b4[e] = col < lim_of_block(j) ? X::from_bits(p.bias[col]) : 0.f;
-            }
-          }
-        }
-#pragma unroll
-        for (int e = 0; e < 4; e++) pre[j][4 * g + e] = acc[i][j][4 * g + e] + b4[e];
-      }
-    }
-    if (OUT == OUT_F32) {
-      if (p.C) {
-#pragma unroll
-        for (int j = 0; j < TJ; j++)
-#pragma unroll
-          for (int g = 0; g < 4; g++) {
-            f32x4_t v = {pre[j][4 * g], pre[j][4 * g + 1], pre[j][4 * g + 2], pre[j][4 * g + 3]};
-            *reinterpret_cast<f32x4_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 4) = v;
-          }
-        wave_lds_sync();
-        flush(i, p.C, p.ldc, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::true_type{}, p.accumulate != 0);
-        wave_lds_sync();
-      }
-    } else {
-      // round to bf16 once (one v_cvt_pk_bf16_f32 per pair); an activation sees the rounded value, as
-      // the unfused layers would
-      uint32_t pk[TJ][8];
-#pragma unroll
-      for (int j = 0; j < TJ; j++)
-#pragma unroll
-        for (int q = 0; q < 8; q++) pk[j][q] = X::pack2(pre[j][2 * q], pre[j][2 * q + 1]);
-      if (p.C) {
-#pragma unroll
-        for (int j = 0; j < TJ; j++)
-#pragma unroll
-          for (int g = 0; g < 4; g++) {
-            u32x2_t v = {pk[j][2 * g], pk[j][2 * g + 1]};
-            *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
-          }
-        wave_lds_sync();
-        flush(i, p.C, p.ldc, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::false_type{}, p.accumulate != 0);
-        wave_lds_sync();
-      }
-      if (EPI != MTP_EPI_NONE && EPI != MTP_EPI_BIAS && EPI != EPI_ROWSUM) {
-#pragma unroll
-        for (int j = 0; j < TJ; j++)
-#pragma unroll
-          for (int q = 0; q < 8; q++) {
-            pre[j][2 * q] = X::lo(pk[j][q]);
-            pre[j][2 * q + 1] = X::hi(pk[j][q]);
-          }
-      }
-      if constexpr (EPI == MTP_EPI_BIAS_GELU || EPI == MTP_EPI_GELU) {
-#pragma unroll
-        for (int j = 0; j < TJ; j++)
-#pragma unroll
-          for (int g = 0; g < 4; g++) {
-            u32x2_t v = {X::pack2(gelu_new_f(pre[j][4 * g]), gelu_new_f(pre[j][4 * g + 1])),
-                         X::pack2(gelu_new_f(pre[j][4 * g + 2]), gelu_new_f(pre[j][4 * g + 3]))};
-            *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
-          }
-        wave_lds_sync();
-        flush(i, p.C2, p.ldc2, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::false_type{}, false);
-        wave_lds_sync();
-      }
-      if constexpr (EPI == MTP_EPI_SWIGLU) {
-        constexpr int HJ = TJ / 2;
-#pragma unroll
-        for (int j = 0; j < HJ; j++)
-#pragma unroll
-          for (int g = 0; g < 4; g++) {
-            float a4[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) a4[e] = silu_f(pre[j][4 * g + e]) * pre[j + HJ][4 * g + e];
-            u32x2_t v = {X::pack2(a4[0], a4[1]), X::pack2(a4[2], a4[3])};
-            *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
-          }
-        wave_lds_sync();
-        auto act_col = [&](int j) -> int { return n0 + wn * (WN / 2) + j * 32; };
-        auto act_lim = [&](int) -> int { return p.half; };
-        flush(i, p.C2, p.ldc2, std::integral_constant<int, HJ>{}, act_col, act_lim, std::false_type{}, false);
-        wave_lds_sync();
-      }
-    }
-  }
+  if constexpr (EPI == EPI_ROWSUM) static_assert(NMF >= TI, "every A fragment of a step must meet an MFMA");
+  gemm_epilogue<BM, BN, EPI, OUT, NW, F16, false, NSTAGE * STAGE_BYTES>(p, acc, rsum, lds, m0, n0, tn, wave, lane);
 }
 
 template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16>
 __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs p) {
   gemm_bf16_body<BM, BN, ALAY, BLAY, EPI, OUT, NW, F16>(p);
+}
+
+template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16>
+__global__ __launch_bounds__(NW * 64) void gemm_q_kernel(const GemmArgs p) {
+  gemm_q_body<ALAY, BLAY, EPI, OUT, NW, F16>(p);
 }
 
 // ---------------------------------------------------------------------------
@@ -950,14 +1354,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs p) {
 struct TileCfg {
   int bm, bn, nw;
   float eff;  // relative speed of one tile's inner loop per flop (256x256 = 1), from measurement
+  bool q;     // the 64-deep main loop (256x256 only)
 };
 // 256x256 exists with 8 waves (2 per SIMD: one wave's barrier and LDS waits are covered by the other's
 // MFMAs, and the epilogue's VALU work is spread over twice the waves) and with 4 waves (128x128 per wave:
 // a third fewer LDS reads per MFMA, accumulators in AGPRs), measured 0-4 % faster on the Llama-3-8B
 // shapes; the narrow tiles were measured best as listed.
 constexpr TileCfg kCfgs[] = {
-    {256, 256, 8, 1.00f}, {256, 192, 4, 0.92f}, {192, 256, 4, 0.92f}, {256, 128, 4, 0.85f}, {128, 256, 8, 0.85f},
-    {256, 256, 4, 1.02f},
+    {256, 256, 8, 1.00f, false}, {256, 192, 4, 0.92f, false}, {192, 256, 4, 0.92f, false}, {256, 128, 4, 0.85f, false},
+    {128, 256, 8, 0.85f, false}, {256, 256, 4, 1.02f, false}, {256, 256, 4, 1.01f, true},   {256, 256, 8, 1.00f, true},
 };
 constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
 
@@ -973,13 +1378,13 @@ constexpr bool cfg_valid(int c) {
 
 template <int EPI>
 int pick_config(const GemmArgs& a) {
-  if (const char* e = getenv("MTP_GEMM_CFG")) {
-    const int c = atoi(e);
+  static MtpTune tune_cfg("MTP_GEMM_CFG"), tune_skip("MTP_GEMM_SKIP");
+  if (tune_cfg.is_set()) {
+    const int c = tune_cfg.get(0);
     if (c >= 0 && c < kNumCfgs) return c;
   }
   const int64_t span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
-  int skip = 0;  // measurement only: bit c set = leave configuration c out of the choice
-  if (const char* e = getenv("MTP_GEMM_SKIP")) skip = atoi(e);
+  const int skip = tune_skip.get(0);  // bit c set = leave configuration c out of the choice
   int best = 0;
   double best_t = 1e300;
   for (int c = 0; c < kNumCfgs; c++) {
@@ -1009,8 +1414,12 @@ int launch_cfg(const GemmArgs& a, hipStream_t s) {
     const int span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
     const int bn_span = (EPI == MTP_EPI_SWIGLU) ? BN / 2 : BN;
     const int tiles_n = (span + bn_span - 1) / bn_span;
-    hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, NW, F16>), dim3((unsigned)(tiles_m * tiles_n)),
-                       dim3(NW * 64), 0, s, a);
+    if constexpr (kCfgs[C].q)
+      hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16>), dim3((unsigned)(tiles_m * tiles_n)), dim3(NW * 64),
+                         0, s, a);
+    else
+      hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, NW, F16>), dim3((unsigned)(tiles_m * tiles_n)),
+                         dim3(NW * 64), 0, s, a);
     MTP_CHECK_LAUNCH("gemm_bf16");
     return MTP_OK;
   }
@@ -1018,7 +1427,10 @@ int launch_cfg(const GemmArgs& a, hipStream_t s) {
 
 template <int ALAY, int BLAY, int EPI, int OUT, bool F16>
 int launch_typed(GemmArgs a, hipStream_t s) {
-  if (const char* e = getenv("MTP_GEMM_DEBUG")) a.debug = atoi(e);
+#ifdef MTP_MEASURE
+  static MtpTune tune_debug("MTP_GEMM_DEBUG");
+  a.debug = tune_debug.get(0);
+#endif
   int c = pick_config<EPI>(a);
   if (!cfg_valid<EPI>(c)) c = 0;
   switch (c) {
@@ -1028,6 +1440,8 @@ int launch_typed(GemmArgs a, hipStream_t s) {
     case 3: return launch_cfg<3, ALAY, BLAY, EPI, OUT, F16>(a, s);
     case 4: return launch_cfg<4, ALAY, BLAY, EPI, OUT, F16>(a, s);
     case 5: return launch_cfg<5, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 6: return launch_cfg<6, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 7: return launch_cfg<7, ALAY, BLAY, EPI, OUT, F16>(a, s);
   }
   return MTP_EINVAL;
 }

@@ -260,8 +260,8 @@ int launch_f32_tile(const F32Args& a, hipStream_t s) {
 template <int ALAY, int BLAY>
 int launch_f32(const F32Args& a, hipStream_t s) {
   auto tiles = [&](int bm, int bn) { return (int64_t)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
-  int force = 0;
-  if (const char* e = getenv("MTP_GEMM_F32_TILE")) force = atoi(e);  // measurement: 1..4 picks a tile
+  static MtpTune tune_tile("MTP_GEMM_F32_TILE");
+  const int force = tune_tile.get(0);  // 1..4 picks a tile
   if (force == 1 || (!force && tiles(128, 128) >= 512)) return launch_f32_tile<ALAY, BLAY, 128, 128>(a, s);
   const bool tall = a.M >= a.N;
   if (force == 2 || force == 3 || (!force && tiles(tall ? 64 : 128, tall ? 128 : 64) >= 512)) {

@@ -731,7 +731,8 @@ GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode, bool may_split 
   // pay for the hand-over), batches up to 8 gain nothing.
   if (may_split && mode != 2 && K % 64 == 0 && groups / c.R < 190) {
     int want = (B > 8 && K >= 8192) ? 0 : -1;
-    if (const char* e = getenv("MTP_GEMV_S")) want = atoi(e);
+    static MtpTune tune_s("MTP_GEMV_S");
+    want = tune_s.get(want);
     const int waves = c.R >= 8 ? 4 : GV_MAX_WAVES;
     for (int sl = 2; want >= 0 && sl <= GV_MAX_SLICES; sl *= 2) {
       if ((K / 64) % (sl * waves) != 0 || (want == 0 && K / 64 / (sl * waves) < 6)) break;
@@ -744,13 +745,14 @@ GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode, bool may_split 
   if (mode == 1 && c.R < 2) c.R = 2;
   c.D = (B > 16 || c.R >= 4) ? 1 : 2;
   while (!depth_ok(K, c.D)) c.D >>= 1;
-  if (const char* e = getenv("MTP_GEMV_R")) {
-    const int r = atoi(e);
+  static MtpTune tune_r("MTP_GEMV_R"), tune_d("MTP_GEMV_D");
+  if (tune_r.is_set()) {
+    const int r = tune_r.get(0);
     if (r == 1 || r == 2 || r == 4 || r == 8) c.R = (mode == 1 && r == 1) ? 2 : r;
     if (c.R * c.D > 4) c.D = c.R >= 4 ? 1 : 4 / c.R;
   }
-  if (const char* e = getenv("MTP_GEMV_D")) {
-    const int d = atoi(e);
+  if (tune_d.is_set()) {
+    const int d = tune_d.get(0);
     if ((d == 1 || d == 2 || d == 4) && c.R * d <= 4 && depth_ok(K, d)) c.D = d;
   }
   if (c.R >= 4) c.D = 1;
@@ -770,11 +772,11 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   const unsigned n_wg = (unsigned)((span + rows_per_wg - 1) / rows_per_wg);
   if (n_wg_out) *n_wg_out = n_wg;
   const int NB = B > 16 ? 2 : 1;
-  int rot_mul = 1;
-  if (const char* e = getenv("MTP_GEMV_ROT")) rot_mul = atoi(e);
+  static MtpTune tune_rot("MTP_GEMV_ROT"), tune_noshift("MTP_GEMV_NOSHIFT");
+  int rot_mul = tune_rot.get(1);
   if (rot_mul < 0) rot_mul = 0;   // the rotation is taken modulo the number of pairs: it must not go negative
-  int flags = 0;                  // bit 0: SwiGLU up rows walk in step with the gate rows (measurement only)
-  if (const char* e = getenv("MTP_GEMV_NOSHIFT")) flags |= atoi(e) ? 1 : 0;
+  int flags = 0;                  // bit 0: SwiGLU up rows walk in step with the gate rows (slower, same result)
+  flags |= tune_noshift.get(0) ? 1 : 0;
   // k slices: counters first (one per row block, zero between launches), then the partial sums
   const int S = workspace ? cfg.S : 1;
   int32_t* karrived = static_cast<int32_t*>(workspace);
@@ -827,8 +829,9 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
 int pick_mixed_groups(int64_t B, int64_t N, int64_t K) {
   const int64_t half = N / 2;
   if (B > 16 || K % 64 != 0 || (K / 64) % GV_MAX_WAVES != 0 || (half + 64) * K >= (1ll << 32)) return 0;
-  if (const char* e = getenv("MTP_GEMV_MIX")) {
-    const int r = atoi(e);
+  static MtpTune tune_mix("MTP_GEMV_MIX");
+  if (tune_mix.is_set()) {
+    const int r = tune_mix.get(0);
     return r >= 1 && r <= 7 ? r : 0;
   }
   const int64_t groups = (half + 7) / 8;
@@ -851,8 +854,8 @@ int launch_gemv_mixed(const void* x, const void* w, const void* bias, void* y, i
                       hipStream_t s, bool f16, GemvFuse fz = GemvFuse{nullptr, nullptr, 0.f, nullptr, nullptr}) {
   const int64_t half = N / 2;
   const unsigned n_wg = (unsigned)((half + 8 * R - 1) / (8 * R));
-  int rot_mul = 1;
-  if (const char* e = getenv("MTP_GEMV_ROT")) rot_mul = atoi(e);
+  static MtpTune tune_rot("MTP_GEMV_ROT");
+  int rot_mul = tune_rot.get(1);
   if (rot_mul < 0) rot_mul = 0;
 #define GVM_T(RR, FF)                                                                                              \
   hipLaunchKernelGGL((gemv_kernel<RR, 1, 3, false, 1, GV_MAX_WAVES, FF, NORM, (RR <= 6)>), dim3(n_wg),                \

@@ -127,6 +127,20 @@ __device__ __forceinline__ float silu_f(float x) { return x * sigmoid_f(x); }
 // ---- host side -------------------------------------------------------------
 void mtp_set_error(const char* fmt, ...);
 
+// Tuning variables (tile or slice choices that never change a result, only which correct kernel runs).  The
+// environment is read once per variable, at its first use, and again only when mtp_reload_tuning() is called:
+// a launch never calls getenv.
+struct MtpTune {
+  const char* name;
+  int value;      // valid when state == 2
+  int state;      // 0 = not read yet, 1 = unset in the environment, 2 = set
+  MtpTune* next;
+  explicit MtpTune(const char* n);
+  // value of the variable, or dflt when it is not set
+  int get(int dflt);
+  bool is_set();
+};
+
 #define MTP_REQUIRE(cond, code, ...)        \
   do {                                      \
     if (!(cond)) {                          \

@@ -23,6 +23,24 @@ def gpu():
     return torch.device("cuda:0")
 
 
+@pytest.fixture
+def set_tuning(monkeypatch):
+    """set_tuning(name, value): put an MTP_* tuning variable into the environment (None removes it) and have the
+    library read it: the library reads its environment once, not per launch.  Undone when the test ends."""
+    from merak_amd import _lib
+
+    def _set(name, value):
+        if value is None:
+            monkeypatch.delenv(name, raising=False)
+        else:
+            monkeypatch.setenv(name, str(value))
+        _lib.lib().mtp_reload_tuning()
+
+    yield _set
+    monkeypatch.undo()
+    _lib.lib().mtp_reload_tuning()
+
+
 @pytest.fixture(autouse=True)
 def _reset_mpu():
     from merak_amd import mpu, set_args

@@ -163,6 +163,25 @@ def test_ce_full_size_llama_vocab(gpu):
     assert (rowsum - expect).abs().max() < 0.05
 
 
+def test_ce_full_size_gpt2_vocab(gpu):
+    """[8192, 50257] fp32 (rows not 16-byte aligned), uniform labels: oracle on a sample of rows; every gradient
+    row sums to zero (softmax sums to one, minus the one-hot)."""
+    n, v = 8192, 50257
+    x = torch.empty(n, v, device=gpu).normal_(generator=torch.Generator(device=gpu).manual_seed(1239))
+    t = torch.randint(0, v, (n,), generator=gen(14))
+    tg = t.to(gpu)
+    loss, m, s, pred = ops.vocab_ce_fwd(x, tg, 0)
+    rows = torch.randperm(n, generator=gen(15))[:48]
+    xs = x[rows.to(gpu)].cpu()
+    g = torch.full((n,), 1.0 / n)
+    ref_loss, ref_grad = R.cross_entropy_fp32(xs, t[rows], 0, g[rows])
+    assert rel(loss.cpu()[rows], ref_loss) < TOL_LOSS
+    assert bool(torch.isfinite(loss).all()) and float(loss.min()) > 0
+    ops.vocab_ce_bwd_(x, tg, m, s, g.to(gpu), 0)
+    assert rel(x[rows.to(gpu)], ref_grad) < TOL_F32
+    assert (x.double().sum(-1).cpu() * n).abs().max() < 1e-3
+
+
 @pytest.mark.parametrize("dtype,n,v", [
     (torch.float32, 64, 50257), (torch.bfloat16, 64, 128256), (torch.float32, 7, 1), (torch.float32, 3, 5),
     (torch.bfloat16, 5, 9), (torch.bfloat16, 4, 1031), (torch.float32, 2, 2048 + 3), (torch.bfloat16, 3, 40000),
@@ -514,7 +533,8 @@ def test_gpt2_small_fp32_full_size(gpu):
 
 
 @pytest.mark.parametrize("name,m,k,n", [("llama8b_qkv", 4096, 4096, 6144), ("llama8b_down", 4096, 14336, 4096),
-                                         ("llama70b_tp8_qkv", 8192, 8192, 1280), ("llama70b_tp8_oproj", 8192, 1024, 8192)])
+                                         ("llama70b_tp8_qkv", 8192, 8192, 1280), ("llama70b_tp8_oproj", 8192, 1024, 8192),
+                                         ("llama70b_tp8_down", 8192, 3584, 8192)])
 def test_linear_full_size_sampled(gpu, name, m, k, n):
     """Full Llama-3-8B and Llama-70B tp=8 shard shapes: oracle on sampled rows of Y, dX and dW; linearity in X over the whole output."""
     g = torch.Generator(device=gpu).manual_seed(1240)
@@ -532,6 +552,36 @@ def test_linear_full_size_sampled(gpu, name, m, k, n):
     ref_dw = R.linear_backward(x.cpu().float(), ws[rn.cpu()], dy[:, rn].cpu().float(), False)[1]
     assert rel(dw[rn], ref_dw) < TOL_BF16
     y2, _ = ops.linear_fwd((x.float() * 2).bfloat16(), w, None, ops.EPI_NONE)     # exact in bf16: scaling by 2
+    assert torch.equal(y2.float(), y.float() * 2)
+
+
+@pytest.mark.parametrize("name,m,k,half", [("llama8b_gate_up", 4096, 4096, 14336), ("llama70b_tp8_gate_up", 8192, 8192, 3584)])
+def test_swiglu_full_size_sampled(gpu, name, m, k, half):
+    """Gate/up column layers with the fused SwiGLU at their full token counts: oracle on sampled rows of the
+    pre-activation, the activation, dX and dW; the pre-activation is linear in X over the whole output."""
+    n = 2 * half
+    g = torch.Generator(device=gpu).manual_seed(1241)
+    x = torch.empty(m, k, device=gpu).normal_(generator=g).bfloat16()
+    w = torch.empty(n, k, device=gpu).normal_(0, 0.02, generator=g).bfloat16()
+    dact = torch.empty(m, half, device=gpu).normal_(generator=g).bfloat16()
+    y, act = ops.linear_fwd(x, w, None, ops.EPI_SWIGLU)
+    assert y.shape == (m, n) and act.shape == (m, half)
+    rm = torch.randperm(m, generator=gen(72))[:32].to(gpu)
+    rn = torch.randperm(n, generator=gen(73))[:32].to(gpu)
+    xs, ws = x[rm].cpu().float(), w.cpu().float()
+    assert rel(y[rm], F.linear(xs, ws)) < TOL_BF16
+    assert rel(act[rm], R.swiglu(y[rm].float().cpu())) < TOL_BF16      # activation of the stored pre-activation
+    _, act_only = ops.linear_fwd(x, w, None, ops.EPI_SWIGLU, want_pre=False)
+    assert torch.equal(act_only, act)
+    dy = ops.activation_bwd(dact, y, ops.EPI_SWIGLU)
+    assert rel(dy[rm], R.swiglu_backward(dact[rm].float().cpu(), y[rm].float().cpu())) < TOL_BF16
+    dx = ops.linear_dgrad(dy, w)
+    dw, _ = ops.linear_wgrad(dy, x, False)
+    dys = dy[rm].cpu().float()
+    assert rel(dx[rm], R.linear_backward(xs, ws, dys, False)[0]) < TOL_BF16
+    ref_dw = R.linear_backward(x.cpu().float(), ws[rn.cpu()], dy[:, rn].cpu().float(), False)[1]
+    assert rel(dw[rn], ref_dw) < TOL_BF16
+    y2, _ = ops.linear_fwd((x.float() * 2).bfloat16(), w, None, ops.EPI_SWIGLU)   # exact in bf16: scaling by 2
     assert torch.equal(y2.float(), y.float() * 2)
 
 
@@ -617,12 +667,12 @@ def test_gemv_and_fused_argmax(gpu, b, n, k):
     (32, 4096, 4096, "none", None, False), (8, 4096, 14336, "none", None, False),      # small k / small batch: uncut
     (32, 6144, 4096, "bias", "4", True), (32, 2048, 4096, "swiglu", "8", True), (24, 1000, 1024, "none", "2", True),
     (3, 4096, 4096, "none", "8", True)])
-def test_gemv_cut_along_k_with_workspace(gpu, monkeypatch, b, n, k, epi, force, cut):
+def test_gemv_cut_along_k_with_workspace(gpu, set_tuning, b, n, k, epi, force, cut):
     """Few-row matrices with a long k run, above 8 batch rows, as k slices whose partial sums meet in a
     workspace (other shapes only when forced): same numbers as the oracle, the same bits on every run, and a
     workspace that can be used again as it is left."""
     if force:
-        monkeypatch.setenv("MTP_GEMV_S", force)
+        set_tuning("MTP_GEMV_S", force)
     g = gen(31)
     x = torch.randn(b, k, generator=g).bfloat16()
     w = (torch.randn(n, k, generator=g) * 0.02).bfloat16()
@@ -950,11 +1000,11 @@ def test_greedy_pick_over_a_vocab_sharded_lm_head(gpu):
 @pytest.mark.parametrize("mix", ["1", "2", "3", "4", "5", "6", "7", None])
 @pytest.mark.parametrize("b,half,k,with_bias", [(1, 14336, 4096, False), (8, 1000, 1024, True), (16, 56, 512, False),
                                                 (3, 3584, 8192, False)])
-def test_gemv_swiglu_mixed_row_groups(gpu, monkeypatch, mix, b, half, k, with_bias):
+def test_gemv_swiglu_mixed_row_groups(gpu, set_tuning, mix, b, half, k, with_bias):
     """SwiGLU GEMV whose 16-row tiles hold 8 gate rows and their 8 up rows, for every number of groups per
     workgroup (forced) and for the automatic choice: same result as the oracle, ragged ends included."""
     if mix is not None:
-        monkeypatch.setenv("MTP_GEMV_MIX", mix)
+        set_tuning("MTP_GEMV_MIX", mix)
     g = gen(41)
     x = torch.randn(b, k, generator=g).bfloat16()
     w = (torch.randn(2 * half, k, generator=g) * 0.03).bfloat16()

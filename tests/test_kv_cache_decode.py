@@ -99,10 +99,10 @@ def test_attn_decode_lengths_and_groups(gpu, n_q, n_kv, lens):
 
 
 @pytest.mark.parametrize("splits", ["1", "3", "16", "64"])
-def test_attn_decode_ragged_batch_any_split_count(gpu, splits, monkeypatch):
+def test_attn_decode_ragged_batch_any_split_count(gpu, splits, set_tuning):
     lens = [1000, 1, 0, 64, 513, 37]
     q, kc, vc, dl, ref = _attn_case(gpu, 6, 32, 8, 1024, lens, seed=4)
-    monkeypatch.setenv("MTP_ATTN_SPLITS", splits)
+    set_tuning("MTP_ATTN_SPLITS", splits)
     out = ops.attn_decode(q, kc, vc, dl)
     assert torch.count_nonzero(out[2]) == 0                      # no tokens: zeros
     for b in range(6):
@@ -281,11 +281,11 @@ def test_block_step_vs_oracle_llama8b_shape(gpu):
         assert rel(kc[b, :, int(pos[b])], kf[b, :, int(pos[b])]) < TOL_BF16
 
 
-def test_negative_rotation_knobs_are_clamped(gpu, monkeypatch):
+def test_negative_rotation_knobs_are_clamped(gpu, set_tuning):
     """The measurement knobs that rotate the walk order are taken modulo a count on the device: negative values
     from the environment are clamped on the host (they used to turn into negative offsets)."""
-    monkeypatch.setenv("MTP_GEMV_ROT", "-3")
-    monkeypatch.setenv("MTP_ATTN_ROT", "-5")
+    set_tuning("MTP_GEMV_ROT", "-3")
+    set_tuning("MTP_ATTN_ROT", "-5")
     g = gen(12)
     x = torch.randn(4, 1024, generator=g).bfloat16()
     w = (torch.randn(512, 1024, generator=g) * 0.05).bfloat16()
@@ -389,8 +389,8 @@ def test_gemv_norm_prologue(gpu, dtype, B, N, K, epi):
 
 
 @pytest.mark.parametrize("groups", [1, 2, 3, 4, 5, 6, 7])
-def test_gemv_norm_prologue_every_mixed_group_count(gpu, groups, monkeypatch):
-    monkeypatch.setenv("MTP_GEMV_MIX", str(groups))
+def test_gemv_norm_prologue_every_mixed_group_count(gpu, groups, set_tuning):
+    set_tuning("MTP_GEMV_MIX", str(groups))
     g = gen(62)
     B, N, K = 6, 2 * 1288, 1024
     x = torch.randn(B, K, generator=g).bfloat16().to(gpu)
@@ -400,7 +400,7 @@ def test_gemv_norm_prologue_every_mixed_group_count(gpu, groups, monkeypatch):
     two = ops.gemv(ops.rmsnorm(x, nw, 1e-6), w, None, ops.EPI_SWIGLU)
     assert rel(fused, two) < TOL_BF16 / 4
     plain = ops.gemv(x, w, None, ops.EPI_SWIGLU)                # the two-set main loop without the norm
-    monkeypatch.setenv("MTP_GEMV_MIX", "0")
+    set_tuning("MTP_GEMV_MIX", "0")
     assert rel(plain, ops.gemv(x, w, None, ops.EPI_SWIGLU)) < TOL_BF16 / 4
 
 

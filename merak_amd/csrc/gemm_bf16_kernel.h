@@ -357,14 +357,26 @@ template <int ROWS, int NW> struct OperandOf<LAY_COL, ROWS, NW> { using type = C
 //                 block row i starts at tile row (i/HI)*BM/2 + wm*32*HI + 32 (i%HI), columns likewise.
 // With SwiGLU both forms put the gate columns into blocks j < TJ/2 and the matching up columns into the others.
 // ---------------------------------------------------------------------------
-template <int BM, int BN, int EPI, int OUT, int NW, bool F16, bool QMAP, int LDS_BYTES, int TI, int TJ>
-__device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16_t (&acc)[TI][TJ], float (&rsum)[TI], char* lds,
-                                              int m0, int n0, int tn, int wave, int lane) {
+//
+// The accumulators come through an accessor, so that both MFMA shapes are served.  Seen from here the wave's part
+// is a TI x TJ grid of 32x32 blocks, and of block (i, j) a lane holds four groups g of four consecutive columns:
+//   BLK = 32 (v_mfma_f32_32x32x16, B fragment first): group g = row l%32, columns 8 g + 4 (l/32) .. +3;
+//   BLK = 16 (v_mfma_f32_16x16x32, B fragment first; the block is 2x2 MFMA blocks): group g = row
+//            16 (g/2) + l%16, columns 16 (g%2) + 4 (l/16) .. +3.
+// accv(i, j, g, e) is element e of group g; rsum_of(i, g) (EPI_ROWSUM only) the lane's part of the k sum of the
+// A row that group g sits in.
+template <int BM, int BN, int EPI, int OUT, int NW, bool F16, bool QMAP, int LDS_BYTES, int TI, int TJ, int BLK,
+          typename AccFn, typename RsumFn>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, AccFn accv, RsumFn rsum_of, char* lds, int m0, int n0,
+                                              int tn, int wave, int lane) {
   using X = X16<F16>;
+  static_assert(BLK == 32 || BLK == 16, "MFMA block: 32x32 or 16x16");
   constexpr int WGM = 2, WGN = NW / 2;
   constexpr int HI = TI / 2, HJ = TJ / 2;
   const int wm = wave / WGN, wn = wave % WGN;
-  const int lh = lane >> 5, l32 = lane & 31;
+  // row (inside the 32-row block) and first column (inside the 32-column block) of group g
+  auto row_off = [&](int g) -> int { return BLK == 32 ? (lane & 31) : 16 * (g >> 1) + (lane & 15); };
+  auto col_off = [&](int g) -> int { return BLK == 32 ? 8 * g + 4 * (lane >> 5) : 16 * (g & 1) + 4 * (lane >> 4); };
   // first tile row of the wave's block row i
   auto blk_row = [&](int i) -> int {
     if (QMAP) return (i / HI) * (BM / 2) + wm * (32 * HI) + (i % HI) * 32;
@@ -375,24 +387,29 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16_t (&acc)
 
     if (tn == 0 && wn == 0) {
 #pragma unroll
-      for (int i = 0; i < TI; i++) {
-        const float t = rsum[i] + __shfl_xor(rsum[i], 32, 64);  // the two k halves of a row
-        const int row = m0 + blk_row(i) + l32;
-        if (lh == 0 && row < p.M) {
-          if (OUT == OUT_F32) {
-            float* q = (float*)p.rowsum + row;
-            *q = p.accumulate ? *q + t : t;
-          } else {
-            uint16_t* q = (uint16_t*)p.rowsum + row;
-            *q = X::to_bits(p.accumulate ? X::from_bits(*q) + t : t);
+      for (int i = 0; i < TI; i++)
+#pragma unroll
+        for (int g = 0; g < (BLK == 32 ? 1 : 4); g += 2) {
+          // the lanes that hold the same row at other k add up: 2 halves (32x32x16) or 4 quarters (16x16x32)
+          float t = rsum_of(i, g);
+          t += __shfl_xor(t, 32, 64);
+          if (BLK == 16) t += __shfl_xor(t, 16, 64);
+          const int row = m0 + blk_row(i) + row_off(g);
+          if (lane < BLK && row < p.M) {
+            if (OUT == OUT_F32) {
+              float* q = (float*)p.rowsum + row;
+              *q = p.accumulate ? *q + t : t;
+            } else {
+              uint16_t* q = (uint16_t*)p.rowsum + row;
+              *q = X::to_bits(p.accumulate ? X::from_bits(*q) + t : t);
+            }
           }
         }
-      }
     }
   }
 
   // ---- epilogue ----------------------------------------------------------------
-  // acc[i][j][r]: row m = m0 + wm*BM/2 + 32i + l32, column block j, n_local = 8*(r/4) + 4*lh + r%4.
+  // group g of block (i, j): row m0 + blk_row(i) + row_off(g), columns col_of_block(j) + col_off(g) .. +3.
   // Stage 32 rows x (BN/2) columns per wave through LDS, then 16-byte row-contiguous stores.
   constexpr int WN = BN / WGN;                     // columns per wave
   constexpr int ESZ = (OUT == OUT_F32) ? 4 : 2;
@@ -527,13 +544,13 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16_t (&acc)
           if (p.bias) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-              const int col = cb + 8 * g + 4 * lh + e;
+              const int col = cb + col_off(g) + e;
               b4[e] = col < lim_of_block(j) ? X::from_bits(p.bias[col]) : 0.f;
             }
           }
         }
 #pragma unroll
-        for (int e = 0; e < 4; e++) pre[j][4 * g + e] = acc[i][j][4 * g + e] + b4[e];
+        for (int e = 0; e < 4; e++) pre[j][4 * g + e] = accv(i, j, g, e) + b4[e];
       }
     }
     if (OUT == OUT_F32) {
@@ -543,7 +560,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16_t (&acc)
 #pragma unroll
           for (int g = 0; g < 4; g++) {
             f32x4_t v = {pre[j][4 * g], pre[j][4 * g + 1], pre[j][4 * g + 2], pre[j][4 * g + 3]};
-            *reinterpret_cast<f32x4_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 4) = v;
+            *reinterpret_cast<f32x4_t*>(stage + row_off(g) * PITCH + (32 * j + col_off(g)) * 4) = v;
           }
         wave_lds_sync();
         flush(i, p.C, p.ldc, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::true_type{}, p.accumulate != 0);
@@ -563,7 +580,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16_t (&acc)
 #pragma unroll
           for (int g = 0; g < 4; g++) {
             u32x2_t v = {pk[j][2 * g], pk[j][2 * g + 1]};
-            *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
+            *reinterpret_cast<u32x2_t*>(stage + row_off(g) * PITCH + (32 * j + col_off(g)) * 2) = v;
           }
         wave_lds_sync();
         flush(i, p.C, p.ldc, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::false_type{}, p.accumulate != 0);
@@ -585,7 +602,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16_t (&acc)
           for (int g = 0; g < 4; g++) {
             u32x2_t v = {X::pack2(gelu_new_f(pre[j][4 * g]), gelu_new_f(pre[j][4 * g + 1])),
                          X::pack2(gelu_new_f(pre[j][4 * g + 2]), gelu_new_f(pre[j][4 * g + 3]))};
-            *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
+            *reinterpret_cast<u32x2_t*>(stage + row_off(g) * PITCH + (32 * j + col_off(g)) * 2) = v;
           }
         wave_lds_sync();
         flush(i, p.C2, p.ldc2, std::integral_constant<int, TJ>{}, col_of_block, lim_of_block, std::false_type{}, false);
@@ -601,7 +618,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16_t (&acc)
 #pragma unroll
             for (int e = 0; e < 4; e++) a4[e] = silu_f(pre[j][4 * g + e]) * pre[j + HJ][4 * g + e];
             u32x2_t v = {X::pack2(a4[0], a4[1]), X::pack2(a4[2], a4[3])};
-            *reinterpret_cast<u32x2_t*>(stage + l32 * PITCH + (32 * j + 8 * g + 4 * lh) * 2) = v;
+            *reinterpret_cast<u32x2_t*>(stage + row_off(g) * PITCH + (32 * j + col_off(g)) * 2) = v;
           }
         wave_lds_sync();
         auto act_col = [&](int j) -> int { return n0 + wn * (WN / 2) + j * 32; };
@@ -634,24 +651,30 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, f32x16_t (&acc)
 // the two units the next half tile reads.  The requests of tiles past the end of k are still issued, with
 // every lane out of range (zero fill, no memory traffic), so that the counting never changes.
 // ---------------------------------------------------------------------------
+//
+// BLK picks the MFMA: 32 = v_mfma_f32_32x32x16 (4 steps of 16 per k-tile), 16 = v_mfma_f32_16x16x32 (2 steps of 32).
+// Per flop the 16x16x32 form moves half the accumulator registers and twice the operand registers, 8 against 10
+// KiB per 32 Kflop in all, and on operands of random sign and mantissa the matrix cores sustain about 15 % more
+// with it at the board's power limit (register-resident loops with 256 accumulator registers per lane: 2120
+// against 1850 TFLOP/s).
 constexpr int QBK = 64;    // k-tile depth
-constexpr int QKS = 4;     // k16 steps per k-tile
 
 // K-contiguous operand: LDS unit = 128 rows x 128 bytes; the 16-byte chunk c of row r sits at position
 // c ^ ((r >> 1) & 7): 16 consecutive rows read at one k cover all 64 banks.  One DMA instruction fills 8 rows
 // (lane l -> row l/8, position l%8, fetching chunk (l%8) ^ swizzle of its row: the 8 lanes of a row still ask
 // for one whole line).  Fragment = one ds_read_b128.
-template <int NW, int WG>
+template <int NW, int WG, int BLK>
 struct RowOperandQ {
   static constexpr int UROWS = 128;                  // rows per unit
   static constexpr int UBYTES = UROWS * QBK * 2;     // 16 KiB
   static constexpr int BYTES = 2 * UBYTES;           // per k-tile buffer
-  static constexpr int H = UROWS / (32 * WG);        // 32-row blocks per wave and unit
+  static constexpr int QKS = BLK == 32 ? 4 : 2;      // MFMA steps per k-tile
+  static constexpr int H = UROWS / (BLK * WG);       // BLK-row blocks per wave and unit
   static constexpr int NU = UROWS / 8 / NW;          // DMA instructions per wave and unit
   static_assert(H >= 1 && NU >= 1, "wave grid too fine for the unit");
   rsrc_t rsrc;
   uint32_t voff[2][NU];
-  uint32_t fo[QKS];
+  uint32_t fo[2][QKS];   // [k-tile buffer][step]: the buffer's 64 KiB do not fit the 16-bit offset field of a read
   int gchunk, K;
 
   // rowmap(r): global row (relative to row0) of tile row r (unit r / 128), or a negative value for "no such row";
@@ -672,11 +695,13 @@ struct RowOperandQ {
         const int64_t gr = rowmap(r);
         voff[u][j] = (gr < 0 || gr >= nrows - row0) ? 0x80000000u : (uint32_t)((gr * ld + gchunk * 8) * 2);
       }
-    // fragment of block b at step kk: row 32 H wsub + 32 b + l32 of the unit, chunk 2 kk + l/32
-    const int l32 = lane & 31, h = lane >> 5;
+    // fragment of block b at step kk: row BLK (H wsub + b) + l % BLK of the unit, 8 k from 8 (64 / BLK) kk + 8 (l / BLK)
+    const int lr = lane & (BLK - 1), h = lane / BLK;
 #pragma unroll
-    for (int kk = 0; kk < QKS; kk++)
-      fo[kk] = (uint32_t)((wsub * 32 * H + l32) * 128 + ((((2 * kk + h) ^ (l32 >> 1)) & 7) << 4));
+    for (int kk = 0; kk < QKS; kk++) {
+      fo[0][kk] = (uint32_t)((wsub * BLK * H + lr) * 128 + (((((64 / BLK) * kk + h) ^ (lr >> 1)) & 7) << 4));
+      fo[1][kk] = fo[0][kk] + 65536;
+    }
   }
   struct Prep {
     uint32_t soff;
@@ -689,35 +714,41 @@ struct RowOperandQ {
   __device__ __forceinline__ void issue(const Prep& pp, uint32_t unit_lds, int wave, int u, int j) const {
     dma16(rsrc, unit_lds + (wave + NW * j) * 1024, pp.dead ? 0x80000000u : voff[u][j], pp.soff);
   }
-  __device__ __forceinline__ bf16x8_t frag(const char* unit, int b, int kk) const {
-    return *reinterpret_cast<const bf16x8_t*>(unit + b * (32 * 128) + fo[kk]);
+  // unit: address of the unit in k-tile buffer 0
+  __device__ __forceinline__ bf16x8_t frag(const char* unit, int buf, int b, int kk) const {
+    return *reinterpret_cast<const bf16x8_t*>(unit + b * (BLK * 128) + fo[buf][kk]);
   }
 };
 
 // Transposed operand (memory [K, rows], rows contiguous): LDS unit = 64 k-rows x 128 rows, 256 bytes per k-row;
-// chunk c of k-row k sits at position c ^ ((k & 3) << 2).  One DMA instruction fills 4 k-rows (lane l -> k-row
-// l/16, position l%16).  Fragment = two ds_read_b64_tr_b16, addressed as in ColOperand.
-template <int NW, int WG>
+// chunk c of k-row k sits at position c ^ ((k & 3) << 2) ^ ((k >> 3 & 1) << 1): the four k-rows a group of 16
+// lanes reads land on four different 64-byte bank groups, and the k-rows 8 apart that the two groups of one
+// ds_read_b64_tr_b16 pass read in the 16x16x32 form land 32 bytes apart.  One DMA instruction fills 4 k-rows
+// (lane l -> k-row l/16, position l%16).  Fragment = two ds_read_b64_tr_b16: in each group of 16 lanes, lane i
+// supplies the address of 4 consecutive rows-elements of one k-row and receives, transposed, 4 consecutive k of
+// one row; BLK = 32: group G holds rows 16 (G%2) .. +15 at k 8 (G/2) .. +7, BLK = 16: rows 0 .. 15 at k 8 G .. +7.
+template <int NW, int WG, int BLK>
 struct ColOperandQ {
   static constexpr int UROWS = 128;
   static constexpr int UBYTES = QBK * UROWS * 2;
   static constexpr int BYTES = 2 * UBYTES;
-  static constexpr int H = UROWS / (32 * WG);
+  static constexpr int QKS = BLK == 32 ? 4 : 2;
+  static constexpr int H = UROWS / (BLK * WG);
   static constexpr int NU = QBK / 4 / NW;
   static_assert(H >= 1 && NU >= 1, "wave grid too fine for the unit");
   const char* base;     // &mem[0][row0]
   int64_t total;        // bytes from base to the end of the matrix
   int64_t ktile_bytes;  // QBK * ld * 2
   uint32_t voff[2][NU];
-  uint32_t lane_base;
-  uint32_t moff[H];
+  uint32_t moff[2][H];   // [k-tile buffer][block], the lane's k-row and element included
 
   __device__ __forceinline__ void init(const uint16_t* mem, int64_t ld, int row0, int K_, int lane, int wave, int wsub) {
     base = reinterpret_cast<const char*>(mem + row0);
     total = ((int64_t)K_ * ld - row0) * 2;
     ktile_bytes = (int64_t)QBK * ld * 2;
     const int ksub = lane >> 4;                        // k-row inside the instruction = k & 3
-    const int c = (lane & 15) ^ (ksub << 2);           // chunk of the unit's 128 rows this lane fetches
+    // chunk of the unit's 128 rows this lane fetches; k >> 3 & 1 = (wave + NW j) >> 1 & 1 = wave >> 1 & 1
+    const int c = (lane & 15) ^ (ksub << 2) ^ (((wave >> 1) & 1) << 1);
 #pragma unroll
     for (int u = 0; u < 2; u++)
 #pragma unroll
@@ -725,14 +756,16 @@ struct ColOperandQ {
         const int krow = 4 * (wave + NW * j) + ksub;
         voff[u][j] = (uint32_t)(((int64_t)krow * ld + u * UROWS + c * 8) * 2);
       }
-    // lane (group G = l/16, i = l%16) addresses k-row 8 (G/2) + i/4 (+16 kk, +4 for the second read) and
-    // elements 16 (G%2) + 4 (i%4) .. +3 of the block
+    // lane (group G = l/16, i = l%16) addresses k-row kg + i/4 (+ (1024 / BLK) kk, +4 for the second read) and
+    // elements eg + 4 (i%4) .. +3 of the block, with (kg, eg) = (8 (G/2), 16 (G%2)) for BLK = 32, (8 G, 0) for 16
     const int G = lane >> 4, i = lane & 15, kq = i >> 2;
-    lane_base = (uint32_t)((8 * (G >> 1) + kq) * (UROWS * 2) + 8 * (i & 1));
+    const int kg = BLK == 32 ? 8 * (G >> 1) : 8 * G, eg = BLK == 32 ? 16 * (G & 1) : 0;
+    const uint32_t lane_base = (uint32_t)((kg + kq) * (UROWS * 2) + 8 * (i & 1));
 #pragma unroll
     for (int b = 0; b < H; b++) {
-      const int c2 = (wsub * 32 * H + 32 * b) / 8 + 2 * (G & 1) + ((i & 3) >> 1);
-      moff[b] = (uint32_t)((c2 ^ (kq << 2)) * 16);
+      const int c2 = (wsub * BLK * H + BLK * b + eg) / 8 + ((i & 3) >> 1);
+      moff[0][b] = lane_base + (uint32_t)((c2 ^ (kq << 2) ^ (((kg >> 3) & 1) << 1)) * 16);
+      moff[1][b] = moff[0][b] + 65536;
     }
   }
   struct Prep {
@@ -745,8 +778,8 @@ struct ColOperandQ {
   __device__ __forceinline__ void issue(const Prep& pp, uint32_t unit_lds, int wave, int u, int j) const {
     dma16(pp.r, unit_lds + (wave + NW * j) * 1024, voff[u][j], 0);
   }
-  __device__ __forceinline__ bf16x8_t frag(const char* unit, int b, int kk) const {
-    const char* a = unit + lane_base + moff[b] + kk * (16 * UROWS * 2);
+  __device__ __forceinline__ bf16x8_t frag(const char* unit, int buf, int b, int kk) const {
+    const char* a = unit + moff[buf][b] + kk * ((QBK / QKS) * UROWS * 2);
     const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
         (bf16x4_t __attribute__((address_space(3)))*)(a));
     const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
@@ -755,8 +788,8 @@ struct ColOperandQ {
   }
 };
 
-template <int LAY, int NW, int WG> struct QOperandOf { using type = RowOperandQ<NW, WG>; };
-template <int NW, int WG> struct QOperandOf<LAY_COL, NW, WG> { using type = ColOperandQ<NW, WG>; };
+template <int LAY, int NW, int WG, int BLK> struct QOperandOf { using type = RowOperandQ<NW, WG, BLK>; };
+template <int NW, int WG, int BLK> struct QOperandOf<LAY_COL, NW, WG, BLK> { using type = ColOperandQ<NW, WG, BLK>; };
 
 // compile-time list of ints, read by index
 template <int... V>
@@ -764,19 +797,23 @@ struct IntList {
   static constexpr int v[sizeof...(V)] = {V...};
 };
 
-template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16>
+template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK>
 __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
   using X = X16<F16>;
   constexpr int BM = 256, BN = 256;
   static_assert(EPI != MTP_EPI_SWIGLU || BLAY == LAY_ROW, "the SwiGLU row interleave is a forward (row B) feature");
   static_assert(NW == 4 || NW == 8, "4 waves (2x2) or 8 waves (2x4) per workgroup");
   constexpr int WGM = 2, WGN = NW / 2;
-  constexpr int TI = BM / (32 * WGM), TJ = BN / (32 * WGN);
-  using AOp = typename QOperandOf<ALAY, NW, WGM>::type;
-  using BOp = typename QOperandOf<BLAY, NW, WGN>::type;
-  constexpr int HI = AOp::H, HJ = BOp::H;
+  constexpr int TI = BM / (BLK * WGM), TJ = BN / (BLK * WGN);   // MFMA blocks per wave in m and n
+  using AOp = typename QOperandOf<ALAY, NW, WGM, BLK>::type;
+  using BOp = typename QOperandOf<BLAY, NW, WGN, BLK>::type;
+  constexpr int HI = AOp::H, HJ = BOp::H, QKS = AOp::QKS;
   static_assert(2 * HI == TI && 2 * HJ == TJ, "two units per operand");
+  using AccT = std::conditional_t<BLK == 32, f32x16_t, f32x4_t>;
+  constexpr int S = 32 / BLK;           // MFMA blocks per 32 rows (columns)
+  constexpr int TI32 = TI / S, TJ32 = TJ / S;
   constexpr int QBUF = AOp::BYTES + BOp::BYTES;   // one k-tile of both operands: 64 KiB
+  static_assert(QBUF == 65536, "the operands keep per-buffer read offsets 64 KiB apart");
   constexpr int LDS_BYTES = 2 * QBUF;
   __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
 
@@ -830,13 +867,13 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
   auto unit_a = [](int buf, int u) constexpr { return buf * QBUF + u * AOp::UBYTES; };
   auto unit_b = [](int buf, int u) constexpr { return buf * QBUF + AOp::BYTES + u * BOp::UBYTES; };
 
-  f32x16_t acc[TI][TJ];
+  AccT acc[TI][TJ];
 #pragma unroll
   for (int i = 0; i < TI; i++)
 #pragma unroll
     for (int j = 0; j < TJ; j++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+      for (int r = 0; r < (BLK == 32 ? 16 : 4); r++) acc[i][j][r] = 0.f;
   float rsum[TI];
 #pragma unroll
   for (int i = 0; i < TI; i++) rsum[i] = 0.f;
@@ -848,9 +885,10 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
   constexpr int HT = 2 * PH;                 // MFMAs per half tile
   constexpr int NDH = AOp::NU + BOp::NU;     // DMA instructions per wave and half tile (one unit of A, one of B)
   static_assert(AOp::NU == BOp::NU, "the units of A and B take the same number of DMA instructions");
-  constexpr int BPOST = PH >= 16 ? 4 : 2;    // MFMAs of a half tile issued behind its barrier
+  constexpr int BPOST = (BLK == 32 ? 1 : 2) * (HI * HJ >= 4 ? 4 : 2);   // MFMAs of a half tile issued behind its barrier
   constexpr int BARRIER_AT = HT - BPOST;
-  // the d-th DMA instruction of a half tile is issued behind MFMA number d HT / NDH + 1 of the half tile
+  // the d-th DMA instruction of a half tile is issued behind MFMA number dma_at(d) of the half tile
+  auto dma_at = [](int d) constexpr { return d * HT / NDH + 1; };
   constexpr int NAFTER = [&]() constexpr {   // DMA instructions of a half tile issued behind its barrier
     int n = 0;
     for (int d = 0; d < NDH; d++) n += (d * HT / NDH + 1) >= BARRIER_AT ? 1 : 0;
@@ -866,7 +904,21 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
     constexpr int MA = decltype(ma_tag)::value, MB = decltype(mb_tag)::value, m = decltype(m_tag)::value;
     constexpr int kk = m / (HI * HJ), w = m % (HI * HJ);
     constexpr int i = w / HJ, j = (i & 1) ? HJ - 1 - w % HJ : w % HJ;
-    acc[MA * HI + i][MB * HJ + j] = X::mfma32(rb[MB][j][kk], ra[MA][i][kk], acc[MA * HI + i][MB * HJ + j]);
+    constexpr int bi = MA * HI + i, bj = MB * HJ + j;   // MFMA block of the wave's part
+    if constexpr (BLK == 32) {
+      acc[bi][bj] = X::mfma32(rb[MB][j][kk], ra[MA][i][kk], acc[bi][bj]);
+    } else {
+      // Inline assembly with the accumulator tied in place: left to itself the register allocator moves the 64
+      // four-register accumulators about (hundreds of v_accvgpr copies per k-tile, and spills).  The statement
+      // hides the instruction from the compiler's hazard checks; what they would cover holds by construction:
+      // an accumulator is touched again 16 MFMAs later at the earliest, the operand registers are written by LDS
+      // reads only (s_waitcnt lgkmcnt, which the compiler does insert for the statement's inputs), and the
+      // first read of an accumulator by another instruction sits behind the wait states after the loop.
+      if constexpr (F16)
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[bi][bj]) : "v"(rb[MB][j][kk]), "v"(ra[MA][i][kk]));
+      else
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[bi][bj]) : "v"(rb[MB][j][kk]), "v"(ra[MA][i][kk]));
+    }
     if constexpr (EPI == EPI_ROWSUM && MB == 0 && j == 0) rsum[MA * HI + i] = X::sum8(ra[MA][i][kk], rsum[MA * HI + i]);
   };
   // f-th fragment read of a phase that refills register set U of A (IS_A) or B from buffer BUF; fragments in the
@@ -876,10 +928,10 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
     constexpr int U = decltype(u_tag)::value, BUF = decltype(buf_tag)::value, f = decltype(f_tag)::value;
     if constexpr (IS_A) {
       constexpr int kk = f / HI, b = f % HI;
-      ra[U][b][kk] = opA.frag(lds + unit_a(BUF, U), b, kk);
+      ra[U][b][kk] = opA.frag(lds + unit_a(0, U), BUF, b, kk);
     } else {
       constexpr int kk = f / HJ, b = f % HJ;
-      rb[U][b][kk] = opB.frag(lds + unit_b(BUF, U), b, kk);
+      rb[U][b][kk] = opB.frag(lds + unit_b(0, U), BUF, b, kk);
     }
   };
   // d-th DMA instruction of the group (A unit UA, B unit UB, buffer BUF): A and B alternate
@@ -971,9 +1023,17 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
     half_tile(kt + 2, EvenH1{});
   }
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+  // the last MFMAs' results must have reached the registers before anything else reads them (see mfma_q)
+  if constexpr (BLK == 16) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   __syncthreads();  // the epilogue reuses the tile buffers
   if (MTP_DBG(p, 2)) return;
-  gemm_epilogue<BM, BN, EPI, OUT, NW, F16, true, LDS_BYTES>(p, acc, rsum, lds, m0, n0, tn, wave, lane);
+  gemm_epilogue<BM, BN, EPI, OUT, NW, F16, true, LDS_BYTES, TI32, TJ32, BLK>(
+      p,
+      [&](int i, int j, int g, int e) -> float {
+        if constexpr (BLK == 32) return acc[i][j][4 * g + e];
+        else return acc[2 * i + (g >> 1)][2 * j + (g & 1)][e];
+      },
+      [&](int i, int g) -> float { return BLK == 32 ? rsum[i] : rsum[2 * i + (g >> 1)]; }, lds, m0, n0, tn, wave, lane);
 }
 
 // The body lives in a __device__ function: it uses inline assembly operands that the host pass over a
@@ -1330,7 +1390,9 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   if (MTP_DBG(p, 2)) return;
 
   if constexpr (EPI == EPI_ROWSUM) static_assert(NMF >= TI, "every A fragment of a step must meet an MFMA");
-  gemm_epilogue<BM, BN, EPI, OUT, NW, F16, false, NSTAGE * STAGE_BYTES>(p, acc, rsum, lds, m0, n0, tn, wave, lane);
+  gemm_epilogue<BM, BN, EPI, OUT, NW, F16, false, NSTAGE * STAGE_BYTES, TI, TJ, 32>(
+      p, [&](int i, int j, int g, int e) -> float { return acc[i][j][4 * g + e]; },
+      [&](int i, int) -> float { return rsum[i]; }, lds, m0, n0, tn, wave, lane);
 }
 
 template <int BM, int BN, int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16>
@@ -1338,9 +1400,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs p) {
   gemm_bf16_body<BM, BN, ALAY, BLAY, EPI, OUT, NW, F16>(p);
 }
 
-template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16>
+template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK>
 __global__ __launch_bounds__(NW * 64) void gemm_q_kernel(const GemmArgs p) {
-  gemm_q_body<ALAY, BLAY, EPI, OUT, NW, F16>(p);
+  gemm_q_body<ALAY, BLAY, EPI, OUT, NW, F16, BLK>(p);
 }
 
 // ---------------------------------------------------------------------------
@@ -1354,15 +1416,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_q_kernel(const GemmArgs p) {
 struct TileCfg {
   int bm, bn, nw;
   float eff;  // relative speed of one tile's inner loop per flop (256x256 = 1), from measurement
-  bool q;     // the 64-deep main loop (256x256 only)
+  int q;      // 0: the 32-deep ring; 32 / 16: the 64-deep main loop (256x256 only) on 32x32x16 / 16x16x32 MFMAs
 };
-// 256x256 exists with 8 waves (2 per SIMD: one wave's barrier and LDS waits are covered by the other's
-// MFMAs, and the epilogue's VALU work is spread over twice the waves) and with 4 waves (128x128 per wave:
-// a third fewer LDS reads per MFMA, accumulators in AGPRs), measured 0-4 % faster on the Llama-3-8B
-// shapes; the narrow tiles were measured best as listed.
+// 256x256 exists as the 32-deep ring (8 waves, or 4 waves with 128x128 per wave) and as the 64-deep loop (4 or 8
+// waves, 32x32x16 or 16x16x32 MFMAs).  Measured on the Llama-3-8B shapes (TFLOP/s, forward / dgrad / wgrad of
+// 4096x28672x4096): ring 4 waves 1290 / 1334 / 1300; 64-deep 32x32x16 4 waves 1378 / 1393 / 1358; 64-deep
+// 16x16x32 4 waves 1490 / 1538 / 1484, 8 waves 1432 / 1502 / 1411.  The narrow tiles (ring only) were measured
+// best as listed.
 constexpr TileCfg kCfgs[] = {
-    {256, 256, 8, 1.00f, false}, {256, 192, 4, 0.92f, false}, {192, 256, 4, 0.92f, false}, {256, 128, 4, 0.85f, false},
-    {128, 256, 8, 0.85f, false}, {256, 256, 4, 1.02f, false}, {256, 256, 4, 1.01f, true},   {256, 256, 8, 1.00f, true},
+    {256, 256, 8, 1.00f, 0}, {256, 192, 4, 0.92f, 0}, {192, 256, 4, 0.92f, 0},  {256, 128, 4, 0.85f, 0},
+    {128, 256, 8, 0.85f, 0}, {256, 256, 4, 1.02f, 0}, {256, 256, 4, 1.08f, 32}, {256, 256, 8, 1.06f, 32},
+    {256, 256, 4, 1.16f, 16}, {256, 256, 8, 1.12f, 16},
 };
 constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
 
@@ -1414,9 +1478,9 @@ int launch_cfg(const GemmArgs& a, hipStream_t s) {
     const int span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
     const int bn_span = (EPI == MTP_EPI_SWIGLU) ? BN / 2 : BN;
     const int tiles_n = (span + bn_span - 1) / bn_span;
-    if constexpr (kCfgs[C].q)
-      hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16>), dim3((unsigned)(tiles_m * tiles_n)), dim3(NW * 64),
-                         0, s, a);
+    if constexpr (kCfgs[C].q != 0)
+      hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16, (kCfgs[C].q ? kCfgs[C].q : 32)>),
+                         dim3((unsigned)(tiles_m * tiles_n)), dim3(NW * 64), 0, s, a);
     else
       hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, NW, F16>), dim3((unsigned)(tiles_m * tiles_n)),
                          dim3(NW * 64), 0, s, a);
@@ -1442,6 +1506,8 @@ int launch_typed(GemmArgs a, hipStream_t s) {
     case 5: return launch_cfg<5, ALAY, BLAY, EPI, OUT, F16>(a, s);
     case 6: return launch_cfg<6, ALAY, BLAY, EPI, OUT, F16>(a, s);
     case 7: return launch_cfg<7, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 8: return launch_cfg<8, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 9: return launch_cfg<9, ALAY, BLAY, EPI, OUT, F16>(a, s);
   }
   return MTP_EINVAL;
 }

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTP_ABI_VERSION 6
+#define MTP_ABI_VERSION 7
 
 /* element types.  MTP_F16 is IEEE half, what the reference's --fp16 sets as
  * params_dtype (Merak/merak_args/args.py:584-585). */
@@ -92,6 +92,33 @@ int mtp_linear_dgrad(const void* dy, const void* w, void* dx,
 int mtp_linear_wgrad(const void* dy, const void* x, void* dw, void* db,
                      int64_t M, int64_t N, int64_t K,
                      int dtype, int dw_dtype, int accumulate, void* stream);
+
+/* The three products above with device scratch.  On the 16-bit path a product
+ * whose 256x256 tiling would leave much of the last round of workgroups idle
+ * (few tiles with a long reduction: one rank's narrow shard of a wide layer)
+ * is cut "stream-K" fashion: the k range of the tiles of that round is dealt
+ * evenly to all compute units, the parts of a tile shared by several workgroups
+ * meet in the scratch and a second small kernel adds them up in k order and
+ * writes the tile, so results are reproducible bit for bit from run to run
+ * (they may differ in the last bit from the call without scratch, which sums
+ * each tile in one piece).
+ * workspace: 16-byte aligned, mtp_linear_workspace_bytes() bytes (about 138 MB,
+ * shape independent); its contents on entry do not matter.  Launches that
+ * share a workspace must not overlap (one workspace per stream).  NULL or too small:
+ * exactly the call without scratch.  The reference has no counterpart (its
+ * F.linear at layers.py:252,354 leaves such choices to the BLAS library). */
+int64_t mtp_linear_workspace_bytes(void);
+int mtp_linear_fwd_ws(const void* x, const void* w, const void* bias,
+                      void* y, void* act, void* workspace, int64_t workspace_bytes,
+                      int64_t M, int64_t N, int64_t K,
+                      int dtype, int epilogue, void* stream);
+int mtp_linear_dgrad_ws(const void* dy, const void* w, void* dx,
+                        void* workspace, int64_t workspace_bytes,
+                        int64_t M, int64_t N, int64_t K, int dtype, void* stream);
+int mtp_linear_wgrad_ws(const void* dy, const void* x, void* dw, void* db,
+                        void* workspace, int64_t workspace_bytes,
+                        int64_t M, int64_t N, int64_t K,
+                        int dtype, int dw_dtype, int accumulate, void* stream);
 
 /* Backward of the fused activations: given dACT and the saved
  * pre-activation Y, writes dY.

@@ -10,13 +10,13 @@
 #define FWD_NAME mtp_gemm_bf16_nt
 #define FWD_LAUNCH(EPI) launch_typed<LAY_ROW, LAY_ROW, EPI, OUT_BF16, false>(a, s)
 int mtp_gemm_f16_nt_impl(const void* A, const void* B, const void* bias, void* C, void* C2, int64_t M, int64_t N,
-                         int64_t K, int epilogue, int f16, hipStream_t s);
+                         int64_t K, int epilogue, int f16, void* ws, hipStream_t s);
 #endif
 
 int FWD_NAME(const void* A, const void* B, const void* bias, void* C, void* C2, int64_t M, int64_t N,
-             int64_t K, int epilogue, int f16, hipStream_t s) {
+             int64_t K, int epilogue, int f16, void* ws, hipStream_t s) {
 #ifndef MTP_FWD_F16
-  if (f16) return mtp_gemm_f16_nt_impl(A, B, bias, C, C2, M, N, K, epilogue, f16, s);
+  if (f16) return mtp_gemm_f16_nt_impl(A, B, bias, C, C2, M, N, K, epilogue, f16, ws, s);
 #endif
   GemmArgs a{};
   a.A = (const uint16_t*)A;
@@ -31,6 +31,7 @@ int FWD_NAME(const void* A, const void* B, const void* bias, void* C, void* C2, 
   a.ldb = K;
   a.ldc = N;
   a.accumulate = 0;
+  a.ws = ws;
   a.half = (int)(N / 2);
   a.ldc2 = (epilogue == MTP_EPI_SWIGLU) ? N / 2 : N;
   switch (epilogue) {

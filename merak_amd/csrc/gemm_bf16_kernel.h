@@ -60,6 +60,11 @@ struct GemmArgs {
   int64_t lda, ldb, ldc, ldc2;
   int accumulate;      // C += result
   int half;            // SwiGLU: number of gate columns (N/2)
+  // Stream-K (64-deep loop, 16x16x32, 4 waves only; sk_wgs == 0: every tile is one workgroup).  The tiles at
+  // positions [0, sk_full) are one workgroup each; the k-tiles of the others, taken as one sequence tile after
+  // tile, are dealt to sk_wgs further workgroups in runs of sk_ipw.  ws: device scratch, see SkLayout.
+  int sk_full, sk_wgs, sk_ipw;
+  void* ws;
 #ifdef MTP_MEASURE
   int debug;           // measurement builds only (MTP_GEMM_DEBUG): 1 = every tile loads tile (0,0), 2 = no epilogue
                        // stores, 4 = every DMA reads out of range (no memory traffic).  Results are wrong with any bit set.
@@ -125,6 +130,15 @@ __device__ __forceinline__ void dma16(rsrc_t rsrc, uint32_t lds_addr, uint32_t v
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
                : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff));
+}
+// The same with the LDS address given as a scalar base plus a compile-time offset: the many destinations of an
+// unrolled loop then cost one live scalar register instead of one each (s_add_u32 leaves its carry in SCC).
+template <int OFFSET>
+__device__ __forceinline__ void dma16_at(rsrc_t rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+  asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff), "n"(OFFSET)
+               : "scc");
 }
 // Register-staged loads, also inline assembly so that their order against the DMA-style waits stays in this
 // file's hands: 64 lanes x 16 bytes from the buffer into four VGPRs ...
@@ -707,12 +721,15 @@ struct RowOperandQ {
     uint32_t soff;
     bool dead;
   };
-  __device__ __forceinline__ Prep prep(int kt) const {
-    return Prep{(uint32_t)(kt * QBK * 2), kt * QBK + gchunk * 8 >= K};  // chunk at or past the end of k: zero fill
+  // kend: first k-tile past the range this workgroup multiplies (requests beyond it are zero fill)
+  __device__ __forceinline__ Prep prep(int kt, int kend) const {
+    return Prep{(uint32_t)(kt * QBK * 2), kt >= kend || kt * QBK + gchunk * 8 >= K};  // chunk at or past the end of k
   }
-  // j-th DMA instruction of this wave for unit u; unit_lds = LDS byte address of the unit
-  __device__ __forceinline__ void issue(const Prep& pp, uint32_t unit_lds, int wave, int u, int j) const {
-    dma16(rsrc, unit_lds + (wave + NW * j) * 1024, pp.dead ? 0x80000000u : voff[u][j], pp.soff);
+  // J-th DMA instruction of this wave for unit U, which sits UNIT_OFF bytes into the tile buffers;
+  // wave_lds = LDS byte address of the tile buffers + 1024 * wave
+  template <int UNIT_OFF, int U, int J>
+  __device__ __forceinline__ void issue(const Prep& pp, uint32_t wave_lds) const {
+    dma16_at<UNIT_OFF + NW * J * 1024>(rsrc, wave_lds, pp.dead ? 0x80000000u : voff[U][J], pp.soff);
   }
   // unit: address of the unit in k-tile buffer 0
   __device__ __forceinline__ bf16x8_t frag(const char* unit, int buf, int b, int kk) const {
@@ -771,12 +788,13 @@ struct ColOperandQ {
   struct Prep {
     rsrc_t r;
   };
-  __device__ __forceinline__ Prep prep(int kt) const {
+  __device__ __forceinline__ Prep prep(int kt, int kend) const {
     // the whole address goes through the range check: k-rows past K read as zero
-    return Prep{make_rsrc(base + kt * ktile_bytes, total - kt * ktile_bytes)};
+    return Prep{make_rsrc(base + kt * ktile_bytes, kt >= kend ? 0 : total - kt * ktile_bytes)};
   }
-  __device__ __forceinline__ void issue(const Prep& pp, uint32_t unit_lds, int wave, int u, int j) const {
-    dma16(pp.r, unit_lds + (wave + NW * j) * 1024, voff[u][j], 0);
+  template <int UNIT_OFF, int U, int J>
+  __device__ __forceinline__ void issue(const Prep& pp, uint32_t wave_lds) const {
+    dma16_at<UNIT_OFF + NW * J * 1024>(pp.r, wave_lds, voff[U][J], 0);
   }
   __device__ __forceinline__ bf16x8_t frag(const char* unit, int buf, int b, int kk) const {
     const char* a = unit + moff[buf][b] + kk * ((QBK / QKS) * UROWS * 2);
@@ -797,10 +815,26 @@ struct IntList {
   static constexpr int v[sizeof...(V)] = {V...};
 };
 
-template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK>
+// Stream-K scratch: two slots per stream workgroup; a slot holds one workgroup's accumulators of a tile whose k
+// range it shares with others: 64 x 16 bytes per lane, lane-interleaved (vector v of thread t at byte
+// (v * 256 + t) * 16), + the row sums of EPI_ROWSUM in vectors 64 and 65.  A workgroup's first slot takes the piece
+// that begins its run of k-tiles, the second the piece that ends it.  gemm_sk_reduce_kernel adds the pieces of
+// every shared tile up, in k order, and writes the tile.
+constexpr int SK_MAX_WGS = 256;
+constexpr int SK_SLOT_VECS = 66;                              // 16-byte vectors per lane and slot
+constexpr int64_t SK_SLOT_BYTES = (int64_t)SK_SLOT_VECS * 256 * 16;
+constexpr int64_t SK_WORKSPACE_BYTES = 2 * SK_MAX_WGS * SK_SLOT_BYTES;
+static_assert(SK_WORKSPACE_BYTES == 2ll * 256 * 66 * 256 * 16, "linear.hip states the same size");
+// slot of the piece of shared tile r (k-tiles [r KT, (r + 1) KT) of the stream) that workgroup w multiplied
+__device__ __forceinline__ int64_t sk_slot_of(int w, int r, int KT, int ipw) {
+  return (int64_t)(2 * w + (w * ipw < r * KT ? 1 : 0)) * SK_SLOT_BYTES;
+}
+
+template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK, bool SK>
 __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
   using X = X16<F16>;
   constexpr int BM = 256, BN = 256;
+  static_assert(!SK || (BLK == 16 && NW == 4), "stream-K is built for the 4-wave 16x16x32 form");
   static_assert(EPI != MTP_EPI_SWIGLU || BLAY == LAY_ROW, "the SwiGLU row interleave is a forward (row B) feature");
   static_assert(NW == 4 || NW == 8, "4 waves (2x2) or 8 waves (2x4) per workgroup");
   constexpr int WGM = 2, WGN = NW / 2;
@@ -817,7 +851,8 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
   constexpr int LDS_BYTES = 2 * QBUF;
   __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
 
-  const int tid = threadIdx.x, lane = tid & 63;
+  const int tid = threadIdx.x;
+  int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
 
@@ -825,8 +860,36 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
   const int n_span = (EPI == MTP_EPI_SWIGLU) ? p.half : p.N;  // SwiGLU tiles cover BN/2 gate + BN/2 up columns
   constexpr int BN_SPAN = (EPI == MTP_EPI_SWIGLU) ? BN / 2 : BN;
   const int tiles_n = (n_span + BN_SPAN - 1) / BN_SPAN;
+  const int KT = (p.K + QBK - 1) / QBK;
+  // This workgroup's run of k-tiles in the sequence "all k-tiles of tile position 0, of position 1, ...": one whole
+  // tile, or (stream-K) sk_ipw k-tiles that may end one tile and begin the next.
+  int it = blockIdx.x * KT, it_end = it + KT;
+  [[maybe_unused]] int sk_w = -1;
+  if constexpr (SK) {
+    if ((int)blockIdx.x >= p.sk_full) {
+      sk_w = blockIdx.x - p.sk_full;
+      it = p.sk_full * KT + sk_w * p.sk_ipw;
+      const int all = tiles_m * tiles_n * KT;
+      it_end = it + p.sk_ipw < all ? it + p.sk_ipw : all;
+    }
+  }
+  // where this wave's DMA instructions put their first KiB
+  const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_addr_of(lds)) + wave * 1024;
+  // byte offsets of the units inside lds
+  auto unit_a = [](int buf, int u) constexpr { return buf * QBUF + u * AOp::UBYTES; };
+  auto unit_b = [](int buf, int u) constexpr { return buf * QBUF + AOp::BYTES + u * BOp::UBYTES; };
+
+ do {
+  // One piece (for all but stream-K workgroups the only one).  Everything a lane derives from its number is
+  // derived again per piece: hoisted out of this loop it would stay live through the main loop, where every
+  // register is taken, and come back from scratch memory on the critical path of the next piece's first requests.
+  if constexpr (SK) asm volatile("" : "+v"(lane));
+  const int pos = it / KT;                         // tile position
+  const int k0 = it - pos * KT;                    // first k-tile of this piece
+  const int k1 = it_end - pos * KT < KT ? it_end - pos * KT : KT;   // one past its last
+  it += k1 - k0;
   int tm, tn;
-  tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  tile_of(pos, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM;
   const int n0 = tn * BN_SPAN;
   const int lm0 = MTP_DBG(p, 1) ? 0 : MTP_DBG(p, 8) ? (tm & 1) * BM : m0;
@@ -861,11 +924,6 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
     }
   }
 #endif
-
-  const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr_of(lds));
-  // byte offsets of the units inside lds
-  auto unit_a = [](int buf, int u) constexpr { return buf * QBUF + u * AOp::UBYTES; };
-  auto unit_b = [](int buf, int u) constexpr { return buf * QBUF + AOp::BYTES + u * BOp::UBYTES; };
 
   AccT acc[TI][TJ];
 #pragma unroll
@@ -940,13 +998,13 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
     constexpr int UA = decltype(ua_tag)::value, UB = decltype(ub_tag)::value, BUF = decltype(buf_tag)::value;
     constexpr int d = decltype(d_tag)::value;
     if constexpr ((d & 1) == 0)
-      opA.issue(pa, lds0 + unit_a(BUF, UA), wave, UA, d >> 1);
+      opA.template issue<unit_a(BUF, UA), UA, (d >> 1)>(pa, lds_wave);
     else
-      opB.issue(pb, lds0 + unit_b(BUF, UB), wave, UB, d >> 1);
+      opB.template issue<unit_b(BUF, UB), UB, (d >> 1)>(pb, lds_wave);
   };
   auto dma_group = [&](int kt, auto ua_tag, auto ub_tag, auto buf_tag) {
-    const auto pa = opA.prep(kt);
-    const auto pb = opB.prep(kt);
+    const auto pa = opA.prep(kt, k1);
+    const auto pb = opB.prep(kt, k1);
     static_for<NDH>([&](auto d) { dma_q(pa, pb, ua_tag, ub_tag, buf_tag, d); });
   };
 
@@ -957,8 +1015,8 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
   // issued well before the barrier (which hands the units over) and has about half a phase to land.
   auto half_tile = [&](int kt_dma, auto desc) {
     using D = decltype(desc);
-    const auto pa = opA.prep(kt_dma);
-    const auto pb = opB.prep(kt_dma);
+    const auto pa = opA.prep(kt_dma, k1);
+    const auto pb = opB.prep(kt_dma, k1);
     __builtin_amdgcn_sched_barrier(0);
     static_for<HT>([&](auto g_tag) {
       constexpr int g = decltype(g_tag)::value;
@@ -995,30 +1053,29 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
   using OddH0 = IntList<0, 1, 0, 0, /**/ 0, 0, 1, /**/ 1, 1, 1, /**/ 0, 1, 1>;   // Q01 Q00; reads B0[t] A1[t]
   using OddH1 = IntList<1, 0, 1, 1, /**/ 1, 0, 0, /**/ 0, 0, 0, /**/ 1, 0, 1>;   // Q10 Q11; reads A0[t+1] B0[t+1]
 
-  const int KT = (p.K + QBK - 1) / QBK;
   {
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     // the four request groups in front of the loop, in the order the loop would have issued them
-    dma_group(0, I0{}, I0{}, I0{});   // A0[0] B0[0]
-    dma_group(0, I1{}, I1{}, I0{});   // A1[0] B1[0]
-    dma_group(1, I0{}, I1{}, I1{});   // A0[1] B1[1]
-    dma_group(1, I1{}, I0{}, I1{});   // A1[1] B0[1]
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NDH) : "memory");   // all of k-tile 0
+    dma_group(k0, I0{}, I0{}, I0{});       // A0[0] B0[0]
+    dma_group(k0, I1{}, I1{}, I0{});       // A1[0] B1[0]
+    dma_group(k0 + 1, I0{}, I1{}, I1{});   // A0[1] B1[1]
+    dma_group(k0 + 1, I1{}, I0{}, I1{});   // A1[1] B0[1]
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NDH) : "memory");   // all of the first k-tile
     __syncthreads();
     static_for<HI * QKS>([&](auto f) { read_q(I1{}, I0{}, I0{}, f); });
     static_for<HJ * QKS>([&](auto f) { read_q(I0{}, I0{}, I0{}, f); });
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __syncthreads();   // everyone holds A0[0], B0[0]: the loop's first requests may overwrite them
   }
-  int kt = 0;
-  for (; kt + 1 < KT; kt += 2) {
+  int kt = k0;
+  for (; kt + 1 < k1; kt += 2) {
     half_tile(kt + 2, EvenH0{});
     half_tile(kt + 2, EvenH1{});
     half_tile(kt + 3, OddH0{});
     half_tile(kt + 3, OddH1{});
   }
-  if (kt < KT) {
+  if (kt < k1) {
     half_tile(kt + 2, EvenH0{});
     half_tile(kt + 2, EvenH1{});
   }
@@ -1027,13 +1084,37 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
   if constexpr (BLK == 16) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   __syncthreads();  // the epilogue reuses the tile buffers
   if (MTP_DBG(p, 2)) return;
-  gemm_epilogue<BM, BN, EPI, OUT, NW, F16, true, LDS_BYTES, TI32, TJ32, BLK>(
-      p,
-      [&](int i, int j, int g, int e) -> float {
-        if constexpr (BLK == 32) return acc[i][j][4 * g + e];
-        else return acc[2 * i + (g >> 1)][2 * j + (g & 1)][e];
-      },
-      [&](int i, int g) -> float { return BLK == 32 ? rsum[i] : rsum[2 * i + (g >> 1)]; }, lds, m0, n0, tn, wave, lane);
+
+  auto write_tile = [&]() {
+    gemm_epilogue<BM, BN, EPI, OUT, NW, F16, true, LDS_BYTES, TI32, TJ32, BLK>(
+        p,
+        [&](int i, int j, int g, int e) -> float {
+          if constexpr (BLK == 32) return acc[i][j][4 * g + e];
+          else return acc[2 * i + (g >> 1)][2 * j + (g & 1)][e];
+        },
+        [&](int i, int g) -> float { return BLK == 32 ? rsum[i] : rsum[2 * i + (g >> 1)]; }, lds, m0, n0, tn, wave, lane);
+  };
+  if constexpr (!SK) {
+    write_tile();
+  } else {
+    if (k0 == 0 && k1 == KT) {
+      write_tile();
+    } else {
+      // part of a tile whose k range is shared: the accumulators go to this workgroup's slot as they are
+      char* q = static_cast<char*>(p.ws) + sk_slot_of(sk_w, pos - p.sk_full, KT, p.sk_ipw) + tid * 16;
+      constexpr int NT = NW * 64;
+#pragma unroll
+      for (int i = 0; i < TI; i++)
+#pragma unroll
+        for (int j = 0; j < TJ; j++) *reinterpret_cast<f32x4_t*>(q + (i * TJ + j) * (NT * 16)) = acc[i][j];
+      if constexpr (EPI == EPI_ROWSUM) {
+        *reinterpret_cast<f32x4_t*>(q + 64 * (NT * 16)) = f32x4_t{rsum[0], rsum[1], rsum[2], rsum[3]};
+        *reinterpret_cast<f32x4_t*>(q + 65 * (NT * 16)) = f32x4_t{rsum[4], rsum[5], rsum[6], rsum[7]};
+      }
+    }
+  }
+  if (SK && it < it_end) __syncthreads();   // the next piece's requests overwrite what the epilogue staged in LDS
+ } while (SK && it < it_end);
 }
 
 // The body lives in a __device__ function: it uses inline assembly operands that the host pass over a
@@ -1400,9 +1481,140 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs p) {
   gemm_bf16_body<BM, BN, ALAY, BLAY, EPI, OUT, NW, F16>(p);
 }
 
-template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK>
+template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK, bool SK>
 __global__ __launch_bounds__(NW * 64) void gemm_q_kernel(const GemmArgs p) {
-  gemm_q_body<ALAY, BLAY, EPI, OUT, NW, F16, BLK>(p);
+  gemm_q_body<ALAY, BLAY, EPI, OUT, NW, F16, BLK, SK>(p);
+}
+
+// Second pass of stream-K: one workgroup per (shared tile, row of 16x16 blocks) adds that row's pieces up in k
+// order and does what the GEMM's epilogue does for a whole tile, on the 8 vectors (16 rows x 128 columns of the
+// wave's part) each of its lanes holds; grid.y == 8 is the bias-gradient row (EPI_ROWSUM).  Thread t here stands
+// for thread t of the GEMM workgroup: same wave, same lane, same blocks.
+template <int EPI, int OUT, bool F16>
+__global__ __launch_bounds__(256) void gemm_sk_reduce_kernel(const GemmArgs p) {
+  using X = X16<F16>;
+  constexpr int BM = 256, BN = 256, TI = 8, TJ = 8, HI = 4, HJ = 4;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  const int KT = (p.K + QBK - 1) / QBK;
+  const int tiles_m = (p.M + BM - 1) / BM;
+  const int n_span = (EPI == MTP_EPI_SWIGLU) ? p.half : p.N;
+  constexpr int BN_SPAN = (EPI == MTP_EPI_SWIGLU) ? BN / 2 : BN;
+  const int tiles_n = (n_span + BN_SPAN - 1) / BN_SPAN;
+  const int r = blockIdx.x;
+  int tm, tn;
+  tile_of(p.sk_full + r, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN_SPAN;
+  const int w_first = r * KT / p.sk_ipw;
+  const int pieces = ((r + 1) * KT - 1) / p.sk_ipw - w_first + 1;
+  if (pieces == 1) return;   // one workgroup had the whole tile and wrote it
+  const char* ws = static_cast<const char*>(p.ws) + tid * 16;
+  const int i = blockIdx.y;
+  if (i == TI) {
+    if constexpr (EPI == EPI_ROWSUM) {
+      if (tn != 0 || wn != 0) return;
+      f32x4_t a = {0.f, 0.f, 0.f, 0.f}, b = a;
+      for (int pc = 0; pc < pieces; pc++) {
+        const char* q = ws + sk_slot_of(w_first + pc, r, KT, p.sk_ipw);
+        const f32x4_t va = *reinterpret_cast<const f32x4_t*>(q + 64 * 4096), vb = *reinterpret_cast<const f32x4_t*>(q + 65 * 4096);
+        a = pc == 0 ? va : a + va;
+        b = pc == 0 ? vb : b + vb;
+      }
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        float t = e < 4 ? a[e & 3] : b[e & 3];   // lanes holding the same row at other k add up
+        t += __shfl_xor(t, 32, 64);
+        t += __shfl_xor(t, 16, 64);
+        const int row = m0 + (e / HI) * (BM / 2) + wm * (16 * HI) + (e % HI) * 16 + (lane & 15);
+        if (lane < 16 && row < p.M) {
+          if (OUT == OUT_F32) {
+            float* q = (float*)p.rowsum + row;
+            *q = p.accumulate ? *q + t : t;
+          } else {
+            uint16_t* q = (uint16_t*)p.rowsum + row;
+            *q = X::to_bits(p.accumulate ? X::from_bits(*q) + t : t);
+          }
+        }
+      }
+    }
+    return;
+  }
+  f32x4_t v[TJ];
+  for (int pc = 0; pc < pieces; pc++) {
+    const char* q = ws + sk_slot_of(w_first + pc, r, KT, p.sk_ipw) + (int64_t)i * TJ * 4096;
+#pragma unroll
+    for (int j = 0; j < TJ; j++) {
+      const f32x4_t t = *reinterpret_cast<const f32x4_t*>(q + j * 4096);
+      v[j] = pc == 0 ? t : v[j] + t;
+    }
+  }
+  const int row = m0 + (i / HI) * (BM / 2) + wm * (16 * HI) + (i % HI) * 16 + (lane & 15);
+  if (row >= p.M) return;
+  // first column of block j, and one past the last valid column for it (as in gemm_epilogue)
+  auto col_of = [&](int j) -> int {
+    if (EPI == MTP_EPI_SWIGLU) return (j < HJ ? 0 : p.half) + n0 + wn * (16 * HJ) + (j % HJ) * 16 + 4 * (lane >> 4);
+    return n0 + (j / HJ) * (BN / 2) + wn * (16 * HJ) + (j % HJ) * 16 + 4 * (lane >> 4);
+  };
+  auto lim_of = [&](int j) -> int { return (EPI == MTP_EPI_SWIGLU && j < HJ) ? p.half : p.N; };
+  float pre[TJ][4];
+#pragma unroll
+  for (int j = 0; j < TJ; j++) {
+    const int col = col_of(j), lim = lim_of(j);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      float bv = 0.f;
+      if (EPI == MTP_EPI_BIAS || EPI == MTP_EPI_BIAS_GELU || EPI == MTP_EPI_SWIGLU)
+        if (p.bias && col + e < lim) bv = X::from_bits(p.bias[col + e]);
+      pre[j][e] = v[j][e] + bv;
+    }
+  }
+  if (OUT == OUT_F32) {
+    if (p.C) {
+#pragma unroll
+      for (int j = 0; j < TJ; j++) {
+        const int col = col_of(j), lim = lim_of(j);
+        float* q = (float*)p.C + (int64_t)row * p.ldc + col;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (col + e < lim) q[e] = p.accumulate ? q[e] + pre[j][e] : pre[j][e];
+      }
+    }
+    return;
+  }
+  // 16-bit outputs: round once; an activation sees the rounded value, as the unfused layers would
+#pragma unroll
+  for (int j = 0; j < TJ; j++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) pre[j][e] = X::from_bits(X::to_bits(pre[j][e]));
+  if (p.C) {
+#pragma unroll
+    for (int j = 0; j < TJ; j++) {
+      const int col = col_of(j), lim = lim_of(j);
+      uint16_t* q = (uint16_t*)p.C + (int64_t)row * p.ldc + col;
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        if (col + e < lim) q[e] = X::to_bits(p.accumulate ? X::from_bits(q[e]) + pre[j][e] : pre[j][e]);
+    }
+  }
+  if constexpr (EPI == MTP_EPI_BIAS_GELU || EPI == MTP_EPI_GELU) {
+#pragma unroll
+    for (int j = 0; j < TJ; j++) {
+      const int col = col_of(j), lim = lim_of(j);
+      uint16_t* q = (uint16_t*)p.C2 + (int64_t)row * p.ldc2 + col;
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        if (col + e < lim) q[e] = X::to_bits(gelu_new_f(pre[j][e]));
+    }
+  }
+  if constexpr (EPI == MTP_EPI_SWIGLU) {
+#pragma unroll
+    for (int j = 0; j < HJ; j++) {
+      const int col = n0 + wn * (16 * HJ) + j * 16 + 4 * (lane >> 4);
+      uint16_t* q = (uint16_t*)p.C2 + (int64_t)row * p.ldc2 + col;
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        if (col + e < p.half) q[e] = X::to_bits(silu_f(pre[j][e]) * pre[j + HJ][e]);
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -1467,6 +1679,38 @@ int pick_config(const GemmArgs& a) {
   return best;
 }
 
+// Stream-K for a 256x256 tiling that leaves most compute units without a tile: the k-tiles of all tiles, taken as
+// one sequence, are dealt evenly to (up to) 256 workgroups; tiles that several workgroups share go through the
+// scratch and gemm_sk_reduce_kernel.  Measured (Llama-70B tp=8 shard, 8192 tokens): 128 tiles with 128 k-tiles
+// each (o-proj dgrad / wgrad) 138 -> 125 us.  It does not pay where at least 160 of the 256 compute units have a
+// tile, nor behind full rounds: the chip runs against its power limit, so the compute units that still work in a
+// part-empty round run at a higher clock and the round costs much less than its tile count suggests (160 tiles
+// with 128 k-tiles: 147 us as they are, 166 us dealt out; 3.5 rounds of 64 k-tiles: 344 against 355 us), while
+// the hand-over costs about 40 us per 128 shared tiles.  MTP_GEMM_SK = 0 switches it off, 1 takes it whenever
+// the last round is part empty, 2 runs every tile as one workgroup through the stream-K kernel.
+inline bool plan_stream_k(GemmArgs& a, int tiles, int KT) {
+  static MtpTune tune_sk("MTP_GEMM_SK");
+  a.sk_wgs = 0;
+  const int force = tune_sk.get(-1);
+  if (!a.ws || force == 0) return false;
+  if (force == 2) {
+    a.sk_full = tiles;
+    a.sk_ipw = KT;
+    return true;
+  }
+  const int R = tiles % SK_MAX_WGS;
+  if (R == 0 || KT < 2 || (int64_t)tiles * KT >= (1ll << 31)) return false;
+  if (force != 1 && !(tiles <= SK_MAX_WGS / 2 && KT >= 32)) return false;
+  // at most about five pieces per tile, at least four k-tiles per piece (one where the whole k is shorter)
+  int ipw = (R * KT + SK_MAX_WGS - 1) / SK_MAX_WGS;
+  if (ipw < KT / 4) ipw = KT / 4;
+  if (ipw < 4) ipw = KT < 4 ? KT : 4;
+  a.sk_full = tiles - R;
+  a.sk_ipw = ipw;
+  a.sk_wgs = (R * KT + ipw - 1) / ipw;
+  return a.sk_wgs <= SK_MAX_WGS;
+}
+
 template <int C, int ALAY, int BLAY, int EPI, int OUT, bool F16>
 int launch_cfg(const GemmArgs& a, hipStream_t s) {
   if constexpr (!cfg_valid<EPI>(C)) {
@@ -1478,8 +1722,23 @@ int launch_cfg(const GemmArgs& a, hipStream_t s) {
     const int span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
     const int bn_span = (EPI == MTP_EPI_SWIGLU) ? BN / 2 : BN;
     const int tiles_n = (span + bn_span - 1) / bn_span;
+    if constexpr (kCfgs[C].q == 16 && NW == 4) {
+      GemmArgs b = a;
+      if (plan_stream_k(b, tiles_m * tiles_n, (a.K + QBK - 1) / QBK)) {
+        hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16, 16, true>), dim3((unsigned)(b.sk_full + b.sk_wgs)),
+                           dim3(NW * 64), 0, s, b);
+        MTP_CHECK_LAUNCH("gemm_bf16");
+        if (b.sk_wgs > 0) {
+          const int shared = tiles_m * tiles_n - b.sk_full;
+          hipLaunchKernelGGL((gemm_sk_reduce_kernel<EPI, OUT, F16>), dim3((unsigned)shared, EPI == EPI_ROWSUM ? 9u : 8u),
+                             dim3(256), 0, s, b);
+          MTP_CHECK_LAUNCH("gemm_bf16 stream-K reduce");
+        }
+        return MTP_OK;
+      }
+    }
     if constexpr (kCfgs[C].q != 0)
-      hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16, (kCfgs[C].q ? kCfgs[C].q : 32)>),
+      hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16, (kCfgs[C].q ? kCfgs[C].q : 32), false>),
                          dim3((unsigned)(tiles_m * tiles_n)), dim3(NW * 64), 0, s, a);
     else
       hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, NW, F16>), dim3((unsigned)(tiles_m * tiles_n)),

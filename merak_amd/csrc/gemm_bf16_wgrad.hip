@@ -3,7 +3,7 @@
 
 // db (may be null): the bias gradient sum_m dY[m, :], in dw's dtype, produced by the same launch
 int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
-                        int dw_dtype, int accumulate, int f16, hipStream_t s) {
+                        int dw_dtype, int accumulate, int f16, void* ws, hipStream_t s) {
   GemmArgs a{};
   a.A = (const uint16_t*)dy;
   a.B = (const uint16_t*)x;
@@ -16,6 +16,7 @@ int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64
   a.ldc = K;
   a.accumulate = accumulate;
   a.rowsum = db;
+  a.ws = ws;
   if (db) {
     if (dw_dtype == MTP_F32) return launch<LAY_COL, LAY_COL, EPI_ROWSUM, OUT_F32>(a, s, f16);
     return launch<LAY_COL, LAY_COL, EPI_ROWSUM, OUT_BF16>(a, s, f16);

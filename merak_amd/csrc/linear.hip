@@ -4,12 +4,15 @@
 #include "mtp_common.h"
 
 // f16 != 0: the 16-bit tensors are IEEE half instead of bf16 (same kernel, other MFMA and conversions)
+// ws: stream-K scratch of MTP_LINEAR_WS_BYTES bytes, or null (every tile is then one workgroup)
 int mtp_gemm_bf16_nt(const void* A, const void* B, const void* bias, void* C, void* C2, int64_t M, int64_t N,
-                     int64_t K, int epilogue, int f16, hipStream_t s);
-int mtp_gemm_bf16_dgrad(const void* dy, const void* w, void* dx, int64_t M, int64_t N, int64_t K, int f16,
+                     int64_t K, int epilogue, int f16, void* ws, hipStream_t s);
+int mtp_gemm_bf16_dgrad(const void* dy, const void* w, void* dx, int64_t M, int64_t N, int64_t K, int f16, void* ws,
                         hipStream_t s);
 int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
-                        int dw_dtype, int accumulate, int f16, hipStream_t s);
+                        int dw_dtype, int accumulate, int f16, void* ws, hipStream_t s);
+// = SK_WORKSPACE_BYTES of gemm_bf16_kernel.h (checked there): 2 slots for each of 256 workgroups
+#define MTP_LINEAR_WS_BYTES (2ll * 256 * 66 * 256 * 16)
 int mtp_gemm_generic(const void* A, int64_t sam, int64_t sak, const void* B, int64_t sbn, int64_t sbk,
                      const void* bias, void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, int out_dtype,
                      int accumulate, hipStream_t s);
@@ -22,6 +25,9 @@ int mtp_act_fwd(const void* y, void* act, int64_t M, int64_t N, int dtype, int s
 namespace {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// the scratch is used only when it is large enough and aligned; otherwise the call runs as without one
+void* usable_ws(void* ws, int64_t bytes) { return (ws && bytes >= MTP_LINEAR_WS_BYTES && aligned16(ws)) ? ws : nullptr; }
 
 int check_dims(const char* what, int64_t M, int64_t N, int64_t K, int dtype) {
   MTP_REQUIRE(M >= 0 && N >= 1 && K >= 1, MTP_EINVAL, "%s: M=%lld N=%lld K=%lld", what, (long long)M, (long long)N,
@@ -47,8 +53,16 @@ bool f32_fast_ok(const void* a, const void* b, int64_t d0, int64_t d1, int64_t b
 
 }  // namespace
 
+extern "C" int64_t mtp_linear_workspace_bytes(void) { return MTP_LINEAR_WS_BYTES; }
+
 extern "C" int mtp_linear_fwd(const void* x, const void* w, const void* bias, void* y, void* act, int64_t M,
                               int64_t N, int64_t K, int dtype, int epilogue, void* stream) {
+  return mtp_linear_fwd_ws(x, w, bias, y, act, nullptr, 0, M, N, K, dtype, epilogue, stream);
+}
+
+extern "C" int mtp_linear_fwd_ws(const void* x, const void* w, const void* bias, void* y, void* act, void* workspace,
+                                 int64_t workspace_bytes, int64_t M, int64_t N, int64_t K, int dtype, int epilogue,
+                                 void* stream) {
   int rc = check_dims("linear_fwd", M, N, K, dtype);
   if (rc) return rc;
   MTP_REQUIRE(epilogue >= MTP_EPI_NONE && epilogue <= MTP_EPI_GELU, MTP_EINVAL, "linear_fwd: unknown epilogue %d",
@@ -69,7 +83,7 @@ extern "C" int mtp_linear_fwd(const void* x, const void* w, const void* bias, vo
   if (is16 && fast_ok(K, K, x, w) && N * K * 2 < (1ll << 31)) {
     int epi = epilogue;
     if (epilogue == MTP_EPI_SWIGLU && !use_bias) use_bias = nullptr;
-    return mtp_gemm_bf16_nt(x, w, use_bias, y, act, M, N, K, epi, dtype == MTP_F16, s);
+    return mtp_gemm_bf16_nt(x, w, use_bias, y, act, M, N, K, epi, dtype == MTP_F16, usable_ws(workspace, workspace_bytes), s);
   }
   if (dtype == MTP_F32 && f32_fast_ok(x, w, K, K, 0, 0) && K * 4 * 128 < (1ll << 31)) {
     void* pre32 = y ? y : (epilogue != MTP_EPI_SWIGLU ? act : nullptr);
@@ -92,13 +106,18 @@ extern "C" int mtp_linear_fwd(const void* x, const void* w, const void* bias, vo
 
 extern "C" int mtp_linear_dgrad(const void* dy, const void* w, void* dx, int64_t M, int64_t N, int64_t K, int dtype,
                                 void* stream) {
+  return mtp_linear_dgrad_ws(dy, w, dx, nullptr, 0, M, N, K, dtype, stream);
+}
+
+extern "C" int mtp_linear_dgrad_ws(const void* dy, const void* w, void* dx, void* workspace, int64_t workspace_bytes,
+                                   int64_t M, int64_t N, int64_t K, int dtype, void* stream) {
   int rc = check_dims("linear_dgrad", M, N, K, dtype);
   if (rc) return rc;
   if (M == 0) return MTP_OK;
   MTP_REQUIRE(dy && w && dx, MTP_EINVAL, "linear_dgrad: null pointer");
   hipStream_t s = (hipStream_t)stream;
   if ((dtype == MTP_BF16 || dtype == MTP_F16) && fast_ok(N, K, dy, w) && aligned16(dx)) {
-    rc = mtp_gemm_bf16_dgrad(dy, w, dx, M, N, K, dtype == MTP_F16, s);
+    rc = mtp_gemm_bf16_dgrad(dy, w, dx, M, N, K, dtype == MTP_F16, usable_ws(workspace, workspace_bytes), s);
     if (rc != MTP_EUNSUPPORTED) return rc;
   }
   if (dtype == MTP_F32 && f32_fast_ok(dy, w, N, K, 0, N * K * 4) && N * 4 * 128 < (1ll << 31))
@@ -109,6 +128,12 @@ extern "C" int mtp_linear_dgrad(const void* dy, const void* w, void* dx, int64_t
 
 extern "C" int mtp_linear_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
                                 int dtype, int dw_dtype, int accumulate, void* stream) {
+  return mtp_linear_wgrad_ws(dy, x, dw, db, nullptr, 0, M, N, K, dtype, dw_dtype, accumulate, stream);
+}
+
+extern "C" int mtp_linear_wgrad_ws(const void* dy, const void* x, void* dw, void* db, void* workspace,
+                                   int64_t workspace_bytes, int64_t M, int64_t N, int64_t K, int dtype, int dw_dtype,
+                                   int accumulate, void* stream) {
   int rc = check_dims("linear_wgrad", M, N, K, dtype);
   if (rc) return rc;
   MTP_REQUIRE(dw_dtype == MTP_F32 || dw_dtype == dtype, MTP_EUNSUPPORTED,
@@ -117,7 +142,8 @@ extern "C" int mtp_linear_wgrad(const void* dy, const void* x, void* dw, void* d
   MTP_REQUIRE(M == 0 || (dy && x), MTP_EINVAL, "linear_wgrad: null input");
   hipStream_t s = (hipStream_t)stream;
   if ((dtype == MTP_BF16 || dtype == MTP_F16) && M > 0 && fast_ok(N, K, dy, x) && aligned16(dw)) {
-    rc = mtp_gemm_bf16_wgrad(dy, x, dw, db, M, N, K, dw_dtype, accumulate, dtype == MTP_F16, s);
+    rc = mtp_gemm_bf16_wgrad(dy, x, dw, db, M, N, K, dw_dtype, accumulate, dtype == MTP_F16,
+                             usable_ws(workspace, workspace_bytes), s);
     if (rc != MTP_EUNSUPPORTED) return rc;
   }
   if (dtype == MTP_F32 && dw_dtype == MTP_F32 && M > 0 && f32_fast_ok(dy, x, N, K, M * N * 4, M * K * 4)) {

@@ -62,6 +62,30 @@ def _contig(t: torch.Tensor) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------------- linear
+_linear_ws_cache = {}
+
+
+def linear_workspace(dev: torch.device) -> torch.Tensor:
+    """Scratch of the 16-bit linear products for the current stream of `dev` (stream-K: tiles whose k range
+    several workgroups share meet there).  One buffer per (device, stream), allocated at first use and kept:
+    launches on one stream are ordered, so they may share it."""
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    key = (idx, torch.cuda.current_stream(dev).cuda_stream)
+    ws = _linear_ws_cache.get(key)
+    if ws is None:
+        ws = torch.empty(_lib.lib().mtp_linear_workspace_bytes(), dtype=torch.uint8, device=dev)
+        _linear_ws_cache[key] = ws
+    return ws
+
+
+def _ws_args(t: torch.Tensor, dev: torch.device):
+    """(pointer, bytes) of the scratch for a product on tensors like t; fp32 products take none"""
+    if t.dtype == torch.float32:
+        return None, 0
+    ws = linear_workspace(dev)
+    return ws.data_ptr(), ws.numel()
+
+
 def linear_fwd(x2d: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], epilogue: int = EPI_NONE,
                want_pre: bool = True) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
     """(y, act) = epilogue(x2d @ w.T + bias).  x2d [M,K], w [N,K] contiguous, same dtype."""
@@ -85,13 +109,14 @@ def linear_fwd(x2d: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
     if has_act:
         act = torch.empty((M, N // 2 if epilogue == EPI_SWIGLU else N), dtype=x2d.dtype, device=dev)
     with torch.cuda.device(dev):
-        rc = _lib.lib().mtp_linear_fwd(_p(x2d), _p(w), _p(bias), _p(y), _p(act), M, N, K, _dt(x2d), epilogue,
-                                       _stream(dev))
+        wsp, wsb = _ws_args(x2d, dev)
+        rc = _lib.lib().mtp_linear_fwd_ws(_p(x2d), _p(w), _p(bias), _p(y), _p(act), wsp, wsb, M, N, K, _dt(x2d),
+                                          epilogue, _stream(dev))
         if rc == -2 and y is None:
             # shapes served by the general kernel need the pre-activation buffer for SwiGLU
             y = torch.empty((M, N), dtype=x2d.dtype, device=dev)
-            rc = _lib.lib().mtp_linear_fwd(_p(x2d), _p(w), _p(bias), _p(y), _p(act), M, N, K, _dt(x2d), epilogue,
-                                           _stream(dev))
+            rc = _lib.lib().mtp_linear_fwd_ws(_p(x2d), _p(w), _p(bias), _p(y), _p(act), wsp, wsb, M, N, K, _dt(x2d),
+                                              epilogue, _stream(dev))
             y = None
         _lib.check(rc, "mtp_linear_fwd")
     return y, act
@@ -108,7 +133,8 @@ def linear_dgrad(dy2d: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     dy2d, w = _contig(dy2d), _contig(w)
     dx = torch.empty((M, K), dtype=dy2d.dtype, device=dev)
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().mtp_linear_dgrad(_p(dy2d), _p(w), _p(dx), M, N, K, _dt(dy2d), _stream(dev)),
+        wsp, wsb = _ws_args(dy2d, dev)
+        _lib.check(_lib.lib().mtp_linear_dgrad_ws(_p(dy2d), _p(w), _p(dx), wsp, wsb, M, N, K, _dt(dy2d), _stream(dev)),
                    "mtp_linear_dgrad")
     return dx
 
@@ -138,8 +164,9 @@ def linear_wgrad(dy2d: torch.Tensor, x2d: torch.Tensor, want_db: bool, out_dtype
     if want_db and (db.numel() != N or not db.is_contiguous() or db.dtype != out_dtype):
         raise ValueError("linear_wgrad: db must be a contiguous [N] tensor of the output dtype")
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().mtp_linear_wgrad(_p(dy2d), _p(x2d), _p(dw), _p(db) if want_db else None, M, N, K,
-                                               _dt(dy2d), _DTYPES[out_dtype], int(accumulate), _stream(dev)),
+        wsp, wsb = _ws_args(dy2d, dev)
+        _lib.check(_lib.lib().mtp_linear_wgrad_ws(_p(dy2d), _p(x2d), _p(dw), _p(db) if want_db else None, wsp, wsb, M, N,
+                                                  K, _dt(dy2d), _DTYPES[out_dtype], int(accumulate), _stream(dev)),
                    "mtp_linear_wgrad")
     return dw, (db if want_db else None)
 

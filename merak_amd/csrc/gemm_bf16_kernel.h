@@ -133,12 +133,19 @@ __device__ __forceinline__ void dma16(rsrc_t rsrc, uint32_t lds_addr, uint32_t v
 }
 // The same with the LDS address given as a scalar base plus a compile-time offset: the many destinations of an
 // unrolled loop then cost one live scalar register instead of one each (s_add_u32 leaves its carry in SCC).
-template <int OFFSET>
+// INST_OFF goes into the instruction's offset field, which moves the LDS address and the memory address alike:
+// instructions that fill consecutive KiB of LDS can share one setting of M0 when each one's VGPR offset has
+// INST_OFF taken off (the range check sees the sum, the true offset).  SET_M0: first instruction of such a run.
+template <bool SET_M0, int LDS_OFF, int INST_OFF>
 __device__ __forceinline__ void dma16_at(rsrc_t rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
-  asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff), "n"(OFFSET)
-               : "scc");
+  static_assert(INST_OFF >= 0 && INST_OFF < 4096, "12-bit instruction offset");
+  if constexpr (SET_M0)
+    asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen offset:%5 lds"
+                 :
+                 : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff), "n"(LDS_OFF), "n"(INST_OFF)
+                 : "scc");
+  else
+    asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:%3 lds" : : "v"(voff), "s"(rsrc), "s"(soff), "n"(INST_OFF));
 }
 // Register-staged loads, also inline assembly so that their order against the DMA-style waits stays in this
 // file's hands: 64 lanes x 16 bytes from the buffer into four VGPRs ...
@@ -676,7 +683,8 @@ constexpr int QBK = 64;    // k-tile depth
 // K-contiguous operand: LDS unit = 128 rows x 128 bytes; the 16-byte chunk c of row r sits at position
 // c ^ ((r >> 1) & 7): 16 consecutive rows read at one k cover all 64 banks.  One DMA instruction fills 8 rows
 // (lane l -> row l/8, position l%8, fetching chunk (l%8) ^ swizzle of its row: the 8 lanes of a row still ask
-// for one whole line).  Fragment = one ds_read_b128.
+// for one whole line); a wave's NU instructions of a unit fill 8 NU consecutive rows, so that they share one
+// setting of M0 (dma16_at).  Fragment = one ds_read_b128.
 template <int NW, int WG, int BLK>
 struct RowOperandQ {
   static constexpr int UROWS = 128;                  // rows per unit
@@ -689,25 +697,26 @@ struct RowOperandQ {
   rsrc_t rsrc;
   uint32_t voff[2][NU];
   uint32_t fo[2][QKS];   // [k-tile buffer][step]: the buffer's 64 KiB do not fit the 16-bit offset field of a read
-  int gchunk, K;
 
   // rowmap(r): global row (relative to row0) of tile row r (unit r / 128), or a negative value for "no such row";
   // wsub: the wave's index along this operand's dimension
   template <typename RowMap>
   __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int row0, int nrows, int K_, int lane,
                                        int wave, int wsub, RowMap rowmap) {
-    K = K_;
+    (void)K_;   // a multiple of the k-tile depth (the host checks): no k-tile is ragged
     rsrc = make_rsrc(base + (int64_t)row0 * ld, (int64_t)(nrows - row0) * ld * 2);
-    // tile row of lane l in instruction q = wave + NW j of unit u: 128 u + 8 q + l/8; its swizzle (row >> 1) & 7
-    // = (4 wave + l/16) & 7 whatever j and u are (8 NW j and 128 u are multiples of 16 rows)
-    gchunk = (lane & 7) ^ ((4 * wave + (lane >> 4)) & 7);
+    // tile row of lane l in instruction j of unit u: 128 u + 8 (NU wave + j) + l/8; its swizzle (row >> 1) & 7
+    // = (4 (NU wave + j) + l/16) & 7
 #pragma unroll
     for (int u = 0; u < 2; u++)
 #pragma unroll
       for (int j = 0; j < NU; j++) {
-        const int r = u * UROWS + (wave + NW * j) * 8 + (lane >> 3);
+        const int q = NU * wave + j;
+        const int gchunk = (lane & 7) ^ ((4 * q + (lane >> 4)) & 7);
+        const int r = u * UROWS + q * 8 + (lane >> 3);
         const int64_t gr = rowmap(r);
-        voff[u][j] = (gr < 0 || gr >= nrows - row0) ? 0x80000000u : (uint32_t)((gr * ld + gchunk * 8) * 2);
+        // a valid row r >= 8 j lies at least 1024 j bytes into the buffer (rows are at least 128 bytes long)
+        voff[u][j] = ((gr < 0 || gr >= nrows - row0) ? 0x80000000u : (uint32_t)((gr * ld + gchunk * 8) * 2)) - 1024u * j;
       }
     // fragment of block b at step kk: row BLK (H wsub + b) + l % BLK of the unit, 8 k from 8 (64 / BLK) kk + 8 (l / BLK)
     const int lr = lane & (BLK - 1), h = lane / BLK;
@@ -718,18 +727,21 @@ struct RowOperandQ {
     }
   }
   struct Prep {
+    rsrc_t r;
     uint32_t soff;
-    bool dead;
   };
-  // kend: first k-tile past the range this workgroup multiplies (requests beyond it are zero fill)
+  // kend: first k-tile past the range this workgroup multiplies: requests beyond it go through an empty resource
+  // (zero fill, no memory traffic), a scalar choice that costs the lanes nothing
   __device__ __forceinline__ Prep prep(int kt, int kend) const {
-    return Prep{(uint32_t)(kt * QBK * 2), kt >= kend || kt * QBK + gchunk * 8 >= K};  // chunk at or past the end of k
+    rsrc_t r = rsrc;
+    if (kt >= kend) r[2] = 0;
+    return Prep{r, (uint32_t)(kt * QBK * 2)};
   }
   // J-th DMA instruction of this wave for unit U, which sits UNIT_OFF bytes into the tile buffers;
-  // wave_lds = LDS byte address of the tile buffers + 1024 * wave
+  // wave_lds = LDS byte address of the tile buffers + 1024 * NU * wave
   template <int UNIT_OFF, int U, int J>
   __device__ __forceinline__ void issue(const Prep& pp, uint32_t wave_lds) const {
-    dma16_at<UNIT_OFF + NW * J * 1024>(rsrc, wave_lds, pp.dead ? 0x80000000u : voff[U][J], pp.soff);
+    dma16_at<J == 0, UNIT_OFF, 1024 * J>(pp.r, wave_lds, voff[U][J], pp.soff);
   }
   // unit: address of the unit in k-tile buffer 0
   __device__ __forceinline__ bf16x8_t frag(const char* unit, int buf, int b, int kk) const {
@@ -764,14 +776,17 @@ struct ColOperandQ {
     total = ((int64_t)K_ * ld - row0) * 2;
     ktile_bytes = (int64_t)QBK * ld * 2;
     const int ksub = lane >> 4;                        // k-row inside the instruction = k & 3
-    // chunk of the unit's 128 rows this lane fetches; k >> 3 & 1 = (wave + NW j) >> 1 & 1 = wave >> 1 & 1
-    const int c = (lane & 15) ^ (ksub << 2) ^ (((wave >> 1) & 1) << 1);
 #pragma unroll
     for (int u = 0; u < 2; u++)
 #pragma unroll
       for (int j = 0; j < NU; j++) {
-        const int krow = 4 * (wave + NW * j) + ksub;
-        voff[u][j] = (uint32_t)(((int64_t)krow * ld + u * UROWS + c * 8) * 2);
+        // a wave's NU instructions of a unit fill 4 NU consecutive k-rows (one setting of M0, see dma16_at)
+        const int q = NU * wave + j;
+        const int krow = 4 * q + ksub;
+        // chunk of the unit's 128 rows this lane fetches; k >> 3 & 1 = q >> 1 & 1
+        const int c = (lane & 15) ^ (ksub << 2) ^ (((q >> 1) & 1) << 1);
+        // k-row 4 j lies at least 1024 j bytes in: rows are at least 256 bytes long (the host checks)
+        voff[u][j] = (uint32_t)(((int64_t)krow * ld + u * UROWS + c * 8) * 2) - 1024u * j;
       }
     // lane (group G = l/16, i = l%16) addresses k-row kg + i/4 (+ (1024 / BLK) kk, +4 for the second read) and
     // elements eg + 4 (i%4) .. +3 of the block, with (kg, eg) = (8 (G/2), 16 (G%2)) for BLK = 32, (8 G, 0) for 16
@@ -794,7 +809,7 @@ struct ColOperandQ {
   }
   template <int UNIT_OFF, int U, int J>
   __device__ __forceinline__ void issue(const Prep& pp, uint32_t wave_lds) const {
-    dma16_at<UNIT_OFF + NW * J * 1024>(pp.r, wave_lds, voff[U][J], 0);
+    dma16_at<J == 0, UNIT_OFF, 1024 * J>(pp.r, wave_lds, voff[U][J], 0);
   }
   __device__ __forceinline__ bf16x8_t frag(const char* unit, int buf, int b, int kk) const {
     const char* a = unit + moff[buf][b] + kk * ((QBK / QKS) * UROWS * 2);
@@ -873,8 +888,9 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
       it_end = it + p.sk_ipw < all ? it + p.sk_ipw : all;
     }
   }
-  // where this wave's DMA instructions put their first KiB
-  const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_addr_of(lds)) + wave * 1024;
+  // where this wave's DMA instructions of a unit put their first KiB
+  static_assert(AOp::NU == BOp::NU, "one wave base serves both operands");
+  const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_addr_of(lds)) + wave * (AOp::NU * 1024);
   // byte offsets of the units inside lds
   auto unit_a = [](int buf, int u) constexpr { return buf * QBUF + u * AOp::UBYTES; };
   auto unit_b = [](int buf, int u) constexpr { return buf * QBUF + AOp::BYTES + u * BOp::UBYTES; };
@@ -992,15 +1008,15 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
       rb[U][b][kk] = opB.frag(lds + unit_b(0, U), BUF, b, kk);
     }
   };
-  // d-th DMA instruction of the group (A unit UA, B unit UB, buffer BUF): A and B alternate
+  // d-th DMA instruction of the group (A unit UA, B unit UB, buffer BUF): A's, then B's (each run shares M0)
   auto dma_q = [&](const typename AOp::Prep& pa, const typename BOp::Prep& pb, auto ua_tag, auto ub_tag, auto buf_tag,
                    auto d_tag) {
     constexpr int UA = decltype(ua_tag)::value, UB = decltype(ub_tag)::value, BUF = decltype(buf_tag)::value;
     constexpr int d = decltype(d_tag)::value;
-    if constexpr ((d & 1) == 0)
-      opA.template issue<unit_a(BUF, UA), UA, (d >> 1)>(pa, lds_wave);
+    if constexpr (d < AOp::NU)
+      opA.template issue<unit_a(BUF, UA), UA, d>(pa, lds_wave);
     else
-      opB.template issue<unit_b(BUF, UB), UB, (d >> 1)>(pb, lds_wave);
+      opB.template issue<unit_b(BUF, UB), UB, d - AOp::NU>(pb, lds_wave);
   };
   auto dma_group = [&](int kt, auto ua_tag, auto ub_tag, auto buf_tag) {
     const auto pa = opA.prep(kt, k1);
@@ -1027,23 +1043,33 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
       constexpr int RSPAN = PH / 2;                // spread over the first half of the phase
       if constexpr (g == BARRIER_AT) {
         // own reads of this half tile done, own requests for the next half tile's units landed ...
+#if defined(MTP_MEASURE) && defined(QX_NOVMWAIT)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // timing only: results are wrong
+#else
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(VM_AT_BARRIER) : "memory");
+#endif
+#if !(defined(MTP_MEASURE) && defined(QX_NOBARRIER))
         __syncthreads();  // ... for every wave
+#endif
         __builtin_amdgcn_sched_barrier(0);
       }
       mfma_q(std::integral_constant<int, MA>{}, std::integral_constant<int, MB>{}, std::integral_constant<int, m>{});
+#if !(defined(MTP_MEASURE) && defined(QX_NODMA))
       static_for<NDH>([&](auto d_tag) {
         constexpr int d = decltype(d_tag)::value;
         if constexpr (d * HT / NDH + 1 == g + 1)
           dma_q(pa, pb, std::integral_constant<int, D::v[10]>{}, std::integral_constant<int, D::v[11]>{},
                 std::integral_constant<int, D::v[12]>{}, d_tag);
       });
+#endif
+#if !(defined(MTP_MEASURE) && defined(QX_NOREAD))
       if constexpr (m < RSPAN) {
         static_for<(m + 1) * NR / RSPAN - m * NR / RSPAN>([&](auto e) {
           read_q(std::integral_constant<int, RA>{}, std::integral_constant<int, RU>{},
                  std::integral_constant<int, RBUF>{}, std::integral_constant<int, m * NR / RSPAN + decltype(e)::value>{});
         });
       }
+#endif
       __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -1652,12 +1678,16 @@ constexpr bool cfg_valid(int c) {
   return true;
 }
 
+// The 64-deep loop takes whole k-tiles only, and rows of at least 256 bytes (its DMA instructions carry part of
+// their address in the offset field, see dma16_at)
+inline bool q_loop_ok(const GemmArgs& a) { return a.K % QBK == 0 && a.lda >= 128 && a.ldb >= 128; }
+
 template <int EPI>
 int pick_config(const GemmArgs& a) {
   static MtpTune tune_cfg("MTP_GEMM_CFG"), tune_skip("MTP_GEMM_SKIP");
   if (tune_cfg.is_set()) {
     const int c = tune_cfg.get(0);
-    if (c >= 0 && c < kNumCfgs) return c;
+    if (c >= 0 && c < kNumCfgs && !(kCfgs[c].q != 0 && !q_loop_ok(a))) return c;
   }
   const int64_t span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
   const int skip = tune_skip.get(0);  // bit c set = leave configuration c out of the choice
@@ -1669,7 +1699,7 @@ int pick_config(const GemmArgs& a) {
     const int bn_span = (EPI == MTP_EPI_SWIGLU) ? t.bn / 2 : t.bn;
     const int64_t tiles = ((a.M + t.bm - 1) / t.bm) * ((span + bn_span - 1) / bn_span);
     const int64_t rounds = (tiles + 255) / 256;
-    if (!cfg_valid<EPI>(c)) continue;
+    if (!cfg_valid<EPI>(c) || (t.q != 0 && !q_loop_ok(a))) continue;
     const double cost = (double)rounds * t.bm * t.bn / t.eff;
     if (cost < best_t * 0.999) {
       best_t = cost;

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTP_ABI_VERSION 7
+#define MTP_ABI_VERSION 8
 
 /* element types.  MTP_F16 is IEEE half, what the reference's --fp16 sets as
  * params_dtype (Merak/merak_args/args.py:584-585). */
@@ -280,6 +280,20 @@ int mtp_gemv_argmax(const void* x, const void* w,
                     int64_t* idx, float* maxval,
                     void* workspace, int64_t workspace_bytes,
                     int64_t B, int64_t N, int64_t K, int dtype, void* stream);
+
+/* mtp_gemv_argmax for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid it): the
+ * scratch is an array inside the library, mtp_gemv_argmax_noalloc_max_bytes()
+ * = 4 MiB per GPU, held until the process ends; a shape whose
+ * mtp_gemv_argmax_workspace_bytes exceeds that returns MTP_EWORKSPACE.  No
+ * call allocates or frees.  All calls on one GPU share that GPU's array:
+ * calls that overlap on one GPU (different streams) race.  Nothing in the
+ * array needs clearing between calls.  It has no counterpart in the
+ * reference. */
+int64_t mtp_gemv_argmax_noalloc_max_bytes(void);
+int mtp_gemv_argmax_noalloc(const void* x, const void* w,
+                            int64_t* idx, float* maxval,
+                            int64_t B, int64_t N, int64_t K, int dtype, void* stream);
 
 /* Row-wise argmax of materialised logits [B,V] (dtype f32, bf16 or f16): the
  * literal torch.argmax(logits, dim=-1) of :227. */

@@ -19,7 +19,7 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmerak_tp_gfx950.so"
 
 MTP_F32, MTP_BF16, MTP_F16 = 0, 1, 2
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_SWIGLU, EPI_GELU = 0, 1, 2, 3, 4
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _i64, _int, _vp = C.c_int64, C.c_int, C.c_void_p
 
@@ -47,6 +47,8 @@ SIGNATURES = {
     "mtp_gemv": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
     "mtp_gemv_argmax_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "mtp_gemv_argmax": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "mtp_gemv_argmax_noalloc_max_bytes": (_i64, []),
+    "mtp_gemv_argmax_noalloc": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "mtp_argmax_rows": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "mtp_sample_workspace_bytes": (_i64, [_i64]),
     "mtp_sample_top_k_top_p": (_int, [_vp, _int, _i64, _i64, C.c_float, _int, C.c_float, _vp, _vp, _vp, _vp, _i64, _vp]),

@@ -24,6 +24,7 @@
 // bit-reproducible run to run.
 #include "mtp_common.h"
 #include <stdlib.h>
+#include <mutex>
 #include <type_traits>
 
 namespace {
@@ -1011,6 +1012,54 @@ extern "C" int mtp_gemv_argmax(const void* x, const void* w, int64_t* idx, float
                      idx, maxval);
   MTP_CHECK_LAUNCH("argmax_finish");
   return MTP_OK;
+}
+
+// ---- the greedy pick for callers that cannot allocate --------------------------------------------------------
+// Same kernels as mtp_gemv_argmax; the per-workgroup partial maxima live in a device array of this library
+// instead of a caller's workspace.  Every GPU holds its own copy of the array at its own address: the address is
+// asked for once per device (hipGetSymbolAddress, with that device current) and kept.
+#define MTP_ARGMAX_STATIC_BYTES (4ll << 20)
+static __device__ __align__(256) unsigned char g_argmax_scratch[MTP_ARGMAX_STATIC_BYTES];
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+// device address of g_argmax_scratch on the current device, or null (error set)
+void* argmax_scratch_ptr() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    mtp_set_error("gemv_argmax_noalloc: hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* q = nullptr;
+    e = hipGetSymbolAddress(&q, HIP_SYMBOL(g_argmax_scratch));
+    if (e != hipSuccess || !q) {
+      mtp_set_error("gemv_argmax_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = q;
+  }
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int64_t mtp_gemv_argmax_noalloc_max_bytes(void) { return MTP_ARGMAX_STATIC_BYTES; }
+
+extern "C" int mtp_gemv_argmax_noalloc(const void* x, const void* w, int64_t* idx, float* maxval, int64_t B, int64_t N,
+                                       int64_t K, int dtype, void* stream) {
+  int rc = check_gemv_args("gemv_argmax_noalloc", x, w, B, N, K, dtype);
+  if (rc) return rc;
+  MTP_REQUIRE(idx, MTP_EINVAL, "gemv_argmax_noalloc: null pointer");
+  const int64_t need = mtp_gemv_argmax_workspace_bytes(B, N, K);
+  MTP_REQUIRE(need <= MTP_ARGMAX_STATIC_BYTES, MTP_EWORKSPACE,
+              "gemv_argmax_noalloc: B=%lld N=%lld needs %lld bytes of scratch, the library holds %lld (use mtp_gemv_argmax "
+              "with a workspace)", (long long)B, (long long)N, (long long)need, (long long)MTP_ARGMAX_STATIC_BYTES);
+  void* scratch = argmax_scratch_ptr();
+  if (!scratch) return MTP_EDEVICE;
+  return mtp_gemv_argmax(x, w, idx, maxval, scratch, MTP_ARGMAX_STATIC_BYTES, B, N, K, dtype, stream);
 }
 
 extern "C" int mtp_argmax_rows(const void* logits, int64_t* idx, int64_t B, int64_t V, int dtype, void* stream) {

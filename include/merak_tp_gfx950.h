@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTP_ABI_VERSION 8
+#define MTP_ABI_VERSION 9
 
 /* element types.  MTP_F16 is IEEE half, what the reference's --fp16 sets as
  * params_dtype (Merak/merak_args/args.py:584-585). */
@@ -92,6 +92,12 @@ int mtp_linear_dgrad(const void* dy, const void* w, void* dx,
 int mtp_linear_wgrad(const void* dy, const void* x, void* dw, void* db,
                      int64_t M, int64_t N, int64_t K,
                      int dtype, int dw_dtype, int accumulate, void* stream);
+
+/* db[N] (+)= sum_m dY[m,:] alone: the bias gradient of F.linear for a layer
+ * whose weight takes no gradient (otherwise mtp_linear_wgrad delivers it with
+ * dW in one launch).  db_dtype: dtype or MTP_F32.  M == 0 writes zeros. */
+int mtp_linear_bias_grad(const void* dy, void* db, int64_t M, int64_t N,
+                         int dtype, int db_dtype, int accumulate, void* stream);
 
 /* The three products above with device scratch.  On the 16-bit path a product
  * whose 256x256 tiling would leave much of the last round of workgroups idle

@@ -157,3 +157,13 @@ extern "C" int mtp_linear_wgrad_ws(const void* dy, const void* x, void* dw, void
   if (db) return mtp_colsum(dy, db, M, N, dtype, dw_dtype, accumulate, s);
   return MTP_OK;
 }
+
+extern "C" int mtp_linear_bias_grad(const void* dy, void* db, int64_t M, int64_t N, int dtype, int db_dtype, int accumulate,
+                                    void* stream) {
+  int rc = check_dims("linear_bias_grad", M, N, 1, dtype);
+  if (rc) return rc;
+  MTP_REQUIRE(db_dtype == MTP_F32 || db_dtype == dtype, MTP_EUNSUPPORTED,
+              "linear_bias_grad: the gradient is fp32 or of the inputs' dtype (inputs %d, db %d)", dtype, db_dtype);
+  MTP_REQUIRE(db && (M == 0 || dy), MTP_EINVAL, "linear_bias_grad: null pointer");
+  return mtp_colsum(dy, db, M, N, dtype, db_dtype, accumulate, (hipStream_t)stream);
+}

@@ -168,7 +168,7 @@ class _LMHeadCrossEntropy(torch.autograd.Function):
     per-position losses), as the one-launch cross entropy does."""
 
     @staticmethod
-    def forward(ctx, hidden, weight, bias, target, assumed_grad, chunk_rows):
+    def forward(ctx, hidden, weight, bias, target, assumed_grad, chunk_rows, accum_dtype):
         vocab_start_index, _ = _vocab_range(weight.shape[0])
         lead = hidden.shape[:-1]
         h2d = hidden.reshape(-1, hidden.shape[-1])
@@ -178,8 +178,12 @@ class _LMHeadCrossEntropy(torch.autograd.Function):
         need_b = bias is not None and ctx.needs_input_grad[2]
         losses = torch.empty((n,), dtype=torch.float32, device=h2d.device)
         dh = torch.empty_like(h2d) if need_h else None
-        dw = torch.zeros_like(weight) if need_w else None
-        db = torch.zeros_like(bias) if need_b else None
+        # The first chunk writes the weight and bias gradients, the later ones add to them (a read-modify-write of
+        # the whole gradient per chunk), in accum_dtype: the weight's dtype, or fp32 with one cast at the end.
+        one_chunk = chunk_rows >= n
+        acc_dt = weight.dtype if one_chunk else accum_dtype
+        dw = torch.empty(weight.shape, dtype=acc_dt, device=weight.device) if need_w else None
+        db = torch.empty(bias.shape, dtype=acc_dt, device=bias.device) if need_b else None
         epi = ops.EPI_BIAS if bias is not None else ops.EPI_NONE
         backward_wanted = need_h or need_w or need_b
         for r0 in range(0, n, chunk_rows):
@@ -189,13 +193,18 @@ class _LMHeadCrossEntropy(torch.autograd.Function):
                 loss_c, _, _, _ = ops.vocab_ce_fwd_bwd_(logits, t1d[r0:r1], vocab_start_index, None, assumed_grad)
                 if need_h:
                     dh[r0:r1] = ops.linear_dgrad(logits, weight)
-                if need_w or need_b:
-                    ops.linear_wgrad(logits, h2d[r0:r1], need_b, dw=dw if need_w else torch.zeros_like(weight),
-                                     db=db, accumulate=True)
+                if need_w:
+                    ops.linear_wgrad(logits, h2d[r0:r1], need_b, dw=dw, db=db, accumulate=r0 > 0)
+                elif need_b:
+                    ops.colsum(logits, db, accumulate=r0 > 0)
             else:
                 loss_c, _, _, _ = ops.vocab_ce_fwd(logits, t1d[r0:r1], vocab_start_index)
             losses[r0:r1] = loss_c
             del logits
+        if dw is not None and dw.dtype != weight.dtype:
+            dw = dw.to(weight.dtype)
+        if db is not None and db.dtype != bias.dtype:
+            db = db.to(bias.dtype)
         ctx.assumed_grad = float(assumed_grad)
         ctx.lead = lead
         ctx.save_for_backward(dh, dw, db)
@@ -213,10 +222,10 @@ class _LMHeadCrossEntropy(torch.autograd.Function):
         if ratio != 1.0:
             # out of place: the saved gradients stay valid for a second backward over a retained graph
             dh, dw, db = (None if t is None else t * ratio for t in (dh, dw, db))
-        return (dh.view(*ctx.lead, dh.shape[-1]) if dh is not None else None), dw, db, None, None, None
+        return (dh.view(*ctx.lead, dh.shape[-1]) if dh is not None else None), dw, db, None, None, None, None
 
 
-def lm_head_cross_entropy(hidden, lm_head, target, loss_scale=1.0, chunk_rows=4096):
+def lm_head_cross_entropy(hidden, lm_head, target, loss_scale=1.0, chunk_rows=4096, grad_accum_dtype=None):
     """Per-position losses of ``vocab_parallel_cross_entropy(lm_head(hidden)[0], target)`` without ever holding
     the full logits: the head's product, the cross entropy and both of the head's backward products run per
     chunk of ``chunk_rows`` tokens, so the largest temporary is [chunk_rows, vocab/p].
@@ -224,8 +233,16 @@ def lm_head_cross_entropy(hidden, lm_head, target, loss_scale=1.0, chunk_rows=40
     ``lm_head``: a ``ColumnParallelLinear(hidden, vocab, gather_output=False)`` (model_parallel.py:143-156) or
     its weight.  The per-position losses must be reduced with one common factor — ``.mean()`` as the
     trainer does (merak_trainer.py:325), times ``loss_scale`` if any; that factor is assumed in forward
-    (``loss_scale / n``) and checked in backward.  Weight gradients are accumulated chunk by chunk in the
-    weight's dtype."""
+    (``loss_scale / n``) and checked in backward.
+
+    What it is and is not: the logits still make their trip through memory, one chunk at a time (product ->
+    cross entropy and gradient in place -> the two backward products); what is saved is memory — the largest
+    temporary is one chunk — not traffic, and every chunk after the first pays a read-modify-write of the whole
+    weight gradient, so on a shape whose full logits fit it is a little slower than the unfused sequence.
+    ``grad_accum_dtype``: dtype the weight (and bias) gradient is summed in across chunks.  Default: the
+    weight's own dtype, which is how the reference's ``.grad`` sums micro-batches (one rounding to 16 bits per
+    chunk: at 32 chunks in bf16 the gradient stays within twice the tolerance of the one-piece product);
+    ``torch.float32`` sums in an fp32 buffer (4 bytes per weight more while the call runs) and rounds once."""
     weight, bias = (lm_head.weight, lm_head.bias) if isinstance(lm_head, torch.nn.Module) else (lm_head, None)
     if get_model_parallel_world_size() != 1:
         raise RuntimeError("lm_head_cross_entropy at tensor-parallel size > 1 needs the MAX/SUM/SUM exchange of "
@@ -235,4 +252,7 @@ def lm_head_cross_entropy(hidden, lm_head, target, loss_scale=1.0, chunk_rows=40
         return torch.zeros(target.shape, dtype=torch.float32, device=hidden.device)
     if weight.shape[0] > ops.vocab_ce_fused_max_vocab(hidden.dtype):
         raise ValueError("vocabulary slice too long for the one-launch cross entropy; use the unfused layers")
-    return _LMHeadCrossEntropy.apply(hidden, weight, bias, target, float(loss_scale) / n, int(chunk_rows))
+    accum = weight.dtype if grad_accum_dtype is None else grad_accum_dtype
+    if accum not in (weight.dtype, torch.float32):
+        raise ValueError("grad_accum_dtype must be the weight's dtype or torch.float32")
+    return _LMHeadCrossEntropy.apply(hidden, weight, bias, target, float(loss_scale) / n, int(chunk_rows), accum)

@@ -171,6 +171,21 @@ def linear_wgrad(dy2d: torch.Tensor, x2d: torch.Tensor, want_db: bool, out_dtype
     return dw, (db if want_db else None)
 
 
+def colsum(dy2d: torch.Tensor, db: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
+    """db (+)= dy2d.sum(0): the bias gradient alone, for a layer whose weight takes none."""
+    dev = _require_gpu(dy2d, db)
+    if dy2d.dim() != 2 or db.numel() != dy2d.shape[1] or not db.is_contiguous():
+        raise ValueError(f"colsum: dy must be [M, N] and db a contiguous [N], got {tuple(dy2d.shape)} and {tuple(db.shape)}")
+    if db.dtype not in (dy2d.dtype, torch.float32):
+        raise TypeError("colsum: db must have dy's dtype or float32")
+    dy2d = _contig(dy2d)
+    M, N = dy2d.shape
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_linear_bias_grad(_p(dy2d), _p(db), M, N, _dt(dy2d), _DTYPES[db.dtype], int(accumulate),
+                                                   _stream(dev)), "mtp_linear_bias_grad")
+    return db
+
+
 def activation_bwd(dact: torch.Tensor, y: torch.Tensor, epilogue: int) -> torch.Tensor:
     dev = _require_gpu(dact, y)
     if y.dim() != 2 or dact.dim() != 2 or dact.dtype != y.dtype:

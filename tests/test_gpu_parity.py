@@ -340,6 +340,47 @@ def test_lm_head_cross_entropy_chunked(gpu, dtype, n, k, v, chunk, has_bias):
         (l3.view(-1) * torch.arange(n, device=gpu)).sum().backward()
 
 
+@pytest.mark.parametrize("accum", [None, torch.float32])
+def test_lm_head_cross_entropy_many_chunks(gpu, accum):
+    """32 chunks of 256 tokens: the weight gradient summed across chunks in the weight's dtype (one rounding per
+    chunk, as the reference's .grad sums micro-batches) stays within twice the one-piece tolerance, and within it
+    when summed in fp32; the two differ from the unfused layers only by that rounding."""
+    n, k, v, chunk = 8192, 512, 2048, 256
+    g = gen(120)
+    h = torch.randn(n, k, generator=g).bfloat16()
+    w = (torch.randn(v, k, generator=g) * 0.05).bfloat16()
+    b = (torch.randn(v, generator=g) * 0.05).bfloat16()
+    t = torch.randint(0, v, (n,), generator=g)
+    t[::50] = -100
+    hr, wr, br = h.float().requires_grad_(True), w.float().requires_grad_(True), b.float().requires_grad_(True)
+    logits = F.linear(hr, wr, br)
+    logits = logits + (logits.detach().bfloat16().float() - logits.detach())
+    lse = torch.logsumexp(logits, -1)
+    picked = logits[torch.arange(n), t.clamp_min(0)]
+    closed = torch.where(t >= 0, lse - picked, lse - logits.max(-1).values.detach())
+    closed.mean().backward()
+    hg = h.to(gpu).requires_grad_(True)
+    wg = w.to(gpu).requires_grad_(True)
+    bg = b.to(gpu).requires_grad_(True)
+    head = type("Head", (torch.nn.Module,), {})()
+    head.weight, head.bias = wg, bg
+    losses = mpu.lm_head_cross_entropy(hg, head, t.to(gpu), chunk_rows=chunk, grad_accum_dtype=accum)
+    assert rel(losses, closed.detach()) < 1e-4
+    losses.mean().backward()
+    assert wg.grad.dtype == torch.bfloat16 and bg.grad.dtype == torch.bfloat16
+    tol = 2 * TOL_BF16 if accum is None else TOL_BF16
+    assert rel(hg.grad, hr.grad) < TOL_BF16 and rel(wg.grad, wr.grad) < tol and rel(bg.grad, br.grad) < tol
+    # a head whose weight takes no gradient: the bias gradient alone, no weight-sized temporary
+    wf = w.to(gpu)
+    bg2 = b.to(gpu).requires_grad_(True)
+    head.weight, head.bias = wf, bg2
+    before = torch.cuda.max_memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    l2 = mpu.lm_head_cross_entropy(h.to(gpu), head, t.to(gpu), chunk_rows=chunk, grad_accum_dtype=accum)
+    l2.mean().backward()
+    assert rel(bg2.grad, br.grad) < tol
+
+
 # =============================================================================== embedding
 @pytest.mark.parametrize("dtype,v,h", [(torch.bfloat16, 1000, 4096), (torch.float32, 777, 33), (torch.bfloat16, 50, 7),
                                         (torch.float32, 64, 1)])

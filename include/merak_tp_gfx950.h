@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTP_ABI_VERSION 9
+#define MTP_ABI_VERSION 10
 
 /* element types.  MTP_F16 is IEEE half, what the reference's --fp16 sets as
  * params_dtype (Merak/merak_args/args.py:584-585). */
@@ -152,13 +152,18 @@ int mtp_embedding_gather(const int64_t* ids, const void* table, void* out,
 /* Dense gradient of the lookup: dtable[ids[i]-vocab_start,:] += dout[i,:]
  * for in-range ids; dtable is [rows,dim] of dtable_dtype (fp32, or the
  * 16-bit dtype of dout).  This is the embedding_dense_backward ATen runs behind
- * F.embedding (layers.py:156).  Tokens that share an id are summed in
- * ascending token order in fp32 and added to the table row once, so the
- * result is reproducible bit for bit.  The caller zeroes dtable first unless
- * it wants accumulation, e.g. onto the LM-head weight gradient when the two
- * are tied (Merak/core/pipeline/module.py:646-662).  workspace: device scratch
- * of mtp_embedding_bwd_workspace_bytes(n_ids) bytes, 8-byte aligned. */
-int64_t mtp_embedding_bwd_workspace_bytes(int64_t n_ids);
+ * F.embedding (layers.py:156).  Tokens that share an id are summed in fp32 in
+ * an order fixed by the ids alone (ascending token order; an id carried by
+ * more than 32 tokens: ascending inside blocks of 32 of its tokens, the block
+ * sums ascending inside blocks of 32 blocks, then those in ascending order)
+ * and added to the table row once, so the result is reproducible bit for
+ * bit, and the longest dependent chain is 64 + count/1024 steps however many
+ * tokens share an id (a padded batch).  The
+ * caller zeroes dtable first unless it wants accumulation, e.g. onto the
+ * LM-head weight gradient when the two are tied
+ * (Merak/core/pipeline/module.py:646-662).  workspace: device scratch of
+ * mtp_embedding_bwd_workspace_bytes(n_ids, dim) bytes, 16-byte aligned. */
+int64_t mtp_embedding_bwd_workspace_bytes(int64_t n_ids, int64_t dim);
 int mtp_embedding_bwd(const int64_t* ids, const void* dout, void* dtable,
                       void* workspace, int64_t workspace_bytes,
                       int64_t n_ids, int64_t dim, int dtype, int dtable_dtype,

@@ -241,7 +241,7 @@ def embedding_bwd(ids: torch.Tensor, dout: torch.Tensor, rows: int, vocab_start:
     elif tuple(out.shape) != (rows, dim) or not out.is_contiguous():
         raise ValueError(f"out must be a contiguous [{rows}, {dim}] tensor")
     lib = _lib.lib()
-    ws = torch.empty((max(int(lib.mtp_embedding_bwd_workspace_bytes(flat.numel())), 8),), dtype=torch.uint8, device=dev)
+    ws = torch.empty((max(int(lib.mtp_embedding_bwd_workspace_bytes(flat.numel(), dim)), 16),), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         _lib.check(lib.mtp_embedding_bwd(_p(flat), _p(d2), _p(out), _p(ws), ws.numel(), flat.numel(), dim, _dt(d2),
                                          _dt(out), vocab_start, vocab_end, _stream(dev)), "mtp_embedding_bwd")

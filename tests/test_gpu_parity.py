@@ -430,13 +430,19 @@ def test_embedding_backward_reproducible(gpu, dtype, n, v, h, lo, hi):
     a = ops.embedding_bwd(ids.to(gpu), dout.to(gpu), hi - lo, lo, hi, dtype=torch.float32)
     b = ops.embedding_bwd(ids.to(gpu), dout.to(gpu), hi - lo, lo, hi, dtype=torch.float32)
     assert rel(a, ref) < TOL_F32 and torch.equal(a, b), "same inputs, same bits"
-    # the documented order: ascending token index, fp32 running sum
-    seq = torch.zeros(h)
-    for i in range(n // 3):
-        seq += dout[i].float()
-    extra = (ids[n // 3:] == lo + 1).nonzero().flatten() + n // 3
-    for i in extra.tolist():
-        seq += dout[i].float()
+    # the documented order: ascending token index in fp32; an id carried by more than 32 tokens: the same inside
+    # blocks of 32 of its tokens, the block sums in ascending order inside blocks of 32 blocks, those in ascending order
+    mine = (ids == lo + 1).nonzero().flatten().tolist()
+    def running(rows):
+        acc = torch.zeros(h)
+        for r in rows:
+            acc += r
+        return acc
+    if len(mine) > 32:
+        blocks = [running([dout[i].float() for i in mine[b:b + 32]]) for b in range(0, len(mine), 32)]
+        seq = running([running(blocks[b:b + 32]) for b in range(0, len(blocks), 32)])
+    else:
+        seq = running([dout[i].float() for i in mine])
     assert torch.equal(a[1].cpu(), seq)
     # accumulation onto an existing gradient (tied LM head), in the table's own dtype
     base = torch.randn(hi - lo, h, generator=gen(29)).to(dtype)
@@ -445,6 +451,35 @@ def test_embedding_backward_reproducible(gpu, dtype, n, v, h, lo, hi):
     untouched = torch.ones(hi - lo, dtype=torch.bool)
     untouched[ids[(ids >= lo) & (ids < hi)] - lo] = False
     assert torch.equal(tied.cpu()[untouched], base[untouched])
+
+
+def test_embedding_backward_padded_batch(gpu):
+    """Half of 8192 tokens carry one id (a padded batch), a few more ids are carried by 33-200 tokens, the rest are
+    Zipf-like: parity with the oracle, the same bits on every run, and a bounded time (the chain of the common id is
+    walked in blocks of 32, not token by token)."""
+    n, v, h = 8192, 32000, 4096
+    g = gen(30)
+    ids = (torch.rand(n, generator=g) ** 4 * v).long().clamp_max(v - 1)
+    ids[torch.randperm(n, generator=g)[: n // 2]] = 2                      # pad id
+    for k, c in ((7, 33), (11, 64), (13, 200), (17, 32)):
+        ids[torch.randperm(n, generator=g)[:c]] = k
+    dout = torch.randn(n, h, generator=g).bfloat16()
+    ref = R.embedding_backward(ids, dout, v, 0, v)
+    a = ops.embedding_bwd(ids.to(gpu), dout.to(gpu), v, 0, v, dtype=torch.float32)
+    b = ops.embedding_bwd(ids.to(gpu), dout.to(gpu), v, 0, v, dtype=torch.float32)
+    assert rel(a, ref) < TOL_F32 and torch.equal(a, b)
+    for k in (2, 7, 11, 13, 17):
+        assert rel(a[k], ref[k]) < TOL_F32, k
+    idg, dg, out = ids.to(gpu), dout.to(gpu), torch.zeros(v, h, device=gpu)
+    ops.embedding_bwd(idg, dg, v, 0, v, out=out)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        ops.embedding_bwd(idg, dg, v, 0, v, out=out)
+    e1.record()
+    torch.cuda.synchronize()
+    assert e0.elapsed_time(e1) / 5 < 2.0, "a common id must not be walked token by token (milliseconds)"
 
 
 def test_embedding_full_size_llama_table(gpu):

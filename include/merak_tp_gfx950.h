@@ -246,10 +246,12 @@ int mtp_gemv(const void* x, const void* w, const void* bias, void* y,
  * part of X); the slices' partial sums meet in the workspace and are added
  * in slice order, so the result is reproducible.  workspace: 16-byte
  * aligned, mtp_gemv_workspace_bytes(B, N, K, epilogue) bytes (0 = this shape
- * is not cut; then workspace may be NULL).  ITS FIRST 4 * ceil(N / 16) BYTES
- * MUST BE ZERO before the first launch that uses it; every launch leaves
- * them zero.  Launches that share a workspace must not overlap.  A NULL or
- * too small workspace gives mtp_gemv's uncut behaviour. */
+ * is not cut; then workspace may be NULL).  ITS FIRST 8192 BYTES MUST BE
+ * ZERO before the first launch that uses it; every launch leaves them zero,
+ * whatever its shape, so one workspace (of the largest size any of them
+ * asks for) serves launches of different shapes in turn.  Launches that
+ * share a workspace must not overlap.  A NULL or too small workspace gives
+ * mtp_gemv's uncut behaviour. */
 int64_t mtp_gemv_workspace_bytes(int64_t B, int64_t N, int64_t K, int epilogue);
 int mtp_gemv_ws(const void* x, const void* w, const void* bias, void* y,
                 void* workspace, int64_t workspace_bytes,

@@ -718,6 +718,10 @@ constexpr int GV_MAX_SLICES = 8;
 
 bool depth_ok(int64_t K, int d) { return d == 1 || (K % 64 == 0 && ((K / 64) % (GV_MAX_WAVES * d)) == 0); }
 
+// The counters take the same 8 KiB whatever the shape, so that one zeroed workspace serves launches of different
+// shapes in turn: with a size that followed N, the partial sums of a matrix with few rows would land where a
+// larger one keeps its counters.  2048 counters cover every shape that is cut (fewer than 190 row blocks).
+constexpr int64_t GV_COUNTER_BYTES = 8192;
 GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode, bool may_split = false) {
   const int64_t groups = ((mode == 1 ? N / 2 : N) + 15) / 16 * (mode == 1 ? 2 : 1);
   // Bytes in flight are what a bandwidth-bound kernel lives on: R*D k-pairs (2 KiB each) per wave.  Large
@@ -730,7 +734,8 @@ GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode, bool may_split 
   // cut instead (each slice reads only its part of X); every wave of a slice gets the same number of pairs.
   // Measured (B = 16 and 32): 4096x14336 gains 17-23 %, matrices with K = 4096 lose (too little k per slice to
   // pay for the hand-over), batches up to 8 gain nothing.
-  if (may_split && mode != 2 && K % 64 == 0 && groups / c.R < 190) {
+  if (may_split && mode != 2 && K % 64 == 0 && groups / c.R < 190 &&
+      groups * (int64_t)sizeof(int32_t) <= GV_COUNTER_BYTES) {
     int want = (B > 8 && K >= 8192) ? 0 : -1;
     static MtpTune tune_s("MTP_GEMV_S");
     want = tune_s.get(want);
@@ -761,7 +766,10 @@ GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode, bool may_split 
 }
 
 // bytes of the arrival counters in front of the partial sums: one per 16 rows covers every configuration
-int64_t gemv_counter_bytes(int64_t N) { return ((N + 15) / 16 * (int64_t)sizeof(int32_t) + 255) / 256 * 256; }
+int64_t gemv_counter_bytes(int64_t N) {
+  (void)N;
+  return GV_COUNTER_BYTES;
+}
 
 template <int MODE, bool NORM = false>
 int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart* part, int64_t B, int64_t N,

@@ -20,6 +20,10 @@ from .mappings import gather_from_model_parallel_region
 from .mappings import reduce_from_model_parallel_region
 from .mappings import scatter_to_model_parallel_region
 
+from .random import get_rng_tracker
+from .random import model_parallel_manual_seed
+from .random import RNGStatesTracker
+
 from .utils import divide
 from .utils import ensure_divisibility
 from .utils import split_tensor_along_last_dim

@@ -87,6 +87,12 @@ class _VocabParallelCrossEntropyFused(torch.autograd.Function):
         logits_2d = vocab_parallel_logits.view(-1, partition_vocab_size)
         target_1d = target.reshape(-1)
         loss, _, _, _ = ops.vocab_ce_fwd_bwd_(logits_2d, target_1d, vocab_start_index, None, assumed_grad)
+        # the kernel wrote through a raw pointer: tell autograd that the caller's logits have changed, so that
+        # another function that saved them for its own backward fails loudly instead of using the gradient.
+        # A view handed out by a custom Function (the linear layers reshape their product) cannot be marked:
+        # autograd refuses to rebuild such a view's history, so there the overwrite is only documented.
+        if not vocab_parallel_logits._is_view():
+            torch.autograd.graph.increment_version(vocab_parallel_logits)
         ctx.assumed_grad = float(assumed_grad)
         ctx.save_for_backward(vocab_parallel_logits)
         loss = loss.view_as(target)
@@ -133,8 +139,12 @@ def vocab_loss_fn(outputs, labels, loss_scale=1.0):
     if isinstance(labels, tuple):
         labels = labels[0]
     n = labels.numel()
+    # The one-launch kernel overwrites the logits with their gradient during forward; that is only wanted when a
+    # backward pass will follow.  Evaluation (no_grad, or logits that take no gradient: the reference's eval_batch
+    # hands the logits back after the loss) runs the plain forward, which leaves the logits as they are.
+    wants_grad = torch.is_grad_enabled() and outputs.requires_grad
     losses = vocab_parallel_cross_entropy(outputs, labels,
-                                          fused_backward_scale=(float(loss_scale) / n) if n else None)
+                                          fused_backward_scale=(float(loss_scale) / n) if (n and wants_grad) else None)
     return torch.mean(losses.view(-1))
 
 

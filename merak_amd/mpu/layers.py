@@ -9,6 +9,8 @@ GPT-2, ``silu(gate) * up`` for Llama) into the GEMM epilogue.
 """
 from __future__ import annotations
 
+import contextlib
+
 import torch
 import torch.nn.init as init
 from torch.nn.parameter import Parameter
@@ -18,21 +20,28 @@ from ..args import get_args
 from .initialize import get_model_parallel_rank, get_model_parallel_world_size
 from .mappings import (copy_to_model_parallel_region, gather_from_model_parallel_region,
                        reduce_from_model_parallel_region, scatter_to_model_parallel_region)
+from .random import get_rng_tracker
 from .utils import VocabUtility, divide
 
 _ACTIVATIONS = {None: None, "gelu_new": "gelu_new", "swiglu": "swiglu"}
 
 
-def _initialize_affine_weight_gpu(weight, init_method, partition_dim, stride=1):
+def _initialize_affine_weight_gpu(weight, init_method, partition_dim, stride=1, rng_context=None):
     """Tag and initialise a device-resident shard (layers.py:44-53).
 
-    The reference draws under its model-parallel RNG fork; the fork only
-    decides which generator state is used, so the caller's ``init_method``
-    runs on whatever generator is current."""
+    The reference draws under ``get_rng_tracker().fork()``, the model-parallel generator state, so that ranks of one
+    tensor-parallel group get different shards from one seed.  Here: under ``rng_context`` when one is given (any
+    context manager), else under this package's tracker when ``mpu.model_parallel_manual_seed`` has registered the
+    model-parallel state, else on the current generator (the reference would refuse; a caller that never seeded
+    the tracker builds one rank's shard with its own generator)."""
     weight.model_parallel = True
     weight.partition_dim = partition_dim
     weight.partition_stride = stride
-    init_method(weight)
+    if rng_context is None:
+        tracker = get_rng_tracker()
+        rng_context = tracker.fork() if tracker.has() else contextlib.nullcontext()
+    with rng_context:
+        init_method(weight)
 
 
 def _initialize_affine_weight_cpu(weight, output_size, input_size, per_partition_size, partition_dim, init_method,

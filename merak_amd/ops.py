@@ -342,7 +342,8 @@ def vocab_ce_rescale_(grad2d: torch.Tensor, grad_rows: torch.Tensor, assumed: fl
 # --------------------------------------------------------------------------- decode
 def gemv_workspace(B: int, N: int, K: int, epilogue: int, device) -> Optional[torch.Tensor]:
     """Zero-filled scratch for ``gemv(..., workspace=)`` or None when this shape runs without one.  One
-    workspace serves any number of launches that do not overlap (take the largest need)."""
+    workspace serves any number of launches, of any shapes, that do not overlap: take the largest need (the
+    counters every launch leaves zero sit in its first 8 KiB whatever the shape)."""
     need = int(_lib.lib().mtp_gemv_workspace_bytes(B, N, K, epilogue))
     return torch.zeros((need,), dtype=torch.uint8, device=device) if need else None
 

@@ -45,6 +45,8 @@ def set_tuning(monkeypatch):
 def _reset_mpu():
     from merak_amd import mpu, set_args
     mpu.destroy_model_parallel()
+    mpu.get_rng_tracker().reset()
     set_args(use_cpu_initialization=True)
     yield
     mpu.destroy_model_parallel()
+    mpu.get_rng_tracker().reset()

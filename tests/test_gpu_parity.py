@@ -265,6 +265,31 @@ def test_ce_vocab_loss_fn_autograd(gpu, dtype):
     assert bool((xg2.grad.view(n, v)[mask.view(n) == 0] == 0).all())
 
 
+def test_ce_vocab_loss_fn_leaves_logits_alone_without_grad(gpu):
+    """Evaluation: under no_grad, or for logits that take no gradient, the loss is the same and the logits the
+    caller gets back are still logits (the reference's eval_batch returns them after the loss)."""
+    n, v = 37, 5000
+    x = torch.randn(n, v, generator=gen(90)).bfloat16()
+    t = torch.randint(0, v, (n,), generator=gen(91))
+    ref, _ = R.cross_entropy_fp32(x, t, 0, torch.full((n,), 1.0 / n))
+    for mode in ("no_grad", "no_requires_grad"):
+        xg = x.to(gpu)
+        if mode == "no_grad":
+            xg.requires_grad_(True)
+            with torch.no_grad():
+                loss = mpu.vocab_loss_fn((xg, None), t.to(gpu))
+        else:
+            loss = mpu.vocab_loss_fn(xg, t.to(gpu))
+        assert abs(loss.item() - ref.mean().item()) < 1e-4
+        assert torch.equal(xg.detach().cpu(), x), mode
+    # training: the forward consumes the logits, and autograd knows they changed
+    xg = x.to(gpu).requires_grad_(True)
+    y = xg * 1.0
+    v0 = y._version
+    mpu.vocab_loss_fn(y, t.to(gpu)).backward()
+    assert y._version > v0 and not torch.equal(y.detach().cpu(), x)
+
+
 def test_ce_one_launch_full_size_llama_vocab(gpu):
     n, v = 8192, 128256
     x = torch.empty(n, v, dtype=torch.bfloat16, device=gpu).normal_(generator=torch.Generator(device=gpu).manual_seed(1239))
@@ -767,6 +792,29 @@ def test_gemv_cut_along_k_with_workspace(gpu, set_tuning, b, n, k, epi, force, c
     if ws is not None:
         assert rel(ops.gemv(xg, wg, bg, e), y1) < TOL_BF16 / 4        # against the uncut form
         assert int(ws[:4 * ((n + 15) // 16)].count_nonzero()) == 0       # counters are back at zero
+
+
+def test_gemv_one_workspace_for_shapes_in_turn(gpu):
+    """Two cut shapes with different numbers of rows alternate on one zeroed workspace: the counters sit at a
+    fixed place, so the partial sums of the matrix with few rows never land in the other one's counters."""
+    g = gen(33)
+    b = 16
+    shapes = [(1024, 8192), (8192, 8192), (1280, 8192), (4096, 14336)]
+    need = max(_lib_bytes(b, n, k) for n, k in shapes)
+    assert need > 0 and min(_lib_bytes(b, n, k) for n, k in shapes) > 0, "every shape here is cut"
+    ws = torch.zeros(need, dtype=torch.uint8, device=gpu)
+    mats = [((torch.randn(n, k, generator=g) * 0.02).bfloat16().to(gpu), torch.randn(b, k, generator=g).bfloat16().to(gpu))
+            for n, k in shapes]
+    for rep in range(2):
+        for w, x in mats:
+            y = ops.gemv(x, w, workspace=ws)
+            assert rel(y, F.linear(x.float(), w.float())) < TOL_BF16
+    assert int(ws[:8192].view(torch.int32).abs().sum()) == 0
+
+
+def _lib_bytes(b, n, k):
+    from merak_amd import _lib
+    return _lib.lib().mtp_gemv_workspace_bytes(b, n, k, _lib.EPI_NONE)
 
 
 def test_argmax_ties_and_nan(gpu):

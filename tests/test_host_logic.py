@@ -266,3 +266,42 @@ def test_input_output_ratio_table_tags_linear_and_conv1d():
     assert isinstance(m.c_attn, ColPara) and m.c_attn.weight.shape == (48, 64)
     assert isinstance(m.lin_same, nn.Linear)                                        # untagged: left alone
     reset_tp_layer_lists()
+
+
+def test_model_parallel_rng_gives_ranks_different_shards():
+    """Device-side initialisation draws under the model-parallel generator state (layers.py:52-53): two ranks of one
+    tensor-parallel group, seeded alike, get different shards; one rank seeded twice gets the same shard; the
+    default generator is left where it was."""
+    from merak_amd.mpu.layers import _initialize_affine_weight_gpu
+    from merak_amd.mpu.random import get_rng_tracker
+
+    def shard(rank, seed=1234):
+        mpu.set_model_parallel_world_size(2)
+        mpu.set_model_parallel_rank(rank)
+        mpu.model_parallel_manual_seed(seed)
+        before = torch.get_rng_state()
+        w = torch.empty(8, 16)
+        _initialize_affine_weight_gpu(w, torch.nn.init.normal_, 0)
+        assert torch.equal(torch.get_rng_state(), before)          # the fork restores the caller's state
+        assert w.model_parallel and w.partition_dim == 0 and w.partition_stride == 1
+        return w
+
+    a, b, a2 = shard(0), shard(1), shard(0)
+    assert not torch.equal(a, b) and torch.equal(a, a2)
+    # a second draw under the same state continues the stream, as the reference's fork does
+    w1, w2 = torch.empty(4), torch.empty(4)
+    mpu.model_parallel_manual_seed(7)
+    _initialize_affine_weight_gpu(w1, torch.nn.init.normal_, 0)
+    _initialize_affine_weight_gpu(w2, torch.nn.init.normal_, 0)
+    assert not torch.equal(w1, w2)
+    # an explicit context wins; without a seeded tracker the current generator is used
+    get_rng_tracker().reset()
+    torch.manual_seed(5)
+    w3 = torch.empty(4)
+    _initialize_affine_weight_gpu(w3, torch.nn.init.normal_, 0)
+    torch.manual_seed(5)
+    assert torch.equal(w3, torch.empty(4).normal_())
+    with pytest.raises(Exception, match="already exists"):
+        t = mpu.RNGStatesTracker()
+        t.add("a", 1)
+        t.add("b", 1)

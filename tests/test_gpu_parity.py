@@ -563,6 +563,82 @@ def test_linear_fwd_bwd_vs_oracle(gpu, dtype, m, n, k):
         assert rel(acc - 1, rdw) < TOL_F32 * 10 and rel(accb - 1, rdb) < TOL_F32 * 10
 
 
+def _every_product_once(gpu, dtype, m, n, k, seed):
+    """Every 16-bit product and epilogue of the linear layers on one shape, as a dict of device tensors."""
+    x, w, b, dy = _lin_inputs(m, n, k, dtype, seed)
+    xg, wg, bg, dyg = x.to(gpu), w.to(gpu), b.to(gpu), dy.to(gpu)
+    out = {}
+    out["y"], _ = ops.linear_fwd(xg, wg, bg, ops.EPI_BIAS)
+    out["pre"], out["gelu"] = ops.linear_fwd(xg, wg, bg, ops.EPI_BIAS_GELU)
+    out["spre"], out["swiglu"] = ops.linear_fwd(xg, wg, None, ops.EPI_SWIGLU)
+    out["dx"] = ops.linear_dgrad(dyg, wg)
+    out["dw"], out["db"] = ops.linear_wgrad(dyg, xg, True)
+    acc, accb = torch.ones(n, k, device=gpu), torch.ones(n, device=gpu)
+    ops.linear_wgrad(dyg, xg, True, dw=acc, db=accb, accumulate=True)
+    out["acc"], out["accb"] = acc, accb
+    return (x, w, b, dy), out
+
+
+def _check_every_product(inputs, out, tol, what):
+    x, w, b, dy = (t.float() for t in inputs)
+    pre = R.column_parallel_linear_forward(x, w, b)[0]
+    assert rel(out["y"], pre) < tol and rel(out["pre"], pre) < tol, what
+    assert rel(out["gelu"], R.gelu_new(pre)) < tol, what
+    assert rel(out["spre"], F.linear(x, w)) < tol, what
+    assert rel(out["swiglu"], R.swiglu(out["spre"].float().cpu())) < tol, what
+    rdx, rdw, rdb = R.linear_backward(x, w, dy, True)
+    assert rel(out["dx"], rdx) < tol and rel(out["dw"], rdw) < tol and rel(out["db"], rdb) < tol, what
+    assert rel(out["acc"] - 1, rdw) < TOL_F32 * 10 and rel(out["accb"] - 1, rdb) < TOL_F32 * 10, what
+
+
+# k, n and m multiples of 64 (every product can take the 64-deep loop), then ragged in all three
+_CFG_SHAPES = [(320, 576, 448), (300, 520, 200), (1100, 1304, 2112)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("cfg", list(range(10)))
+def test_every_tile_configuration_vs_oracle(gpu, set_tuning, dtype, cfg):
+    """Each tile configuration forced in turn (one that cannot serve a shape or epilogue falls back to the
+    automatic choice): every product and epilogue against the oracle, and the same bits on a second run."""
+    set_tuning("MTP_GEMM_CFG", cfg)
+    for (m, n, k) in _CFG_SHAPES:
+        inputs, out = _every_product_once(gpu, dtype, m, n, k, 300 + cfg)
+        _check_every_product(inputs, out, TOL_BF16, (cfg, m, n, k))
+        _, again = _every_product_once(gpu, dtype, m, n, k, 300 + cfg)
+        for name in out:
+            assert torch.equal(out[name], again[name]), (cfg, m, n, k, name)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("cfg", [8, None])
+def test_stream_k_forced_vs_oracle(gpu, set_tuning, mode, cfg):
+    """Stream-K switched off, taken wherever the last round is part empty, and with every tile going through its
+    kernel: against the oracle, the same bits on every run (the pieces are summed in k order by a second kernel,
+    no atomics), and the three modes within rounding of one another."""
+    set_tuning("MTP_GEMM_SK", mode)
+    set_tuning("MTP_GEMM_CFG", cfg)
+    for (m, n, k) in _CFG_SHAPES + [(256, 512, 4096), (512, 768, 8192)]:
+        inputs, out = _every_product_once(gpu, torch.bfloat16, m, n, k, 330)
+        _check_every_product(inputs, out, TOL_BF16, (mode, cfg, m, n, k))
+        for _ in range(2):
+            _, again = _every_product_once(gpu, torch.bfloat16, m, n, k, 330)
+            for name in out:
+                assert torch.equal(out[name], again[name]), (mode, cfg, m, n, k, name)
+
+
+def test_measurement_switches_are_not_in_the_shipped_library(gpu, set_tuning):
+    """MTP_GEMM_DEBUG turns parts of the product off in a measurement build (-DMTP_MEASURE).  The library that
+    ships must not know the variable: with it set, results still match the oracle and are the bits of a run
+    without it."""
+    inputs, plain = _every_product_once(gpu, torch.bfloat16, 320, 576, 448, 340)
+    for value in (1, 2, 4, 255):
+        set_tuning("MTP_GEMM_DEBUG", value)
+        _, out = _every_product_once(gpu, torch.bfloat16, 320, 576, 448, 340)
+        _check_every_product(inputs, out, TOL_BF16, value)
+        for name in out:
+            assert torch.equal(out[name], plain[name]), (value, name)
+
+
 @pytest.mark.parametrize("dtype,m,n,k", [(torch.float32, 512, 3072, 768), (torch.bfloat16, 512, 3072, 768),
                                           (torch.bfloat16, 200, 136, 72), (torch.float32, 33, 20, 10)])
 def test_bias_gelu_epilogue(gpu, dtype, m, n, k):

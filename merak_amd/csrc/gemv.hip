@@ -30,6 +30,7 @@
 namespace {
 
 constexpr int GV_MAX_WAVES = 8;  // waves per workgroup: 8, or 4 for the register-heavy configurations
+constexpr int GV_MAX_SLICES = 8; // slices along k, one workgroup each
 
 struct ArgPart {
   float v;
@@ -478,12 +479,22 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
 
   if (MODE != 2 && gridDim.y > 1) {
     // k slices: hand the partial over with device-scope stores, count arrivals; the last slice to arrive sums
-    // all of them in slice order (its own included, read back), so the result does not depend on who is last
+    // all of them in slice order (its own included, read back), so the result does not depend on who is last.
+    // Two values per access, and a thread asks for all it will sum before it looks at the first: the sum is a
+    // single round trip to the memory-side cache whatever the batch and the number of row groups.
     constexpr int FIN = 16 * R;
+    constexpr int PER = (16 * NB * FIN / 2 + GV_THREADS - 1) / GV_THREADS;   // pairs of values per thread
     const int S = gridDim.y, cnt = B * FIN;
-    float* mine = kpart + ((int64_t)blockIdx.x * S + blockIdx.y) * cnt;
-    for (int e = tid; e < cnt; e += GV_THREADS)
-      __hip_atomic_store(mine + e, fin[e / FIN][e % FIN], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint64_t* mine = reinterpret_cast<uint64_t*>(kpart + ((int64_t)blockIdx.x * S + blockIdx.y) * cnt);
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int e = 2 * (i * GV_THREADS + tid);
+      if (e < cnt) {
+        const float lo = fin[e / FIN][e % FIN], hi = fin[(e + 1) / FIN][(e + 1) % FIN];
+        __hip_atomic_store(mine + (e >> 1), ((uint64_t)__float_as_uint(hi) << 32) | __float_as_uint(lo), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     __shared__ int last_one;
@@ -494,16 +505,31 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
     }
     __syncthreads();
     if (!last_one) return;
-    const float* all = kpart + (int64_t)blockIdx.x * S * cnt;
-    for (int e = tid; e < cnt; e += GV_THREADS) {
-      float v[8];
+    const uint64_t* all = reinterpret_cast<const uint64_t*>(kpart + (int64_t)blockIdx.x * S * cnt);
+    const int64_t slice_stride = cnt >> 1;
+    uint64_t v[PER][GV_MAX_SLICES];
 #pragma unroll
-      for (int sl = 0; sl < 8; sl++)
-        v[sl] = sl < S ? __hip_atomic_load(all + (int64_t)sl * cnt + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
-      float sum = v[0];
+    for (int i = 0; i < PER; i++) {
+      const int e = 2 * (i * GV_THREADS + tid);
 #pragma unroll
-      for (int sl = 1; sl < 8; sl++) sum += v[sl];
-      fin[e / FIN][e % FIN] = sum;
+      for (int sl = 0; sl < GV_MAX_SLICES; sl++)
+        v[i][sl] = (e < cnt && sl < S)
+                       ? __hip_atomic_load(all + sl * slice_stride + (e >> 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                       : 0ull;
+    }
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int e = 2 * (i * GV_THREADS + tid);
+      if (e < cnt) {
+        float lo = __uint_as_float((uint32_t)v[i][0]), hi = __uint_as_float((uint32_t)(v[i][0] >> 32));
+#pragma unroll
+        for (int sl = 1; sl < GV_MAX_SLICES; sl++) {   // slices beyond S hold +0: adding them changes nothing
+          lo += __uint_as_float((uint32_t)v[i][sl]);
+          hi += __uint_as_float((uint32_t)(v[i][sl] >> 32));
+        }
+        fin[e / FIN][e % FIN] = lo;
+        fin[(e + 1) / FIN][(e + 1) % FIN] = hi;
+      }
     }
     __syncthreads();
   }
@@ -714,7 +740,6 @@ struct GemvCfg {
   int D;  // k-pairs in flight per wave and step
   int S;  // slices along k, one workgroup each (needs a workspace); 1 = the workgroup walks all of k
 };
-constexpr int GV_MAX_SLICES = 8;
 
 bool depth_ok(int64_t K, int d) { return d == 1 || (K % 64 == 0 && ((K / 64) % (GV_MAX_WAVES * d)) == 0); }
 

@@ -39,9 +39,26 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3     # MI355X fp32 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# HBM bytes per launch of the largest GEMMs, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file
-# scaled by a 1 GiB copy kernel (x2.000 / x1.000): profiles/hbm_traffic_fetch_write_size.txt
-HBM_TRAFFIC_BYTES = {"gate_up.fwd": 1.763e9, "gate_up.wgrad": 1.645e9, "down.dgrad": 0.889e9}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hbm_traffic_fetch_write_size.txt")
+
+
+def measured_traffic():
+    """HBM bytes per launch from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary: its lines
+    `traffic_bytes <kernel of this file> <bytes>` and `measured_at <commit>`.  ({}, None) when the file is absent:
+    the figure is a measurement of a profiler run, never a constant of this script."""
+    rows, stamp = {}, None
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                t = line.split()
+                if len(t) >= 3 and t[0] == "traffic_bytes":
+                    rows[t[1]] = float(t[2])
+                elif len(t) >= 2 and t[0] == "measured_at":
+                    stamp = t[1]
+    except OSError:
+        pass
+    return rows, stamp
+
 
 LLAMA8B = [  # (name, K, N, epilogue)
     ("qkv", 4096, 6144, "none"),
@@ -323,6 +340,12 @@ def secondary(dev, timer, reps, with_cpu):
     eb_ms = timer.run("emb.bwd", lambda: ops.embedding_bwd(ids, dout, v, 0, v, out=dtab), reps)
     ebz_ms = timer.run("emb.bwd0", lambda: ops.embedding_bwd(ids, dout, v, 0, v), max(3, reps // 4))
     out["embedding_c4"].update({"bwd_scatter_us": round(eb_ms * 1e3, 1), "bwd_with_zero_fill_us": round(ebz_ms * 1e3, 1)})
+    # the same scatter when half of the batch is one padding id, and when every id is the same
+    ids_pad = ids.clone()
+    ids_pad[torch.randperm(n, generator=gen(13))[: n // 2].to(dev)] = 2
+    ids_one = torch.full_like(ids, 7)
+    for nm, ii in (("bwd_scatter_half_padded_us", ids_pad), ("bwd_scatter_one_id_us", ids_one)):
+        out["embedding_c4"][nm] = round(timer.run("emb." + nm, lambda: ops.embedding_bwd(ii, dout, v, 0, v, out=dtab), reps) * 1e3, 1)
     del dout, dtab
     # --- LM head + cross entropy at the C4 shape: full logits vs one chunk of rows at a time
     from merak_amd import mpu
@@ -382,7 +405,8 @@ def secondary(dev, timer, reps, with_cpu):
     ms3 = timer.run("c3.step", lambda: linear_step(w3), max(3, reps // 2))
     fl3 = sum(L["flops"] for L in w3)
     out["linear_c3_llama70b_tp8"] = {"ms_per_step": round(ms3, 4), "tflops": round(fl3 / ms3 / 1e9, 1),
-                                     "frac_bf16_peak": round(fl3 / ms3 / 1e9 / PEAK_BF16_TFLOPS, 4)}
+                                     "frac_bf16_peak": round(fl3 / ms3 / 1e9 / PEAK_BF16_TFLOPS, 4),
+                                     "tokens": 8192, "kernels": per_kernel(w3, timer, max(3, reps // 2))}
     del w3
     # --- GPT-2-small fp32 (config 1): Column 768->3072 bias+GeLU, Row 3072->768 bias
     M1 = 8192
@@ -418,9 +442,17 @@ def secondary(dev, timer, reps, with_cpu):
     p_ms = timer.run("mfma", lambda: _lib.check(_lib.lib().mtp_mfma_peak(sink.data_ptr(), 4096, iters, 0, st), "peak"), 3)
     r_ms = timer.run("mfma_r", lambda: _lib.check(_lib.lib().mtp_mfma_peak(sink.data_ptr(), 4096, iters, 1, st), "peak"), 3)
     del src, dst
-    # the nine GEMMs of the headline step through the vendor library (torch.matmul, i.e. hipBLASLt) and through
-    # this library on the same operands, launch by launch in turn so that both see the same clocks: what the
-    # board's power management grants depends on what ran in the milliseconds before
+    out["vendor_blas_same_gemms"] = vendor_compare(dev, reps)
+    out["device_reference"] = {"copy_1GiB_GBs_read_plus_write": round(2 * src_bytes / c_ms / 1e6, 1),
+                               "mfma_loop_bf16_tflops_smooth_operands": round(4096 * iters * 32 * 32 * 16 * 2 / p_ms / 1e9, 1),
+                               "mfma_loop_bf16_tflops_random_operands": round(4096 * iters * 32 * 32 * 16 * 2 / r_ms / 1e9, 1)}
+    return out
+
+
+def vendor_compare(dev, reps, kinds=("fwd", "dgrad", "wgrad")):
+    """The plain GEMMs of the headline step through the vendor library (torch.matmul, i.e. hipBLASLt) and through
+    this library on the same operands, launch by launch in turn so that both see the same clocks: what the
+    board's power management grants depends on what ran in the milliseconds before."""
     from merak_amd import ops
     w2 = build_linear_workload(dev, LLAMA8B, 4096, 100)
     rows, v_sum, o_sum, fl_sum = {}, 0.0, 0.0, 0.0
@@ -430,6 +462,8 @@ def secondary(dev, timer, reps, with_cpu):
                  ("dgrad", lambda: gdy @ L["w"], lambda: ops.linear_dgrad(gdy, L["w"])),
                  ("wgrad", lambda: gdy.t() @ L["x"], lambda: ops.linear_wgrad(gdy, L["x"], False)))
         for kind, vendor_fn, own_fn in pairs:
+            if kind not in kinds:
+                continue
             vendor_fn(), own_fn()
             torch.cuda.synchronize()
             ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(2 * reps)]
@@ -439,18 +473,15 @@ def secondary(dev, timer, reps, with_cpu):
             v_ms = statistics.mean(e0.elapsed_time(e1) for e0, e1, _ in ev)
             o_ms = statistics.mean(e1.elapsed_time(e2) for _, e1, e2 in ev)
             fl = 2.0 * L["M"] * L["N"] * L["K"]
-            rows[f"{L['name']}.{kind}"] = {"vendor_tflops": round(fl / v_ms / 1e9, 1), "this_library_tflops": round(fl / o_ms / 1e9, 1)}
+            rows[f"{L['name']}.{kind}"] = {"M": L["M"], "N": L["N"], "K": L["K"], "vendor_ms": round(v_ms, 4),
+                                           "this_library_ms": round(o_ms, 4), "vendor_tflops": round(fl / v_ms / 1e9, 1),
+                                           "this_library_tflops": round(fl / o_ms / 1e9, 1)}
             v_sum, o_sum, fl_sum = v_sum + v_ms, o_sum + o_ms, fl_sum + fl
         del gdy
-    out["vendor_blas_same_gemms"] = {"vendor_sum_ms": round(v_sum, 4), "vendor_tflops": round(fl_sum / v_sum / 1e9, 1),
-                                     "this_library_sum_ms": round(o_sum, 4), "this_library_tflops": round(fl_sum / o_sum / 1e9, 1),
-                                     "note": "plain GEMMs, alternating launches; the headline step also fuses SwiGLU into gate_up.fwd",
-                                     "per_gemm": rows}
-    del w2
-    out["device_reference"] = {"copy_1GiB_GBs_read_plus_write": round(2 * src_bytes / c_ms / 1e6, 1),
-                               "mfma_loop_bf16_tflops_smooth_operands": round(4096 * iters * 32 * 32 * 16 * 2 / p_ms / 1e9, 1),
-                               "mfma_loop_bf16_tflops_random_operands": round(4096 * iters * 32 * 32 * 16 * 2 / r_ms / 1e9, 1)}
-    return out
+    return {"vendor_sum_ms": round(v_sum, 4), "vendor_tflops": round(fl_sum / v_sum / 1e9, 1),
+            "this_library_sum_ms": round(o_sum, 4), "this_library_tflops": round(fl_sum / o_sum / 1e9, 1),
+            "note": "plain GEMMs, alternating launches; the headline step also fuses SwiGLU into gate_up.fwd",
+            "per_gemm": rows}
 
 
 def main():
@@ -462,6 +493,10 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="headline only (no secondary figures)")
     ap.add_argument("--cpu-tokens", type=int, default=4096,
                     help="tokens of the workload the CPU baseline runs (default: all 4096, about 13 s on 16 cores)")
+    ap.add_argument("--only", choices=["gemm-fwd-vs-vendor", "gemm-vs-vendor"], default=None,
+                    help="launch nothing but the forward GEMMs (or all nine plain GEMMs) of the headline step, each "
+                         "through the vendor library and through this one in turn, and print their times: the "
+                         "program to put behind `rocprofv3 --pmc ... --` or `--kernel-trace` for a counter comparison")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (no collectives, one rank's share "
@@ -474,6 +509,12 @@ def main():
     _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.only:
+        kinds = ("fwd",) if args.only == "gemm-fwd-vs-vendor" else ("fwd", "dgrad", "wgrad")
+        res = vendor_compare(dev, max(3, args.steps), kinds)
+        print(json.dumps({"mode": args.only, "launches_per_gemm_and_library": 2 * max(3, args.steps) + 1, **res}))
+        return
 
     M = 4096
     work = build_linear_workload(dev, LLAMA8B, M, 20)
@@ -494,9 +535,12 @@ def main():
     kernels = per_kernel(work, timer, reps)
     gemms = [k for k in kernels if "tflops" in k]
     dom = max(gemms, key=lambda k: k["ms"])
+    traffic, stamp = measured_traffic()
     roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4),
-                "traffic": HBM_TRAFFIC_BYTES.get(dom["kernel"]),
+                "traffic": traffic.get(dom["kernel"]),
+                "traffic_source": (f"profiles/hbm_traffic_fetch_write_size.txt, measured at commit {stamp}"
+                                   if dom["kernel"] in traffic else None),
                 "launch_ms": dom["ms"], "flops_per_launch": 2.0 * dom["M"] * dom["N"] * dom["K"]}
     # what the matrix cores sustain on this board with no memory traffic at all (register-resident MFMA loop on
     # operands of random sign and mantissa): the chip runs against its power limit well below the published peak

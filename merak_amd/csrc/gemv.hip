@@ -271,37 +271,93 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
     load_w(pq0, a);
     load_x(pq0, b);
   };
+  // The two halves of group r's k-pair as MFMA operands.  GUARD: a0 / a1 are the halves themselves.  Otherwise pick
+  // them per lane out of loads A and B; the second half then sits 8 lanes away inside its group of 16 (row i^8 at
+  // position i): one DPP rotation per register puts it in place.
+  auto halves = [&](const bf16x8_t& a0, const bf16x8_t& a1, bf16x8_t& h0, bf16x8_t& h1) {
+    h0 = a0;
+    h1 = a1;
+    if (!GUARD) {
+      h0 = low ? a0 : a1;
+      const u32x4_t t = __builtin_bit_cast(u32x4_t, low ? a1 : a0);
+      u32x4_t rt;
+      rt.x = rot8_in_row(t.x); rt.y = rot8_in_row(t.y); rt.z = rot8_in_row(t.z); rt.w = rot8_in_row(t.w);
+      h1 = __builtin_bit_cast(bf16x8_t, rt);
+    }
+  };
+  // (the single-set loop takes the first halves of all batch tiles before the second ones: two dependent
+  // products never stand next to each other inside its pinned sections)
+  auto multiply_group = [&](int r, const bf16x8_t& h0, const bf16x8_t& h1, bf16x8_t (&bx)[XS][NB][2]) {
+    if constexpr (PP) {
+      if (MIX) {
+        // rows 0-7 (gate) belong to k position 0, rows 8-15 (up) to position 1: both products, two accumulators
+        acc[r][0] = X::mfma16(h0, bx[0][0][0], acc[r][0]);
+        acc[r][0] = X::mfma16(h1, bx[0][0][1], acc[r][0]);
+        acc_up[r] = X::mfma16(h0, bx[XS - 1][0][0], acc_up[r]);
+        acc_up[r] = X::mfma16(h1, bx[XS - 1][0][1], acc_up[r]);
+        return;
+      }
+      const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+        acc[r][nb] = X::mfma16(h0, bx[xs][nb][0], acc[r][nb]);
+        acc[r][nb] = X::mfma16(h1, bx[xs][nb][1], acc[r][nb]);
+      }
+    } else {
+      if (MIX) {
+        acc[r][0] = X::mfma16(h0, bx[0][0][0], acc[r][0]);
+        acc_up[r] = X::mfma16(h0, bx[XS - 1][0][0], acc_up[r]);
+        acc[r][0] = X::mfma16(h1, bx[0][0][1], acc[r][0]);
+        acc_up[r] = X::mfma16(h1, bx[XS - 1][0][1], acc_up[r]);
+        return;
+      }
+      const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) acc[r][nb] = X::mfma16(h0, bx[xs][nb][0], acc[r][nb]);
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) acc[r][nb] = X::mfma16(h1, bx[xs][nb][1], acc[r][nb]);
+    }
+  };
   auto multiply = [&](bf16x8_t (&a_cur)[D][R][2], bf16x8_t (&b_cur)[D][XS][NB][2]) {
 #pragma unroll
     for (int d = 0; d < D; d++)
 #pragma unroll
       for (int r = 0; r < R; r++) {
-        // GUARD: a[0] / a[1] are the halves themselves.  Otherwise pick them per lane out of loads A and
-        // B; the second half then sits 8 lanes away inside its group of 16 (row i^8 at position i): one
-        // DPP rotation per register puts it in place.
-        bf16x8_t h0 = a_cur[d][r][0], h1 = a_cur[d][r][1];
-        if (!GUARD) {
-          h0 = low ? a_cur[d][r][0] : a_cur[d][r][1];
-          const u32x4_t t = __builtin_bit_cast(u32x4_t, low ? a_cur[d][r][1] : a_cur[d][r][0]);
-          u32x4_t rt;
-          rt.x = rot8_in_row(t.x); rt.y = rot8_in_row(t.y); rt.z = rot8_in_row(t.z); rt.w = rot8_in_row(t.w);
-          h1 = __builtin_bit_cast(bf16x8_t, rt);
-        }
-        if (MIX) {
-          // rows 0-7 (gate) belong to k position 0, rows 8-15 (up) to position 1: both products, two accumulators
-          acc[r][0] = X::mfma16(h0, b_cur[d][0][0][0], acc[r][0]);
-          acc[r][0] = X::mfma16(h1, b_cur[d][0][0][1], acc[r][0]);
-          acc_up[r] = X::mfma16(h0, b_cur[d][XS - 1][0][0], acc_up[r]);
-          acc_up[r] = X::mfma16(h1, b_cur[d][XS - 1][0][1], acc_up[r]);
-          continue;
-        }
-        const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-          acc[r][nb] = X::mfma16(h0, b_cur[d][xs][nb][0], acc[r][nb]);
-          acc[r][nb] = X::mfma16(h1, b_cur[d][xs][nb][1], acc[r][nb]);
-        }
+        bf16x8_t h0, h1;
+        halves(a_cur[d][r][0], a_cur[d][r][1], h0, h1);
+        multiply_group(r, h0, h1, b_cur[d]);
       }
+  };
+  // One step with a single set of weight registers: group after group, the two registers of a group are taken,
+  // asked for again at once for the next step (pair pq_next), and only then multiplied; the order is pinned, so the
+  // wait in front of a group covers that group's two loads alone and fifteen of sixteen requests stay in flight
+  // while the step is multiplied.  (Left to itself the compiler gathers the selects of all groups at the top of
+  // the loop behind one wait for every load: nothing in flight during the products.)  The X fragments of the
+  // next step are asked for first, into the second set.
+  auto roll_step = [&](int64_t pq_next, bf16x8_t (&a)[D][R][2], bf16x8_t (&b_cur)[D][XS][NB][2],
+                       bf16x8_t (&b_nxt)[D][XS][NB][2]) {
+    load_x(pq_next, b_nxt);
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+      int64_t ks[2];
+      pair_k(pq_next, d, ks);
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        bf16x8_t h0, h1;
+        halves(a[d][r][0], a[d][r][1], h0, h1);
+        __builtin_amdgcn_sched_barrier(0);   // the two registers are free from here on: the requests reuse them
+        if (MIX) {
+          a[d][r][0] = load_frag_nt(wbase[r] + ks[0] + offa[r], true);
+          a[d][r][1] = load_frag_nt(wbase[r] + ks[1] + offb[r], true);
+        } else {
+          const int64_t k = ks[(XS == 2 && r >= R / 2) ? 1 : 0];
+          a[d][r][0] = load_frag_nt(wbase[r] + k + offa[r], !GUARD || (k + 8 * lg < K));
+          a[d][r][1] = load_frag_nt(wbase[r] + k + offb[r], !GUARD || (k + 32 + 8 * lg < K));
+        }
+        multiply_group(r, h0, h1, b_cur[d]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
   };
 
   // NORM prologue, part 1: everything it reads is asked for before the first weights, folded after them, so
@@ -406,25 +462,21 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
         multiply(a_s0, b_s0);
       }
     } else {
-      for (int64_t it = 1; it < n_it; it++) {
+      // one set of weight registers (a_s0), two of X fragments used in turn
+      int64_t it = 1;
+      for (; it + 1 < n_it; it += 2) {
         advance();
-        load_set(pq, a_s1, b_s1);
-        multiply(a_s0, b_s0);
-#pragma unroll
-        for (int d = 0; d < D; d++) {
-#pragma unroll
-          for (int r = 0; r < R; r++)
-#pragma unroll
-            for (int hf = 0; hf < 2; hf++) a_s0[d][r][hf] = a_s1[d][r][hf];
-#pragma unroll
-          for (int xs = 0; xs < XS; xs++)
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-              for (int hf = 0; hf < 2; hf++) b_s0[d][xs][nb][hf] = b_s1[d][xs][nb][hf];
-        }
+        roll_step(pq, a_s0, b_s0, b_s1);
+        advance();
+        roll_step(pq, a_s0, b_s1, b_s0);
       }
-      multiply(a_s0, b_s0);
+      if (it < n_it) {
+        advance();
+        roll_step(pq, a_s0, b_s0, b_s1);
+        multiply(a_s0, b_s1);
+      } else {
+        multiply(a_s0, b_s0);
+      }
     }
   }
 
@@ -759,18 +811,34 @@ GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode, bool may_split 
   // cut instead (each slice reads only its part of X); every wave of a slice gets the same number of pairs.
   // Measured (B = 16 and 32): 4096x14336 gains 17-23 %, matrices with K = 4096 lose (too little k per slice to
   // pay for the hand-over), batches up to 8 gain nothing.
-  if (may_split && mode != 2 && K % 64 == 0 && groups / c.R < 190 &&
-      groups * (int64_t)sizeof(int32_t) <= GV_COUNTER_BYTES) {
+  // Above 16 rows the cut is tried with 4 row groups (8 waves) first: 4096x14336 at 32 rows as 64 row blocks x 4
+  // slices takes 26.7 us, as 32 x 8 (8 groups, 4 waves) 29.6 us.  MTP_GEMV_R forces the row groups here too.
+  if (may_split && mode != 2 && K % 64 == 0 && groups * (int64_t)sizeof(int32_t) <= GV_COUNTER_BYTES) {
     int want = (B > 8 && K >= 8192) ? 0 : -1;
-    static MtpTune tune_s("MTP_GEMV_S");
+    static MtpTune tune_s("MTP_GEMV_S"), tune_r0("MTP_GEMV_R");
     want = tune_s.get(want);
-    const int waves = c.R >= 8 ? 4 : GV_MAX_WAVES;
-    for (int sl = 2; want >= 0 && sl <= GV_MAX_SLICES; sl *= 2) {
-      if ((K / 64) % (sl * waves) != 0 || (want == 0 && K / 64 / (sl * waves) < 6)) break;
-      c.S = sl;
-      if (want ? sl >= want : groups / c.R * sl >= 190) break;
+    const int forced_r = tune_r0.get(0);
+    const int cand[2] = {B > 16 ? 4 : c.R, c.R};
+    GemvCfg best = c;
+    int64_t best_wgs = 0;
+    for (int ci = 0; ci < 2 && want >= 0; ci++) {
+      GemvCfg t = c;
+      t.R = (forced_r == 2 || forced_r == 4 || forced_r == 8) ? forced_r : cand[ci];
+      if (groups / t.R >= 190) continue;
+      const int waves = t.R >= 8 ? 4 : GV_MAX_WAVES;
+      for (int sl = 2; sl <= GV_MAX_SLICES; sl *= 2) {
+        if ((K / 64) % (sl * waves) != 0 || (want == 0 && K / 64 / (sl * waves) < 6)) break;
+        t.S = sl;
+        if (want ? sl >= want : groups / t.R * sl >= 190) break;
+      }
+      const int64_t wgs = groups / t.R * t.S;
+      if (t.S > 1 && wgs > best_wgs) {
+        best = t;
+        best_wgs = wgs;
+      }
+      if (best_wgs >= 190) break;
     }
-    if (c.S > 1) return c;
+    if (best.S > 1) return best;
   }
   while (c.R > 1 && groups / c.R < 190) c.R >>= 1;
   if (mode == 1 && c.R < 2) c.R = 2;

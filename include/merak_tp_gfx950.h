@@ -107,7 +107,12 @@ int mtp_linear_bias_grad(const void* dy, void* db, int64_t M, int64_t N,
  * meet in the scratch and a second small kernel adds them up in k order and
  * writes the tile, so results are reproducible bit for bit from run to run
  * (they may differ in the last bit from the call without scratch, which sums
- * each tile in one piece).
+ * each tile in one piece).  On the fp32 path a product with fewer 128x128
+ * output tiles than compute units and a long reduction (a weight gradient) is
+ * cut into up to 8 slices along k, one workgroup per tile and slice; the
+ * slices meet in the scratch and a second kernel adds them in slice order
+ * (reproducible bit for bit as well); it takes a scratch of any size and cuts
+ * only when the slices fit.
  * workspace: 16-byte aligned, mtp_linear_workspace_bytes() bytes (about 138 MB,
  * shape independent); its contents on entry do not matter.  Launches that
  * share a workspace must not overlap (one workspace per stream).  NULL or too small:

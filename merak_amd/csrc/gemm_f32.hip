@@ -37,6 +37,12 @@ struct F32Args {
   int M, N, K;
   int64_t lda, ldb, ldc;
   int accumulate;
+  // k slices (gridDim.y > 1): slice y multiplies k in [y * kslice, min(K, (y + 1) * kslice)) and stores its tile, as
+  // it is, into part + y * M * N (row length N) and its row sums into part_rowsum + y * M; f32_slices_sum_kernel
+  // adds the slices up in slice order
+  int kslice;
+  float* part;
+  float* part_rowsum;
 };
 
 // One operand tile of ROWS (rows of A / rows of B; 128 or 64) x 16 k.
@@ -113,7 +119,19 @@ struct FOperand {
 };
 
 template <int ALAY, int BLAY, int BM, int BN>
-__global__ __launch_bounds__(256) void gemm_f32_kernel(const F32Args p) {
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const F32Args q) {
+  F32Args p = q;
+  if (gridDim.y > 1) {
+    const int k0 = (int)blockIdx.y * q.kslice;
+    p.K = min(q.K - k0, q.kslice);
+    p.A = q.A + (ALAY == LAY_ROW ? (int64_t)k0 : (int64_t)k0 * q.lda);
+    p.B = q.B + (BLAY == LAY_ROW ? (int64_t)k0 : (int64_t)k0 * q.ldb);
+    p.C = q.part + (int64_t)blockIdx.y * q.M * q.N;
+    p.ldc = q.N;
+    p.bias = nullptr;
+    p.accumulate = 0;
+    p.rowsum = q.rowsum ? q.part_rowsum + (int64_t)blockIdx.y * q.M : nullptr;
+  }
   using AOp = FOperand<ALAY, BM>;
   using BOp = FOperand<BLAY, BN>;
   constexpr int STAGE = AOp::BYTES + BOp::BYTES;
@@ -247,21 +265,67 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const F32Args p) {
   }
 }
 
+// C[m][n] (+)= sum over the slices, in slice order, (+ bias[n]); rowsum likewise.  Four columns per thread.
+__global__ __launch_bounds__(256) void f32_slices_sum_kernel(const F32Args p, int S) {
+  const int64_t quads = ((int64_t)p.M * p.N) >> 2;   // N % 4 == 0 on this path
+  const int64_t slice = (int64_t)p.M * p.N;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < quads; i += (int64_t)gridDim.x * 256) {
+    f32x4_t v = *reinterpret_cast<const f32x4_t*>(p.part + 4 * i);
+    for (int sl = 1; sl < S; sl++) v += *reinterpret_cast<const f32x4_t*>(p.part + sl * slice + 4 * i);
+    const int64_t m = (4 * i) / p.N, n = (4 * i) - m * p.N;
+    if (p.bias) v += f32x4_t{p.bias[n], p.bias[n + 1], p.bias[n + 2], p.bias[n + 3]};
+    float* c = p.C + m * p.ldc + n;
+    if (p.accumulate) v += f32x4_t{c[0], c[1], c[2], c[3]};
+    c[0] = v.x; c[1] = v.y; c[2] = v.z; c[3] = v.w;
+  }
+  if (p.rowsum) {
+    for (int64_t m = (int64_t)blockIdx.x * 256 + threadIdx.x; m < p.M; m += (int64_t)gridDim.x * 256) {
+      float t = p.part_rowsum[m];
+      for (int sl = 1; sl < S; sl++) t += p.part_rowsum[(int64_t)sl * p.M + m];
+      p.rowsum[m] = p.accumulate ? p.rowsum[m] + t : t;
+    }
+  }
+}
+
 template <int ALAY, int BLAY, int BM, int BN>
-int launch_f32_tile(const F32Args& a, hipStream_t s) {
+int launch_f32_tile(const F32Args& a, hipStream_t s, int slices = 1) {
   const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
-  hipLaunchKernelGGL((gemm_f32_kernel<ALAY, BLAY, BM, BN>), dim3((unsigned)tiles), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((gemm_f32_kernel<ALAY, BLAY, BM, BN>), dim3((unsigned)tiles, (unsigned)slices), dim3(256), 0, s, a);
   MTP_CHECK_LAUNCH("gemm_f32");
+  if (slices > 1) {
+    const int64_t quads = ((int64_t)a.M * a.N) >> 2;
+    const unsigned wgs = (unsigned)((quads + 255) / 256 < 2048 ? (quads + 255) / 256 : 2048);
+    hipLaunchKernelGGL(f32_slices_sum_kernel, dim3(wgs ? wgs : 1u), dim3(256), 0, s, a, slices);
+    MTP_CHECK_LAUNCH("gemm_f32 slices");
+  }
   return MTP_OK;
 }
 
 // 128x128 unless that leaves CUs idle: three workgroups fit a CU, so below 512 tiles the tile is halved
 // along the longer side, and once more if that is still not enough.
+// Fewer 128x128 output tiles than CUs and a long k (the weight gradient of an fp32 layer: 3072 x 768 outputs over
+// 8192 tokens): with a workspace the 128x128 tiling is kept and k is cut into up to 8 slices of at least 512, one
+// workgroup per (tile, slice), until about a thousand workgroups exist; a second kernel adds the slices in slice
+// order (bit-reproducible).  Measured on 3072 x 768 x 8192: 441 us as 576 tiles of 64x64 (which read every operand
+// element twice as often per flop), 521 / 390 / 340 us with 2 / 4 / 8 slices.
+// MTP_GEMM_F32_SLICES = 1 switches the cut off, 2 / 4 / 8 force it.
 template <int ALAY, int BLAY>
-int launch_f32(const F32Args& a, hipStream_t s) {
+int launch_f32(F32Args a, hipStream_t s, void* ws, int64_t ws_bytes) {
   auto tiles = [&](int bm, int bn) { return (int64_t)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
-  static MtpTune tune_tile("MTP_GEMM_F32_TILE");
+  static MtpTune tune_tile("MTP_GEMM_F32_TILE"), tune_slices("MTP_GEMM_F32_SLICES");
   const int force = tune_tile.get(0);  // 1..4 picks a tile
+  const int want = tune_slices.get(0);
+  if (ws && !force && a.N % 4 == 0 && (want > 1 || tiles(128, 128) < 256)) {
+    int S = 1;
+    while (S < 8 && (want ? S < want : tiles(128, 128) * S < 1024) && a.K / (2 * S) >= 512) S *= 2;
+    const int64_t need = (int64_t)S * ((int64_t)a.M * a.N + a.M) * 4;
+    if (S > 1 && need <= ws_bytes && want != 1) {
+      a.kslice = (((a.K + S - 1) / S) + FBK - 1) / FBK * FBK;   // whole k-tiles per slice
+      a.part = static_cast<float*>(ws);
+      a.part_rowsum = a.part + (int64_t)S * a.M * a.N;
+      return launch_f32_tile<ALAY, BLAY, 128, 128>(a, s, S);
+    }
+  }
   if (force == 1 || (!force && tiles(128, 128) >= 512)) return launch_f32_tile<ALAY, BLAY, 128, 128>(a, s);
   const bool tall = a.M >= a.N;
   if (force == 2 || force == 3 || (!force && tiles(tall ? 64 : 128, tall ? 128 : 64) >= 512)) {
@@ -276,16 +340,17 @@ int launch_f32(const F32Args& a, hipStream_t s) {
 // kind 0: C[M,N] = A[M,K] B[N,K]^T (+bias); 1: C[M,N] = A[M,K] B[K,N]; 2: C[M,N] (+)= A[K,M]^T B[K,N] and,
 // if rowsum is given, rowsum[m] (+)= sum_k A[k,m]
 int mtp_gemm_f32(int kind, const float* A, int64_t lda, const float* B, int64_t ldb, const float* bias, float* C,
-                 float* rowsum, int64_t ldc, int64_t M, int64_t N, int64_t K, int accumulate, hipStream_t s) {
+                 float* rowsum, int64_t ldc, int64_t M, int64_t N, int64_t K, int accumulate, void* ws, int64_t ws_bytes,
+                 hipStream_t s) {
   F32Args a{};
   a.A = A; a.B = B; a.bias = bias; a.C = C; a.rowsum = rowsum;
   a.M = (int)M; a.N = (int)N; a.K = (int)K;
   a.lda = lda; a.ldb = ldb; a.ldc = ldc;
   a.accumulate = accumulate;
   switch (kind) {
-    case 0: return launch_f32<LAY_ROW, LAY_ROW>(a, s);
-    case 1: return launch_f32<LAY_ROW, LAY_COL>(a, s);
-    case 2: return launch_f32<LAY_COL, LAY_COL>(a, s);
+    case 0: return launch_f32<LAY_ROW, LAY_ROW>(a, s, ws, ws_bytes);
+    case 1: return launch_f32<LAY_ROW, LAY_COL>(a, s, ws, ws_bytes);
+    case 2: return launch_f32<LAY_COL, LAY_COL>(a, s, ws, ws_bytes);
   }
   mtp_set_error("gemm_f32: unknown kind %d", kind);
   return MTP_EINVAL;

@@ -16,8 +16,10 @@ int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64
 int mtp_gemm_generic(const void* A, int64_t sam, int64_t sak, const void* B, int64_t sbn, int64_t sbk,
                      const void* bias, void* C, int64_t ldc, int64_t M, int64_t N, int64_t K, int dtype, int out_dtype,
                      int accumulate, hipStream_t s);
+// ws: scratch for the cut along k (any size: the cut is taken when it fits), or null
 int mtp_gemm_f32(int kind, const float* A, int64_t lda, const float* B, int64_t ldb, const float* bias, float* C,
-                 float* rowsum, int64_t ldc, int64_t M, int64_t N, int64_t K, int accumulate, hipStream_t s);
+                 float* rowsum, int64_t ldc, int64_t M, int64_t N, int64_t K, int accumulate, void* ws, int64_t ws_bytes,
+                 hipStream_t s);
 int mtp_colsum(const void* dy, void* db, int64_t M, int64_t N, int dtype, int out_dtype, int accumulate,
                hipStream_t s);
 int mtp_act_fwd(const void* y, void* act, int64_t M, int64_t N, int dtype, int swiglu, hipStream_t s);
@@ -28,6 +30,8 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 // the scratch is used only when it is large enough and aligned; otherwise the call runs as without one
 void* usable_ws(void* ws, int64_t bytes) { return (ws && bytes >= MTP_LINEAR_WS_BYTES && aligned16(ws)) ? ws : nullptr; }
+// the fp32 products take a scratch of any size (their cut along k is sized to it)
+void* f32_ws(void* ws, int64_t bytes) { return (ws && bytes > 0 && aligned16(ws)) ? ws : nullptr; }
 
 int check_dims(const char* what, int64_t M, int64_t N, int64_t K, int dtype) {
   MTP_REQUIRE(M >= 0 && N >= 1 && K >= 1, MTP_EINVAL, "%s: M=%lld N=%lld K=%lld", what, (long long)M, (long long)N,
@@ -88,7 +92,8 @@ extern "C" int mtp_linear_fwd_ws(const void* x, const void* w, const void* bias,
   if (dtype == MTP_F32 && f32_fast_ok(x, w, K, K, 0, 0) && K * 4 * 128 < (1ll << 31)) {
     void* pre32 = y ? y : (epilogue != MTP_EPI_SWIGLU ? act : nullptr);
     MTP_REQUIRE(pre32, MTP_EUNSUPPORTED, "linear_fwd: this shape needs the pre-activation buffer y");
-    rc = mtp_gemm_f32(0, (const float*)x, K, (const float*)w, K, (const float*)use_bias, (float*)pre32, nullptr, N, M, N, K, 0, s);
+    rc = mtp_gemm_f32(0, (const float*)x, K, (const float*)w, K, (const float*)use_bias, (float*)pre32, nullptr, N, M, N, K, 0,
+                      f32_ws(workspace, workspace_bytes), workspace_bytes, s);
     if (rc) return rc;
     if (has_act) return mtp_act_fwd(pre32, act, M, N, dtype, epilogue == MTP_EPI_SWIGLU, s);
     return MTP_OK;
@@ -121,7 +126,8 @@ extern "C" int mtp_linear_dgrad_ws(const void* dy, const void* w, void* dx, void
     if (rc != MTP_EUNSUPPORTED) return rc;
   }
   if (dtype == MTP_F32 && f32_fast_ok(dy, w, N, K, 0, N * K * 4) && N * 4 * 128 < (1ll << 31))
-    return mtp_gemm_f32(1, (const float*)dy, N, (const float*)w, K, nullptr, (float*)dx, nullptr, K, M, K, N, 0, s);
+    return mtp_gemm_f32(1, (const float*)dy, N, (const float*)w, K, nullptr, (float*)dx, nullptr, K, M, K, N, 0,
+                        f32_ws(workspace, workspace_bytes), workspace_bytes, s);
   // dX[m,k] = sum_n dY[m,n] W[n,k]: A = dY (N,1), B(k,n) = W[n*K + k]
   return mtp_gemm_generic(dy, N, 1, w, 1, K, nullptr, dx, K, M, K, N, dtype, dtype, 0, s);
 }
@@ -149,7 +155,7 @@ extern "C" int mtp_linear_wgrad_ws(const void* dy, const void* x, void* dw, void
   if (dtype == MTP_F32 && dw_dtype == MTP_F32 && M > 0 && f32_fast_ok(dy, x, N, K, M * N * 4, M * K * 4)) {
     // the bias gradient (column sums of dY = row sums of the A operand) rides along in the first tile column
     return mtp_gemm_f32(2, (const float*)dy, N, (const float*)x, K, nullptr, (float*)dw, (float*)db, K, N, K, M,
-                        accumulate, s);
+                        accumulate, f32_ws(workspace, workspace_bytes), workspace_bytes, s);
   }
   // dW[n,k] = sum_m dY[m,n] X[m,k]: A(n,m) = dY[m*N + n], B(k,m) = X[m*K + k]; M == 0 writes zeros
   rc = mtp_gemm_generic(dy, 1, N, x, 1, K, nullptr, dw, K, N, K, M, dtype, dw_dtype, accumulate, s);

@@ -66,9 +66,9 @@ _linear_ws_cache = {}
 
 
 def linear_workspace(dev: torch.device) -> torch.Tensor:
-    """Scratch of the 16-bit linear products for the current stream of `dev` (stream-K: tiles whose k range
-    several workgroups share meet there).  One buffer per (device, stream), allocated at first use and kept:
-    launches on one stream are ordered, so they may share it."""
+    """Scratch of the linear products for the current stream of `dev` (16-bit: stream-K, tiles whose k range
+    several workgroups share meet there; fp32: the slices of a product that is cut along k).  One buffer per
+    (device, stream), allocated at first use and kept: launches on one stream are ordered, so they may share it."""
     idx = dev.index if dev.index is not None else torch.cuda.current_device()
     key = (idx, torch.cuda.current_stream(dev).cuda_stream)
     ws = _linear_ws_cache.get(key)
@@ -79,9 +79,7 @@ def linear_workspace(dev: torch.device) -> torch.Tensor:
 
 
 def _ws_args(t: torch.Tensor, dev: torch.device):
-    """(pointer, bytes) of the scratch for a product on tensors like t; fp32 products take none"""
-    if t.dtype == torch.float32:
-        return None, 0
+    """(pointer, bytes) of the scratch for a product on tensors like t"""
     ws = linear_workspace(dev)
     return ws.data_ptr(), ws.numel()
 

@@ -626,6 +626,35 @@ def test_stream_k_forced_vs_oracle(gpu, set_tuning, mode, cfg):
                 assert torch.equal(out[name], again[name]), (mode, cfg, m, n, k, name)
 
 
+@pytest.mark.parametrize("slices", [1, 2, 4, 8, None])
+def test_fp32_products_cut_along_k(gpu, set_tuning, slices):
+    """fp32 products with few output tiles and a long k are cut into slices along k (one workgroup per tile and
+    slice, a second kernel adds the slices in slice order): switched off, forced to 2 / 4 / 8 and as chosen, against
+    the oracle, with bias, bias gradient and accumulation, ragged shapes included, and the same bits on every run."""
+    set_tuning("MTP_GEMM_F32_SLICES", slices)
+    for (m, n, k) in ((4096, 768, 256), (8192, 384, 132), (2100, 260, 520)):
+        x, w, b, dy = _lin_inputs(m, n, k, torch.float32, 350)
+        xg, wg, bg, dyg = x.to(gpu), w.to(gpu), b.to(gpu), dy.to(gpu)
+        rdx, rdw, rdb = R.linear_backward(x, w, dy, True)
+        outs = []
+        for _ in range(2):
+            dw, db = ops.linear_wgrad(dyg, xg, True)                      # k of this product = m tokens
+            acc, accb = torch.ones(n, k, device=gpu), torch.ones(n, device=gpu)
+            ops.linear_wgrad(dyg, xg, True, dw=acc, db=accb, accumulate=True)
+            y, _ = ops.linear_fwd(dyg, wg.t().contiguous(), None, ops.EPI_NONE)   # [m, k] = dy w: k of the product = n
+            outs.append((dw, db, acc, accb, y))
+        dw, db, acc, accb, y = outs[0]
+        assert rel(dw, rdw) < TOL_F32 and rel(db, rdb) < TOL_F32, (slices, m, n, k)
+        assert rel(acc - 1, rdw) < TOL_F32 * 10 and rel(accb - 1, rdb) < TOL_F32 * 10, (slices, m, n, k)
+        assert rel(y, rdx) < TOL_F32, (slices, m, n, k)
+        for a, b2 in zip(outs[0], outs[1]):
+            assert torch.equal(a, b2), (slices, m, n, k)
+    # a product with a bias whose k is long: forward of a narrow layer over many features
+    x, w, b, _ = _lin_inputs(96, 200, 4096, torch.float32, 351)
+    y, _ = ops.linear_fwd(x.to(gpu), w.to(gpu), b.to(gpu), ops.EPI_BIAS)
+    assert rel(y, R.column_parallel_linear_forward(x, w, b)[0]) < TOL_F32
+
+
 def test_measurement_switches_are_not_in_the_shipped_library(gpu, set_tuning):
     """MTP_GEMM_DEBUG turns parts of the product off in a measurement build (-DMTP_MEASURE).  The library that
     ships must not know the variable: with it set, results still match the oracle and are the bits of a run

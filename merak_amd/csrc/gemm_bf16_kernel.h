@@ -1682,6 +1682,20 @@ constexpr bool cfg_valid(int c) {
 // their address in the offset field, see dma16_at)
 inline bool q_loop_ok(const GemmArgs& a) { return a.K % QBK == 0 && a.lda >= 128 && a.ldb >= 128; }
 
+// Mixed tiling for the 64-deep loop.  One and a half rounds of 256x256 tiles take the time of two (QKV of
+// Llama-3-8B: 384 tiles).  Where the tiles of the half-empty round form whole tile columns (or rows) of the output,
+// the product is launched in two parts instead: the whole round on the 64-deep loop, the remaining columns (rows)
+// as twice as many 256x128 (128x256) tiles of the 32-deep ring loop, which fit one round and take 0.72-0.78 of a
+// full tile's time.  Measured: QKV forward 4096 x 6144 x 4096 1215 -> 1332 TFLOP/s, its weight gradient 1210 ->
+// 1258 (the 256x192 tiling they ran on before: 1150-1165).  Not with the SwiGLU epilogue (its tiles interleave
+// two column ranges); the bias gradient (row sums of A) only splits along rows.  MTP_GEMM_MIXED = 0 switches it off.
+struct MixedSplit {
+  int dim;   // 0: none, 1: columns [at, N) go to the second launch, 2: rows [at, M)
+  int at;
+};
+template <int EPI>
+MixedSplit plan_mixed(const GemmArgs& a);
+
 template <int EPI>
 int pick_config(const GemmArgs& a) {
   static MtpTune tune_cfg("MTP_GEMM_CFG"), tune_skip("MTP_GEMM_SKIP");
@@ -1700,13 +1714,29 @@ int pick_config(const GemmArgs& a) {
     const int64_t tiles = ((a.M + t.bm - 1) / t.bm) * ((span + bn_span - 1) / bn_span);
     const int64_t rounds = (tiles + 255) / 256;
     if (!cfg_valid<EPI>(c) || (t.q != 0 && !q_loop_ok(a))) continue;
-    const double cost = (double)rounds * t.bm * t.bn / t.eff;
+    double cost = (double)rounds * t.bm * t.bn / t.eff;
+    if (t.q == 16 && t.nw == 4 && plan_mixed<EPI>(a).dim != 0) cost = ((double)(tiles / 256) + 0.78) * t.bm * t.bn / t.eff;
     if (cost < best_t * 0.999) {
       best_t = cost;
       best = c;
     }
   }
   return best;
+}
+
+template <int EPI>
+MixedSplit plan_mixed(const GemmArgs& a) {
+  static MtpTune tune_mixed("MTP_GEMM_MIXED");
+  if (tune_mixed.get(1) == 0 || EPI == MTP_EPI_SWIGLU || !q_loop_ok(a)) return MixedSplit{0, 0};
+  const int tiles_m = (a.M + 255) / 256, tiles_n = (a.N + 255) / 256;
+  const int64_t tiles = (int64_t)tiles_m * tiles_n;
+  const int R = (int)(tiles % 256);
+  // only behind a single whole round: behind three, the half-empty round already costs less than a full one
+  // (down dgrad 4096 x 14336 x 4096, 3.5 rounds: 339 us in one launch, 346 us in two)
+  if (tiles / 256 != 1 || R == 0 || R > 128) return MixedSplit{0, 0};
+  if (EPI != EPI_ROWSUM && R % tiles_m == 0 && cfg_valid<EPI>(3)) return MixedSplit{1, (tiles_n - R / tiles_m) * 256};
+  if (R % tiles_n == 0 && cfg_valid<EPI>(4)) return MixedSplit{2, (tiles_m - R / tiles_n) * 256};
+  return MixedSplit{0, 0};
 }
 
 // Stream-K for a 256x256 tiling that leaves most compute units without a tile: the k-tiles of all tiles, taken as
@@ -1786,6 +1816,33 @@ int launch_typed(GemmArgs a, hipStream_t s) {
 #endif
   int c = pick_config<EPI>(a);
   if (!cfg_valid<EPI>(c)) c = 0;
+  static MtpTune tune_forced("MTP_GEMM_CFG");
+  if (c == 8 && !tune_forced.is_set()) {
+    const MixedSplit ms = plan_mixed<EPI>(a);
+    constexpr int64_t esz = OUT == OUT_F32 ? 4 : 2;
+    if (ms.dim == 1) {
+      GemmArgs a1 = a, a2 = a;
+      a1.N = ms.at;
+      a2.N = a.N - ms.at;
+      a2.B = a.B + (BLAY == LAY_ROW ? (int64_t)ms.at * a.ldb : (int64_t)ms.at);
+      a2.C = a.C ? (char*)a.C + (int64_t)ms.at * esz : nullptr;
+      a2.C2 = a.C2 ? (char*)a.C2 + (int64_t)ms.at * 2 : nullptr;
+      a2.bias = a.bias ? a.bias + ms.at : nullptr;
+      const int rc = launch_cfg<8, ALAY, BLAY, EPI, OUT, F16>(a1, s);
+      return rc ? rc : launch_cfg<3, ALAY, BLAY, EPI, OUT, F16>(a2, s);
+    }
+    if (ms.dim == 2) {
+      GemmArgs a1 = a, a2 = a;
+      a1.M = ms.at;
+      a2.M = a.M - ms.at;
+      a2.A = a.A + (ALAY == LAY_ROW ? (int64_t)ms.at * a.lda : (int64_t)ms.at);
+      a2.C = a.C ? (char*)a.C + (int64_t)ms.at * a.ldc * esz : nullptr;
+      a2.C2 = a.C2 ? (char*)a.C2 + (int64_t)ms.at * a.ldc2 * 2 : nullptr;
+      a2.rowsum = a.rowsum ? (char*)a.rowsum + (int64_t)ms.at * esz : nullptr;
+      const int rc = launch_cfg<8, ALAY, BLAY, EPI, OUT, F16>(a1, s);
+      return rc ? rc : launch_cfg<4, ALAY, BLAY, EPI, OUT, F16>(a2, s);
+    }
+  }
   switch (c) {
     case 0: return launch_cfg<0, ALAY, BLAY, EPI, OUT, F16>(a, s);
     case 1: return launch_cfg<1, ALAY, BLAY, EPI, OUT, F16>(a, s);

@@ -655,6 +655,40 @@ def test_fp32_products_cut_along_k(gpu, set_tuning, slices):
     assert rel(y, R.column_parallel_linear_forward(x, w, b)[0]) < TOL_F32
 
 
+@pytest.mark.parametrize("mixed", [None, 0])
+def test_mixed_tiling_vs_oracle(gpu, set_tuning, mixed):
+    """One and a half rounds of 256x256 tiles are launched as one round on the 64-deep loop plus one round of
+    half-size tiles on the ring loop (columns for the forward product, rows for the weight gradient): with it
+    and with it switched off, against the oracle on sampled rows and columns of both parts, ragged edges, bias +
+    GELU, bias gradient and accumulation; the same bits on every run."""
+    set_tuning("MTP_GEMM_MIXED", mixed)
+    m, n, k = 4096, 6100, 4096          # 16 x 24 tiles forward, 24 x 16 for the weight gradient
+    g = torch.Generator(device=gpu).manual_seed(1242)
+    x = torch.empty(m, k, device=gpu).normal_(generator=g).bfloat16()
+    w = torch.empty(n, k, device=gpu).normal_(0, 0.02, generator=g).bfloat16()
+    b = torch.empty(n, device=gpu).normal_(0, 0.5, generator=g).bfloat16()
+    dy = torch.empty(m, n, device=gpu).normal_(generator=g).bfloat16()
+    rm = torch.randperm(m, generator=gen(74))[:24].to(gpu)
+    rn = torch.cat([torch.randperm(n, generator=gen(75))[:20], torch.tensor([0, 4095, 4096, 4097, n - 1])]).to(gpu)
+    xs, ws, bs = x[rm].cpu().float(), w.cpu().float(), b.cpu().float()
+    runs = []
+    for _ in range(2):
+        y, act = ops.linear_fwd(x, w, b, ops.EPI_BIAS_GELU)
+        dw, db = ops.linear_wgrad(dy, x, True)
+        acc, accb = torch.ones(n, k, device=gpu), torch.ones(n, device=gpu)
+        ops.linear_wgrad(dy, x, True, dw=acc, db=accb, accumulate=True)
+        runs.append((y, act, dw, db, acc, accb))
+    y, act, dw, db, acc, accb = runs[0]
+    pre = R.column_parallel_linear_forward(xs, ws, bs)[0]
+    assert rel(y[rm], pre) < TOL_BF16 and rel(act[rm], R.gelu_new(y[rm].float().cpu())) < TOL_BF16
+    ref_dw = dy[:, rn].cpu().float().t() @ x.cpu().float()
+    ref_db = dy.cpu().float().sum(0)
+    assert rel(dw[rn], ref_dw) < TOL_BF16 and rel(db, ref_db) < TOL_BF16
+    assert rel(acc[rn] - 1, ref_dw) < TOL_F32 * 10 and rel(accb - 1, ref_db) < TOL_F32 * 10
+    for a, c in zip(runs[0], runs[1]):
+        assert torch.equal(a, c)
+
+
 def test_measurement_switches_are_not_in_the_shipped_library(gpu, set_tuning):
     """MTP_GEMM_DEBUG turns parts of the product off in a measurement build (-DMTP_MEASURE).  The library that
     ships must not know the variable: with it set, results still match the oracle and are the bits of a run

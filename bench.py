@@ -8,7 +8,8 @@ backward, bf16 with fp32 accumulate, on 4096 tokens:
     QKV 4096->6144, gate/up 4096->2x14336 with fused SwiGLU, down 14336->4096.
 A step is: 3 forwards (Y = X W^T, SwiGLU fused into the gate/up epilogue), the
 SwiGLU backward, 3 input gradients (dX = dY W) and 3 weight gradients
-(dW = dY^T X).  FLOPs counted: 6*M*K*N per layer (4947.8 GFLOP per step); the
+(dW = dY^T X), the two gradients of a layer through the one call the layers'
+backward makes (one launch where their tiles share rounds of workgroups).  FLOPs counted: 6*M*K*N per layer (4947.8 GFLOP per step); the
 activation work is executed inside the timed region but not counted.
 
 Inputs are resident in HBM before the timed region.  Timing: W warm-up steps,
@@ -132,8 +133,7 @@ def linear_step(work):
         g = L["dy"]
         if L["epi"] == ops.EPI_SWIGLU:
             g = ops.activation_bwd(g, y, ops.EPI_SWIGLU)
-        ops.linear_dgrad(g, L["w"])
-        ops.linear_wgrad(g, L["x"], False)
+        ops.linear_bwd(g, L["x"], L["w"], False)     # dX and dW: one call, as the layers' backward makes it
 
 
 def per_kernel(work, timer, reps):

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTP_ABI_VERSION 10
+#define MTP_ABI_VERSION 11
 
 /* element types.  MTP_F16 is IEEE half, what the reference's --fp16 sets as
  * params_dtype (Merak/merak_args/args.py:584-585). */
@@ -130,6 +130,22 @@ int mtp_linear_wgrad_ws(const void* dy, const void* x, void* dw, void* db,
                         void* workspace, int64_t workspace_bytes,
                         int64_t M, int64_t N, int64_t K,
                         int dtype, int dw_dtype, int accumulate, void* stream);
+
+/* Input gradient and weight gradient of one layer, dX = dY W and dW (+)= dY^T X
+ * (db likewise, may be NULL), what autograd derives for F.linear at
+ * layers.py:252,354 — the two calls above as one.  Where both products run on
+ * the 64-deep bf16 / fp16 loop and their 256x256 tiles together fill fewer
+ * rounds of 256 workgroups than apart (896 + 896 tiles: 7 rounds instead of
+ * 4 + 4), they go out as ONE launch; the results are those of mtp_linear_dgrad
+ * + mtp_linear_wgrad to the rounding order of the sums (another tile
+ * configuration may serve a product there), and the same bits on every run.
+ * In every other case it is those two calls, one after the other.  Same
+ * workspace rules. */
+int mtp_linear_bwd_ws(const void* dy, const void* x, const void* w,
+                      void* dx, void* dw, void* db,
+                      void* workspace, int64_t workspace_bytes,
+                      int64_t M, int64_t N, int64_t K,
+                      int dtype, int dw_dtype, int accumulate, void* stream);
 
 /* Backward of the fused activations: given dACT and the saved
  * pre-activation Y, writes dY.

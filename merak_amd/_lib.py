@@ -19,7 +19,7 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmerak_tp_gfx950.so"
 
 MTP_F32, MTP_BF16, MTP_F16 = 0, 1, 2
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_SWIGLU, EPI_GELU = 0, 1, 2, 3, 4
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 _i64, _int, _vp = C.c_int64, C.c_int, C.c_void_p
 
@@ -36,6 +36,7 @@ SIGNATURES = {
     "mtp_linear_fwd_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "mtp_linear_dgrad_ws": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "mtp_linear_wgrad_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
+    "mtp_linear_bwd_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
     "mtp_activation_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "mtp_embedding_gather": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "mtp_embedding_bwd_workspace_bytes": (_i64, [_i64, _i64]),

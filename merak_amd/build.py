@@ -28,6 +28,7 @@ LIB_DIR = PKG_DIR / "lib"
 LIB_PATH = LIB_DIR / "libmerak_tp_gfx950.so"
 
 SOURCES = [
+    "gemm_bf16_bwd.hip",
     "api.hip",
     "vocab_ce.hip",
     "embedding.hip",

@@ -845,8 +845,11 @@ __device__ __forceinline__ int64_t sk_slot_of(int w, int r, int KT, int ipw) {
   return (int64_t)(2 * w + (w * ipw < r * KT ? 1 : 0)) * SK_SLOT_BYTES;
 }
 
+// bid: this workgroup's index among the workgroups of the product p (blockIdx.x, or less where one launch holds
+// two products); lds: the workgroup's Q_LDS_BYTES of LDS, 1 KiB aligned
+constexpr int Q_LDS_BYTES = 2 * 65536;
 template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK, bool SK>
-__device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
+__device__ __forceinline__ void gemm_q_body(const GemmArgs& p, const int bid, char* lds) {
   using X = X16<F16>;
   constexpr int BM = 256, BN = 256;
   static_assert(!SK || (BLK == 16 && NW == 4), "stream-K is built for the 4-wave 16x16x32 form");
@@ -864,7 +867,7 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
   constexpr int QBUF = AOp::BYTES + BOp::BYTES;   // one k-tile of both operands: 64 KiB
   static_assert(QBUF == 65536, "the operands keep per-buffer read offsets 64 KiB apart");
   constexpr int LDS_BYTES = 2 * QBUF;
-  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+  static_assert(LDS_BYTES == Q_LDS_BYTES, "the kernels allocate Q_LDS_BYTES");
 
   const int tid = threadIdx.x;
   int lane = tid & 63;
@@ -878,11 +881,11 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p) {
   const int KT = (p.K + QBK - 1) / QBK;
   // This workgroup's run of k-tiles in the sequence "all k-tiles of tile position 0, of position 1, ...": one whole
   // tile, or (stream-K) sk_ipw k-tiles that may end one tile and begin the next.
-  int it = blockIdx.x * KT, it_end = it + KT;
+  int it = bid * KT, it_end = it + KT;
   [[maybe_unused]] int sk_w = -1;
   if constexpr (SK) {
-    if ((int)blockIdx.x >= p.sk_full) {
-      sk_w = blockIdx.x - p.sk_full;
+    if (bid >= p.sk_full) {
+      sk_w = bid - p.sk_full;
       it = p.sk_full * KT + sk_w * p.sk_ipw;
       const int all = tiles_m * tiles_n * KT;
       it_end = it + p.sk_ipw < all ? it + p.sk_ipw : all;
@@ -1509,7 +1512,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs p) {
 
 template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK, bool SK>
 __global__ __launch_bounds__(NW * 64) void gemm_q_kernel(const GemmArgs p) {
-  gemm_q_body<ALAY, BLAY, EPI, OUT, NW, F16, BLK, SK>(p);
+  __shared__ __attribute__((aligned(1024))) char lds[Q_LDS_BYTES];
+  gemm_q_body<ALAY, BLAY, EPI, OUT, NW, F16, BLK, SK>(p, (int)blockIdx.x, lds);
+}
+
+// Input gradient and weight gradient of one layer in one launch: workgroups [0, n1) are the tiles of p1 (dX = dY W),
+// the others the tiles of p2 (dW = dY^T X, with or without the bias gradient).  The tiles of both products fill
+// the rounds of 256 workgroups together: 896 + 896 tiles of Llama-3-8B's down layer are 7 whole rounds instead of
+// twice 3.5, 128 + 128 of the Llama-70B shard's o-proj one round instead of two launches cut along k.
+template <int EPI2, int OUT2, bool F16>
+__global__ __launch_bounds__(256) void gemm_q_bwd_kernel(const GemmArgs p1, const GemmArgs p2, const int n1) {
+  __shared__ __attribute__((aligned(1024))) char lds[Q_LDS_BYTES];
+  if ((int)blockIdx.x < n1)
+    gemm_q_body<LAY_ROW, LAY_COL, MTP_EPI_NONE, OUT_BF16, 4, F16, 16, false>(p1, (int)blockIdx.x, lds);
+  else
+    gemm_q_body<LAY_COL, LAY_COL, EPI2, OUT2, 4, F16, 16, false>(p2, (int)blockIdx.x - n1, lds);
 }
 
 // Second pass of stream-K: one workgroup per (shared tile, row of 16x16 blocks) adds that row's pieces up in k

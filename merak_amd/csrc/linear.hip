@@ -11,6 +11,9 @@ int mtp_gemm_bf16_dgrad(const void* dy, const void* w, void* dx, int64_t M, int6
                         hipStream_t s);
 int mtp_gemm_bf16_wgrad(const void* dy, const void* x, void* dw, void* db, int64_t M, int64_t N, int64_t K,
                         int dw_dtype, int accumulate, int f16, void* ws, hipStream_t s);
+// both of the above, in one launch where that saves a round of workgroups
+int mtp_gemm_bf16_bwd(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db, int64_t M, int64_t N,
+                      int64_t K, int dw_dtype, int accumulate, int f16, void* ws, hipStream_t s);
 // = SK_WORKSPACE_BYTES of gemm_bf16_kernel.h (checked there): 2 slots for each of 256 workgroups
 #define MTP_LINEAR_WS_BYTES (2ll * 256 * 66 * 256 * 16)
 int mtp_gemm_generic(const void* A, int64_t sam, int64_t sak, const void* B, int64_t sbn, int64_t sbk,
@@ -162,6 +165,26 @@ extern "C" int mtp_linear_wgrad_ws(const void* dy, const void* x, void* dw, void
   if (rc) return rc;
   if (db) return mtp_colsum(dy, db, M, N, dtype, dw_dtype, accumulate, s);
   return MTP_OK;
+}
+
+extern "C" int mtp_linear_bwd_ws(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db,
+                                 void* workspace, int64_t workspace_bytes, int64_t M, int64_t N, int64_t K, int dtype,
+                                 int dw_dtype, int accumulate, void* stream) {
+  int rc = check_dims("linear_bwd", M, N, K, dtype);
+  if (rc) return rc;
+  MTP_REQUIRE(dw_dtype == MTP_F32 || dw_dtype == dtype, MTP_EUNSUPPORTED,
+              "linear_bwd: gradients are fp32 or of the inputs' dtype (inputs %d, dw %d)", dtype, dw_dtype);
+  MTP_REQUIRE(dx && dw, MTP_EINVAL, "linear_bwd: null output");
+  MTP_REQUIRE(M == 0 || (dy && x && w), MTP_EINVAL, "linear_bwd: null input");
+  if ((dtype == MTP_BF16 || dtype == MTP_F16) && M > 0 && fast_ok(N, K, dy, w) && fast_ok(N, K, dy, x) && aligned16(dx) &&
+      aligned16(dw)) {
+    rc = mtp_gemm_bf16_bwd(dy, x, w, dx, dw, db, M, N, K, dw_dtype, accumulate, dtype == MTP_F16,
+                           usable_ws(workspace, workspace_bytes), (hipStream_t)stream);
+    if (rc != MTP_EUNSUPPORTED) return rc;
+  }
+  rc = mtp_linear_dgrad_ws(dy, w, dx, workspace, workspace_bytes, M, N, K, dtype, stream);
+  if (rc) return rc;
+  return mtp_linear_wgrad_ws(dy, x, dw, db, workspace, workspace_bytes, M, N, K, dtype, dw_dtype, accumulate, stream);
 }
 
 extern "C" int mtp_linear_bias_grad(const void* dy, void* db, int64_t M, int64_t N, int dtype, int db_dtype, int accumulate,

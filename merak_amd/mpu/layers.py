@@ -81,7 +81,7 @@ class _LinearFunction(torch.autograd.Function):
     """y = x W^T (+ b), optionally followed by a fused activation.
 
     backward: dX = dY W, dW = dY^T X, db = sum dY — what autograd derives for
-    ``F.linear`` (layers.py:252,354), each one kernel launch."""
+    ``F.linear`` (layers.py:252,354), one call of the library for all three."""
 
     @staticmethod
     def forward(ctx, x, weight, bias, activation):
@@ -110,9 +110,13 @@ class _LinearFunction(torch.autograd.Function):
         if ctx.activation is not None:
             g2d = ops.activation_bwd(g2d, pre, ctx.epi)
         dx = dw = db = None
+        want_db = ctx.has_bias and ctx.needs_input_grad[2]
+        if ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and g2d.shape[0] > 0:
+            # both products in one call (one launch where their tiles share rounds of workgroups)
+            dx, dw, db = ops.linear_bwd(g2d, x2d, weight, want_db)
+            return dx.view(*ctx.lead, weight.shape[1]), dw, db, None
         if ctx.needs_input_grad[0]:
             dx = ops.linear_dgrad(g2d, weight).view(*ctx.lead, weight.shape[1])
-        want_db = ctx.has_bias and ctx.needs_input_grad[2]
         if ctx.needs_input_grad[1]:
             dw, db = ops.linear_wgrad(g2d, x2d, want_db)
         elif want_db:

@@ -169,6 +169,41 @@ def linear_wgrad(dy2d: torch.Tensor, x2d: torch.Tensor, want_db: bool, out_dtype
     return dw, (db if want_db else None)
 
 
+def linear_bwd(dy2d: torch.Tensor, x2d: torch.Tensor, w: torch.Tensor, want_db: bool,
+               out_dtype: Optional[torch.dtype] = None, dw: Optional[torch.Tensor] = None,
+               db: Optional[torch.Tensor] = None, accumulate: bool = False):
+    """(dx, dw, db) = (dy w, dy^T x, sum of dy's rows): linear_dgrad and linear_wgrad of one layer as one call, and
+    as one launch where the tiles of the two products together fill fewer rounds of workgroups than apart."""
+    dev = _require_gpu(dy2d, x2d, w, dw, db)
+    if dy2d.dim() != 2 or x2d.dim() != 2 or w.dim() != 2:
+        raise ValueError("linear_bwd: dy [M, N], x [M, K] and weight [N, K] must be 2-d")
+    M, N = dy2d.shape
+    K = x2d.shape[1]
+    if x2d.shape[0] != M or tuple(w.shape) != (N, K):
+        raise ValueError(f"linear_bwd: shapes dy {tuple(dy2d.shape)}, x {tuple(x2d.shape)}, weight {tuple(w.shape)}")
+    if not (dy2d.dtype == x2d.dtype == w.dtype):
+        raise TypeError("linear_bwd: dy, x and weight must share a dtype")
+    out_dtype = out_dtype or (dw.dtype if dw is not None else dy2d.dtype)
+    if accumulate and dw is None:
+        raise ValueError("linear_bwd: accumulate needs the gradient buffers")
+    dy2d, x2d, w = _contig(dy2d), _contig(x2d), _contig(w)
+    dx = torch.empty((M, K), dtype=dy2d.dtype, device=dev)
+    if dw is None:
+        dw = torch.empty((N, K), dtype=out_dtype, device=dev)
+    if want_db and db is None:
+        db = torch.empty((N,), dtype=out_dtype, device=dev)
+    if tuple(dw.shape) != (N, K) or dw.dtype != out_dtype or not dw.is_contiguous():
+        raise ValueError("linear_bwd: dw must be a contiguous [N, K] tensor of out_dtype")
+    if want_db and (tuple(db.shape) != (N,) or db.dtype != out_dtype or not db.is_contiguous()):
+        raise ValueError("linear_bwd: db must be a contiguous [N] tensor of out_dtype")
+    with torch.cuda.device(dev):
+        wsp, wsb = _ws_args(dy2d, dev)
+        _lib.check(_lib.lib().mtp_linear_bwd_ws(_p(dy2d), _p(x2d), _p(w), _p(dx), _p(dw), _p(db) if want_db else None,
+                                                wsp, wsb, M, N, K, _dt(dy2d), _DTYPES[out_dtype], int(accumulate),
+                                                _stream(dev)), "mtp_linear_bwd")
+    return dx, dw, (db if want_db else None)
+
+
 def colsum(dy2d: torch.Tensor, db: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
     """db (+)= dy2d.sum(0): the bias gradient alone, for a layer whose weight takes none."""
     dev = _require_gpu(dy2d, db)

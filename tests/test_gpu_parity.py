@@ -689,6 +689,45 @@ def test_mixed_tiling_vs_oracle(gpu, set_tuning, mixed):
         assert torch.equal(a, c)
 
 
+@pytest.mark.parametrize("name,m,n,k", [("llama8b_down", 4096, 4096, 14336), ("llama70b_tp8_oproj", 8192, 8192, 1024),
+                                         ("ragged", 1792, 2304, 3000), ("small", 300, 520, 448)])
+def test_layer_backward_in_one_call(gpu, set_tuning, name, m, n, k):
+    """mtp_linear_bwd: input and weight gradient of a layer as one call — one launch where the tiles of the two
+    products together fill fewer rounds of workgroups (the first two shapes, and 84 + 108 tiles of the third,
+    whose outputs end inside a tile), two launches otherwise.  The same bits as the two separate calls without scratch, with bias gradient, fp32
+    accumulation into existing gradients, and on every run; the oracle on sampled rows."""
+    g = torch.Generator(device=gpu).manual_seed(1243)
+    x = torch.empty(m, k, device=gpu).normal_(generator=g).bfloat16()
+    w = torch.empty(n, k, device=gpu).normal_(0, 0.02, generator=g).bfloat16()
+    dy = torch.empty(m, n, device=gpu).normal_(generator=g).bfloat16()
+    set_tuning("MTP_GEMM_PAIR", 0)
+    set_tuning("MTP_GEMM_SK", 0)             # the pair never cuts a tile along k
+    dx0, dw0, db0 = ops.linear_bwd(dy, x, w, True)
+    acc0, accb0 = torch.ones(n, k, device=gpu), torch.ones(n, device=gpu)
+    ops.linear_bwd(dy, x, w, True, dw=acc0, db=accb0, accumulate=True)
+    set_tuning("MTP_GEMM_PAIR", None)
+    set_tuning("MTP_GEMM_SK", None)
+    runs = []
+    for _ in range(2):
+        dx, dw, db = ops.linear_bwd(dy, x, w, True)
+        acc, accb = torch.ones(n, k, device=gpu), torch.ones(n, device=gpu)
+        dx2, _, _ = ops.linear_bwd(dy, x, w, True, dw=acc, db=accb, accumulate=True)
+        _, dw_nodb, none = ops.linear_bwd(dy, x, w, False)
+        assert none is None and torch.equal(dx2, dx) and torch.equal(dw_nodb, dw)
+        runs.append((dx, dw, db, acc, accb))
+    for a, b in zip(runs[0], runs[1]):
+        assert torch.equal(a, b), name                      # the same bits on every run
+    # against the two separate launches: the same sums, possibly in another tile configuration's order
+    for a, b, tol in ((dx, dx0, 3e-3), (dw, dw0, 3e-3), (db, db0, 3e-3), (acc, acc0, 1e-5), (accb, accb0, 1e-5)):
+        assert rel(a, b) < tol, name
+    rm = torch.randperm(m, generator=gen(76))[:16].to(gpu)
+    rn = torch.randperm(n, generator=gen(77))[:16].to(gpu)
+    ws = w.cpu().float()
+    assert rel(dx[rm], dy[rm].cpu().float() @ ws) < TOL_BF16
+    assert rel(dw[rn], dy[:, rn].cpu().float().t() @ x.cpu().float()) < TOL_BF16
+    assert rel(db, dy.cpu().float().sum(0)) < TOL_BF16
+
+
 def test_measurement_switches_are_not_in_the_shipped_library(gpu, set_tuning):
     """MTP_GEMM_DEBUG turns parts of the product off in a measurement build (-DMTP_MEASURE).  The library that
     ships must not know the variable: with it set, results still match the oracle and are the bits of a run

@@ -1518,15 +1518,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_q_kernel(const GemmArgs p) {
 
 // Input gradient and weight gradient of one layer in one launch: workgroups [0, n1) are the tiles of p1 (dX = dY W),
 // the others the tiles of p2 (dW = dY^T X, with or without the bias gradient).  The tiles of both products fill
-// the rounds of 256 workgroups together: 896 + 896 tiles of Llama-3-8B's down layer are 7 whole rounds instead of
-// twice 3.5, 128 + 128 of the Llama-70B shard's o-proj one round instead of two launches cut along k.
+// the 256 compute units together: 896 + 896 tiles of Llama-3-8B's down layer are 7 whole rounds instead of twice
+// 3.5, 128 + 128 of the Llama-70B shard's o-proj one round instead of two launches cut along k, and the 160 long
+// tiles of that shard's QKV weight gradient leave 96 compute units to its input gradient's 1024 short ones.
+// The tiles of the product with the longer k come first (n1 > 0: p1's n1 tiles, then p2's; n1 < 0: p2's -n1 tiles,
+// then p1's): workgroups are handed out in index order as compute units fall free, so the long tiles start at once
+// and the short ones fill in behind them.
 template <int EPI2, int OUT2, bool F16>
 __global__ __launch_bounds__(256) void gemm_q_bwd_kernel(const GemmArgs p1, const GemmArgs p2, const int n1) {
   __shared__ __attribute__((aligned(1024))) char lds[Q_LDS_BYTES];
-  if ((int)blockIdx.x < n1)
-    gemm_q_body<LAY_ROW, LAY_COL, MTP_EPI_NONE, OUT_BF16, 4, F16, 16, false>(p1, (int)blockIdx.x, lds);
+  const int bid = (int)blockIdx.x;
+  const bool first = n1 > 0 ? bid < n1 : bid >= -n1;      // this workgroup multiplies a tile of p1
+  if (first)
+    gemm_q_body<LAY_ROW, LAY_COL, MTP_EPI_NONE, OUT_BF16, 4, F16, 16, false>(p1, n1 > 0 ? bid : bid + n1, lds);
   else
-    gemm_q_body<LAY_COL, LAY_COL, EPI2, OUT2, 4, F16, 16, false>(p2, (int)blockIdx.x - n1, lds);
+    gemm_q_body<LAY_COL, LAY_COL, EPI2, OUT2, 4, F16, 16, false>(p2, n1 > 0 ? bid - n1 : bid, lds);
 }
 
 // Second pass of stream-K: one workgroup per (shared tile, row of 16x16 blocks) adds that row's pieces up in k

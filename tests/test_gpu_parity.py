@@ -690,6 +690,7 @@ def test_mixed_tiling_vs_oracle(gpu, set_tuning, mixed):
 
 
 @pytest.mark.parametrize("name,m,n,k", [("llama8b_down", 4096, 4096, 14336), ("llama70b_tp8_oproj", 8192, 8192, 1024),
+                                         ("llama70b_tp8_qkv", 8192, 1280, 8192),     # the weight gradient's long tiles go first
                                          ("ragged", 1792, 2304, 3000), ("small", 300, 520, 448)])
 def test_layer_backward_in_one_call(gpu, set_tuning, name, m, n, k):
     """mtp_linear_bwd: input and weight gradient of a layer as one call — one launch where the tiles of the two

@@ -150,6 +150,10 @@ def per_kernel(work, timer, reps):
             ms = timer.run(f"{L['name']}.{kind}", fn, reps)
             rows.append(dict(kernel=f"{L['name']}.{kind}", M=M, N=N, K=K, ms=round(ms, 4),
                              tflops=round(2.0 * M * N * K / ms / 1e9, 1)))
+        # both gradients through the one call the step makes (one launch where their tiles share rounds of workgroups)
+        ms = timer.run(f"{L['name']}.bwd", lambda: ops.linear_bwd(g, L["x"], L["w"], False), reps)
+        rows.append(dict(kernel=f"{L['name']}.dgrad+wgrad", M=M, N=N, K=K, ms=round(ms, 4),
+                         tflops_both=round(4.0 * M * N * K / ms / 1e9, 1)))
         if L["epi"] == ops.EPI_SWIGLU:
             ms = timer.run(f"{L['name']}.swiglu_bwd", lambda: ops.activation_bwd(L["dy"], y, ops.EPI_SWIGLU), reps)
             rows.append(dict(kernel=f"{L['name']}.swiglu_bwd", ms=round(ms, 4),

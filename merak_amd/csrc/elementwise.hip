@@ -132,19 +132,22 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ d
 // ---- measurement -------------------------------------------------------------
 __global__ __launch_bounds__(256) void stream_copy_kernel(const u32x4_t* __restrict__ src, u32x4_t* __restrict__ dst,
                                                           int64_t nvec) {
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  for (; i + 3 * stride < nvec; i += 4 * stride) {
-    u32x4_t a = __builtin_nontemporal_load(src + i);
-    u32x4_t b = __builtin_nontemporal_load(src + i + stride);
-    u32x4_t c = __builtin_nontemporal_load(src + i + 2 * stride);
-    u32x4_t d = __builtin_nontemporal_load(src + i + 3 * stride);
-    __builtin_nontemporal_store(a, dst + i);
-    __builtin_nontemporal_store(b, dst + i + stride);
-    __builtin_nontemporal_store(c, dst + i + 2 * stride);
-    __builtin_nontemporal_store(d, dst + i + 3 * stride);
+  // Workgroup b copies the 16 KiB pieces b, b + grid, ...: four vectors per lane, 4 KiB apart.  Contiguous
+  // pieces per workgroup move 5.6-5.8 TB/s (read + write) on an MI355X; the same loop with the four vectors a
+  // whole grid apart (every workgroup touching four far-apart 4 KiB pieces per step) moves 4.3-5.1 TB/s.
+  constexpr int U = 4;
+  const int64_t pieces = nvec / (256 * U);
+  for (int64_t c = blockIdx.x; c < pieces; c += gridDim.x) {
+    const int64_t i = c * (256 * U) + threadIdx.x;
+    u32x4_t v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = __builtin_nontemporal_load(src + i + u * 256);
+#pragma unroll
+    for (int u = 0; u < U; u++) __builtin_nontemporal_store(v[u], dst + i + u * 256);
   }
-  for (; i < nvec; i += stride) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+  // what is left of the last piece
+  for (int64_t i = pieces * (256 * U) + (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256)
+    __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
 // Register-resident MFMA loop.  What the matrix cores sustain depends on the operand bits, because the chip
@@ -263,7 +266,7 @@ extern "C" int mtp_stream_copy(const void* src, void* dst, int64_t bytes, void* 
               "stream_copy: buffers must be 16-byte aligned");
   const int64_t nvec = bytes / 16;
   int64_t blocks = (nvec + 256 * 4 - 1) / (256 * 4);
-  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (blocks > 256 * 64) blocks = 256 * 64;
   hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                      (const u32x4_t*)src, (u32x4_t*)dst, nvec);
   MTP_CHECK_LAUNCH("stream_copy");

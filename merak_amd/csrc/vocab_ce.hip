@@ -130,8 +130,8 @@ __device__ __forceinline__ void ms_accumulate(MaxSum& acc, const float* f) {
   acc.s = s;
 }
 
-template <typename T>
-__global__ __launch_bounds__(CE_THREADS) void vocab_ce_fwd_kernel(
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void vocab_ce_fwd_kernel(
     const T* __restrict__ logits, const int64_t* __restrict__ target, float* __restrict__ loss,
     float* __restrict__ row_max, float* __restrict__ row_sumexp, float* __restrict__ pred, int64_t V,
     int64_t vocab_start) {
@@ -149,18 +149,17 @@ __global__ __launch_bounds__(CE_THREADS) void vocab_ce_fwd_kernel(
   MaxSum acc{NEG_BIG, 0.0f};
 
   int64_t i = tid;
-  for (; i + (UNROLL - 1) * CE_THREADS < nvec; i += UNROLL * CE_THREADS) {
+  for (; i + (UNROLL - 1) * NT < nvec; i += UNROLL * NT) {
     u32x4_t v[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; u++) v[u] = __builtin_nontemporal_load(vp + i + u * CE_THREADS);
+    for (int u = 0; u < UNROLL; u++) v[u] = __builtin_nontemporal_load(vp + i + u * NT);
+    // the step's vectors as one block: one running-maximum update (and one rescaling exponential) per step
+    float f[UNROLL * EPV];
 #pragma unroll
-    for (int u = 0; u < UNROLL; u++) {
-      float f[EPV];
-      Elem<T>::unpack(v[u], f);
-      ms_accumulate<EPV>(acc, f);
-    }
+    for (int u = 0; u < UNROLL; u++) Elem<T>::unpack(v[u], f + u * EPV);
+    ms_accumulate<UNROLL * EPV>(acc, f);
   }
-  for (; i < nvec; i += CE_THREADS) {
+  for (; i < nvec; i += NT) {
     u32x4_t v = __builtin_nontemporal_load(vp + i);
     float f[EPV];
     Elem<T>::unpack(v, f);
@@ -185,7 +184,7 @@ __global__ __launch_bounds__(CE_THREADS) void vocab_ce_fwd_kernel(
     other.s = __shfl_xor(acc.s, o, 64);
     acc = ms_combine(acc, other);
   }
-  __shared__ float sm[CE_WAVES], ss[CE_WAVES];
+  __shared__ float sm[(NT / MTP_WAVE)], ss[(NT / MTP_WAVE)];
   if ((tid & 63) == 0) {
     sm[tid >> 6] = acc.m;
     ss[tid >> 6] = acc.s;
@@ -194,7 +193,7 @@ __global__ __launch_bounds__(CE_THREADS) void vocab_ce_fwd_kernel(
   if (tid == 0) {
     MaxSum t{sm[0], ss[0]};
 #pragma unroll
-    for (int w = 1; w < CE_WAVES; w++) t = ms_combine(t, MaxSum{sm[w], ss[w]});
+    for (int w = 1; w < (NT / MTP_WAVE); w++) t = ms_combine(t, MaxSum{sm[w], ss[w]});
     t.s *= ms_residual_scale(t.m);
     const int64_t tl = target[row] - vocab_start;
     const bool in_range = tl >= 0 && tl < V;
@@ -206,8 +205,8 @@ __global__ __launch_bounds__(CE_THREADS) void vocab_ce_fwd_kernel(
   }
 }
 
-template <typename T>
-__global__ __launch_bounds__(CE_THREADS) void vocab_ce_bwd_kernel(
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void vocab_ce_bwd_kernel(
     T* __restrict__ logits, const int64_t* __restrict__ target, const float* __restrict__ row_max,
     const float* __restrict__ row_sumexp, const float* __restrict__ grad_out, int64_t V, int64_t vocab_start) {
   constexpr int EPV = Elem<T>::EPV;
@@ -233,27 +232,27 @@ __global__ __launch_bounds__(CE_THREADS) void vocab_ce_bwd_kernel(
   const int64_t tv = (tl >= head) ? (tl - head) : -1;
 
   int64_t i = tid;
-  for (; i + (UNROLL - 1) * CE_THREADS < nvec; i += UNROLL * CE_THREADS) {
+  for (; i + (UNROLL - 1) * NT < nvec; i += UNROLL * NT) {
     u32x4_t v[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; u++) v[u] = __builtin_nontemporal_load(vp + i + u * CE_THREADS);
+    for (int u = 0; u < UNROLL; u++) v[u] = __builtin_nontemporal_load(vp + i + u * NT);
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
       float f[EPV];
       Elem<T>::unpack(v[u], f);
 #pragma unroll
       for (int e = 0; e < EPV; e++) f[e] = (from_softmax ? f[e] : __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc))) * scale;
-      const int64_t base = (i + u * CE_THREADS) * EPV;
+      const int64_t base = (i + u * NT) * EPV;
       if ((uint64_t)(tv - base) < (uint64_t)EPV) {
         const int e = (int)(tv - base);
 #pragma unroll
         for (int q = 0; q < EPV; q++)
           if (q == e) f[q] -= g;
       }
-      __builtin_nontemporal_store(Elem<T>::pack(f), vp + i + u * CE_THREADS);
+      __builtin_nontemporal_store(Elem<T>::pack(f), vp + i + u * NT);
     }
   }
-  for (; i < nvec; i += CE_THREADS) {
+  for (; i < nvec; i += NT) {
     u32x4_t v = __builtin_nontemporal_load(vp + i);
     float f[EPV];
     Elem<T>::unpack(v, f);
@@ -324,46 +323,54 @@ __global__ __launch_bounds__(FU_THREADS) void vocab_ce_fused_kernel(
 
   __shared__ float red_m[FU_WAVES], red_s[FU_WAVES];
 
-  // row maximum
-  float lm = fe;
+  // Row maximum and sum of exponentials in one pass over the registers, two vectors at a time in the order they
+  // arrive (the running maximum and the shifted sum of the forward kernel), so that this arithmetic runs while
+  // the rest of the row is still on its way: as a pass of its own behind a barrier it cost 93 us of the 844 a
+  // bf16 [8192, 128256] matrix took.
+  MaxSum acc{NEG_BIG, 0.0f};
+  if (has_edge) ms_accumulate<1>(acc, &fe);
 #pragma unroll
-  for (int u = 0; u < NV; u++)
-    if (tid + u * FU_THREADS < nvec) {
+  for (int u = 0; u < NV; u += 2) {
+    if (u + 1 < NV && tid + (u + 1) * FU_THREADS < nvec) {
+      float f[2 * EPV];
+      Elem<T>::unpack(v[u], f);
+      Elem<T>::unpack(v[u + 1], f + EPV);
+      ms_accumulate<2 * EPV>(acc, f);
+    } else if (tid + u * FU_THREADS < nvec) {
       float f[EPV];
       Elem<T>::unpack(v[u], f);
-#pragma unroll
-      for (int e = 0; e < EPV; e++) lm = fmaxf(lm, f[e]);
+      ms_accumulate<EPV>(acc, f);
     }
-  // keep the row as loaded: without this the compiler carries the unpacked floats of one phase into the
-  // next, which doubles the registers a bf16 row needs
+  }
+  // keep the row as loaded: without this the compiler carries the unpacked floats into the gradient pass, which
+  // doubles the registers a bf16 row needs
 #pragma unroll
   for (int u = 0; u < NV; u++) asm volatile("" : "+v"(v[u]));
-  lm = wave_max(lm);
-  if ((tid & 63) == 0) red_m[tid >> 6] = lm;
-  __syncthreads();
-  float m = red_m[0];
 #pragma unroll
-  for (int w = 1; w < FU_WAVES; w++) m = fmaxf(m, red_m[w]);
+  for (int o = 32; o > 0; o >>= 1) {
+    MaxSum other;
+    other.m = __shfl_xor(acc.m, o, 64);
+    other.s = __shfl_xor(acc.s, o, 64);
+    acc = ms_combine(acc, other);
+  }
+  if ((tid & 63) == 0) {
+    red_m[tid >> 6] = acc.m;
+    red_s[tid >> 6] = acc.s;
+  }
+  __syncthreads();
+  // every wave combines the 16 waves' pairs on its own lanes (16 lanes hold one copy) and takes lane 0's result
+  static_assert(FU_WAVES == 16, "the cross-wave butterfly is written for 16 waves");
+  MaxSum tot{red_m[tid & 15], red_s[tid & 15]};
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) {
+    MaxSum other;
+    other.m = __shfl_xor(tot.m, o, 64);
+    other.s = __shfl_xor(tot.s, o, 64);
+    tot = ms_combine(tot, other);
+  }
+  const float m = __shfl(tot.m, 0, 64);
+  const float s_raw = __shfl(tot.s, 0, 64);   // sum of exp2(x*c - fl(m*c)): the forward kernel's shifted sum
   const float mc = mul_rn(m, LOG2E);
-
-  // sum of exponentials, same term as the two-kernel path: exp2(fma(x, c, -fl(m*c)))
-  float ls = has_edge ? __builtin_amdgcn_exp2f(__builtin_fmaf(fe, LOG2E, -mc)) : 0.0f;
-#pragma unroll
-  for (int u = 0; u < NV; u++)
-    if (tid + u * FU_THREADS < nvec) {
-      float f[EPV];
-      Elem<T>::unpack(v[u], f);
-#pragma unroll
-      for (int e = 0; e < EPV; e++) ls += __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc));
-    }
-#pragma unroll
-  for (int u = 0; u < NV; u++) asm volatile("" : "+v"(v[u]));
-  ls = wave_sum(ls);
-  if ((tid & 63) == 0) red_s[tid >> 6] = ls;
-  __syncthreads();
-  float s_raw = red_s[0];
-#pragma unroll
-  for (int w = 1; w < FU_WAVES; w++) s_raw += red_s[w];
   const float resid = ms_residual_scale(m);
 
   if (tid == 0) {
@@ -398,6 +405,117 @@ __global__ __launch_bounds__(FU_THREADS) void vocab_ce_fused_kernel(
     if (edge_j == tl) f -= g;
     Elem<T>::st(rp + edge_j, f);
   }
+}
+
+// Backward with the row held in registers: every lane of a 1024-lane workgroup loads its NV vectors of the row,
+// the workgroup meets at a barrier, then every lane rewrites them.  The memory sees the row as one burst of reads
+// followed by one burst of writes (250 KiB each for a bf16 row of 128256) instead of 16 KiB steps that alternate
+// between the two: a plain in-place copy moves 6.1 TB/s in this shape against 5.1 TB/s in steps.  Same arithmetic
+// per element as vocab_ce_bwd_kernel, so the same bits.
+template <typename T, int NV>
+__global__ __launch_bounds__(FU_THREADS) void vocab_ce_bwd_row_kernel(
+    T* __restrict__ logits, const int64_t* __restrict__ target, const float* __restrict__ row_max,
+    const float* __restrict__ row_sumexp, const float* __restrict__ grad_out, int64_t V, int64_t vocab_start) {
+  constexpr int EPV = Elem<T>::EPV;
+  const int64_t row = blockIdx.x;
+  T* rp = logits + row * V;
+  const int tid = threadIdx.x;
+
+  int head;
+  int64_t nvec64;
+  row_split(rp, V, head, nvec64);
+  const int nvec = (int)nvec64;  // the host checked nvec <= NV * FU_THREADS
+  u32x4_t* vp = reinterpret_cast<u32x4_t*>(rp + head);
+  const int tail0 = head + nvec * EPV;
+  const int n_edge = head + (int)(V - tail0);
+  const int edge_j = tid < head ? tid : tail0 + (tid - head);
+  const bool has_edge = tid < n_edge;
+
+  u32x4_t v[NV] = {};
+#pragma unroll
+  for (int u = 0; u < NV; u++)
+    if (tid + u * FU_THREADS < nvec) v[u] = __builtin_nontemporal_load(vp + tid + u * FU_THREADS);
+  float fe = 0.0f;
+  if (has_edge) fe = Elem<T>::ld(rp + edge_j);
+
+  const float g = grad_out ? grad_out[row] : 1.0f;
+  const bool from_softmax = row_max == nullptr;
+  const float mc = from_softmax ? 0.0f : mul_rn(row_max[row], LOG2E);
+  const float scale = from_softmax ? g : g * ms_residual_scale(row_max[row]) / row_sumexp[row];
+  int64_t tl = target[row] - vocab_start;
+  if (tl < 0 || tl >= V) tl = -1;
+  const int tv = (tl >= head) ? (int)(tl - head) : -1;
+#pragma unroll
+  for (int u = 0; u < NV; u++) asm volatile("" : "+v"(v[u]));   // every load issued before the first is waited for
+  __syncthreads();   // the whole row has been asked for (and has arrived for this wave) before anyone writes
+
+#pragma unroll
+  for (int u = 0; u < NV; u++)
+    if (tid + u * FU_THREADS < nvec) {
+      float f[EPV];
+      Elem<T>::unpack(v[u], f);
+#pragma unroll
+      for (int e = 0; e < EPV; e++) f[e] = (from_softmax ? f[e] : __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc))) * scale;
+      const int base = (tid + u * FU_THREADS) * EPV;
+      if ((unsigned)(tv - base) < (unsigned)EPV) {
+        const int e = tv - base;
+#pragma unroll
+        for (int q = 0; q < EPV; q++)
+          if (q == e) f[q] -= g;
+      }
+      __builtin_nontemporal_store(Elem<T>::pack(f), vp + tid + u * FU_THREADS);
+    }
+  if (has_edge) {
+    float f = (from_softmax ? fe : __builtin_amdgcn_exp2f(__builtin_fmaf(fe, LOG2E, -mc))) * scale;
+    if (edge_j == tl) f -= g;
+    Elem<T>::st(rp + edge_j, f);
+  }
+}
+
+// Rows of at least two unrolled steps of a 1024-lane workgroup are walked by 1024 lanes (64 KiB per step; bf16
+// [8192, 128256] forward 312 -> 305 us, fp32 [8192, 50257] 254 -> 240 us: fewer, larger streams, and a last wave
+// of workgroups that is a sixteenth of the launch instead of a quarter), shorter rows by 256 (a 1024-lane step
+// would cover a 32000-element bf16 row only once, in its slower single-vector loop).
+template <typename T>
+bool long_row(int64_t vocab) { return vocab / Elem<T>::EPV >= 2 * 4 * 1024; }
+
+template <typename T>
+void launch_fwd(const void* logits, const int64_t* target, float* loss, float* row_max, float* row_sumexp, float* pred,
+                int64_t n_rows, int64_t vocab, int64_t vocab_start, hipStream_t s) {
+  if (long_row<T>(vocab))
+    hipLaunchKernelGGL((vocab_ce_fwd_kernel<T, 1024>), dim3((unsigned)n_rows), dim3(1024), 0, s, (const T*)logits,
+                       target, loss, row_max, row_sumexp, pred, vocab, vocab_start);
+  else
+    hipLaunchKernelGGL((vocab_ce_fwd_kernel<T, CE_THREADS>), dim3((unsigned)n_rows), dim3(CE_THREADS), 0, s,
+                       (const T*)logits, target, loss, row_max, row_sumexp, pred, vocab, vocab_start);
+}
+
+template <typename T>
+void launch_bwd(void* logits, const int64_t* target, const float* row_max, const float* row_sumexp,
+                const float* grad_out, int64_t n_rows, int64_t vocab, int64_t vocab_start, hipStream_t s) {
+  static MtpTune tune_row("MTP_CE_BWD_ROW");
+  const int64_t need = (vocab / Elem<T>::EPV + FU_THREADS - 1) / FU_THREADS;
+#define MTP_BWD_ROW_CASE(NV)                                                                                     \
+  if (need <= NV) {                                                                                              \
+    hipLaunchKernelGGL((vocab_ce_bwd_row_kernel<T, NV>), dim3((unsigned)n_rows), dim3(FU_THREADS), 0, s,         \
+                       (T*)logits, target, row_max, row_sumexp, grad_out, vocab, vocab_start);                   \
+    return;                                                                                                      \
+  }
+  // rows of at least a quarter of what 1024 lanes hold; shorter rows are served as well by the stepping kernel
+  if (tune_row.get(1) != 0 && need >= 4) {
+    MTP_BWD_ROW_CASE(4)
+    MTP_BWD_ROW_CASE(8)
+    MTP_BWD_ROW_CASE(12)
+    MTP_BWD_ROW_CASE(16)
+    MTP_BWD_ROW_CASE(20)
+  }
+#undef MTP_BWD_ROW_CASE
+  if (long_row<T>(vocab))
+    hipLaunchKernelGGL((vocab_ce_bwd_kernel<T, 1024>), dim3((unsigned)n_rows), dim3(1024), 0, s, (T*)logits, target,
+                       row_max, row_sumexp, grad_out, vocab, vocab_start);
+  else
+    hipLaunchKernelGGL((vocab_ce_bwd_kernel<T, CE_THREADS>), dim3((unsigned)n_rows), dim3(CE_THREADS), 0, s, (T*)logits,
+                       target, row_max, row_sumexp, grad_out, vocab, vocab_start);
 }
 
 // grad[i,:] *= grad_rows[i] / assumed, skipped for rows where the two are equal
@@ -477,19 +595,15 @@ extern "C" int mtp_vocab_ce_fwd(const void* logits, const int64_t* target, float
   if (n_rows == 0) return MTP_OK;
   MTP_REQUIRE(logits && target && loss && row_max && row_sumexp && pred, MTP_EINVAL, "vocab_ce_fwd: null pointer");
   hipStream_t s = (hipStream_t)stream;
-  dim3 grid((unsigned)n_rows), block(CE_THREADS);
   if (dtype == MTP_F32) {
     MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 3) == 0, MTP_EINVAL, "vocab_ce_fwd: fp32 logits not 4-byte aligned");
-    hipLaunchKernelGGL(vocab_ce_fwd_kernel<float>, grid, block, 0, s, (const float*)logits, target, loss, row_max,
-                       row_sumexp, pred, vocab, vocab_start);
+    launch_fwd<float>(logits, target, loss, row_max, row_sumexp, pred, n_rows, vocab, vocab_start, s);
   } else if (dtype == MTP_BF16) {
     MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL, "vocab_ce_fwd: bf16 logits not 2-byte aligned");
-    hipLaunchKernelGGL(vocab_ce_fwd_kernel<uint16_t>, grid, block, 0, s, (const uint16_t*)logits, target, loss,
-                       row_max, row_sumexp, pred, vocab, vocab_start);
+    launch_fwd<uint16_t>(logits, target, loss, row_max, row_sumexp, pred, n_rows, vocab, vocab_start, s);
   } else if (dtype == MTP_F16) {
     MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL, "vocab_ce_fwd: fp16 logits not 2-byte aligned");
-    hipLaunchKernelGGL(vocab_ce_fwd_kernel<f16s>, grid, block, 0, s, (const f16s*)logits, target, loss, row_max,
-                       row_sumexp, pred, vocab, vocab_start);
+    launch_fwd<f16s>(logits, target, loss, row_max, row_sumexp, pred, n_rows, vocab, vocab_start, s);
   } else {
     MTP_REQUIRE(false, MTP_EINVAL, "vocab_ce_fwd: unknown dtype %d", dtype);
   }
@@ -508,19 +622,15 @@ extern "C" int mtp_vocab_ce_bwd(void* logits, const int64_t* target, const float
   MTP_REQUIRE((row_max == nullptr) == (row_sumexp == nullptr), MTP_EINVAL,
               "vocab_ce_bwd: row_max and row_sumexp must both be given or both be null");
   hipStream_t s = (hipStream_t)stream;
-  dim3 grid((unsigned)n_rows), block(CE_THREADS);
   if (dtype == MTP_F32) {
     MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 3) == 0, MTP_EINVAL, "vocab_ce_bwd: fp32 logits not 4-byte aligned");
-    hipLaunchKernelGGL(vocab_ce_bwd_kernel<float>, grid, block, 0, s, (float*)logits, target, row_max, row_sumexp,
-                       grad_out, vocab, vocab_start);
+    launch_bwd<float>(logits, target, row_max, row_sumexp, grad_out, n_rows, vocab, vocab_start, s);
   } else if (dtype == MTP_BF16) {
     MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL, "vocab_ce_bwd: bf16 logits not 2-byte aligned");
-    hipLaunchKernelGGL(vocab_ce_bwd_kernel<uint16_t>, grid, block, 0, s, (uint16_t*)logits, target, row_max,
-                       row_sumexp, grad_out, vocab, vocab_start);
+    launch_bwd<uint16_t>(logits, target, row_max, row_sumexp, grad_out, n_rows, vocab, vocab_start, s);
   } else if (dtype == MTP_F16) {
     MTP_REQUIRE((reinterpret_cast<uintptr_t>(logits) & 1) == 0, MTP_EINVAL, "vocab_ce_bwd: fp16 logits not 2-byte aligned");
-    hipLaunchKernelGGL(vocab_ce_bwd_kernel<f16s>, grid, block, 0, s, (f16s*)logits, target, row_max, row_sumexp,
-                       grad_out, vocab, vocab_start);
+    launch_bwd<f16s>(logits, target, row_max, row_sumexp, grad_out, n_rows, vocab, vocab_start, s);
   } else {
     MTP_REQUIRE(false, MTP_EINVAL, "vocab_ce_bwd: unknown dtype %d", dtype);
   }

@@ -742,6 +742,17 @@ def test_measurement_switches_are_not_in_the_shipped_library(gpu, set_tuning):
             assert torch.equal(out[name], plain[name]), (value, name)
 
 
+@pytest.mark.parametrize("nbytes", [16, 16 * 1023, 16384, 16384 * 7 + 48, 16 * (4096 * 64 * 3 + 1025)])
+def test_reference_copy_kernel_copies_every_byte(gpu, nbytes):
+    """mtp_stream_copy (the bandwidth reference bench.py quotes): whole 16 KiB pieces and what is left of the last."""
+    from merak_amd import _lib
+    src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=gen(77)).to(gpu)
+    dst = torch.zeros(nbytes + 64, dtype=torch.uint8, device=gpu)
+    st = torch.cuda.current_stream().cuda_stream
+    _lib.check(_lib.lib().mtp_stream_copy(src.data_ptr(), dst.data_ptr(), nbytes, st), "copy")
+    assert torch.equal(dst[:nbytes], src) and int(dst[nbytes:].sum()) == 0
+
+
 @pytest.mark.parametrize("dtype,m,n,k", [(torch.float32, 512, 3072, 768), (torch.bfloat16, 512, 3072, 768),
                                           (torch.bfloat16, 200, 136, 72), (torch.float32, 33, 20, 10)])
 def test_bias_gelu_epilogue(gpu, dtype, m, n, k):

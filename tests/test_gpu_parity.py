@@ -90,8 +90,9 @@ def test_ce_autograd_function_matches_reference_semantics(gpu):
     assert rel(y.view(n, v), torch.softmax(x.view(n, v), -1)) < TOL_F32 and rel(l2.view(-1), ref_loss) < TOL_LOSS
 
 
-def test_ce_bf16_loss_dtype_flag_and_materialized_backward(gpu):
-    n, v = 16, 4096
+@pytest.mark.parametrize("v", [4096, 40000])   # rows walked in steps / rows held in registers by the backward
+def test_ce_bf16_loss_dtype_flag_and_materialized_backward(gpu, v):
+    n = 16
     x = torch.randn(n, v, generator=gen(6)).bfloat16()
     t = torch.randint(0, v, (n,), generator=gen(7))
     g = torch.rand(n, generator=gen(8))

@@ -9,9 +9,17 @@
  *
  * Return value: 0 on success, a negative MTP_E* code otherwise.  After a
  * failure mtp_last_error() returns a thread-local, human readable reason.
- * The library is re-entrant: it keeps no mutable global state apart from
- * that thread-local error string (backward passes call it from PyTorch's
- * autograd worker thread while forward runs on the main thread).
+ * The library is re-entrant (backward passes call it from PyTorch's autograd
+ * worker thread while forward runs on the main thread).  What it keeps
+ * between calls, all of it guarded:
+ *   - the thread-local error string;
+ *   - the values of the MTP_* tuning variables, read from the environment at
+ *     first use and again on mtp_reload_tuning() (one list, behind a mutex;
+ *     the values are atomics);
+ *   - for mtp_gemv_argmax_noalloc only: a 4 MiB file-scope device array per
+ *     GPU and the table of its per-device addresses (filled once per device
+ *     under a mutex).  Calls of that entry point that overlap on one GPU
+ *     share the array and race; no other entry point touches it.
  *
  * File:line citations name the interface in the reference tree
  * (HPDL-Group/Merak) that each entry point stands in for.

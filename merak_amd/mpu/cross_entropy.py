@@ -89,8 +89,9 @@ class _VocabParallelCrossEntropyFused(torch.autograd.Function):
         loss, _, _, _ = ops.vocab_ce_fwd_bwd_(logits_2d, target_1d, vocab_start_index, None, assumed_grad)
         # the kernel wrote through a raw pointer: tell autograd that the caller's logits have changed, so that
         # another function that saved them for its own backward fails loudly instead of using the gradient.
-        # A view handed out by a custom Function (the linear layers reshape their product) cannot be marked:
-        # autograd refuses to rebuild such a view's history, so there the overwrite is only documented.
+        # The linear layers return tensors that own their storage, so their logits are marked.  A view handed out
+        # by some other custom Function cannot be: autograd refuses to rebuild such a view's history, and there
+        # the overwrite is only documented.
         if not vocab_parallel_logits._is_view():
             torch.autograd.graph.increment_version(vocab_parallel_logits)
         ctx.assumed_grad = float(assumed_grad)

@@ -94,21 +94,22 @@ class _LinearFunction(torch.autograd.Function):
         else:
             epi = ops.EPI_SWIGLU
         need_pre = activation is None or any(ctx.needs_input_grad[:3])
-        y, act = ops.linear_fwd(x2d, weight, bias, epi, want_pre=need_pre)
+        # outputs are allocated in their final shape: what this function returns owns its storage (a view made here
+        # could not be version-bumped by a later in-place consumer such as the one-launch cross entropy)
+        y, act = ops.linear_fwd(x2d, weight, bias, epi, want_pre=need_pre, lead=tuple(lead))
         ctx.activation = activation
         ctx.epi = epi
         ctx.has_bias = bias is not None
         ctx.lead = lead
         ctx.save_for_backward(x2d, weight, y if activation is not None else None)
-        out = y if activation is None else act
-        return out.view(*lead, out.shape[-1])
+        return y if activation is None else act
 
     @staticmethod
     def backward(ctx, grad_out):
         x2d, weight, pre = ctx.saved_tensors
         g2d = grad_out.reshape(-1, grad_out.shape[-1])
         if ctx.activation is not None:
-            g2d = ops.activation_bwd(g2d, pre, ctx.epi)
+            g2d = ops.activation_bwd(g2d, pre.view(-1, pre.shape[-1]), ctx.epi)
         dx = dw = db = None
         want_db = ctx.has_bias and ctx.needs_input_grad[2]
         if ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and g2d.shape[0] > 0:

@@ -16,21 +16,21 @@ MODEL_PARALLEL_RNG = "model-parallel-rng"
 
 
 def _get_state():
-    return torch.cuda.get_rng_state() if torch.cuda.is_available() else torch.get_rng_state()
+    """(CPU generator state, current GPU's generator state or None): a shard may be drawn on either device
+    (use_cpu_initialization builds it on the host, the device path on the GPU), so both are tracked."""
+    return (torch.get_rng_state(), torch.cuda.get_rng_state() if torch.cuda.is_available() else None)
 
 
 def _set_state(state):
-    if torch.cuda.is_available():
-        torch.cuda.set_rng_state(state)
-    else:
-        torch.set_rng_state(state)
+    cpu, gpu = state
+    torch.set_rng_state(cpu)
+    if gpu is not None and torch.cuda.is_available():
+        torch.cuda.set_rng_state(gpu)
 
 
 def _seed(seed):
-    if torch.cuda.is_available():
-        torch.cuda.manual_seed(seed)
-    else:
-        torch.manual_seed(seed)
+    # torch.manual_seed seeds the CPU generator and every GPU's
+    torch.manual_seed(seed)
 
 
 class RNGStatesTracker:

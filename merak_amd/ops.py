@@ -7,6 +7,7 @@ there is no fallback path.
 """
 from __future__ import annotations
 
+import threading
 from typing import Optional, Tuple
 
 import torch
@@ -63,6 +64,7 @@ def _contig(t: torch.Tensor) -> torch.Tensor:
 
 # --------------------------------------------------------------------------- linear
 _linear_ws_cache = {}
+_linear_ws_lock = threading.Lock()   # forward runs on the caller's thread, backward on autograd's worker thread
 
 
 def linear_workspace(dev: torch.device) -> torch.Tensor:
@@ -71,10 +73,11 @@ def linear_workspace(dev: torch.device) -> torch.Tensor:
     (device, stream), allocated at first use and kept: launches on one stream are ordered, so they may share it."""
     idx = dev.index if dev.index is not None else torch.cuda.current_device()
     key = (idx, torch.cuda.current_stream(dev).cuda_stream)
-    ws = _linear_ws_cache.get(key)
-    if ws is None:
-        ws = torch.empty(_lib.lib().mtp_linear_workspace_bytes(), dtype=torch.uint8, device=dev)
-        _linear_ws_cache[key] = ws
+    with _linear_ws_lock:
+        ws = _linear_ws_cache.get(key)
+        if ws is None:
+            ws = torch.empty(_lib.lib().mtp_linear_workspace_bytes(), dtype=torch.uint8, device=dev)
+            _linear_ws_cache[key] = ws
     return ws
 
 
@@ -85,8 +88,11 @@ def _ws_args(t: torch.Tensor, dev: torch.device):
 
 
 def linear_fwd(x2d: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], epilogue: int = EPI_NONE,
-               want_pre: bool = True) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
-    """(y, act) = epilogue(x2d @ w.T + bias).  x2d [M,K], w [N,K] contiguous, same dtype."""
+               want_pre: bool = True, lead: Optional[Tuple[int, ...]] = None
+               ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """(y, act) = epilogue(x2d @ w.T + bias).  x2d [M,K], w [N,K] contiguous, same dtype.  lead: leading
+    dimensions (product M) to allocate the outputs with, so that a caller whose input was [*lead, K] gets
+    [*lead, N] tensors that own their storage instead of views of [M, N] ones."""
     dev = _require_gpu(x2d, w, bias)
     if x2d.dim() != 2 or w.dim() != 2:
         raise ValueError(f"linear_fwd: x must be [M, K] and weight [N, K], got {tuple(x2d.shape)} and {tuple(w.shape)}")
@@ -102,10 +108,17 @@ def linear_fwd(x2d: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
         raise ValueError(f"linear_fwd: SwiGLU needs an even number of weight rows, got {N}")
     x2d, w = _contig(x2d), _contig(w)
     has_act = epilogue in (EPI_BIAS_GELU, EPI_SWIGLU, EPI_GELU)
-    y = torch.empty((M, N), dtype=x2d.dtype, device=dev) if (want_pre or not has_act) else None
+    rows = (M,) if lead is None else tuple(lead)
+    if lead is not None:
+        prod = 1
+        for d in rows:
+            prod *= d
+        if prod != M:
+            raise ValueError(f"linear_fwd: leading dimensions {rows} do not hold {M} rows")
+    y = torch.empty(rows + (N,), dtype=x2d.dtype, device=dev) if (want_pre or not has_act) else None
     act = None
     if has_act:
-        act = torch.empty((M, N // 2 if epilogue == EPI_SWIGLU else N), dtype=x2d.dtype, device=dev)
+        act = torch.empty(rows + (N // 2 if epilogue == EPI_SWIGLU else N,), dtype=x2d.dtype, device=dev)
     with torch.cuda.device(dev):
         wsp, wsb = _ws_args(x2d, dev)
         rc = _lib.lib().mtp_linear_fwd_ws(_p(x2d), _p(w), _p(bias), _p(y), _p(act), wsp, wsb, M, N, K, _dt(x2d),

@@ -728,6 +728,7 @@ def test_layer_backward_in_one_call(gpu, set_tuning, name, m, n, k):
     assert rel(dx[rm], dy[rm].cpu().float() @ ws) < TOL_BF16
     assert rel(dw[rn], dy[:, rn].cpu().float().t() @ x.cpu().float()) < TOL_BF16
     assert rel(db, dy.cpu().float().sum(0)) < TOL_BF16
+    _whole_gradients_by_blocks(x, w, dy, dx, dw, name)
 
 
 def test_measurement_switches_are_not_in_the_shipped_library(gpu, set_tuning):
@@ -824,6 +825,30 @@ def test_gpt2_small_fp32_full_size(gpu):
         assert rel(p.grad, r.grad) < TOL_F32
 
 
+def _whole_gradients_by_blocks(x, w, dy, dx, dw, what, blk=32):
+    """Every element of both gradients in a checked number.  Sums over blocks of `blk` rows commute with the products:
+    dX summed over the rows of a block = (dY summed over those rows) W, and dW summed over the columns of a block =
+    dY^T (X summed over those columns).  Both sides in fp32 on the device (torch's fp32 matmul on the small side), compared
+    per blk x blk block of the output, so that one wrong tile anywhere shows as a block far beyond the rounding of the
+    16-bit gradients (2^-9 per element)."""
+    m, k = x.shape
+    n = w.shape[0]
+    mb, kb = m // blk, k // blk
+    xf, wf, dyf = x.float(), w.float(), dy.float()
+    got_dx = dx.float()[: mb * blk].view(mb, blk, k).sum(1)                      # [m/blk, k]
+    ref_dx = dyf[: mb * blk].view(mb, blk, n).sum(1) @ wf
+    got_dw = dw.float()[:, : kb * blk].view(n, kb, blk).sum(2)                   # [n, k/blk]
+    ref_dw = dyf.t() @ xf[:, : kb * blk].view(m, kb, blk).sum(2)
+    for name, got, ref, axis in (("dx", got_dx[:, : kb * blk].reshape(mb, kb, blk), ref_dx[:, : kb * blk].reshape(mb, kb, blk), 2),
+                                 ("dw", got_dw[: n // blk * blk].reshape(n // blk, blk, kb), ref_dw[: n // blk * blk].reshape(n // blk, blk, kb), 1)):
+        err = (got - ref).double().norm(dim=axis)
+        mag = ref.double().norm(dim=axis)
+        # a block's reference can be small by chance: measure against the typical block as well
+        worst = (err / torch.maximum(mag, mag.median())).max().item()
+        assert worst < 2 * TOL_BF16, (what, name, worst)
+
+
+
 @pytest.mark.parametrize("name,m,k,n", [("llama8b_qkv", 4096, 4096, 6144), ("llama8b_down", 4096, 14336, 4096),
                                          ("llama70b_tp8_qkv", 8192, 8192, 1280), ("llama70b_tp8_oproj", 8192, 1024, 8192),
                                          ("llama70b_tp8_down", 8192, 3584, 8192)])
@@ -843,6 +868,7 @@ def test_linear_full_size_sampled(gpu, name, m, k, n):
     assert rel(dx[rm], R.linear_backward(xs, ws, dys, False)[0]) < TOL_BF16
     ref_dw = R.linear_backward(x.cpu().float(), ws[rn.cpu()], dy[:, rn].cpu().float(), False)[1]
     assert rel(dw[rn], ref_dw) < TOL_BF16
+    _whole_gradients_by_blocks(x, w, dy, dx, dw, name)
     y2, _ = ops.linear_fwd((x.float() * 2).bfloat16(), w, None, ops.EPI_NONE)     # exact in bf16: scaling by 2
     assert torch.equal(y2.float(), y.float() * 2)
 
@@ -873,6 +899,7 @@ def test_swiglu_full_size_sampled(gpu, name, m, k, half):
     assert rel(dx[rm], R.linear_backward(xs, ws, dys, False)[0]) < TOL_BF16
     ref_dw = R.linear_backward(x.cpu().float(), ws[rn.cpu()], dy[:, rn].cpu().float(), False)[1]
     assert rel(dw[rn], ref_dw) < TOL_BF16
+    _whole_gradients_by_blocks(x, w, dy, dx, dw, name)
     y2, _ = ops.linear_fwd((x.float() * 2).bfloat16(), w, None, ops.EPI_SWIGLU)   # exact in bf16: scaling by 2
     assert torch.equal(y2.float(), y.float() * 2)
 
@@ -895,6 +922,52 @@ def test_module_surface_on_gpu(gpu):
     assert dev_layer.weight.is_cuda and dev_layer.bias.is_cuda
     empty, _ = dev_layer(torch.empty(0, 64, device=gpu))
     assert empty.shape == (0, 64)
+
+
+def test_model_parallel_rng_on_the_device(gpu):
+    """The device path of the weight initialisation (layers.py:44-53): shards drawn on the GPU under the
+    model-parallel generator state: the same shard for one rank seeded twice, different shards for two ranks of one
+    group, the device's default generator state (and the host's) left where it was."""
+    from merak_amd.mpu.layers import _initialize_affine_weight_gpu
+
+    def shard(rank, seed=1234):
+        mpu.set_model_parallel_world_size(2)
+        mpu.set_model_parallel_rank(rank)
+        mpu.model_parallel_manual_seed(seed)
+        before_gpu, before_cpu = torch.cuda.get_rng_state(gpu), torch.get_rng_state()
+        w = torch.empty(8, 16, device=gpu)
+        _initialize_affine_weight_gpu(w, torch.nn.init.normal_, 0)
+        assert torch.equal(torch.cuda.get_rng_state(gpu), before_gpu) and torch.equal(torch.get_rng_state(), before_cpu)
+        return w
+
+    a, b, a2 = shard(0), shard(1), shard(0)
+    assert not torch.equal(a, b) and torch.equal(a, a2)
+    # host-resident weights on a machine with a GPU draw under the same tracker
+    mpu.model_parallel_manual_seed(99)
+    c1 = torch.empty(4, 4)
+    _initialize_affine_weight_gpu(c1, torch.nn.init.normal_, 0)
+    mpu.model_parallel_manual_seed(99)
+    c2 = torch.empty(4, 4)
+    _initialize_affine_weight_gpu(c2, torch.nn.init.normal_, 0)
+    assert torch.equal(c1, c2)
+
+
+def test_one_launch_ce_marks_the_layer_logits_as_overwritten(gpu):
+    """The one-launch cross entropy overwrites the logits with their gradient during forward.  The logits a
+    ColumnParallelLinear returns own their storage (no view), so the overwrite is recorded: another function that
+    saved those logits for its own backward fails loudly instead of using gradients as if they were logits."""
+    set_args(use_cpu_initialization=True, params_dtype=torch.bfloat16)
+    col = mpu.ColumnParallelLinear(64, 512, bias=False, gather_output=False).to(gpu)
+    x = torch.randn(4, 8, 64, generator=gen(90)).bfloat16().to(gpu).requires_grad_(True)
+    tgt = torch.randint(0, 512, (4, 8), generator=gen(91)).to(gpu)
+    logits, _ = col(x)
+    assert logits.shape == (4, 8, 512) and not logits._is_view()
+    other = (logits * logits).sum()             # saves the logits for its backward
+    loss = mpu.vocab_loss_fn(logits, tgt)       # overwrites them
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        other.backward(retain_graph=True)
+    loss.backward()
+    assert x.grad is not None and torch.isfinite(x.grad.float()).all()
 
 
 def test_modules_cast_to_bf16_after_construction(gpu):

@@ -328,10 +328,19 @@ def secondary(dev, timer, reps, with_cpu):
             pass
         torch.set_num_threads(cores)
         made = False
-        if not dist.is_initialized():
-            dist.init_process_group("gloo", init_method="tcp://127.0.0.1:29577", rank=0, world_size=1)
-            made = True
-        grp = dist.new_group([0], backend="gloo")
+        # gloo announces its connections on stdout, which carries this script's one JSON line: send the
+        # process's stdout to stderr while the group is built
+        sys.stdout.flush()
+        keep = os.dup(1)
+        os.dup2(2, 1)
+        try:
+            if not dist.is_initialized():
+                dist.init_process_group("gloo", init_method="tcp://127.0.0.1:29577", rank=0, world_size=1)
+                made = True
+            grp = dist.new_group([0], backend="gloo")
+        finally:
+            os.dup2(keep, 1)
+            os.close(keep)
         ts, gs = tgt[:rows].cpu(), go[:rows].cpu()
         t0 = time.perf_counter()
         for _ in range(3):
@@ -475,9 +484,14 @@ def secondary(dev, timer, reps, with_cpu):
     r_ms = timer.run("mfma_r", lambda: _lib.check(_lib.lib().mtp_mfma_peak(sink.data_ptr(), 4096, iters, 1, st), "peak"), 3)
     del src, dst
     out["vendor_blas_same_gemms"] = vendor_compare(dev, reps)
+    gi = 128 * 1024
+    g0 = timer.run("mfma_g0", lambda: _lib.check(_lib.lib().mtp_mfma_peak_gemm_loop(sink.data_ptr(), 1024, gi, 0, st), "peak"), 3)
+    g1 = timer.run("mfma_g1", lambda: _lib.check(_lib.lib().mtp_mfma_peak_gemm_loop(sink.data_ptr(), 1024, gi, 1, st), "peak"), 3)
     out["device_reference"] = {"copy_1GiB_GBs_read_plus_write": round(2 * src_bytes / c_ms / 1e6, 1),
-                               "mfma_loop_bf16_tflops_smooth_operands": round(4096 * iters * 32 * 32 * 16 * 2 / p_ms / 1e9, 1),
-                               "mfma_loop_bf16_tflops_random_operands": round(4096 * iters * 32 * 32 * 16 * 2 / r_ms / 1e9, 1)}
+                               "mfma_32x32x16_4acc_tflops_smooth_operands": round(4096 * iters * 32 * 32 * 16 * 2 / p_ms / 1e9, 1),
+                               "mfma_32x32x16_4acc_tflops_random_operands": round(4096 * iters * 32 * 32 * 16 * 2 / r_ms / 1e9, 1),
+                               "mfma_16x16x32_gemm_loop_tflops_smooth_operands": round(1024 * gi * 16 * 16 * 32 * 2 / g0 / 1e9, 1),
+                               "mfma_16x16x32_gemm_loop_tflops_random_operands": round(1024 * gi * 16 * 16 * 32 * 2 / g1 / 1e9, 1)}
     return out
 
 
@@ -516,6 +530,44 @@ def vendor_compare(dev, reps, kinds=("fwd", "dgrad", "wgrad")):
             "per_gemm": rows}
 
 
+def gemm_loop_parts(dev, reps):
+    """Where the time of the 64-deep GEMM loop goes: the gate/up forward launch of the headline step (with the SwiGLU
+    epilogue, and as a plain product) timed whole, with its DMA requests answered out of range (instructions issued,
+    LDS written, no memory traffic), with no DMA requests at all, with no fragment reads from LDS, and with neither.
+    Needs the measurement build of the library (python -m merak_amd.build --measure; MERAK_AMD_LIB points at it):
+    the switched-off forms compute wrong results and do not exist in the library that ships."""
+    from merak_amd import ops, _lib
+    lib = _lib.lib()
+    L = build_linear_workload(dev, LLAMA8B, 4096, 20)[1]
+    flops = 2.0 * L["M"] * L["N"] * L["K"]
+    variants = (("whole", 0), ("dma_answered_out_of_range", 4), ("no_dma_requests", 16), ("no_lds_fragment_reads", 32),
+                ("no_dma_requests_no_lds_reads", 48))
+    forms = (("swiglu", ops.EPI_SWIGLU), ("plain", ops.EPI_NONE))
+    acc = {(f, v): [] for f, _ in forms for v, _ in variants}
+    timer = Timer()
+    try:
+        for _ in range(3):                      # the variants in turn, three times: all see the same clocks
+            for v, bits in variants:
+                os.environ["MTP_GEMM_DEBUG"] = str(bits)
+                lib.mtp_reload_tuning()
+                for f, epi in forms:
+                    acc[(f, v)].append(timer.run(f"{f}.{v}", lambda: ops.linear_fwd(L["x"], L["w"], None, epi, want_pre=True), reps))
+    finally:
+        os.environ.pop("MTP_GEMM_DEBUG", None)
+        lib.mtp_reload_tuning()
+    out = {}
+    for f, _ in forms:
+        whole = statistics.mean(acc[(f, "whole")])
+        out[f] = {v: {"ms": round(statistics.mean(acc[(f, v)]), 4), "tflops_equivalent": round(flops / statistics.mean(acc[(f, v)]) / 1e9, 1),
+                      "share_of_whole": round(statistics.mean(acc[(f, v)]) / whole, 4)} for v, _ in variants}
+    sink = torch.empty(64 * 1024, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    gi = 128 * 1024
+    g1 = timer.run("mfma_g1", lambda: _lib.check(lib.mtp_mfma_peak_gemm_loop(sink.data_ptr(), 1024, gi, 1, st), "peak"), 5)
+    out["mfma_16x16x32_gemm_loop_tflops_random_operands"] = round(1024 * gi * 16 * 16 * 32 * 2 / g1 / 1e9, 1)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -525,10 +577,12 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="headline only (no secondary figures)")
     ap.add_argument("--cpu-tokens", type=int, default=4096,
                     help="tokens of the workload the CPU baseline runs (default: all 4096, about 13 s on 16 cores)")
-    ap.add_argument("--only", choices=["gemm-fwd-vs-vendor", "gemm-vs-vendor"], default=None,
+    ap.add_argument("--only", choices=["gemm-fwd-vs-vendor", "gemm-vs-vendor", "gemm-loop-parts"], default=None,
                     help="launch nothing but the forward GEMMs (or all nine plain GEMMs) of the headline step, each "
                          "through the vendor library and through this one in turn, and print their times: the "
-                         "program to put behind `rocprofv3 --pmc ... --` or `--kernel-trace` for a counter comparison")
+                         "program to put behind `rocprofv3 --pmc ... --` or `--kernel-trace` for a counter comparison; "
+                         "gemm-loop-parts: the gate/up forward launch with parts of its main loop switched off "
+                         "(measurement build of the library only)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (no collectives, one rank's share "
@@ -542,6 +596,13 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.only == "gemm-loop-parts":
+        if "measure" not in os.environ.get("MERAK_AMD_LIB", ""):
+            print("gemm-loop-parts needs the measurement build: python -m merak_amd.build --measure, then "
+                  "MERAK_AMD_LIB=merak_amd/lib/libmerak_tp_gfx950_measure.so", file=sys.stderr)
+            sys.exit(2)
+        print(json.dumps({"mode": args.only, **gemm_loop_parts(dev, max(3, args.steps))}))
+        return
     if args.only:
         kinds = ("fwd",) if args.only == "gemm-fwd-vs-vendor" else ("fwd", "dgrad", "wgrad")
         res = vendor_compare(dev, max(3, args.steps), kinds)
@@ -576,11 +637,17 @@ def main():
                 "launch_ms": dom["ms"], "flops_per_launch": 2.0 * dom["M"] * dom["N"] * dom["K"]}
     # what the matrix cores sustain on this board with no memory traffic at all (register-resident MFMA loop on
     # operands of random sign and mantissa): the chip runs against its power limit well below the published peak
+    # The ceiling probe is the GEMM's own instruction stream: v_mfma_f32_16x16x32_bf16 on 64 accumulator quads, 32
+    # operand fragments walked in the loop's quadrant order, one wave per SIMD, 128 MFMAs per pass, nothing else.
     sink = torch.empty(64 * 4096, device=dev)
     st = torch.cuda.current_stream().cuda_stream
-    r_ms = timer.run("mfma_r", lambda: _lib.check(_lib.lib().mtp_mfma_peak(sink.data_ptr(), 4096, 8192, 1, st), "peak"), 12)
-    roofline["mfma_loop_random_operands"] = round(4096 * 8192 * 32 * 32 * 16 * 2 / r_ms / 1e9, 1)
+    g_iters = 128 * 1024
+    r_ms = timer.run("mfma_g", lambda: _lib.check(_lib.lib().mtp_mfma_peak_gemm_loop(sink.data_ptr(), 1024, g_iters, 1, st),
+                                                  "peak"), 12)
+    roofline["mfma_loop_random_operands"] = round(1024 * g_iters * 16 * 16 * 32 * 2 / r_ms / 1e9, 1)
+    roofline["mfma_loop"] = "v_mfma_f32_16x16x32_bf16, 64 accumulator quads, 1024 waves, register-resident"
     roofline["frac_of_mfma_loop"] = round(dom["tflops"] / roofline["mfma_loop_random_operands"], 4)
+    roofline["launch_ms_median"] = round(timer.median[dom["kernel"]], 4)
     del work, sink
     result = {
         "metric": "TP-shard linear fwd+bwd TFLOP/s (% bf16 peak); vocab-CE HBM GB/s",

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define MTP_ABI_VERSION 11
+#define MTP_ABI_VERSION 12
 
 /* element types.  MTP_F16 is IEEE half, what the reference's --fp16 sets as
  * params_dtype (Merak/merak_args/args.py:584-585). */
@@ -127,6 +127,12 @@ int mtp_linear_bias_grad(const void* dy, void* db, int64_t M, int64_t N,
  * exactly the call without scratch.  The reference has no counterpart (its
  * F.linear at layers.py:252,354 leaves such choices to the BLAS library). */
 int64_t mtp_linear_workspace_bytes(void);
+/* Bytes of scratch a product of a layer with these sizes (M tokens, N output
+ * features, K input features) can make use of — kind 0 forward, 1 input
+ * gradient, 2 weight gradient, 3 both gradients — or 0 if it never touches
+ * the scratch (most shapes): lets a caller allocate only when it pays.  Never
+ * more than mtp_linear_workspace_bytes() on the 16-bit path. */
+int64_t mtp_linear_workspace_need(int kind, int64_t M, int64_t N, int64_t K, int dtype);
 int mtp_linear_fwd_ws(const void* x, const void* w, const void* bias,
                       void* y, void* act, void* workspace, int64_t workspace_bytes,
                       int64_t M, int64_t N, int64_t K,
@@ -285,6 +291,22 @@ int64_t mtp_gemv_workspace_bytes(int64_t B, int64_t N, int64_t K, int epilogue);
 int mtp_gemv_ws(const void* x, const void* w, const void* bias, void* y,
                 void* workspace, int64_t workspace_bytes,
                 int64_t B, int64_t N, int64_t K, int epilogue, int dtype, void* stream);
+
+/* Two products over the same activations in one call:
+ *   y1   [B, N1]   = x W1^T (+ bias1)
+ *   act2 [B, N2/2] = silu(G) * U, (G | U) = x W2^T (+ bias2), W2 = [gate rows | up rows]
+ * — what a block whose QKV and gate/up projections read the same rows computes
+ * (the decode step of Merak/inference/text_generation_inference.py:199-203 on
+ * the linears of one block).  Above 16 batch rows both products go out as one
+ * grid, so that the smaller one does not start and drain the chip on its own;
+ * otherwise (and for shapes the one grid does not take) the call is the two
+ * launches of mtp_gemv_ws, with the same workspace rules.  act2 has the bits
+ * of the separate call; y1 is summed along k in the order of the one grid's
+ * larger row blocks (equal to the separate call to rounding). */
+int mtp_gemv_pair(const void* x, const void* w1, const void* bias1, void* y1, int64_t N1,
+                  const void* w2, const void* bias2, void* act2, int64_t N2,
+                  void* workspace, int64_t workspace_bytes,
+                  int64_t B, int64_t K, int dtype, void* stream);
 
 /* mtp_gemv_ws with what a decoder block puts around its linears (HF
  * LlamaDecoderLayer.forward: `residual + hidden_states`, LlamaRMSNorm in
@@ -447,6 +469,14 @@ int mtp_stream_copy(const void* src, void* dst, int64_t bytes, void* stream);
  * because the chip runs against its power limit.  Reports nothing itself:
  * time it with events. */
 int mtp_mfma_peak(float* sink, int64_t n_waves, int64_t iters, int random_data, void* stream);
+
+/* The same for the instruction stream of the 64-deep GEMM loop: iters x
+ * v_mfma_f32_16x16x32_bf16 per wave (iters a multiple of 128) on 64
+ * accumulator quads with 32 register-resident operand fragments walked in
+ * the GEMM's quadrant order; no LDS reads, no memory traffic.  Launch it on
+ * 1024 waves (one per SIMD, as the GEMM runs) for the ceiling of that loop on
+ * this board.  No counterpart in the reference: a measurement aid. */
+int mtp_mfma_peak_gemm_loop(float* sink, int64_t n_waves, int64_t iters, int random_data, void* stream);
 
 #ifdef __cplusplus
 }

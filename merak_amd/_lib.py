@@ -19,7 +19,7 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmerak_tp_gfx950.so"
 
 MTP_F32, MTP_BF16, MTP_F16 = 0, 1, 2
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_SWIGLU, EPI_GELU = 0, 1, 2, 3, 4
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 _i64, _int, _vp = C.c_int64, C.c_int, C.c_void_p
 
@@ -33,6 +33,7 @@ SIGNATURES = {
     "mtp_linear_wgrad": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _int, _vp]),
     "mtp_linear_bias_grad": (_int, [_vp, _vp, _i64, _i64, _int, _int, _int, _vp]),
     "mtp_linear_workspace_bytes": (_i64, []),
+    "mtp_linear_workspace_need": (_i64, [_int, _i64, _i64, _i64, _int]),
     "mtp_linear_fwd_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "mtp_linear_dgrad_ws": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "mtp_linear_wgrad_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
@@ -57,6 +58,7 @@ SIGNATURES = {
     "mtp_gemv_workspace_bytes": (_i64, [_i64, _i64, _i64, _int]),
     "mtp_gemv_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "mtp_gemv_norm_fits": (_int, [_i64, _i64]),
+    "mtp_gemv_pair": (_int, [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _int, _vp]),
     "mtp_gemv_fused": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, C.c_float, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int,
                               _int, _vp]),
     "mtp_rmsnorm": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, C.c_float, _int, _vp]),
@@ -68,6 +70,7 @@ SIGNATURES = {
     "mtp_reload_tuning": (None, []),
     "mtp_stream_copy": (_int, [_vp, _vp, _i64, _vp]),
     "mtp_mfma_peak": (_int, [_vp, _i64, _i64, _int, _vp]),
+    "mtp_mfma_peak_gemm_loop": (_int, [_vp, _i64, _i64, _int, _vp]),
 }
 
 _lock = threading.Lock()

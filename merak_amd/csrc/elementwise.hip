@@ -195,6 +195,65 @@ __global__ __launch_bounds__(256) void mfma_peak_kernel(float* __restrict__ sink
   sink[(int64_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// The same measurement for the instruction stream of the 64-deep GEMM loop: v_mfma_f32_16x16x32_bf16 on 64
+// accumulator quads (the whole accumulator file), operands from 32 register-resident fragments (two units of four
+// 16-row blocks of A and of B, two k steps each) walked quadrant by quadrant as the GEMM walks a k-tile: 128 MFMAs
+// per pass, no LDS reads, no memory traffic, no barriers.  One wave per SIMD, like the GEMM.  What this loop
+// sustains is the ceiling of the GEMM's main loop on this board at its power limit.
+__device__ __forceinline__ void mfma_gemm_loop_body(float* __restrict__ sink, int64_t iters, int random_data) {
+  const int lane = threadIdx.x & 63;
+  bf16x8_t ra[2][4][2], rb[2][4][2];
+  uint32_t rng = 0x9e3779b9u * (uint32_t)(blockIdx.x * 256 + threadIdx.x + 1);
+#pragma unroll
+  for (int f = 0; f < 32; f++) {
+    u32x4_t v;
+    uint32_t* pv = reinterpret_cast<uint32_t*>(&v);
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      if (random_data) {
+        rng ^= rng << 13; rng ^= rng >> 17; rng ^= rng << 5;
+        pv[q] = (rng & 0x80ff80ffu) | 0x3f003f00u;      // sign and mantissa random, values in +-[0.5, 2)
+      } else {
+        pv[q] = pack_bf16x2(0.001f * (lane + 2 * q + f), 0.001f * (lane + 2 * q + 1 + f));
+      }
+    }
+    if (f < 16) ra[f >> 3][(f >> 1) & 3][f & 1] = __builtin_bit_cast(bf16x8_t, v);
+    else rb[(f >> 3) & 1][(f >> 1) & 3][f & 1] = __builtin_bit_cast(bf16x8_t, v);
+  }
+  f32x4_t acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int j = 0; j < 8; j++) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int64_t it = 0; it < iters; it += 128) {
+#pragma unroll
+    for (int qd = 0; qd < 4; qd++) {          // Q00 Q01 Q11 Q10: consecutive quadrants share a unit
+      const int MA = qd >> 1, MB = (qd & 1) ^ MA;
+#pragma unroll
+      for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+          for (int jj = 0; jj < 4; jj++) {
+            const int j = (i & 1) ? 3 - jj : jj;
+            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                         : "+a"(acc[MA * 4 + i][MB * 4 + j])
+                         : "v"(rb[MB][j][kk]), "v"(ra[MA][i][kk]));
+          }
+    }
+  }
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last results reach the registers before they are read
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int j = 0; j < 8; j++) t += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+  sink[(int64_t)blockIdx.x * blockDim.x + threadIdx.x] = t;
+}
+__global__ __launch_bounds__(256) void mfma_gemm_loop_kernel(float* __restrict__ sink, int64_t iters, int random_data) {
+  mfma_gemm_loop_body(sink, iters, random_data);
+}
+
 unsigned grid_for(int64_t work_items) {
   int64_t b = (work_items + 255) / 256;
   if (b > 256 * 32) b = 256 * 32;
@@ -279,5 +338,14 @@ extern "C" int mtp_mfma_peak(float* sink, int64_t n_waves, int64_t iters, int ra
   hipLaunchKernelGGL(mfma_peak_kernel, dim3((unsigned)(n_waves / 4)), dim3(256), 0, (hipStream_t)stream, sink, iters,
                      random_data);
   MTP_CHECK_LAUNCH("mfma_peak");
+  return MTP_OK;
+}
+
+extern "C" int mtp_mfma_peak_gemm_loop(float* sink, int64_t n_waves, int64_t iters, int random_data, void* stream) {
+  MTP_REQUIRE(sink && n_waves >= 4 && n_waves % 4 == 0 && iters >= 128 && iters % 128 == 0, MTP_EINVAL,
+              "mfma_peak_gemm_loop: n_waves must be a positive multiple of 4 and iters of 128");
+  hipLaunchKernelGGL(mfma_gemm_loop_kernel, dim3((unsigned)(n_waves / 4)), dim3(256), 0, (hipStream_t)stream, sink, iters,
+                     random_data);
+  MTP_CHECK_LAUNCH("mfma_peak_gemm_loop");
   return MTP_OK;
 }

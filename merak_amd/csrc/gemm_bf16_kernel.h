@@ -136,6 +136,11 @@ __device__ __forceinline__ void dma16(rsrc_t rsrc, uint32_t lds_addr, uint32_t v
 // INST_OFF goes into the instruction's offset field, which moves the LDS address and the memory address alike:
 // instructions that fill consecutive KiB of LDS can share one setting of M0 when each one's VGPR offset has
 // INST_OFF taken off (the range check sees the sum, the true offset).  SET_M0: first instruction of such a run.
+// The statements that follow a setting one read M0 without saying so (an inline-assembly statement can name M0
+// neither as an input nor as a clobber: it is a reserved register, which the compiler never allocates and writes
+// only where it lowers an instruction that needs it).  Between the statements of a run this file therefore puts
+// MFMAs, LDS reads and scalar address arithmetic only: no indexed register access, no messages, no LDS-direct
+// builtins, nothing that is lowered through M0.
 template <bool SET_M0, int LDS_OFF, int INST_OFF>
 __device__ __forceinline__ void dma16_at(rsrc_t rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
   static_assert(INST_OFF >= 0 && INST_OFF < 4096, "12-bit instruction offset");
@@ -386,21 +391,25 @@ template <int ROWS, int NW> struct OperandOf<LAY_COL, ROWS, NW> { using type = C
 //            16 (g/2) + l%16, columns 16 (g%2) + 4 (l/16) .. +3.
 // accv(i, j, g, e) is element e of group g; rsum_of(i, g) (EPI_ROWSUM only) the lane's part of the k sum of the
 // A row that group g sits in.
-template <int BM, int BN, int EPI, int OUT, int NW, bool F16, bool QMAP, int LDS_BYTES, int TI, int TJ, int BLK,
+// The wave grid is WGM x WGN.  Along a dimension with one wave only (the 64-deep loop's 160- and 192-wide tiles:
+// 4 x 1 or 1 x 4 waves) the two units lie side by side and the wave's blocks are simply consecutive.
+template <int BM, int BN, int EPI, int OUT, int WGM, int WGN, bool F16, bool QMAP, int LDS_BYTES, int TI, int TJ, int BLK,
           typename AccFn, typename RsumFn>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, AccFn accv, RsumFn rsum_of, char* lds, int m0, int n0,
                                               int tn, int wave, int lane) {
   using X = X16<F16>;
   static_assert(BLK == 32 || BLK == 16, "MFMA block: 32x32 or 16x16");
-  constexpr int WGM = 2, WGN = NW / 2;
+  constexpr int NW = WGM * WGN;
   constexpr int HI = TI / 2, HJ = TJ / 2;
+  constexpr bool QM = QMAP && WGM > 1, QN = QMAP && WGN > 1;    // unit mapping along m / n
+  static_assert((!QM || TI % 2 == 0) && (!QN || TJ % 2 == 0), "two units of whole 32-wide blocks per wave");
   const int wm = wave / WGN, wn = wave % WGN;
   // row (inside the 32-row block) and first column (inside the 32-column block) of group g
   auto row_off = [&](int g) -> int { return BLK == 32 ? (lane & 31) : 16 * (g >> 1) + (lane & 15); };
   auto col_off = [&](int g) -> int { return BLK == 32 ? 8 * g + 4 * (lane >> 5) : 16 * (g & 1) + 4 * (lane >> 4); };
   // first tile row of the wave's block row i
   auto blk_row = [&](int i) -> int {
-    if (QMAP) return (i / HI) * (BM / 2) + wm * (32 * HI) + (i % HI) * 32;
+    if (QM) return (i / HI) * (BM / 2) + wm * (32 * HI) + (i % HI) * 32;
     return wm * (BM / WGM) + 32 * i;
   };
 
@@ -444,7 +453,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, AccFn accv, Rsu
       const int hj = TJ / 2;
       return (j < hj ? 0 : p.half) + n0 + wn * (WN / 2) + (j % hj) * 32;
     }
-    if (QMAP) return n0 + (j / HJ) * (BN / 2) + wn * (32 * HJ) + (j % HJ) * 32;
+    if (QN) return n0 + (j / HJ) * (BN / 2) + wn * (32 * HJ) + (j % HJ) * 32;
     return n0 + wn * WN + j * 32;
   };
   // first column past the valid range of block j: SwiGLU gate blocks end at `half` (the columns after it
@@ -457,45 +466,64 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, AccFn accv, Rsu
   // The whole tile lies inside the matrix: the epilogue needs no bounds checks.
   const bool tile_inside = m0 + BM <= p.M && (EPI == MTP_EPI_SWIGLU ? n0 + BN / 2 <= p.half : n0 + BN <= p.N);
 
+  // Fast path of flush, for the blocks [JB, JB + NB) of the staged row (NB a power of two, at most 4): 16-byte
+  // aligned rows of a tile that is completely inside: lane l owns chunk l % CPR of rows l / CPR, l / CPR + 64 / CPR,
+  // ...; one address computation, then constant strides.
+  auto flush_piece = [&](int i, void* out, int64_t ld, auto jb_tag, auto nb_tag, auto colfn, auto f32_tag, bool accumulate) {
+    constexpr int JB = decltype(jb_tag)::value, NB = decltype(nb_tag)::value;
+    constexpr bool f32out = decltype(f32_tag)::value;
+    constexpr int esz_c = f32out ? 4 : 2;
+    constexpr int CPR = NB * 32 * esz_c / 16;                              // 16-byte chunks per staged row piece
+    static_assert(CPR == 4 || CPR == 8 || CPR == 16 || CPR == 32, "a power of two of lanes per row");
+    constexpr int RPI = 64 / CPR, ITERS = 32 / RPI;
+    const int r0 = lane / CPR, cc = lane % CPR;
+    const int e0 = cc * (16 / esz_c);
+    const int col = colfn(JB + (e0 >> 5)) + (e0 & 31);
+    char* gp = (char*)out + ((int64_t)(m0 + blk_row(i) + r0) * ld + col) * esz_c;
+    const char* sp = stage + r0 * PITCH + JB * 32 * esz_c + cc * 16;
+    const int64_t gstride = (int64_t)RPI * ld * esz_c;
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) {
+      u32x4_t v = *reinterpret_cast<const u32x4_t*>(sp + it * RPI * PITCH);
+      u32x4_t* q = reinterpret_cast<u32x4_t*>(gp + it * gstride);
+      if (accumulate) {
+        const u32x4_t o = *q;
+        if (f32out) {
+          v.x = __float_as_uint(__uint_as_float(v.x) + __uint_as_float(o.x));
+          v.y = __float_as_uint(__uint_as_float(v.y) + __uint_as_float(o.y));
+          v.z = __float_as_uint(__uint_as_float(v.z) + __uint_as_float(o.z));
+          v.w = __float_as_uint(__uint_as_float(v.w) + __uint_as_float(o.w));
+        } else {
+          v.x = X::pack2(X::lo(v.x) + X::lo(o.x), X::hi(v.x) + X::hi(o.x));
+          v.y = X::pack2(X::lo(v.y) + X::lo(o.y), X::hi(v.y) + X::hi(o.y));
+          v.z = X::pack2(X::lo(v.z) + X::lo(o.z), X::hi(v.z) + X::hi(o.z));
+          v.w = X::pack2(X::lo(v.w) + X::lo(o.w), X::hi(v.w) + X::hi(o.w));
+        }
+      }
+      __builtin_nontemporal_store(v, q);  // written once, read by a later kernel: keep it out of the way of A/B in L2
+    }
+  };
   auto flush = [&](int i, void* out, int64_t ld, auto nblk_tag, auto colfn, auto limfn, auto f32_tag, bool accumulate) {
     constexpr int nblk = decltype(nblk_tag)::value;
     constexpr bool f32out = decltype(f32_tag)::value;
     {
-      // Fast path: 16-byte aligned rows of a tile that is completely inside: lane l owns chunk l % CPR of
-      // rows l / CPR, l / CPR + 64 / CPR, ...; one address computation, then constant strides.
       constexpr int esz_c = f32out ? 4 : 2;
-      constexpr int CPR = nblk * 32 * esz_c / 16;                            // 16-byte chunks per staged row
-      constexpr int CPRP = CPR <= 4 ? 4 : CPR <= 8 ? 8 : CPR <= 16 ? 16 : 32;  // lanes per row (power of two)
-      constexpr int RPI = 64 / CPRP, ITERS = 32 / RPI;
-      const int r0 = lane / CPRP, cc = lane % CPRP;
-      const int e0 = cc * (16 / esz_c);
-      const int col = colfn(e0 >> 5) + (e0 & 31);
-      char* gp = (char*)out + ((int64_t)(m0 + blk_row(i) + r0) * ld + col) * esz_c;
       const bool aligned = ((reinterpret_cast<uintptr_t>(out) | (uintptr_t)(ld * esz_c)) & 15) == 0;
       if (tile_inside && aligned) {
-        if (CPRP != CPR && cc >= CPR) return;
-        const char* sp = stage + r0 * PITCH + cc * 16;
-        const int64_t gstride = (int64_t)RPI * ld * esz_c;
-#pragma unroll
-        for (int it = 0; it < ITERS; it++) {
-          u32x4_t v = *reinterpret_cast<const u32x4_t*>(sp + it * RPI * PITCH);
-          u32x4_t* q = reinterpret_cast<u32x4_t*>(gp + it * gstride);
-          if (accumulate) {
-            const u32x4_t o = *q;
-            if (f32out) {
-              v.x = __float_as_uint(__uint_as_float(v.x) + __uint_as_float(o.x));
-              v.y = __float_as_uint(__uint_as_float(v.y) + __uint_as_float(o.y));
-              v.z = __float_as_uint(__uint_as_float(v.z) + __uint_as_float(o.z));
-              v.w = __float_as_uint(__uint_as_float(v.w) + __uint_as_float(o.w));
-            } else {
-              v.x = X::pack2(X::lo(v.x) + X::lo(o.x), X::hi(v.x) + X::hi(o.x));
-              v.y = X::pack2(X::lo(v.y) + X::lo(o.y), X::hi(v.y) + X::hi(o.y));
-              v.z = X::pack2(X::lo(v.z) + X::lo(o.z), X::hi(v.z) + X::hi(o.z));
-              v.w = X::pack2(X::lo(v.w) + X::lo(o.w), X::hi(v.w) + X::hi(o.w));
-            }
-          }
-          __builtin_nontemporal_store(v, q);  // written once, read by a later kernel: keep it out of the way of A/B in L2
-        }
+        // the staged row goes out in pieces of 4, 2 and 1 blocks (a 5-block row: 4 + 1), each with a power of two
+        // of lanes per row
+        constexpr int STEP = 4;
+        constexpr int N4 = nblk / STEP, REM = nblk % STEP;
+        static_for<N4>([&](auto t) {
+          flush_piece(i, out, ld, std::integral_constant<int, decltype(t)::value * STEP>{}, std::integral_constant<int, STEP>{},
+                      colfn, f32_tag, accumulate);
+        });
+        if constexpr (REM >= 2)
+          flush_piece(i, out, ld, std::integral_constant<int, N4 * STEP>{}, std::integral_constant<int, 2>{}, colfn, f32_tag,
+                      accumulate);
+        if constexpr (REM % 2 == 1)
+          flush_piece(i, out, ld, std::integral_constant<int, N4 * STEP + (REM >= 2 ? 2 : 0)>{}, std::integral_constant<int, 1>{},
+                      colfn, f32_tag, accumulate);
         return;
       }
     }
@@ -685,20 +713,23 @@ constexpr int QBK = 64;    // k-tile depth
 // (lane l -> row l/8, position l%8, fetching chunk (l%8) ^ swizzle of its row: the 8 lanes of a row still ask
 // for one whole line); a wave's NU instructions of a unit fill 8 NU consecutive rows, so that they share one
 // setting of M0 (dma16_at).  Fragment = one ds_read_b128.
-template <int NW, int WG, int BLK>
+//
+// UR = rows per unit: 128 (256-row tile), or 96 / 80 for the 192- and 160-row tiles, whose units are padded in LDS
+// to the rows the waves' DMA instructions cover (8 NU NW); the instructions of the padding rows read out of range.
+template <int NW, int WG, int BLK, int UR = 128>
 struct RowOperandQ {
-  static constexpr int UROWS = 128;                  // rows per unit
-  static constexpr int UBYTES = UROWS * QBK * 2;     // 16 KiB
+  static constexpr int UROWS = UR;                   // rows per unit
+  static constexpr int NU = (UROWS / 8 + NW - 1) / NW;   // DMA instructions per wave and unit
+  static constexpr int UBYTES = NU * NW * 8 * QBK * 2;   // 16 KiB at 128 rows
   static constexpr int BYTES = 2 * UBYTES;           // per k-tile buffer
   static constexpr int QKS = BLK == 32 ? 4 : 2;      // MFMA steps per k-tile
   static constexpr int H = UROWS / (BLK * WG);       // BLK-row blocks per wave and unit
-  static constexpr int NU = UROWS / 8 / NW;          // DMA instructions per wave and unit
-  static_assert(H >= 1 && NU >= 1, "wave grid too fine for the unit");
+  static_assert(H >= 1 && NU >= 1 && H * BLK * WG == UROWS && UROWS % 8 == 0, "wave grid does not divide the unit");
   rsrc_t rsrc;
   uint32_t voff[2][NU];
   uint32_t fo[2][QKS];   // [k-tile buffer][step]: the buffer's 64 KiB do not fit the 16-bit offset field of a read
 
-  // rowmap(r): global row (relative to row0) of tile row r (unit r / 128), or a negative value for "no such row";
+  // rowmap(r): global row (relative to row0) of tile row r (unit r / UROWS), or a negative value for "no such row";
   // wsub: the wave's index along this operand's dimension
   template <typename RowMap>
   __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int row0, int nrows, int K_, int lane,
@@ -713,8 +744,8 @@ struct RowOperandQ {
       for (int j = 0; j < NU; j++) {
         const int q = NU * wave + j;
         const int gchunk = (lane & 7) ^ ((4 * q + (lane >> 4)) & 7);
-        const int r = u * UROWS + q * 8 + (lane >> 3);
-        const int64_t gr = rowmap(r);
+        const int ru = q * 8 + (lane >> 3);                       // row inside the (padded) unit
+        const int64_t gr = ru < UROWS ? rowmap(u * UROWS + ru) : -1;
         // a valid row r >= 8 j lies at least 1024 j bytes into the buffer (rows are at least 128 bytes long)
         voff[u][j] = ((gr < 0 || gr >= nrows - row0) ? 0x80000000u : (uint32_t)((gr * ld + gchunk * 8) * 2)) - 1024u * j;
       }
@@ -756,15 +787,19 @@ struct RowOperandQ {
 // (lane l -> k-row l/16, position l%16).  Fragment = two ds_read_b64_tr_b16: in each group of 16 lanes, lane i
 // supplies the address of 4 consecutive rows-elements of one k-row and receives, transposed, 4 consecutive k of
 // one row; BLK = 32: group G holds rows 16 (G%2) .. +15 at k 8 (G/2) .. +7, BLK = 16: rows 0 .. 15 at k 8 G .. +7.
-template <int NW, int WG, int BLK>
+//
+// UR = rows per unit.  Units of 96 / 80 rows keep the 256-byte k-rows in LDS; the lanes whose chunk lies past the
+// unit's rows read out of range (zero fill, no memory traffic).
+template <int NW, int WG, int BLK, int UR = 128>
 struct ColOperandQ {
-  static constexpr int UROWS = 128;
-  static constexpr int UBYTES = QBK * UROWS * 2;
+  static constexpr int UROWS = UR;
+  static constexpr int LROWS_U = 128;                // rows of a k-row in LDS
+  static constexpr int UBYTES = QBK * LROWS_U * 2;
   static constexpr int BYTES = 2 * UBYTES;
   static constexpr int QKS = BLK == 32 ? 4 : 2;
   static constexpr int H = UROWS / (BLK * WG);
   static constexpr int NU = QBK / 4 / NW;
-  static_assert(H >= 1 && NU >= 1, "wave grid too fine for the unit");
+  static_assert(H >= 1 && NU >= 1 && H * BLK * WG == UROWS && UROWS % 8 == 0, "wave grid does not divide the unit");
   const char* base;     // &mem[0][row0]
   int64_t total;        // bytes from base to the end of the matrix
   int64_t ktile_bytes;  // QBK * ld * 2
@@ -786,13 +821,13 @@ struct ColOperandQ {
         // chunk of the unit's 128 rows this lane fetches; k >> 3 & 1 = q >> 1 & 1
         const int c = (lane & 15) ^ (ksub << 2) ^ (((q >> 1) & 1) << 1);
         // k-row 4 j lies at least 1024 j bytes in: rows are at least 256 bytes long (the host checks)
-        voff[u][j] = (uint32_t)(((int64_t)krow * ld + u * UROWS + c * 8) * 2) - 1024u * j;
+        voff[u][j] = (c * 8 < UROWS ? (uint32_t)(((int64_t)krow * ld + u * UROWS + c * 8) * 2) : 0x80000000u) - 1024u * j;
       }
     // lane (group G = l/16, i = l%16) addresses k-row kg + i/4 (+ (1024 / BLK) kk, +4 for the second read) and
     // elements eg + 4 (i%4) .. +3 of the block, with (kg, eg) = (8 (G/2), 16 (G%2)) for BLK = 32, (8 G, 0) for 16
     const int G = lane >> 4, i = lane & 15, kq = i >> 2;
     const int kg = BLK == 32 ? 8 * (G >> 1) : 8 * G, eg = BLK == 32 ? 16 * (G & 1) : 0;
-    const uint32_t lane_base = (uint32_t)((kg + kq) * (UROWS * 2) + 8 * (i & 1));
+    const uint32_t lane_base = (uint32_t)((kg + kq) * (LROWS_U * 2) + 8 * (i & 1));
 #pragma unroll
     for (int b = 0; b < H; b++) {
       const int c2 = (wsub * BLK * H + BLK * b + eg) / 8 + ((i & 3) >> 1);
@@ -812,17 +847,17 @@ struct ColOperandQ {
     dma16_at<J == 0, UNIT_OFF, 1024 * J>(pp.r, wave_lds, voff[U][J], 0);
   }
   __device__ __forceinline__ bf16x8_t frag(const char* unit, int buf, int b, int kk) const {
-    const char* a = unit + moff[buf][b] + kk * ((QBK / QKS) * UROWS * 2);
+    const char* a = unit + moff[buf][b] + kk * ((QBK / QKS) * LROWS_U * 2);
     const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
         (bf16x4_t __attribute__((address_space(3)))*)(a));
     const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-        (bf16x4_t __attribute__((address_space(3)))*)(a + 4 * UROWS * 2));
+        (bf16x4_t __attribute__((address_space(3)))*)(a + 4 * LROWS_U * 2));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   }
 };
 
-template <int LAY, int NW, int WG, int BLK> struct QOperandOf { using type = RowOperandQ<NW, WG, BLK>; };
-template <int NW, int WG, int BLK> struct QOperandOf<LAY_COL, NW, WG, BLK> { using type = ColOperandQ<NW, WG, BLK>; };
+template <int LAY, int NW, int WG, int BLK, int UR> struct QOperandOf { using type = RowOperandQ<NW, WG, BLK, UR>; };
+template <int NW, int WG, int BLK, int UR> struct QOperandOf<LAY_COL, NW, WG, BLK, UR> { using type = ColOperandQ<NW, WG, BLK, UR>; };
 
 // compile-time list of ints, read by index
 template <int... V>
@@ -847,25 +882,38 @@ __device__ __forceinline__ int64_t sk_slot_of(int w, int r, int KT, int ipw) {
 
 // bid: this workgroup's index among the workgroups of the product p (blockIdx.x, or less where one launch holds
 // two products); lds: the workgroup's Q_LDS_BYTES of LDS, 1 KiB aligned
+//
+// BM x BN: 256 x 256 (waves 2 x 2, or 2 x 4 with 8 waves), or a tile narrowed along one dimension to 192 or 160 for
+// products whose 256 x 256 tiling fills the 256 compute units badly (8192 x 1280 is 160 tiles of 256 x 256 and 256
+// of 256 x 160).  A narrow tile's four waves stand in one line along the wide dimension (4 x 1 for 256 x BN, 1 x 4
+// for BM x 256): each wave owns 64 rows (columns) of the wide operand, 32 in either unit, and the narrow operand
+// whole, whose units of BN / 2 = 80 or 96 rows are 5 or 6 blocks of 16.
 constexpr int Q_LDS_BYTES = 2 * 65536;
-template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK, bool SK>
+//
+// OFF (measurement builds only, results wrong): bit 0 = the main loop issues no DMA requests, bit 1 = it reads no
+// fragments from LDS (the MFMAs keep multiplying the first k-tile's fragments): what the loop costs without either.
+template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK, bool SK, int BM = 256, int BN = 256, int OFF = 0>
 __device__ __forceinline__ void gemm_q_body(const GemmArgs& p, const int bid, char* lds) {
   using X = X16<F16>;
-  constexpr int BM = 256, BN = 256;
+  constexpr bool NARROW = BM != 256 || BN != 256;
+  static_assert(BM == 256 || BN == 256, "at most one dimension of the tile is narrowed");
+  static_assert(!NARROW || (BLK == 16 && NW == 4 && !SK && EPI != MTP_EPI_SWIGLU),
+                "narrow tiles: 4 waves, 16x16x32, whole tiles, no SwiGLU interleave");
   static_assert(!SK || (BLK == 16 && NW == 4), "stream-K is built for the 4-wave 16x16x32 form");
   static_assert(EPI != MTP_EPI_SWIGLU || BLAY == LAY_ROW, "the SwiGLU row interleave is a forward (row B) feature");
   static_assert(NW == 4 || NW == 8, "4 waves (2x2) or 8 waves (2x4) per workgroup");
-  constexpr int WGM = 2, WGN = NW / 2;
+  constexpr int WGM = BN != 256 ? 4 : BM != 256 ? 1 : 2, WGN = NW / WGM;
   constexpr int TI = BM / (BLK * WGM), TJ = BN / (BLK * WGN);   // MFMA blocks per wave in m and n
-  using AOp = typename QOperandOf<ALAY, NW, WGM, BLK>::type;
-  using BOp = typename QOperandOf<BLAY, NW, WGN, BLK>::type;
+  using AOp = typename QOperandOf<ALAY, NW, WGM, BLK, BM / 2>::type;
+  using BOp = typename QOperandOf<BLAY, NW, WGN, BLK, BN / 2>::type;
   constexpr int HI = AOp::H, HJ = BOp::H, QKS = AOp::QKS;
   static_assert(2 * HI == TI && 2 * HJ == TJ, "two units per operand");
   using AccT = std::conditional_t<BLK == 32, f32x16_t, f32x4_t>;
   constexpr int S = 32 / BLK;           // MFMA blocks per 32 rows (columns)
   constexpr int TI32 = TI / S, TJ32 = TJ / S;
-  constexpr int QBUF = AOp::BYTES + BOp::BYTES;   // one k-tile of both operands: 64 KiB
-  static_assert(QBUF == 65536, "the operands keep per-buffer read offsets 64 KiB apart");
+  static_assert(TI32 * S == TI && TJ32 * S == TJ, "whole 32 x 32 blocks per wave");
+  constexpr int QBUF = 65536;                     // one k-tile of both operands: at most 64 KiB, buffers 64 KiB apart
+  static_assert(AOp::BYTES + BOp::BYTES <= QBUF, "the operands keep per-buffer read offsets 64 KiB apart");
   constexpr int LDS_BYTES = 2 * QBUF;
   static_assert(LDS_BYTES == Q_LDS_BYTES, "the kernels allocate Q_LDS_BYTES");
 
@@ -891,9 +939,10 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p, const int bid, ch
       it_end = it + p.sk_ipw < all ? it + p.sk_ipw : all;
     }
   }
-  // where this wave's DMA instructions of a unit put their first KiB
-  static_assert(AOp::NU == BOp::NU, "one wave base serves both operands");
-  const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_addr_of(lds)) + wave * (AOp::NU * 1024);
+  // where this wave's DMA instructions of a unit of A (of B) put their first KiB
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane(lds_addr_of(lds));
+  const uint32_t lds_wave_a = lds_base + wave * (AOp::NU * 1024);
+  const uint32_t lds_wave_b = AOp::NU == BOp::NU ? lds_wave_a : lds_base + wave * (BOp::NU * 1024);
   // byte offsets of the units inside lds
   auto unit_a = [](int buf, int u) constexpr { return buf * QBUF + u * AOp::UBYTES; };
   auto unit_b = [](int buf, int u) constexpr { return buf * QBUF + AOp::BYTES + u * BOp::UBYTES; };
@@ -961,7 +1010,6 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p, const int bid, ch
   constexpr int PH = HI * HJ * QKS;          // MFMAs per phase (one quadrant)
   constexpr int HT = 2 * PH;                 // MFMAs per half tile
   constexpr int NDH = AOp::NU + BOp::NU;     // DMA instructions per wave and half tile (one unit of A, one of B)
-  static_assert(AOp::NU == BOp::NU, "the units of A and B take the same number of DMA instructions");
   constexpr int BPOST = (BLK == 32 ? 1 : 2) * (HI * HJ >= 4 ? 4 : 2);   // MFMAs of a half tile issued behind its barrier
   constexpr int BARRIER_AT = HT - BPOST;
   // the d-th DMA instruction of a half tile is issued behind MFMA number dma_at(d) of the half tile
@@ -1017,9 +1065,9 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p, const int bid, ch
     constexpr int UA = decltype(ua_tag)::value, UB = decltype(ub_tag)::value, BUF = decltype(buf_tag)::value;
     constexpr int d = decltype(d_tag)::value;
     if constexpr (d < AOp::NU)
-      opA.template issue<unit_a(BUF, UA), UA, d>(pa, lds_wave);
+      opA.template issue<unit_a(BUF, UA), UA, d>(pa, lds_wave_a);
     else
-      opB.template issue<unit_b(BUF, UB), UB, d - AOp::NU>(pb, lds_wave);
+      opB.template issue<unit_b(BUF, UB), UB, d - AOp::NU>(pb, lds_wave_b);
   };
   auto dma_group = [&](int kt, auto ua_tag, auto ub_tag, auto buf_tag) {
     const auto pa = opA.prep(kt, k1);
@@ -1057,22 +1105,19 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p, const int bid, ch
         __builtin_amdgcn_sched_barrier(0);
       }
       mfma_q(std::integral_constant<int, MA>{}, std::integral_constant<int, MB>{}, std::integral_constant<int, m>{});
-#if !(defined(MTP_MEASURE) && defined(QX_NODMA))
-      static_for<NDH>([&](auto d_tag) {
-        constexpr int d = decltype(d_tag)::value;
-        if constexpr (d * HT / NDH + 1 == g + 1)
-          dma_q(pa, pb, std::integral_constant<int, D::v[10]>{}, std::integral_constant<int, D::v[11]>{},
-                std::integral_constant<int, D::v[12]>{}, d_tag);
-      });
-#endif
-#if !(defined(MTP_MEASURE) && defined(QX_NOREAD))
-      if constexpr (m < RSPAN) {
+      if constexpr (!(OFF & 1))
+        static_for<NDH>([&](auto d_tag) {
+          constexpr int d = decltype(d_tag)::value;
+          if constexpr (d * HT / NDH + 1 == g + 1)
+            dma_q(pa, pb, std::integral_constant<int, D::v[10]>{}, std::integral_constant<int, D::v[11]>{},
+                  std::integral_constant<int, D::v[12]>{}, d_tag);
+        });
+      if constexpr (!(OFF & 2) && m < RSPAN) {
         static_for<(m + 1) * NR / RSPAN - m * NR / RSPAN>([&](auto e) {
           read_q(std::integral_constant<int, RA>{}, std::integral_constant<int, RU>{},
                  std::integral_constant<int, RBUF>{}, std::integral_constant<int, m * NR / RSPAN + decltype(e)::value>{});
         });
       }
-#endif
       __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -1115,7 +1160,7 @@ __device__ __forceinline__ void gemm_q_body(const GemmArgs& p, const int bid, ch
   if (MTP_DBG(p, 2)) return;
 
   auto write_tile = [&]() {
-    gemm_epilogue<BM, BN, EPI, OUT, NW, F16, true, LDS_BYTES, TI32, TJ32, BLK>(
+    gemm_epilogue<BM, BN, EPI, OUT, WGM, WGN, F16, true, LDS_BYTES, TI32, TJ32, BLK>(
         p,
         [&](int i, int j, int g, int e) -> float {
           if constexpr (BLK == 32) return acc[i][j][4 * g + e];
@@ -1500,7 +1545,7 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmArgs& p) {
   if (MTP_DBG(p, 2)) return;
 
   if constexpr (EPI == EPI_ROWSUM) static_assert(NMF >= TI, "every A fragment of a step must meet an MFMA");
-  gemm_epilogue<BM, BN, EPI, OUT, NW, F16, false, NSTAGE * STAGE_BYTES, TI, TJ, 32>(
+  gemm_epilogue<BM, BN, EPI, OUT, WGM, WGN, F16, false, NSTAGE * STAGE_BYTES, TI, TJ, 32>(
       p, [&](int i, int j, int g, int e) -> float { return acc[i][j][4 * g + e]; },
       [&](int i, int) -> float { return rsum[i]; }, lds, m0, n0, tn, wave, lane);
 }
@@ -1510,10 +1555,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs p) {
   gemm_bf16_body<BM, BN, ALAY, BLAY, EPI, OUT, NW, F16>(p);
 }
 
-template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK, bool SK>
+template <int ALAY, int BLAY, int EPI, int OUT, int NW, bool F16, int BLK, bool SK, int BM = 256, int BN = 256, int OFF = 0>
 __global__ __launch_bounds__(NW * 64) void gemm_q_kernel(const GemmArgs p) {
   __shared__ __attribute__((aligned(1024))) char lds[Q_LDS_BYTES];
-  gemm_q_body<ALAY, BLAY, EPI, OUT, NW, F16, BLK, SK>(p, (int)blockIdx.x, lds);
+  gemm_q_body<ALAY, BLAY, EPI, OUT, NW, F16, BLK, SK, BM, BN, OFF>(p, (int)blockIdx.x, lds);
 }
 
 // Input gradient and weight gradient of one layer in one launch: workgroups [0, n1) are the tiles of p1 (dX = dY W),
@@ -1674,6 +1719,12 @@ __global__ __launch_bounds__(256) void gemm_sk_reduce_kernel(const GemmArgs p) {
 // multiple of 256 (or well below 256) finish sooner with a narrower tile.  pick_config() estimates
 // rounds x tile cost for each configuration that the kernel at hand was built with.
 // ---------------------------------------------------------------------------
+#ifndef MTP_EFF_192
+#define MTP_EFF_192 1.05f
+#endif
+#ifndef MTP_EFF_160
+#define MTP_EFF_160 1.05f
+#endif
 struct TileCfg {
   int bm, bn, nw;
   float eff;  // relative speed of one tile's inner loop per flop (256x256 = 1), from measurement
@@ -1684,16 +1735,25 @@ struct TileCfg {
 // 4096x28672x4096): ring 4 waves 1290 / 1334 / 1300; 64-deep 32x32x16 4 waves 1378 / 1393 / 1358; 64-deep
 // 16x16x32 4 waves 1490 / 1538 / 1484, 8 waves 1432 / 1502 / 1411.  The narrow tiles (ring only) were measured
 // best as listed.
+// Configurations 10-13: the 64-deep loop on tiles narrowed to 192 or 160 along n (forward: a layer with few output
+// features per rank) or along m (weight gradient of such a layer); each is built for that one product only.
 constexpr TileCfg kCfgs[] = {
     {256, 256, 8, 1.00f, 0}, {256, 192, 4, 0.92f, 0}, {192, 256, 4, 0.92f, 0},  {256, 128, 4, 0.85f, 0},
     {128, 256, 8, 0.85f, 0}, {256, 256, 4, 1.02f, 0}, {256, 256, 4, 1.08f, 32}, {256, 256, 8, 1.06f, 32},
     {256, 256, 4, 1.16f, 16}, {256, 256, 8, 1.12f, 16},
+    {256, 192, 4, MTP_EFF_192, 16}, {192, 256, 4, MTP_EFF_192, 16}, {256, 160, 4, MTP_EFF_160, 16}, {160, 256, 4, MTP_EFF_160, 16},
 };
 constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
 
-template <int EPI>
+// Can configuration c serve the product (A layout, B layout) with epilogue EPI?  (It is instantiated only then.)
+template <int EPI, int ALAY = LAY_ROW, int BLAY = LAY_ROW>
 constexpr bool cfg_valid(int c) {
   const TileCfg t = kCfgs[c];
+  if (t.q != 0 && (t.bm != 256 || t.bn != 256)) {
+    if (EPI == MTP_EPI_SWIGLU) return false;
+    // narrow along n: the forward product; narrow along m: the weight gradient
+    return t.bn != 256 ? (ALAY == LAY_ROW && BLAY == LAY_ROW) : (ALAY == LAY_COL && BLAY == LAY_COL);
+  }
   const int wgn = t.nw / 2;
   if (t.bn % (32 * wgn) != 0) return false;
   const int tj = t.bn / (32 * wgn);
@@ -1719,12 +1779,12 @@ struct MixedSplit {
 template <int EPI>
 MixedSplit plan_mixed(const GemmArgs& a);
 
-template <int EPI>
+template <int EPI, int ALAY = LAY_ROW, int BLAY = LAY_ROW>
 int pick_config(const GemmArgs& a) {
   static MtpTune tune_cfg("MTP_GEMM_CFG"), tune_skip("MTP_GEMM_SKIP");
   if (tune_cfg.is_set()) {
     const int c = tune_cfg.get(0);
-    if (c >= 0 && c < kNumCfgs && !(kCfgs[c].q != 0 && !q_loop_ok(a))) return c;
+    if (c >= 0 && c < kNumCfgs && cfg_valid<EPI, ALAY, BLAY>(c) && !(kCfgs[c].q != 0 && !q_loop_ok(a))) return c;
   }
   const int64_t span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
   const int skip = tune_skip.get(0);  // bit c set = leave configuration c out of the choice
@@ -1736,9 +1796,9 @@ int pick_config(const GemmArgs& a) {
     const int bn_span = (EPI == MTP_EPI_SWIGLU) ? t.bn / 2 : t.bn;
     const int64_t tiles = ((a.M + t.bm - 1) / t.bm) * ((span + bn_span - 1) / bn_span);
     const int64_t rounds = (tiles + 255) / 256;
-    if (!cfg_valid<EPI>(c) || (t.q != 0 && !q_loop_ok(a))) continue;
+    if (!cfg_valid<EPI, ALAY, BLAY>(c) || (t.q != 0 && !q_loop_ok(a))) continue;
     double cost = (double)rounds * t.bm * t.bn / t.eff;
-    if (t.q == 16 && t.nw == 4 && plan_mixed<EPI>(a).dim != 0) cost = ((double)(tiles / 256) + 0.78) * t.bm * t.bn / t.eff;
+    if (t.q == 16 && t.nw == 4 && t.bm == 256 && t.bn == 256 && plan_mixed<EPI>(a).dim != 0) cost = ((double)(tiles / 256) + 0.78) * t.bm * t.bn / t.eff;
     if (cost < best_t * 0.999) {
       best_t = cost;
       best = c;
@@ -1796,7 +1856,7 @@ inline bool plan_stream_k(GemmArgs& a, int tiles, int KT) {
 
 template <int C, int ALAY, int BLAY, int EPI, int OUT, bool F16>
 int launch_cfg(const GemmArgs& a, hipStream_t s) {
-  if constexpr (!cfg_valid<EPI>(C)) {
+  if constexpr (!cfg_valid<EPI, ALAY, BLAY>(C)) {
     mtp_set_error("gemm_bf16: tile configuration %d cannot serve this epilogue", C);
     return MTP_EINVAL;
   } else {
@@ -1805,7 +1865,7 @@ int launch_cfg(const GemmArgs& a, hipStream_t s) {
     const int span = (EPI == MTP_EPI_SWIGLU) ? a.half : a.N;
     const int bn_span = (EPI == MTP_EPI_SWIGLU) ? BN / 2 : BN;
     const int tiles_n = (span + bn_span - 1) / bn_span;
-    if constexpr (kCfgs[C].q == 16 && NW == 4) {
+    if constexpr (kCfgs[C].q == 16 && NW == 4 && BM == 256 && BN == 256) {
       GemmArgs b = a;
       if (plan_stream_k(b, tiles_m * tiles_n, (a.K + QBK - 1) / QBK)) {
         hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16, 16, true>), dim3((unsigned)(b.sk_full + b.sk_wgs)),
@@ -1820,8 +1880,24 @@ int launch_cfg(const GemmArgs& a, hipStream_t s) {
         return MTP_OK;
       }
     }
+#ifdef MTP_MEASURE
+    // measurement builds: the forward product's 64-deep loop with its DMA requests (debug bit 16) and / or its
+    // fragment reads (bit 32) left out, for the decomposition of the loop's time; results are wrong
+    if constexpr (C == 8 && ALAY == LAY_ROW && BLAY == LAY_ROW && !F16 && OUT == OUT_BF16 &&
+                  (EPI == MTP_EPI_NONE || EPI == MTP_EPI_SWIGLU)) {
+      const int off = (a.debug >> 4) & 3;
+      const dim3 grid((unsigned)(tiles_m * tiles_n)), block(NW * 64);
+      if (off == 1) hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16, 16, false, 256, 256, 1>), grid, block, 0, s, a);
+      if (off == 2) hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16, 16, false, 256, 256, 2>), grid, block, 0, s, a);
+      if (off == 3) hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16, 16, false, 256, 256, 3>), grid, block, 0, s, a);
+      if (off != 0) {
+        MTP_CHECK_LAUNCH("gemm_bf16 (parts of the loop off)");
+        return MTP_OK;
+      }
+    }
+#endif
     if constexpr (kCfgs[C].q != 0)
-      hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16, (kCfgs[C].q ? kCfgs[C].q : 32), false>),
+      hipLaunchKernelGGL((gemm_q_kernel<ALAY, BLAY, EPI, OUT, NW, F16, (kCfgs[C].q ? kCfgs[C].q : 32), false, BM, BN>),
                          dim3((unsigned)(tiles_m * tiles_n)), dim3(NW * 64), 0, s, a);
     else
       hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, ALAY, BLAY, EPI, OUT, NW, F16>), dim3((unsigned)(tiles_m * tiles_n)),
@@ -1837,8 +1913,8 @@ int launch_typed(GemmArgs a, hipStream_t s) {
   static MtpTune tune_debug("MTP_GEMM_DEBUG");
   a.debug = tune_debug.get(0);
 #endif
-  int c = pick_config<EPI>(a);
-  if (!cfg_valid<EPI>(c)) c = 0;
+  int c = pick_config<EPI, ALAY, BLAY>(a);
+  if (!cfg_valid<EPI, ALAY, BLAY>(c)) c = 0;
   static MtpTune tune_forced("MTP_GEMM_CFG");
   if (c == 8 && !tune_forced.is_set()) {
     const MixedSplit ms = plan_mixed<EPI>(a);
@@ -1877,6 +1953,10 @@ int launch_typed(GemmArgs a, hipStream_t s) {
     case 7: return launch_cfg<7, ALAY, BLAY, EPI, OUT, F16>(a, s);
     case 8: return launch_cfg<8, ALAY, BLAY, EPI, OUT, F16>(a, s);
     case 9: return launch_cfg<9, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 10: return launch_cfg<10, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 11: return launch_cfg<11, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 12: return launch_cfg<12, ALAY, BLAY, EPI, OUT, F16>(a, s);
+    case 13: return launch_cfg<13, ALAY, BLAY, EPI, OUT, F16>(a, s);
   }
   return MTP_EINVAL;
 }

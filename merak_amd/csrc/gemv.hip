@@ -32,10 +32,8 @@ namespace {
 constexpr int GV_MAX_WAVES = 8;  // waves per workgroup: 8, or 4 for the register-heavy configurations
 constexpr int GV_MAX_SLICES = 8; // slices along k, one workgroup each
 
-struct ArgPart {
-  float v;
-  int32_t i;
-};
+// a workgroup's best (value, index) of one batch row, packed: see arg_key
+typedef uint64_t ArgPart;
 
 // torch.argmax ordering: NaN beats everything, ties go to the lower index
 __device__ __forceinline__ bool arg_better(float va, int64_t ia, float vb, int64_t ib) {
@@ -105,19 +103,60 @@ struct GemvFuse {
 // into two accumulators, and each lane keeps the one whose rows it owns.
 // W waves split K.  Configurations whose registers allow only 8 waves per CU run as two independent workgroups of
 // 4 waves rather than one of 8: while one sums its partial tiles and writes its outputs the other keeps streaming.
+// Everything a launch hands to a workgroup.
+struct GemvArgs {
+  const uint16_t* x;
+  const uint16_t* w;
+  const uint16_t* bias;
+  uint16_t* y;
+  ArgPart* part;
+  int B;
+  int64_t N, K;
+  int rot_mul;
+  int64_t ld;
+  float* kpart;
+  int32_t* karrived;
+  int flags;
+  GemvFuse fz;
+};
+
+// LDS of one workgroup, carved out of one buffer (so that a launch that holds two kinds of workgroups needs the
+// larger of the two, not their sum): the partial tiles of the waves, the finished tile, the "I am last" cell, and
+// with NORM the normalised rows of X and their scales.
+template <int R, int NB, int W, bool NORM>
+struct GemvLds {
+  static constexpr int GP = (R * NB <= 8) ? R : 8 / NB;            // row groups per reduction phase
+  static constexpr int XL_PAD = 32, XL_ELEMS = 8 * (4096 + XL_PAD);
+  static constexpr int PART = 0;                                    // float [W][GP][NB][4][64]
+  static constexpr int PART_BYTES = W * GP * NB * 4 * 64 * 4;
+  static constexpr int FIN = PART + PART_BYTES;                     // float [16 NB][16 R + 1]
+  static constexpr int FIN_BYTES = 16 * NB * (16 * R + 1) * 4;
+  static constexpr int LAST = (FIN + FIN_BYTES + 15) / 16 * 16;     // int
+  static constexpr int RSTD = LAST + 16;                            // float [32]
+  static constexpr int XL = RSTD + 128;                             // uint16_t [XL_ELEMS]
+  static constexpr int BYTES = NORM ? XL + XL_ELEMS * 2 : RSTD;
+};
+
+// bx, by, gy: the workgroup's place (row block, k slice) and the number of k slices; smem: GemvLds<...>::BYTES of LDS
 template <int R, int NB, int MODE, bool GUARD, int D, int W, bool F16, bool NORM, bool PP>
-__global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __restrict__ x,
-                                                          const uint16_t* __restrict__ w,
-                                                          const uint16_t* __restrict__ bias,
-                                                          uint16_t* __restrict__ y, ArgPart* __restrict__ part,
-                                                          int B, int64_t N, int64_t K, int rot_mul, int64_t ld,
-                                                          float* __restrict__ kpart, int32_t* __restrict__ karrived,
-                                                          int flags, const GemvFuse fz) {
+__device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, const int by, const int gy, char* smem) {
+  const uint16_t* __restrict__ x = ga.x;
+  const uint16_t* __restrict__ w = ga.w;
+  const uint16_t* __restrict__ bias = ga.bias;
+  uint16_t* __restrict__ y = ga.y;
+  ArgPart* __restrict__ part = ga.part;
+  const int B = ga.B;
+  const int64_t N = ga.N, K = ga.K, ld = ga.ld;
+  const int rot_mul = ga.rot_mul, flags = ga.flags;
+  float* __restrict__ kpart = ga.kpart;
+  int32_t* __restrict__ karrived = ga.karrived;
+  const GemvFuse& fz = ga.fz;
+  using L = GemvLds<R, NB, W, NORM>;
   static_assert(!NORM || (!GUARD && MODE != 2), "the norm prologue needs K % 64 == 0 and a stored output");
-  // K is the extent along k that this workgroup covers and ld the row stride of X and W: with gridDim.y > 1
-  // the k range is cut into gridDim.y slices of K elements, one workgroup per (row block, slice); the
+  // K is the extent along k that this workgroup covers and ld the row stride of X and W: with gy > 1
+  // the k range is cut into gy slices of K elements, one workgroup per (row block, slice); the
   // slices' partial sums meet in `kpart` and the slice that delivers last adds them up in slice order.
-  const int64_t koff = (int64_t)blockIdx.y * K;
+  const int64_t koff = (int64_t)by * K;
   using X = X16<F16>;   // bf16 or IEEE half: the MFMA and the conversions of the epilogue
   constexpr int GV_WAVES = W, GV_THREADS = W * MTP_WAVE;
   const int tid = threadIdx.x;
@@ -137,14 +176,14 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   for (int r = 0; r < R; r++) {
     int64_t row0, lim;
     if (MODE == 3) {
-      row0 = (int64_t)blockIdx.x * (8 * R) + 8 * r;
+      row0 = (int64_t)bx * (8 * R) + 8 * r;
       lim = half;
     } else if (MODE == 1) {
-      const int64_t j0 = (int64_t)blockIdx.x * (8 * R);
+      const int64_t j0 = (int64_t)bx * (8 * R);
       row0 = (r < R / 2) ? j0 + 16 * r : half + j0 + 16 * (r - R / 2);
       lim = (r < R / 2) ? half : N;
     } else {
-      row0 = (int64_t)blockIdx.x * (16 * R) + 16 * r;
+      row0 = (int64_t)bx * (16 * R) + 16 * r;
       lim = N;
     }
     if (row0 >= lim) row0 = lim - 1;                 // a group entirely past the end reads the last row
@@ -188,7 +227,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   // (rows being a power-of-two apart) live in the same few memory channels.
   // (Summation order along k therefore differs between workgroups: equal weight rows that live in different
   // workgroups give logits that are equal to rounding, not necessarily bit for bit.)
-  const int64_t rot = GUARD || (pairs % GV_MAX_WAVES) ? 0 : ((int64_t)(blockIdx.x + blockIdx.y) * rot_mul) % pairs;
+  const int64_t rot = GUARD || (pairs % GV_MAX_WAVES) ? 0 : ((int64_t)(bx + by) * rot_mul) % pairs;
 
   static_assert(MODE != 3 || (NB == 1 && !GUARD && D == 1), "mixed SwiGLU groups: one batch tile, K % 64 == 0, depth 1");
   constexpr bool MIX = MODE == 3;
@@ -218,9 +257,9 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   bf16x8_t a_s1[D][R][2], b_s1[D][XS][NB][2];
   // NORM: RMSNorm(X) is built once per workgroup in LDS, rows padded so that the 16-byte fragment reads of four
   // batch rows fall into different banks
-  constexpr int XL_PAD = 32, XL_ELEMS = 8 * (4096 + XL_PAD);
+  constexpr int XL_PAD = L::XL_PAD;
   [[maybe_unused]] const int xl_ld = (int)K + XL_PAD;
-  __shared__ uint16_t x_lds[NORM ? XL_ELEMS : 8];
+  [[maybe_unused]] uint16_t* x_lds = reinterpret_cast<uint16_t*>(smem + L::XL);
   const int b_row = li < B ? li : B - 1;
   // GUARD: K is not a multiple of 64, the last pair is partly (or half) past the end of the rows
   auto pair_k = [&](int64_t pq0, int d, int64_t (&ks)[2]) {
@@ -399,7 +438,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
     if (n_it > 0) load_x(pq, b_s0);
   } else {
     // part 2: scale of every row, then the normalised rows into LDS
-    __shared__ float rstd_lds[32];
+    float* rstd_lds = reinterpret_cast<float*>(smem + L::RSTD);
     {
       float s = 0.f;
 #pragma unroll
@@ -491,7 +530,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
       for (int i = 0; i < EPT; i++) {
         const int e = i * GV_THREADS + tid;
         const int b = e / (16 * R), rl = e - b * (16 * R);
-        const int64_t n = (int64_t)blockIdx.x * (16 * R) + rl;
+        const int64_t n = (int64_t)bx * (16 * R) + rl;
         rres[i] = (e < B * 16 * R && n < N) ? fz.residual[(int64_t)b * N + n] : (uint16_t)0;
       }
     }
@@ -506,9 +545,9 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   // ---- sum the 8 k-slices through LDS: up to 8 tiles (row group x batch tile) per wave at a time, i.e. one
   // phase (two barriers) for all but the largest configuration ---------------------------------------------
   // part_lds[w][group][nb][j][lane]; fin[b][local row]
-  constexpr int GP = (R * NB <= 8) ? R : 8 / NB;  // row groups per phase
-  __shared__ float part_lds[GV_WAVES][GP][NB][4][64];
-  __shared__ float fin[16 * NB][16 * R + 1];
+  constexpr int GP = L::GP;  // row groups per phase
+  float (*part_lds)[GP][NB][4][64] = reinterpret_cast<float (*)[GP][NB][4][64]>(smem + L::PART);
+  float (*fin)[16 * R + 1] = reinterpret_cast<float (*)[16 * R + 1]>(smem + L::FIN);
 #pragma unroll
   for (int r0 = 0; r0 < R; r0 += GP) {
 #pragma unroll
@@ -529,15 +568,15 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
     __syncthreads();
   }
 
-  if (MODE != 2 && gridDim.y > 1) {
+  if (MODE != 2 && gy > 1) {
     // k slices: hand the partial over with device-scope stores, count arrivals; the last slice to arrive sums
     // all of them in slice order (its own included, read back), so the result does not depend on who is last.
     // Two values per access, and a thread asks for all it will sum before it looks at the first: the sum is a
     // single round trip to the memory-side cache whatever the batch and the number of row groups.
     constexpr int FIN = 16 * R;
     constexpr int PER = (16 * NB * FIN / 2 + GV_THREADS - 1) / GV_THREADS;   // pairs of values per thread
-    const int S = gridDim.y, cnt = B * FIN;
-    uint64_t* mine = reinterpret_cast<uint64_t*>(kpart + ((int64_t)blockIdx.x * S + blockIdx.y) * cnt);
+    const int S = gy, cnt = B * FIN;
+    uint64_t* mine = reinterpret_cast<uint64_t*>(kpart + ((int64_t)bx * S + by) * cnt);
 #pragma unroll
     for (int i = 0; i < PER; i++) {
       const int e = 2 * (i * GV_THREADS + tid);
@@ -549,15 +588,15 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    __shared__ int last_one;
+    int* last_one = reinterpret_cast<int*>(smem + L::LAST);
     if (tid == 0) {
-      const int seen = __hip_atomic_fetch_add(karrived + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      last_one = seen == S - 1;
-      if (last_one) __hip_atomic_store(karrived + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int seen = __hip_atomic_fetch_add(karrived + bx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *last_one = seen == S - 1;
+      if (*last_one) __hip_atomic_store(karrived + bx, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    if (!last_one) return;
-    const uint64_t* all = reinterpret_cast<const uint64_t*>(kpart + (int64_t)blockIdx.x * S * cnt);
+    if (!*last_one) return;
+    const uint64_t* all = reinterpret_cast<const uint64_t*>(kpart + (int64_t)bx * S * cnt);
     const int64_t slice_stride = cnt >> 1;
     uint64_t v[PER][GV_MAX_SLICES];
 #pragma unroll
@@ -588,7 +627,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
 
   if (MODE == 3) {
     // fin[b][16 r + i]: i < 8 gate row j0 + 8 r + i, i >= 8 the up row of gate row j0 + 8 r + i - 8
-    const int64_t j0 = (int64_t)blockIdx.x * (8 * R);
+    const int64_t j0 = (int64_t)bx * (8 * R);
     for (int e = tid; e < B * 8 * R; e += GV_THREADS) {
       const int b = e / (8 * R), rl = e - b * (8 * R);
       const int64_t jn = j0 + rl;
@@ -607,7 +646,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   } else if (MODE == 0) {
     // 16 consecutive lanes hold 16 consecutive output rows of one batch row: their squares meet in one
     // partial sum (fixed butterfly order), which is what the norm prologue of the next linear adds up
-    const int64_t n0 = (int64_t)blockIdx.x * (16 * R);
+    const int64_t n0 = (int64_t)bx * (16 * R);
     const int total = B * 16 * R;
     const int64_t parts_out = (N + 15) >> 4;
 #pragma unroll
@@ -635,7 +674,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
       }
     }
   } else if (MODE == 1) {
-    const int64_t j0 = (int64_t)blockIdx.x * (8 * R);
+    const int64_t j0 = (int64_t)bx * (8 * R);
     for (int e = tid; e < B * 8 * R; e += GV_THREADS) {
       const int b = e / (8 * R), rl = e - b * (8 * R);
       const int64_t jn = j0 + rl;
@@ -654,7 +693,7 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
   } else {
     // 512 / (16 NB) lanes per batch row: each folds its share of the 16 R rows, then a butterfly inside the
     // lane group.  (value, index) travel as one 64-bit key whose unsigned maximum is torch.argmax's choice.
-    const int64_t n0 = (int64_t)blockIdx.x * (16 * R);
+    const int64_t n0 = (int64_t)bx * (16 * R);
     constexpr int TPB = GV_THREADS / (16 * NB);
     const int b = tid / TPB, sub = tid % TPB;
     uint64_t key = 0;
@@ -671,65 +710,71 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const uint16_t* __re
       const uint64_t ok = (uint64_t)__shfl_xor((long long)key, o, 64);
       key = ok > key ? ok : key;
     }
-    if (sub == 0 && b < B) part[(int64_t)blockIdx.x * B + b] = ArgPart{arg_key_value(key), arg_key_index(key)};
+    // (Finishing the pick inside this launch — every workgroup counts itself in at a counter, the last one of a
+    // group folds the group's keys, the last group the groups — was built and measured: the counter's round trip
+    // at the end of every one of 1000-2000 workgroups costs more than the second kernel it saves, 157 -> 175-183 us
+    // at 1-8 batch rows, no change at 32.)
+    if (sub == 0 && b < B) part[(int64_t)bx * B + b] = key;
   }
+}
+
+template <int R, int NB, int MODE, bool GUARD, int D, int W, bool F16, bool NORM, bool PP>
+__global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const GemvArgs ga) {
+  __shared__ __attribute__((aligned(16))) char smem[GemvLds<R, NB, W, NORM>::BYTES];
+  gemv_body<R, NB, MODE, GUARD, D, W, F16, NORM, PP>(ga, (int)blockIdx.x, (int)blockIdx.y, (int)gridDim.y, smem);
+}
+
+// Two products over the same X in one grid.  The grid is the second product's (SwiGLU: one workgroup per row block,
+// as when it runs alone); the first n1 workgroups multiply a row block of the first product (plain store) before
+// their own.  A product with few rows (QKV beside gate/up) then neither starts nor drains the chip in a launch of
+// its own, and the grid stays at the second product's size (these configurations hold one workgroup per compute
+// unit: a grid with more workgroups than compute units would run its last few alone).
+// Tried and dropped: the first product's row blocks as workgroups of their own in front of the second's (272
+// workgroups: 82 us against 63 us for the two launches, with one or two workgroups per compute unit alike).
+template <int R1, int R2, int MODE2, int NB, int W, bool F16>
+__global__ __launch_bounds__(W * MTP_WAVE) void gemv_pair_kernel(const GemvArgs g1, const GemvArgs g2, const int n1) {
+  using L1 = GemvLds<R1, NB, W, false>;
+  using L2 = GemvLds<R2, NB, W, false>;
+  __shared__ __attribute__((aligned(16))) char smem[L1::BYTES > L2::BYTES ? L1::BYTES : L2::BYTES];
+  const int bid = (int)blockIdx.x;
+  if (bid < n1) {
+    gemv_body<R1, NB, 0, false, 1, W, F16, false, true>(g1, bid, 0, 1, smem);
+    __syncthreads();   // the second product reuses the LDS
+  }
+  gemv_body<R2, NB, MODE2, false, 1, W, F16, false, true>(g2, bid, 0, 1, smem);
 }
 
 // One workgroup per batch row folds that row's per-workgroup partials.  The kernel is a chain of memory
 // latencies (its input was written a moment ago by other CUs), so every thread asks for eight partials
 // before it looks at the first: 256 threads cover 2048 partials per round trip.
 constexpr int AF_THREADS = 256, AF_WAVES = AF_THREADS / MTP_WAVE, AF_DEPTH = 8;
-__global__ __launch_bounds__(AF_THREADS) void argmax_finish_kernel(const ArgPart* __restrict__ part, int n_part, int B,
+__global__ __launch_bounds__(AF_THREADS) void argmax_finish_kernel(const uint64_t* __restrict__ part, int n_part, int B,
                                                                    int64_t* __restrict__ idx, float* __restrict__ maxval) {
   const int b = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  float bv = 0.f;
-  int64_t bi = INT64_MAX;
-  bool have = false;
+  uint64_t best = 0;
   for (int p0 = threadIdx.x; p0 < n_part; p0 += AF_THREADS * AF_DEPTH) {
-    ArgPart a[AF_DEPTH];
+    uint64_t a[AF_DEPTH];
 #pragma unroll
     for (int u = 0; u < AF_DEPTH; u++) {
       const int p = p0 + u * AF_THREADS;
       a[u] = part[(int64_t)(p < n_part ? p : p0) * B + b];   // past the end: the first one again (changes nothing)
     }
 #pragma unroll
-    for (int u = 0; u < AF_DEPTH; u++)
-      if (!have || arg_better(a[u].v, a[u].i, bv, bi)) {
-        bv = a[u].v;
-        bi = a[u].i;
-        have = true;
-      }
+    for (int u = 0; u < AF_DEPTH; u++) best = a[u] > best ? a[u] : best;
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
-    const float ov = __shfl_xor(bv, o, 64);
-    const int64_t oi = __shfl_xor(bi, o, 64);
-    const int oh = __shfl_xor((int)have, o, 64);
-    if (oh && (!have || arg_better(ov, oi, bv, bi))) {
-      bv = ov;
-      bi = oi;
-      have = true;
-    }
+    const uint64_t ok = (uint64_t)__shfl_xor((long long)best, o, 64);
+    best = ok > best ? ok : best;
   }
-  __shared__ float sv[AF_WAVES];
-  __shared__ int64_t si[AF_WAVES];
-  __shared__ int sh[AF_WAVES];
-  if (lane == 0) {
-    sv[wave] = bv;
-    si[wave] = bi;
-    sh[wave] = have;
-  }
+  __shared__ uint64_t sk[AF_WAVES];
+  if (lane == 0) sk[wave] = best;
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int wv = 1; wv < AF_WAVES; wv++)
-      if (sh[wv] && (!have || arg_better(sv[wv], si[wv], bv, bi))) {
-        bv = sv[wv];
-        bi = si[wv];
-        have = true;
-      }
-    idx[b] = bi;
-    if (maxval) maxval[b] = bv;
+    for (int wv = 1; wv < AF_WAVES; wv++) best = sk[wv] > best ? sk[wv] : best;
+    idx[b] = arg_key_index(best);
+    if (maxval) maxval[b] = arg_key_value(best);
   }
 }
 
@@ -886,11 +931,11 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
   const int64_t k_slice = K / S;
 // two operand sets wherever the registers hold them (8 waves: 256 per lane)
 #define GV_PP(RR, NNB) (MODE != 2)
+  const GemvArgs ga{(const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part, (int)B, N, k_slice,
+                    rot_mul, K, kpart, karrived, flags, fz};
 #define GV_LAUNCH_T(RR, NNB, GG, DD, FF)                                                                        \
   hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD, (RR >= 8 ? 4 : 8), FF, NORM, GV_PP(RR, NNB)>), dim3(n_wg, S), \
-                     dim3((RR >= 8 ? 4 : 8) * MTP_WAVE), 0, s,                                                  \
-                     (const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part, (int)B, \
-                     N, k_slice, rot_mul, K, kpart, karrived, flags, fz)
+                     dim3((RR >= 8 ? 4 : 8) * MTP_WAVE), 0, s, ga)
 #define GV_LAUNCH(RR, NNB, GG, DD)                 \
   do {                                             \
     if (f16) GV_LAUNCH_T(RR, NNB, GG, DD, true);   \
@@ -959,11 +1004,11 @@ int launch_gemv_mixed(const void* x, const void* w, const void* bias, void* y, i
   static MtpTune tune_rot("MTP_GEMV_ROT");
   int rot_mul = tune_rot.get(1);
   if (rot_mul < 0) rot_mul = 0;
+  const GemvArgs ga{(const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, nullptr, (int)B, N, K,
+                    rot_mul, K, nullptr, nullptr, 0, fz};
 #define GVM_T(RR, FF)                                                                                              \
   hipLaunchKernelGGL((gemv_kernel<RR, 1, 3, false, 1, GV_MAX_WAVES, FF, NORM, (RR <= 6)>), dim3(n_wg),                \
-                     dim3(GV_MAX_WAVES * MTP_WAVE), 0, s, (const uint16_t*)x, (const uint16_t*)w,                 \
-                     (const uint16_t*)bias, (uint16_t*)y, (ArgPart*)nullptr, (int)B, N, K, rot_mul, K,            \
-                     (float*)nullptr, (int32_t*)nullptr, 0, fz)
+                     dim3(GV_MAX_WAVES * MTP_WAVE), 0, s, ga)
 #define GVM(RR)                  \
   case RR:                       \
     if (f16) GVM_T(RR, true);    \
@@ -1058,6 +1103,72 @@ extern "C" int mtp_gemv_ws(const void* x, const void* w, const void* bias, void*
 
 extern "C" int mtp_gemv_norm_fits(int64_t B, int64_t K) { return gemv_norm_fits(B, K) ? 1 : 0; }
 
+// Two products over the same activations: y1 = x W1^T (+ bias1), act2 = SwiGLU(x W2^T (+ bias2)).  Above 16 batch
+// rows (two batch tiles: the shape whose launches pay most for starting and draining on their own) and for the
+// usual sizes both go out as one grid of 4-wave workgroups, the first product's row blocks in front; everything
+// else runs as the two launches mtp_gemv_ws would make.  MTP_GEMV_PAIR = 0 keeps the two launches.
+extern "C" int mtp_gemv_pair(const void* x, const void* w1, const void* bias1, void* y1, int64_t N1, const void* w2,
+                             const void* bias2, void* act2, int64_t N2, void* workspace, int64_t workspace_bytes,
+                             int64_t B, int64_t K, int dtype, void* stream) {
+  int rc = check_gemv_args("gemv_pair", x, w1, B, N1, K, dtype);
+  if (rc) return rc;
+  rc = check_gemv_args("gemv_pair", x, w2, B, N2, K, dtype);
+  if (rc) return rc;
+  MTP_REQUIRE(y1 && act2, MTP_EINVAL, "gemv_pair: null output");
+  MTP_REQUIRE(y1 != x && act2 != x, MTP_EINVAL, "gemv_pair: an output must not be the input");
+  MTP_REQUIRE(N2 % 2 == 0, MTP_EINVAL, "gemv_pair: SwiGLU needs an even N2, got %lld", (long long)N2);
+  static MtpTune tune_pair("MTP_GEMV_PAIR");
+  hipStream_t s = (hipStream_t)stream;
+  const bool f16 = dtype == MTP_F16;
+  const int64_t half2 = N2 / 2;
+  // one grid: two batch tiles, whole 64-element pairs, a second product that fills the chip with 8-group
+  // workgroups by itself, 32-bit row offsets inside a workgroup's rows
+  const bool one_grid = tune_pair.get(1) != 0 && B > 16 && K % 64 == 0 && pick_gemv_cfg(B, N2, K, 1).R == 8 &&
+                        pick_gemv_cfg(B, N2, K, 1).S == 1 && 128 * K < (1ll << 31);
+  if (!one_grid) {
+    rc = mtp_gemv_ws(x, w1, bias1, y1, workspace, workspace_bytes, B, N1, K, bias1 ? MTP_EPI_BIAS : MTP_EPI_NONE, dtype, stream);
+    if (rc) return rc;
+    return mtp_gemv_ws(x, w2, bias2, act2, workspace, workspace_bytes, B, N2, K, MTP_EPI_SWIGLU, dtype, stream);
+  }
+  static MtpTune tune_rot("MTP_GEMV_ROT"), tune_noshift("MTP_GEMV_NOSHIFT");
+  int rot_mul = tune_rot.get(1);
+  if (rot_mul < 0) rot_mul = 0;
+  const int flags = tune_noshift.get(0) ? 1 : 0;
+  const GemvFuse none{nullptr, nullptr, 0.f, nullptr, nullptr};
+  const GemvArgs g1{(const uint16_t*)x, (const uint16_t*)w1, (const uint16_t*)bias1, (uint16_t*)y1, nullptr, (int)B, N1, K,
+                    rot_mul, K, nullptr, nullptr, flags, none};
+  const GemvArgs g2{(const uint16_t*)x, (const uint16_t*)w2, (const uint16_t*)bias2, (uint16_t*)act2, nullptr, (int)B, N2, K,
+                    rot_mul, K, nullptr, nullptr, flags, none};
+  // the first product's rows in blocks of 16 R1 rows, as few rows per block as still leaves no more blocks than
+  // the second product has workgroups
+  const unsigned n2 = (unsigned)((half2 + 63) / 64);
+  int r1 = 1;
+  while (r1 < 8 && (N1 + 16 * r1 - 1) / (16 * r1) > (int64_t)n2) r1 *= 2;
+  const unsigned n1 = (unsigned)((N1 + 16 * r1 - 1) / (16 * r1));
+  if (n1 > n2) {
+    rc = mtp_gemv_ws(x, w1, bias1, y1, workspace, workspace_bytes, B, N1, K, bias1 ? MTP_EPI_BIAS : MTP_EPI_NONE, dtype, stream);
+    if (rc) return rc;
+    return mtp_gemv_ws(x, w2, bias2, act2, workspace, workspace_bytes, B, N2, K, MTP_EPI_SWIGLU, dtype, stream);
+  }
+#define GVP_T(RR, FF) \
+  hipLaunchKernelGGL((gemv_pair_kernel<RR, 8, 1, 2, 4, FF>), dim3(n2), dim3(4 * MTP_WAVE), 0, s, g1, g2, (int)n1)
+#define GVP(RR)                \
+  case RR:                     \
+    if (f16) GVP_T(RR, true);  \
+    else GVP_T(RR, false);     \
+    break
+  switch (r1) {
+    GVP(1);
+    GVP(2);
+    GVP(4);
+    GVP(8);
+  }
+#undef GVP
+#undef GVP_T
+  MTP_CHECK_LAUNCH("gemv_pair");
+  return MTP_OK;
+}
+
 extern "C" int mtp_gemv_fused(const void* x, const void* w, const void* bias, void* y, const void* norm_weight,
                               const float* sumsq_in, float eps, const void* residual, float* sumsq_out,
                               void* workspace, int64_t workspace_bytes, int64_t B, int64_t N, int64_t K, int epilogue,
@@ -1091,7 +1202,7 @@ extern "C" int mtp_gemv(const void* x, const void* w, const void* bias, void* y,
 extern "C" int64_t mtp_gemv_argmax_workspace_bytes(int64_t B, int64_t N, int64_t K) {
   (void)K;
   if (B < 1 || N < 1) return 0;
-  // one partial per (workgroup, batch row); the smallest workgroup owns 16 rows
+  // one key per (workgroup, batch row); the smallest workgroup owns 16 rows
   return ((N + 15) / 16) * B * (int64_t)sizeof(ArgPart);
 }
 
@@ -1109,8 +1220,8 @@ extern "C" int mtp_gemv_argmax(const void* x, const void* w, int64_t* idx, float
   rc = launch_gemv<2>(x, w, nullptr, nullptr, (ArgPart*)workspace, B, N, K, pick_gemv_cfg(B, N, K, 2), s, &n_wg,
                       dtype == MTP_F16);
   if (rc) return rc;
-  hipLaunchKernelGGL(argmax_finish_kernel, dim3((unsigned)B), dim3(AF_THREADS), 0, s, (const ArgPart*)workspace, (int)n_wg, (int)B,
-                     idx, maxval);
+  hipLaunchKernelGGL(argmax_finish_kernel, dim3((unsigned)B), dim3(AF_THREADS), 0, s, (const ArgPart*)workspace, (int)n_wg,
+                     (int)B, idx, maxval);
   MTP_CHECK_LAUNCH("argmax_finish");
   return MTP_OK;
 }

@@ -62,6 +62,36 @@ bool f32_fast_ok(const void* a, const void* b, int64_t d0, int64_t d1, int64_t b
 
 extern "C" int64_t mtp_linear_workspace_bytes(void) { return MTP_LINEAR_WS_BYTES; }
 
+// Scratch a product of these sizes can make use of: 0 for the (many) shapes that never touch it.  An upper bound of
+// what the kernels' own planning takes (gemm_bf16_kernel.h plan_stream_k, gemm_f32.hip launch_f32): a call with
+// this much never runs without scratch where it would have used some.
+extern "C" int64_t mtp_linear_workspace_need(int kind, int64_t M, int64_t N, int64_t K, int dtype) {
+  if (M <= 0 || N <= 0 || K <= 0 || kind < 0 || kind > 3) return 0;
+  static MtpTune tune_sk("MTP_GEMM_SK"), tune_slices("MTP_GEMM_F32_SLICES");
+  // (rows, columns, reduction length) of the product: forward, input gradient, weight gradient
+  const int64_t dims[3][3] = {{M, N, K}, {M, K, N}, {N, K, M}};
+  int64_t need = 0;
+  for (int p = 0; p < 3; p++) {
+    if (!(kind == p || (kind == 3 && p >= 1))) continue;
+    const int64_t r = dims[p][0], c = dims[p][1], k = dims[p][2];
+    if (dtype == MTP_F32) {
+      // cut along k: fewer 128x128 tiles than compute units (or forced), up to 8 slices of the output and its row sums
+      const int64_t tiles = ((r + 127) / 128) * ((c + 127) / 128);
+      if ((tiles < 256 || tune_slices.get(0) > 1) && k >= 1024 && tune_slices.get(0) != 1) {
+        const int64_t b = 8 * (r * c + r) * 4;
+        need = b > need ? b : need;
+      }
+    } else {
+      // stream-K: at most half the compute units have a 256x256 tile and k is long (or forced)
+      const int64_t tiles = ((r + 255) / 256) * ((c + 255) / 256);
+      const int force = tune_sk.get(-1);
+      if (force != 0 && k % 64 == 0 && (force > 0 || (tiles <= 128 && k / 64 >= 32)))
+        need = MTP_LINEAR_WS_BYTES > need ? MTP_LINEAR_WS_BYTES : need;
+    }
+  }
+  return need;
+}
+
 extern "C" int mtp_linear_fwd(const void* x, const void* w, const void* bias, void* y, void* act, int64_t M,
                               int64_t N, int64_t K, int dtype, int epilogue, void* stream) {
   return mtp_linear_fwd_ws(x, w, bias, y, act, nullptr, 0, M, N, K, dtype, epilogue, stream);

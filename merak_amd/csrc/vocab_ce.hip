@@ -281,195 +281,256 @@ __global__ __launch_bounds__(NT) void vocab_ce_bwd_kernel(
 }
 
 // ---- forward and backward in one pass ---------------------------------------
-// One 1024-lane workgroup per row keeps the whole row in registers (NV 16-byte
-// vectors per lane): loaded once, reduced to (max, sum-exp), then rewritten in
-// place as (softmax - onehot) * g.  HBM sees one read and one write of the row
+// One 1024-lane workgroup keeps a whole row in registers (NV 16-byte vectors per lane): loaded once, reduced to
+// (max, sum-exp), then rewritten in place as (softmax - onehot) * g.  HBM sees one read and one write of the row
 // instead of two reads and a write.
+//
+// A workgroup takes rows b, b + gridDim.x, ...: launched with fewer workgroups than rows it is persistent and asks
+// for the next row's vectors right behind the stores of the current one, so that the next row is on its way while
+// this one's stores drain; launched with gridDim.x = n_rows it is one workgroup per row (row_kernel_grid).
 constexpr int FU_THREADS = 1024;
 constexpr int FU_WAVES = FU_THREADS / MTP_WAVE;
+
+// where a row's aligned 16-byte vectors and its scalar edges lie
+template <typename T>
+struct RowGeo {
+  T* rp;
+  u32x4_t* vp;
+  int head, nvec, edge_j;
+  bool has_edge;
+  __device__ __forceinline__ void set(T* logits, int64_t row, int64_t V, int tid) {
+    constexpr int EPV = Elem<T>::EPV;
+    rp = logits + row * V;
+    int64_t nvec64;
+    row_split(rp, V, head, nvec64);
+    nvec = (int)nvec64;  // the host checked nvec <= NV * FU_THREADS
+    vp = reinterpret_cast<u32x4_t*>(rp + head);
+    const int tail0 = head + nvec * EPV;
+    const int n_edge = head + (int)(V - tail0);
+    edge_j = tid < head ? tid : tail0 + (tid - head);
+    has_edge = tid < n_edge;
+  }
+};
 
 template <typename T, int NV>
 __global__ __launch_bounds__(FU_THREADS) void vocab_ce_fused_kernel(
     T* __restrict__ logits, const int64_t* __restrict__ target, const float* __restrict__ grad_rows,
     float grad_scale, float* __restrict__ loss, float* __restrict__ row_max, float* __restrict__ row_sumexp,
-    float* __restrict__ pred, int64_t V, int64_t vocab_start) {
+    float* __restrict__ pred, int64_t V, int64_t vocab_start, int64_t n_rows) {
   constexpr int EPV = Elem<T>::EPV;
-  const int64_t row = blockIdx.x;
-  T* rp = logits + row * V;
   const int tid = threadIdx.x;
+  int64_t row = blockIdx.x;
+  if (row >= n_rows) return;
 
-  int head;
-  int64_t nvec64;
-  row_split(rp, V, head, nvec64);
-  const int nvec = (int)nvec64;  // the host checked nvec <= NV * FU_THREADS
-  u32x4_t* vp = reinterpret_cast<u32x4_t*>(rp + head);
-  const int tail0 = head + nvec * EPV;
-  const int n_edge = head + (int)(V - tail0);
-  const int edge_j = tid < head ? tid : tail0 + (tid - head);
-  const bool has_edge = tid < n_edge;
-
+  RowGeo<T> geo;
+  geo.set(logits, row, V, tid);
   u32x4_t v[NV] = {};
 #pragma unroll
   for (int u = 0; u < NV; u++)
-    if (tid + u * FU_THREADS < nvec) v[u] = __builtin_nontemporal_load(vp + tid + u * FU_THREADS);
+    if (tid + u * FU_THREADS < geo.nvec) v[u] = __builtin_nontemporal_load(geo.vp + tid + u * FU_THREADS);
   float fe = NEG_BIG;
-  if (has_edge) fe = Elem<T>::ld(rp + edge_j);
+  if (geo.has_edge) fe = Elem<T>::ld(geo.rp + geo.edge_j);
 
-  int64_t tl = target[row] - vocab_start;
-  if (tl < 0 || tl >= V) tl = -1;
-  float x_t = 0.0f;
-  if (tid == 0 && tl >= 0) x_t = Elem<T>::ld(rp + tl);  // read before any lane of this row stores
-  const float g = (grad_rows ? grad_rows[row] : 1.0f) * grad_scale;
+  // two sets of the cross-wave cells, used by alternate rows: a wave that is already reducing the next row must
+  // not overwrite cells another wave still reads for this one (one barrier per row lies between a set's uses)
+  __shared__ float red_m[2][FU_WAVES], red_s[2][FU_WAVES];
+  int par = 0;
 
-  __shared__ float red_m[FU_WAVES], red_s[FU_WAVES];
+  for (;;) {
+    int64_t tl = target[row] - vocab_start;
+    if (tl < 0 || tl >= V) tl = -1;
+    float x_t = 0.0f;
+    if (tid == 0 && tl >= 0) x_t = Elem<T>::ld(geo.rp + tl);  // read before any lane stores to this row
+    const float g = (grad_rows ? grad_rows[row] : 1.0f) * grad_scale;
 
-  // Row maximum and sum of exponentials in one pass over the registers, two vectors at a time in the order they
-  // arrive (the running maximum and the shifted sum of the forward kernel), so that this arithmetic runs while
-  // the rest of the row is still on its way: as a pass of its own behind a barrier it cost 93 us of the 844 a
-  // bf16 [8192, 128256] matrix took.
-  MaxSum acc{NEG_BIG, 0.0f};
-  if (has_edge) ms_accumulate<1>(acc, &fe);
+    // Row maximum and sum of exponentials in one pass over the registers, two vectors at a time in the order they
+    // arrive (the running maximum and the shifted sum of the forward kernel), so that this arithmetic runs while
+    // the rest of the row is still on its way.
+    MaxSum acc{NEG_BIG, 0.0f};
+    if (geo.has_edge) ms_accumulate<1>(acc, &fe);
 #pragma unroll
-  for (int u = 0; u < NV; u += 2) {
-    if (u + 1 < NV && tid + (u + 1) * FU_THREADS < nvec) {
-      float f[2 * EPV];
-      Elem<T>::unpack(v[u], f);
-      Elem<T>::unpack(v[u + 1], f + EPV);
-      ms_accumulate<2 * EPV>(acc, f);
-    } else if (tid + u * FU_THREADS < nvec) {
-      float f[EPV];
-      Elem<T>::unpack(v[u], f);
-      ms_accumulate<EPV>(acc, f);
-    }
-  }
-  // keep the row as loaded: without this the compiler carries the unpacked floats into the gradient pass, which
-  // doubles the registers a bf16 row needs
-#pragma unroll
-  for (int u = 0; u < NV; u++) asm volatile("" : "+v"(v[u]));
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    MaxSum other;
-    other.m = __shfl_xor(acc.m, o, 64);
-    other.s = __shfl_xor(acc.s, o, 64);
-    acc = ms_combine(acc, other);
-  }
-  if ((tid & 63) == 0) {
-    red_m[tid >> 6] = acc.m;
-    red_s[tid >> 6] = acc.s;
-  }
-  __syncthreads();
-  // every wave combines the 16 waves' pairs on its own lanes (16 lanes hold one copy) and takes lane 0's result
-  static_assert(FU_WAVES == 16, "the cross-wave butterfly is written for 16 waves");
-  MaxSum tot{red_m[tid & 15], red_s[tid & 15]};
-#pragma unroll
-  for (int o = 8; o > 0; o >>= 1) {
-    MaxSum other;
-    other.m = __shfl_xor(tot.m, o, 64);
-    other.s = __shfl_xor(tot.s, o, 64);
-    tot = ms_combine(tot, other);
-  }
-  const float m = __shfl(tot.m, 0, 64);
-  const float s_raw = __shfl(tot.s, 0, 64);   // sum of exp2(x*c - fl(m*c)): the forward kernel's shifted sum
-  const float mc = mul_rn(m, LOG2E);
-  const float resid = ms_residual_scale(m);
-
-  if (tid == 0) {
-    const float s = s_raw * resid;
-    row_max[row] = m;
-    row_sumexp[row] = s;
-    pred[row] = x_t;
-    loss[row] = logf(s) - (tl >= 0 ? (x_t - m) : 0.0f);
-  }
-
-  // gradient, in place
-  const float scale = g / s_raw;  // exp2(x*c - fl(m*c)) / s_raw = softmax: the residual cancels
-  const int tv = (tl >= head) ? (int)(tl - head) : -1;
-#pragma unroll
-  for (int u = 0; u < NV; u++)
-    if (tid + u * FU_THREADS < nvec) {
-      float f[EPV];
-      Elem<T>::unpack(v[u], f);
-#pragma unroll
-      for (int e = 0; e < EPV; e++) f[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc)) * scale;
-      const int base = (tid + u * FU_THREADS) * EPV;
-      if ((unsigned)(tv - base) < (unsigned)EPV) {
-        const int e = tv - base;
-#pragma unroll
-        for (int q = 0; q < EPV; q++)
-          if (q == e) f[q] -= g;
+    for (int u = 0; u < NV; u += 2) {
+      if (u + 1 < NV && tid + (u + 1) * FU_THREADS < geo.nvec) {
+        float f[2 * EPV];
+        Elem<T>::unpack(v[u], f);
+        Elem<T>::unpack(v[u + 1], f + EPV);
+        ms_accumulate<2 * EPV>(acc, f);
+      } else if (tid + u * FU_THREADS < geo.nvec) {
+        float f[EPV];
+        Elem<T>::unpack(v[u], f);
+        ms_accumulate<EPV>(acc, f);
       }
-      __builtin_nontemporal_store(Elem<T>::pack(f), vp + tid + u * FU_THREADS);
     }
-  if (has_edge) {
-    float f = __builtin_amdgcn_exp2f(__builtin_fmaf(fe, LOG2E, -mc)) * scale;
-    if (edge_j == tl) f -= g;
-    Elem<T>::st(rp + edge_j, f);
+    // keep the row as loaded: without this the compiler carries the unpacked floats into the gradient pass, which
+    // doubles the registers a bf16 row needs
+#pragma unroll
+    for (int u = 0; u < NV; u++) asm volatile("" : "+v"(v[u]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      MaxSum other;
+      other.m = __shfl_xor(acc.m, o, 64);
+      other.s = __shfl_xor(acc.s, o, 64);
+      acc = ms_combine(acc, other);
+    }
+    if ((tid & 63) == 0) {
+      red_m[par][tid >> 6] = acc.m;
+      red_s[par][tid >> 6] = acc.s;
+    }
+    __syncthreads();
+    // every wave combines the 16 waves' pairs on its own lanes (16 lanes hold one copy) and takes lane 0's result
+    static_assert(FU_WAVES == 16, "the cross-wave butterfly is written for 16 waves");
+    MaxSum tot{red_m[par][tid & 15], red_s[par][tid & 15]};
+    par ^= 1;
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) {
+      MaxSum other;
+      other.m = __shfl_xor(tot.m, o, 64);
+      other.s = __shfl_xor(tot.s, o, 64);
+      tot = ms_combine(tot, other);
+    }
+    const float m = __shfl(tot.m, 0, 64);
+    const float s_raw = __shfl(tot.s, 0, 64);   // sum of exp2(x*c - fl(m*c)): the forward kernel's shifted sum
+    const float mc = mul_rn(m, LOG2E);
+
+    if (tid == 0) {
+      const float s = s_raw * ms_residual_scale(m);
+      row_max[row] = m;
+      row_sumexp[row] = s;
+      pred[row] = x_t;
+      loss[row] = logf(s) - (tl >= 0 ? (x_t - m) : 0.0f);
+    }
+
+    // gradient, in place
+    const int64_t next = row + gridDim.x;
+    const bool more = next < n_rows;
+    RowGeo<T> gn = geo;
+    if (more) gn.set(logits, next, V, tid);
+    const float scale = g / s_raw;  // exp2(x*c - fl(m*c)) / s_raw = softmax: the residual cancels
+    const int tv = (tl >= geo.head) ? (int)(tl - geo.head) : -1;
+#pragma unroll
+    for (int u = 0; u < NV; u++) {
+      if (tid + u * FU_THREADS < geo.nvec) {
+        float f[EPV];
+        Elem<T>::unpack(v[u], f);
+#pragma unroll
+        for (int e = 0; e < EPV; e++) f[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc)) * scale;
+        const int base = (tid + u * FU_THREADS) * EPV;
+        if ((unsigned)(tv - base) < (unsigned)EPV) {
+          const int e = tv - base;
+#pragma unroll
+          for (int q = 0; q < EPV; q++)
+            if (q == e) f[q] -= g;
+        }
+        __builtin_nontemporal_store(Elem<T>::pack(f), geo.vp + tid + u * FU_THREADS);
+      }
+    }
+    if (geo.has_edge) {
+      float f = __builtin_amdgcn_exp2f(__builtin_fmaf(fe, LOG2E, -mc)) * scale;
+      if (geo.edge_j == tl) f -= g;
+      Elem<T>::st(geo.rp + geo.edge_j, f);
+    }
+    if (!more) break;
+    // the next row is asked for behind the last store of this one, as one burst: reads mixed into the write burst
+    // vector by vector cost 6 % (the memory then turns between reading and writing all the time)
+#pragma unroll
+    for (int u = 0; u < NV; u++)
+      if (tid + u * FU_THREADS < gn.nvec) v[u] = __builtin_nontemporal_load(gn.vp + tid + u * FU_THREADS);
+    fe = NEG_BIG;
+    if (gn.has_edge) fe = Elem<T>::ld(gn.rp + gn.edge_j);
+    geo = gn;
+    row = next;
   }
 }
 
 // Backward with the row held in registers: every lane of a 1024-lane workgroup loads its NV vectors of the row,
 // the workgroup meets at a barrier, then every lane rewrites them.  The memory sees the row as one burst of reads
-// followed by one burst of writes (250 KiB each for a bf16 row of 128256) instead of 16 KiB steps that alternate
-// between the two: a plain in-place copy moves 6.1 TB/s in this shape against 5.1 TB/s in steps.  Same arithmetic
-// per element as vocab_ce_bwd_kernel, so the same bits.
+// and one burst of writes (250 KiB each for a bf16 row of 128256) instead of 16 KiB steps that alternate
+// between the two.  Walks rows b, b + gridDim.x, ... like the kernel above (one row per workgroup by default).
+// Same arithmetic per element as vocab_ce_bwd_kernel, so the same bits.
 template <typename T, int NV>
 __global__ __launch_bounds__(FU_THREADS) void vocab_ce_bwd_row_kernel(
     T* __restrict__ logits, const int64_t* __restrict__ target, const float* __restrict__ row_max,
-    const float* __restrict__ row_sumexp, const float* __restrict__ grad_out, int64_t V, int64_t vocab_start) {
+    const float* __restrict__ row_sumexp, const float* __restrict__ grad_out, int64_t V, int64_t vocab_start,
+    int64_t n_rows) {
   constexpr int EPV = Elem<T>::EPV;
-  const int64_t row = blockIdx.x;
-  T* rp = logits + row * V;
   const int tid = threadIdx.x;
+  int64_t row = blockIdx.x;
+  if (row >= n_rows) return;
 
-  int head;
-  int64_t nvec64;
-  row_split(rp, V, head, nvec64);
-  const int nvec = (int)nvec64;  // the host checked nvec <= NV * FU_THREADS
-  u32x4_t* vp = reinterpret_cast<u32x4_t*>(rp + head);
-  const int tail0 = head + nvec * EPV;
-  const int n_edge = head + (int)(V - tail0);
-  const int edge_j = tid < head ? tid : tail0 + (tid - head);
-  const bool has_edge = tid < n_edge;
-
+  RowGeo<T> geo;
+  geo.set(logits, row, V, tid);
   u32x4_t v[NV] = {};
 #pragma unroll
   for (int u = 0; u < NV; u++)
-    if (tid + u * FU_THREADS < nvec) v[u] = __builtin_nontemporal_load(vp + tid + u * FU_THREADS);
+    if (tid + u * FU_THREADS < geo.nvec) v[u] = __builtin_nontemporal_load(geo.vp + tid + u * FU_THREADS);
   float fe = 0.0f;
-  if (has_edge) fe = Elem<T>::ld(rp + edge_j);
-
-  const float g = grad_out ? grad_out[row] : 1.0f;
+  if (geo.has_edge) fe = Elem<T>::ld(geo.rp + geo.edge_j);
   const bool from_softmax = row_max == nullptr;
-  const float mc = from_softmax ? 0.0f : mul_rn(row_max[row], LOG2E);
-  const float scale = from_softmax ? g : g * ms_residual_scale(row_max[row]) / row_sumexp[row];
-  int64_t tl = target[row] - vocab_start;
-  if (tl < 0 || tl >= V) tl = -1;
-  const int tv = (tl >= head) ? (int)(tl - head) : -1;
+
+  for (;;) {
+    const float g = grad_out ? grad_out[row] : 1.0f;
+    const float mc = from_softmax ? 0.0f : mul_rn(row_max[row], LOG2E);
+    const float scale = from_softmax ? g : g * ms_residual_scale(row_max[row]) / row_sumexp[row];
+    int64_t tl = target[row] - vocab_start;
+    if (tl < 0 || tl >= V) tl = -1;
+    const int tv = (tl >= geo.head) ? (int)(tl - geo.head) : -1;
+    const int64_t next = row + gridDim.x;
+    const bool more = next < n_rows;
+    RowGeo<T> gn = geo;
+    if (more) gn.set(logits, next, V, tid);
 #pragma unroll
-  for (int u = 0; u < NV; u++) asm volatile("" : "+v"(v[u]));   // every load issued before the first is waited for
-  __syncthreads();   // the whole row has been asked for (and has arrived for this wave) before anyone writes
+    for (int u = 0; u < NV; u++) asm volatile("" : "+v"(v[u]));   // the whole row has arrived for this wave ...
+    __syncthreads();                                              // ... and for every wave, before anyone writes
 
 #pragma unroll
-  for (int u = 0; u < NV; u++)
-    if (tid + u * FU_THREADS < nvec) {
-      float f[EPV];
-      Elem<T>::unpack(v[u], f);
+    for (int u = 0; u < NV; u++) {
+      if (tid + u * FU_THREADS < geo.nvec) {
+        float f[EPV];
+        Elem<T>::unpack(v[u], f);
 #pragma unroll
-      for (int e = 0; e < EPV; e++) f[e] = (from_softmax ? f[e] : __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc))) * scale;
-      const int base = (tid + u * FU_THREADS) * EPV;
-      if ((unsigned)(tv - base) < (unsigned)EPV) {
-        const int e = tv - base;
+        for (int e = 0; e < EPV; e++) f[e] = (from_softmax ? f[e] : __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], LOG2E, -mc))) * scale;
+        const int base = (tid + u * FU_THREADS) * EPV;
+        if ((unsigned)(tv - base) < (unsigned)EPV) {
+          const int e = tv - base;
 #pragma unroll
-        for (int q = 0; q < EPV; q++)
-          if (q == e) f[q] -= g;
+          for (int q = 0; q < EPV; q++)
+            if (q == e) f[q] -= g;
+        }
+        __builtin_nontemporal_store(Elem<T>::pack(f), geo.vp + tid + u * FU_THREADS);
       }
-      __builtin_nontemporal_store(Elem<T>::pack(f), vp + tid + u * FU_THREADS);
     }
-  if (has_edge) {
-    float f = (from_softmax ? fe : __builtin_amdgcn_exp2f(__builtin_fmaf(fe, LOG2E, -mc))) * scale;
-    if (edge_j == tl) f -= g;
-    Elem<T>::st(rp + edge_j, f);
+    if (geo.has_edge) {
+      float f = (from_softmax ? fe : __builtin_amdgcn_exp2f(__builtin_fmaf(fe, LOG2E, -mc))) * scale;
+      if (geo.edge_j == tl) f -= g;
+      Elem<T>::st(geo.rp + geo.edge_j, f);
+    }
+    if (!more) break;
+#pragma unroll
+    for (int u = 0; u < NV; u++)
+      if (tid + u * FU_THREADS < gn.nvec) v[u] = __builtin_nontemporal_load(gn.vp + tid + u * FU_THREADS);
+    fe = 0.0f;
+    if (gn.has_edge) fe = Elem<T>::ld(gn.rp + gn.edge_j);
+    geo = gn;
+    row = next;
   }
+}
+
+// Workgroups of the register-resident kernels: persistent (one per compute unit — each holds a row's worth of the
+// register file — every one walking its share of the rows) or one per row.  Measured on [8192, 128256] bf16 and
+// [8192, 50257] fp32: the one-launch kernel on 16-bit rows gains from walking (788 -> 759 us: the next row is on
+// its way while the loss of this one is written, and a workgroup's start — target, target logit, row gradient,
+// three dependent reads — happens once instead of per row); on fp32 rows it loses (634 -> 671 us) and the backward
+// kernel, which has no such start, loses on both (741 -> 771, 630 -> 670 us): a workgroup that ends with its
+// stores in flight hands the compute unit to the next row's loads sooner than a loop that, counting its memory
+// operations in order, cannot look at the new row before those stores have landed.  Asking for the next row
+// vector by vector between the stores of this one is worse still (+6 %: the memory then turns between reading
+// and writing all the time).  MTP_CE_PERSIST = 0 / 1 forces one workgroup per row / walking for all of them.
+inline unsigned row_kernel_grid(int64_t n_rows, bool walk_by_default) {
+  static MtpTune tune_persist("MTP_CE_PERSIST");
+  const int per = tune_persist.get(walk_by_default ? 1 : 0);
+  if (per <= 0) return (unsigned)n_rows;
+  const int64_t wgs = 256ll * per;
+  return (unsigned)(n_rows < wgs ? n_rows : wgs);
 }
 
 // Rows of at least two unrolled steps of a 1024-lane workgroup are walked by 1024 lanes (64 KiB per step; bf16
@@ -497,8 +558,8 @@ void launch_bwd(void* logits, const int64_t* target, const float* row_max, const
   const int64_t need = (vocab / Elem<T>::EPV + FU_THREADS - 1) / FU_THREADS;
 #define MTP_BWD_ROW_CASE(NV)                                                                                     \
   if (need <= NV) {                                                                                              \
-    hipLaunchKernelGGL((vocab_ce_bwd_row_kernel<T, NV>), dim3((unsigned)n_rows), dim3(FU_THREADS), 0, s,         \
-                       (T*)logits, target, row_max, row_sumexp, grad_out, vocab, vocab_start);                   \
+    hipLaunchKernelGGL((vocab_ce_bwd_row_kernel<T, NV>), dim3(row_kernel_grid(n_rows, false)), dim3(FU_THREADS), 0, s, \
+                       (T*)logits, target, row_max, row_sumexp, grad_out, vocab, vocab_start, n_rows);           \
     return;                                                                                                      \
   }
   // rows of at least a quarter of what 1024 lanes hold; shorter rows are served as well by the stepping kernel
@@ -554,8 +615,8 @@ template <typename T, int NV>
 void launch_fused(void* logits, const int64_t* target, const float* grad_rows, float grad_scale, float* loss,
                   float* row_max, float* row_sumexp, float* pred, int64_t n_rows, int64_t vocab,
                   int64_t vocab_start, hipStream_t s) {
-  hipLaunchKernelGGL((vocab_ce_fused_kernel<T, NV>), dim3((unsigned)n_rows), dim3(FU_THREADS), 0, s, (T*)logits,
-                     target, grad_rows, grad_scale, loss, row_max, row_sumexp, pred, vocab, vocab_start);
+  hipLaunchKernelGGL((vocab_ce_fused_kernel<T, NV>), dim3(row_kernel_grid(n_rows, sizeof(T) == 2)), dim3(FU_THREADS), 0, s, (T*)logits,
+                     target, grad_rows, grad_scale, loss, row_max, row_sumexp, pred, vocab, vocab_start, n_rows);
 }
 
 template <typename T>

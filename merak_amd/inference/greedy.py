@@ -54,9 +54,7 @@ class DecodeStep:
 
     def __init__(self, w_qkv, w_gate_up, w_down, w_lm_head, max_batch: int = 32):
         self.w_qkv, self.w_gate_up, self.w_down, self.w_lm_head = w_qkv, w_gate_up, w_down, w_lm_head
-        from .. import _lib
-        need = _lib.lib().mtp_gemv_argmax_workspace_bytes(max_batch, w_lm_head.shape[0], w_lm_head.shape[1])
-        self.workspace = torch.empty((need,), dtype=torch.uint8, device=w_lm_head.device)
+        self.workspace = ops.argmax_workspace(max_batch, w_lm_head.shape[0], w_lm_head.shape[1], w_lm_head.device)
         # scratch of the linears that are cut along k at this batch size (the launches follow each other)
         self.max_batch = max_batch
         self._gemv_ws = {}
@@ -71,8 +69,8 @@ class DecodeStep:
 
     def __call__(self, x: torch.Tensor):
         ws = self._ws(x.shape[0])
-        qkv = ops.gemv(x, self.w_qkv, workspace=ws)
-        h = ops.gemv(x, self.w_gate_up, None, ops.EPI_SWIGLU, workspace=ws)
+        # QKV and gate/up read the same rows: one call (one grid above 16 rows)
+        qkv, h = ops.gemv_pair(x, self.w_qkv, self.w_gate_up, workspace=ws)
         out = ops.gemv(h, self.w_down, workspace=ws)
         token = greedy_next_token(out, self.w_lm_head, self.workspace)
         return qkv, out, token

@@ -82,9 +82,7 @@ class LlamaDecoder:
         self.v_cache = [torch.zeros((batch, n_kv_heads, max_len, head_dim), dtype=dt, device=dev) for _ in blocks]
         self.lens = torch.zeros((batch,), dtype=torch.int64, device=dev)
         self.host_len_bound = 0           # upper bound of self.lens kept on the host
-        from .. import _lib
-        need = _lib.lib().mtp_gemv_argmax_workspace_bytes(batch, lm_head.shape[0], lm_head.shape[1])
-        self.argmax_ws = torch.empty((max(int(need), 8),), dtype=torch.uint8, device=dev)
+        self.argmax_ws = ops.argmax_workspace(batch, lm_head.shape[0], lm_head.shape[1], dev)
         # the number of splits, and with it the need, does not shrink when the length bound grows
         self.attn_ws = ops.attn_workspace(batch, n_q_heads, n_kv_heads, max_len, dev)
         w0 = blocks[0]

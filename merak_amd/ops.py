@@ -67,23 +67,38 @@ _linear_ws_cache = {}
 _linear_ws_lock = threading.Lock()   # forward runs on the caller's thread, backward on autograd's worker thread
 
 
-def linear_workspace(dev: torch.device) -> torch.Tensor:
+def linear_workspace(dev: torch.device, nbytes: Optional[int] = None) -> torch.Tensor:
     """Scratch of the linear products for the current stream of `dev` (16-bit: stream-K, tiles whose k range
-    several workgroups share meet there; fp32: the slices of a product that is cut along k).  One buffer per
-    (device, stream), allocated at first use and kept: launches on one stream are ordered, so they may share it."""
+    several workgroups share meet there; fp32: the slices of a product that is cut along k), at least `nbytes`
+    long (default: the 16-bit path's full size).  One buffer per (device, stream), allocated when a product first
+    asks for scratch and grown when a later one asks for more: launches on one stream are ordered, so they may
+    share it.  ``release_workspaces()`` drops them all."""
     idx = dev.index if dev.index is not None else torch.cuda.current_device()
     key = (idx, torch.cuda.current_stream(dev).cuda_stream)
+    if nbytes is None:
+        nbytes = _lib.lib().mtp_linear_workspace_bytes()
     with _linear_ws_lock:
         ws = _linear_ws_cache.get(key)
-        if ws is None:
-            ws = torch.empty(_lib.lib().mtp_linear_workspace_bytes(), dtype=torch.uint8, device=dev)
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.empty(int(nbytes), dtype=torch.uint8, device=dev)
             _linear_ws_cache[key] = ws
     return ws
 
 
-def _ws_args(t: torch.Tensor, dev: torch.device):
-    """(pointer, bytes) of the scratch for a product on tensors like t"""
-    ws = linear_workspace(dev)
+def release_workspaces() -> None:
+    """Forget the cached scratch buffers of the linear products (they are allocated again on demand)."""
+    with _linear_ws_lock:
+        _linear_ws_cache.clear()
+
+
+def _ws_args(kind: int, M: int, N: int, K: int, t: torch.Tensor, dev: torch.device):
+    """(pointer, bytes) of the scratch for product `kind` (0 forward, 1 input gradient, 2 weight gradient, 3 both
+    gradients) of a layer with M tokens, N output and K input features on tensors like t; (None, 0) for the shapes
+    that never use scratch, which then allocate nothing."""
+    need = _lib.lib().mtp_linear_workspace_need(kind, M, N, K, _dt(t))
+    if need <= 0:
+        return None, 0
+    ws = linear_workspace(dev, need)
     return ws.data_ptr(), ws.numel()
 
 
@@ -120,7 +135,7 @@ def linear_fwd(x2d: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
     if has_act:
         act = torch.empty(rows + (N // 2 if epilogue == EPI_SWIGLU else N,), dtype=x2d.dtype, device=dev)
     with torch.cuda.device(dev):
-        wsp, wsb = _ws_args(x2d, dev)
+        wsp, wsb = _ws_args(0, M, N, K, x2d, dev)
         rc = _lib.lib().mtp_linear_fwd_ws(_p(x2d), _p(w), _p(bias), _p(y), _p(act), wsp, wsb, M, N, K, _dt(x2d),
                                           epilogue, _stream(dev))
         if rc == -2 and y is None:
@@ -144,7 +159,7 @@ def linear_dgrad(dy2d: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     dy2d, w = _contig(dy2d), _contig(w)
     dx = torch.empty((M, K), dtype=dy2d.dtype, device=dev)
     with torch.cuda.device(dev):
-        wsp, wsb = _ws_args(dy2d, dev)
+        wsp, wsb = _ws_args(1, M, N, K, dy2d, dev)
         _lib.check(_lib.lib().mtp_linear_dgrad_ws(_p(dy2d), _p(w), _p(dx), wsp, wsb, M, N, K, _dt(dy2d), _stream(dev)),
                    "mtp_linear_dgrad")
     return dx
@@ -175,7 +190,7 @@ def linear_wgrad(dy2d: torch.Tensor, x2d: torch.Tensor, want_db: bool, out_dtype
     if want_db and (db.numel() != N or not db.is_contiguous() or db.dtype != out_dtype):
         raise ValueError("linear_wgrad: db must be a contiguous [N] tensor of the output dtype")
     with torch.cuda.device(dev):
-        wsp, wsb = _ws_args(dy2d, dev)
+        wsp, wsb = _ws_args(2, M, N, K, dy2d, dev)
         _lib.check(_lib.lib().mtp_linear_wgrad_ws(_p(dy2d), _p(x2d), _p(dw), _p(db) if want_db else None, wsp, wsb, M, N,
                                                   K, _dt(dy2d), _DTYPES[out_dtype], int(accumulate), _stream(dev)),
                    "mtp_linear_wgrad")
@@ -210,7 +225,7 @@ def linear_bwd(dy2d: torch.Tensor, x2d: torch.Tensor, w: torch.Tensor, want_db: 
     if want_db and (tuple(db.shape) != (N,) or db.dtype != out_dtype or not db.is_contiguous()):
         raise ValueError("linear_bwd: db must be a contiguous [N] tensor of out_dtype")
     with torch.cuda.device(dev):
-        wsp, wsb = _ws_args(dy2d, dev)
+        wsp, wsb = _ws_args(3, M, N, K, dy2d, dev)
         _lib.check(_lib.lib().mtp_linear_bwd_ws(_p(dy2d), _p(x2d), _p(w), _p(dx), _p(dw), _p(db) if want_db else None,
                                                 wsp, wsb, M, N, K, _dt(dy2d), _DTYPES[out_dtype], int(accumulate),
                                                 _stream(dev)), "mtp_linear_bwd")
@@ -423,6 +438,27 @@ def gemv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     return y
 
 
+def gemv_pair(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, bias1: Optional[torch.Tensor] = None,
+              bias2: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):
+    """``(x @ w1.T (+ bias1), swiglu(x @ w2.T (+ bias2)))``: two products over the same rows in one call (one
+    launch above 16 rows, the two launches of ``gemv`` otherwise)."""
+    dev = _require_gpu(x, w1, w2, bias1, bias2, workspace)
+    dt = _decode_dtype("gemv_pair", x, w1, bias1)
+    _decode_dtype("gemv_pair", x, w2, bias2)
+    B, N1, K = _gemv_shapes("gemv_pair", x, w1, bias1)
+    _, N2, K2 = _gemv_shapes("gemv_pair", x, w2, bias2)
+    if K2 != K or N2 % 2:
+        raise ValueError(f"gemv_pair: second weight must be [2 * I, {K}], got {tuple(w2.shape)}")
+    x, w1, w2 = _contig(x), _contig(w1), _contig(w2)
+    y1 = torch.empty((B, N1), dtype=dt, device=dev)
+    act2 = torch.empty((B, N2 // 2), dtype=dt, device=dev)
+    wbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mtp_gemv_pair(_p(x), _p(w1), _p(bias1), _p(y1), N1, _p(w2), _p(bias2), _p(act2), N2,
+                                            _p(workspace), wbytes, B, K, _DTYPES[dt], _stream(dev)), "mtp_gemv_pair")
+    return y1, act2
+
+
 def gemv_norm_fits(B: int, K: int) -> bool:
     """Whether ``gemv_fused`` can take the RMSNorm of a [B, K] input inside the product (B K <= 8 x 4096, K % 512 == 0, K <= 8192)."""
     return bool(_lib.lib().mtp_gemv_norm_fits(B, K))
@@ -464,6 +500,12 @@ def gemv_fused(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = 
     return (out, sumsq) if want_sumsq else out
 
 
+def argmax_workspace(B: int, N: int, K: int, dev: torch.device) -> torch.Tensor:
+    """Scratch for ``gemv_argmax`` on shapes up to [B, K] x [N, K] (nothing in it needs clearing)."""
+    need = _lib.lib().mtp_gemv_argmax_workspace_bytes(B, N, K)
+    return torch.empty((max(int(need), 8),), dtype=torch.uint8, device=dev)
+
+
 def gemv_argmax(x: torch.Tensor, w: torch.Tensor, workspace: Optional[torch.Tensor] = None):
     """-> (idx int64 [B], maxval fp32 [B]) without materialising the logits."""
     dev = _require_gpu(x, w, workspace)
@@ -472,7 +514,7 @@ def gemv_argmax(x: torch.Tensor, w: torch.Tensor, workspace: Optional[torch.Tens
     x, w = _contig(x), _contig(w)
     need = _lib.lib().mtp_gemv_argmax_workspace_bytes(B, N, K)
     if workspace is None:
-        workspace = torch.empty((need,), dtype=torch.uint8, device=dev)
+        workspace = argmax_workspace(B, N, K, dev)
     idx = torch.empty((B,), dtype=torch.int64, device=dev)
     val = torch.empty((B,), dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):

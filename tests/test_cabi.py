@@ -26,7 +26,7 @@ def test_header_symbols_are_exported_and_bound():
 
 def test_loader_and_versions():
     lib = _lib.lib()
-    assert lib.mtp_abi_version() == _lib.ABI_VERSION == 11
+    assert lib.mtp_abi_version() == _lib.ABI_VERSION == 12
     hdr = open(os.path.join(ROOT, "include", "merak_tp_gfx950.h")).read()
     assert f"#define MTP_ABI_VERSION {_lib.ABI_VERSION}" in hdr
     for name, val in (("MTP_F32", _lib.MTP_F32), ("MTP_BF16", _lib.MTP_BF16), ("MTP_EPI_NONE", _lib.EPI_NONE),

@@ -211,6 +211,36 @@ def test_ce_one_launch_forward_backward(gpu, dtype, n, v):
     assert rel(c, R.cross_entropy_fp32(x, t, 0, torch.full((n,), 1.0 / n))[1]) < tol_g
 
 
+@pytest.mark.parametrize("dtype,n,v", [(torch.bfloat16, 700, 40000), (torch.float32, 523, 4 * 4096 + 1),
+                                        (torch.bfloat16, 257, 8192 * 8 - 3), (torch.float16, 300, 32768)])
+def test_ce_row_kernels_walk_their_rows(gpu, set_tuning, dtype, n, v):
+    """The register-resident kernels (one-launch forward+backward, row backward) either take one row per workgroup
+    or walk rows b, b + 256, ... as persistent workgroups, asking for the next row behind the stores of the current
+    one (the default depends on the kernel and the element size; MTP_CE_PERSIST forces either): more rows than
+    workgroups (two or three per workgroup, the last round part empty), rows whose 16-byte alignment changes from
+    row to row.  Against the oracle, and the same bits in every form."""
+    x = torch.randn(n, v, generator=gen(114)).to(dtype)
+    t = torch.randint(0, v, (n,), generator=gen(115))
+    t[torch.randperm(n, generator=gen(116))[: n // 20]] = -100
+    gr = torch.rand(n, generator=gen(117)) + 0.5
+    ref_loss, ref_grad = R.cross_entropy_fp32(x, t, 0, gr * 0.5)
+    tol_g = TOL_F32 if dtype == torch.float32 else TOL_BF16
+    outs = []
+    for persist in (None, 0, 1, 2):
+        set_tuning("MTP_CE_PERSIST", persist)
+        a, b = x.to(gpu), x.to(gpu)
+        loss, m, s, pred = ops.vocab_ce_fwd_bwd_(a, t.to(gpu), 0, gr.to(gpu), 0.5)
+        _, m2, s2, _ = ops.vocab_ce_fwd(b, t.to(gpu), 0)
+        ops.vocab_ce_bwd_(b, t.to(gpu), m2, s2, (gr * 0.5).to(gpu), 0)
+        outs.append((a, b, loss, m, s, pred))
+    a, b, loss = outs[0][:3]
+    assert (loss.cpu() - ref_loss).abs().max() <= TOL_LOSS * max(ref_loss.abs().max().item(), 0.1)
+    assert rel(a, ref_grad) < tol_g and rel(b, ref_grad) < tol_g
+    for other in outs[1:]:
+        for p, q in zip(outs[0], other):
+            assert torch.equal(p, q)
+
+
 def test_ce_one_launch_vocab_slice_and_limits(gpu):
     n, v, start = 8, 1002, 3006
     x = torch.randn(n, v, generator=gen(18)).bfloat16()
@@ -593,11 +623,12 @@ def _check_every_product(inputs, out, tol, what):
 
 
 # k, n and m multiples of 64 (every product can take the 64-deep loop), then ragged in all three
-_CFG_SHAPES = [(320, 576, 448), (300, 520, 200), (1100, 1304, 2112)]
+# (the third has 33 k-tiles of 64 forward; the fourth gives the weight gradient 17 k-tiles and ragged tiles of every width)
+_CFG_SHAPES = [(320, 576, 448), (300, 520, 200), (1100, 1304, 2112), (1088, 1000, 648)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("cfg", list(range(10)))
+@pytest.mark.parametrize("cfg", list(range(14)))
 def test_every_tile_configuration_vs_oracle(gpu, set_tuning, dtype, cfg):
     """Each tile configuration forced in turn (one that cannot serve a shape or epilogue falls back to the
     automatic choice): every product and epilogue against the oracle, and the same bits on a second run."""
@@ -1074,6 +1105,52 @@ def test_gemv_one_workspace_for_shapes_in_turn(gpu):
             y = ops.gemv(x, w, workspace=ws)
             assert rel(y, F.linear(x.float(), w.float())) < TOL_BF16
     assert int(ws[:8192].view(torch.int32).abs().sum()) == 0
+
+
+def test_argmax_one_workspace_for_shapes_in_turn(gpu):
+    """One workspace serves greedy picks of different shapes in turn (nothing in it needs clearing): fewer workgroups
+    than batch rows, thousands of them, two batch tiles."""
+    shapes = [(3, 48, 64), (32, 128256, 512), (7, 5000, 256), (20, 40000, 128), (1, 70000, 64), (32, 1000, 72)]
+    ws = ops.argmax_workspace(32, 128256, 512, gpu)
+    ws.fill_(0xA5)
+    for rep in range(2):
+        for (b, n, k) in shapes:
+            x = torch.randn(b, k, generator=gen(190 + b)).bfloat16()
+            w = (torch.randn(n, k, generator=gen(191 + b)) * 0.02).bfloat16()
+            ref = F.linear(x.float(), w.float())
+            idx, val = ops.gemv_argmax(x.to(gpu), w.to(gpu), ws)
+            idx2, val2 = ops.gemv_argmax(x.to(gpu), w.to(gpu))
+            assert torch.equal(idx, idx2) and torch.equal(val, val2), (rep, b, n, k)
+            # bf16 products: a near tie may fall the other way than in fp32, the winning value may not
+            assert rel(val, ref.max(-1).values) < TOL_F32 and (idx.cpu() == ref.argmax(-1)).float().mean() >= 0.9
+
+
+@pytest.mark.parametrize("b,n1,half,k,bias", [(32, 6144, 14336, 4096, False), (17, 1000, 4096, 1024, True),
+                                               (8, 6144, 14336, 4096, False), (32, 130, 200, 264, True),
+                                               (20, 1280, 3584, 8192, False)])
+def test_gemv_pair_is_the_two_products(gpu, set_tuning, b, n1, half, k, bias):
+    """mtp_gemv_pair: QKV-like and gate/up-like products over the same rows in one call — one grid above 16 rows
+    for the shapes it takes, two launches otherwise: the results of the two separate calls, and the oracle."""
+    x = torch.randn(b, k, generator=gen(290)).bfloat16()
+    w1 = (torch.randn(n1, k, generator=gen(291)) * 0.02).bfloat16()
+    w2 = (torch.randn(2 * half, k, generator=gen(292)) * 0.02).bfloat16()
+    b1 = (torch.randn(n1, generator=gen(293)) * 0.1).bfloat16() if bias else None
+    b2 = (torch.randn(2 * half, generator=gen(294)) * 0.1).bfloat16() if bias else None
+    dev = lambda t: None if t is None else t.to(gpu)
+    xg, w1g, w2g, b1g, b2g = dev(x), dev(w1), dev(w2), dev(b1), dev(b2)
+    y1 = ops.gemv(xg, w1g, b1g, ops.EPI_BIAS if bias else ops.EPI_NONE)
+    a2 = ops.gemv(xg, w2g, b2g, ops.EPI_SWIGLU)
+    for pair in (None, 0):
+        set_tuning("MTP_GEMV_PAIR", pair)
+        p1, p2 = ops.gemv_pair(xg, w1g, w2g, b1g, b2g)
+        # the second product runs in the configuration it has on its own: the same bits; the first one's row blocks
+        # are larger in the one grid (another order of the sums along k): the same values to rounding
+        assert torch.equal(p2, a2) and rel(p1, y1) < 3e-3, pair
+        if pair == 0:
+            assert torch.equal(p1, y1)
+    ref1 = F.linear(x.float(), w1.float(), None if b1 is None else b1.float())
+    pre = F.linear(x.float(), w2.float(), None if b2 is None else b2.float()).bfloat16().float()
+    assert rel(y1, ref1) < TOL_BF16 and rel(a2, R.swiglu(pre)) < TOL_BF16
 
 
 def _lib_bytes(b, n, k):

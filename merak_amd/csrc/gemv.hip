@@ -118,6 +118,7 @@ struct GemvArgs {
   int32_t* karrived;
   int flags;
   GemvFuse fz;
+  int n_part;     // MODE 2: row blocks of the launch = keys per batch row in `part` ([B][n_part])
 };
 
 // LDS of one workgroup, carved out of one buffer (so that a launch that holds two kinds of workgroups needs the
@@ -714,7 +715,8 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
     // group folds the group's keys, the last group the groups — was built and measured: the counter's round trip
     // at the end of every one of 1000-2000 workgroups costs more than the second kernel it saves, 157 -> 175-183 us
     // at 1-8 batch rows, no change at 32.)
-    if (sub == 0 && b < B) part[(int64_t)bx * B + b] = key;
+    // [batch row][row block]: the finishing kernel's lanes then read neighbouring keys
+    if (sub == 0 && b < B) part[(int64_t)b * ga.n_part + bx] = key;
   }
 }
 
@@ -758,7 +760,7 @@ __global__ __launch_bounds__(AF_THREADS) void argmax_finish_kernel(const uint64_
 #pragma unroll
     for (int u = 0; u < AF_DEPTH; u++) {
       const int p = p0 + u * AF_THREADS;
-      a[u] = part[(int64_t)(p < n_part ? p : p0) * B + b];   // past the end: the first one again (changes nothing)
+      a[u] = part[(int64_t)b * n_part + (p < n_part ? p : p0)];   // past the end: the first one again (changes nothing)
     }
 #pragma unroll
     for (int u = 0; u < AF_DEPTH; u++) best = a[u] > best ? a[u] : best;
@@ -932,7 +934,7 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
 // two operand sets wherever the registers hold them (8 waves: 256 per lane)
 #define GV_PP(RR, NNB) (MODE != 2)
   const GemvArgs ga{(const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, part, (int)B, N, k_slice,
-                    rot_mul, K, kpart, karrived, flags, fz};
+                    rot_mul, K, kpart, karrived, flags, fz, (int)n_wg};
 #define GV_LAUNCH_T(RR, NNB, GG, DD, FF)                                                                        \
   hipLaunchKernelGGL((gemv_kernel<RR, NNB, MODE, GG, DD, (RR >= 8 ? 4 : 8), FF, NORM, GV_PP(RR, NNB)>), dim3(n_wg, S), \
                      dim3((RR >= 8 ? 4 : 8) * MTP_WAVE), 0, s, ga)
@@ -1005,7 +1007,7 @@ int launch_gemv_mixed(const void* x, const void* w, const void* bias, void* y, i
   int rot_mul = tune_rot.get(1);
   if (rot_mul < 0) rot_mul = 0;
   const GemvArgs ga{(const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, nullptr, (int)B, N, K,
-                    rot_mul, K, nullptr, nullptr, 0, fz};
+                    rot_mul, K, nullptr, nullptr, 0, fz, 0};
 #define GVM_T(RR, FF)                                                                                              \
   hipLaunchKernelGGL((gemv_kernel<RR, 1, 3, false, 1, GV_MAX_WAVES, FF, NORM, (RR <= 6)>), dim3(n_wg),                \
                      dim3(GV_MAX_WAVES * MTP_WAVE), 0, s, ga)
@@ -1136,9 +1138,9 @@ extern "C" int mtp_gemv_pair(const void* x, const void* w1, const void* bias1, v
   const int flags = tune_noshift.get(0) ? 1 : 0;
   const GemvFuse none{nullptr, nullptr, 0.f, nullptr, nullptr};
   const GemvArgs g1{(const uint16_t*)x, (const uint16_t*)w1, (const uint16_t*)bias1, (uint16_t*)y1, nullptr, (int)B, N1, K,
-                    rot_mul, K, nullptr, nullptr, flags, none};
+                    rot_mul, K, nullptr, nullptr, flags, none, 0};
   const GemvArgs g2{(const uint16_t*)x, (const uint16_t*)w2, (const uint16_t*)bias2, (uint16_t*)act2, nullptr, (int)B, N2, K,
-                    rot_mul, K, nullptr, nullptr, flags, none};
+                    rot_mul, K, nullptr, nullptr, flags, none, 0};
   // the first product's rows in blocks of 16 R1 rows, as few rows per block as still leaves no more blocks than
   // the second product has workgroups
   const unsigned n2 = (unsigned)((half2 + 63) / 64);

@@ -312,7 +312,9 @@ struct RowGeo {
   }
 };
 
-template <typename T, int NV>
+// WALK: the workgroup may have more than one row (gridDim.x < n_rows); without it the loop below runs once and
+// nothing of the next row's bookkeeping takes registers.
+template <typename T, int NV, bool WALK>
 __global__ __launch_bounds__(FU_THREADS) void vocab_ce_fused_kernel(
     T* __restrict__ logits, const int64_t* __restrict__ target, const float* __restrict__ grad_rows,
     float grad_scale, float* __restrict__ loss, float* __restrict__ row_max, float* __restrict__ row_sumexp,
@@ -402,7 +404,7 @@ __global__ __launch_bounds__(FU_THREADS) void vocab_ce_fused_kernel(
 
     // gradient, in place
     const int64_t next = row + gridDim.x;
-    const bool more = next < n_rows;
+    const bool more = WALK && next < n_rows;
     RowGeo<T> gn = geo;
     if (more) gn.set(logits, next, V, tid);
     const float scale = g / s_raw;  // exp2(x*c - fl(m*c)) / s_raw = softmax: the residual cancels
@@ -447,7 +449,7 @@ __global__ __launch_bounds__(FU_THREADS) void vocab_ce_fused_kernel(
 // and one burst of writes (250 KiB each for a bf16 row of 128256) instead of 16 KiB steps that alternate
 // between the two.  Walks rows b, b + gridDim.x, ... like the kernel above (one row per workgroup by default).
 // Same arithmetic per element as vocab_ce_bwd_kernel, so the same bits.
-template <typename T, int NV>
+template <typename T, int NV, bool WALK>
 __global__ __launch_bounds__(FU_THREADS) void vocab_ce_bwd_row_kernel(
     T* __restrict__ logits, const int64_t* __restrict__ target, const float* __restrict__ row_max,
     const float* __restrict__ row_sumexp, const float* __restrict__ grad_out, int64_t V, int64_t vocab_start,
@@ -475,7 +477,7 @@ __global__ __launch_bounds__(FU_THREADS) void vocab_ce_bwd_row_kernel(
     if (tl < 0 || tl >= V) tl = -1;
     const int tv = (tl >= geo.head) ? (int)(tl - geo.head) : -1;
     const int64_t next = row + gridDim.x;
-    const bool more = next < n_rows;
+    const bool more = WALK && next < n_rows;
     RowGeo<T> gn = geo;
     if (more) gn.set(logits, next, V, tid);
 #pragma unroll
@@ -558,8 +560,13 @@ void launch_bwd(void* logits, const int64_t* target, const float* row_max, const
   const int64_t need = (vocab / Elem<T>::EPV + FU_THREADS - 1) / FU_THREADS;
 #define MTP_BWD_ROW_CASE(NV)                                                                                     \
   if (need <= NV) {                                                                                              \
-    hipLaunchKernelGGL((vocab_ce_bwd_row_kernel<T, NV>), dim3(row_kernel_grid(n_rows, false)), dim3(FU_THREADS), 0, s, \
-                       (T*)logits, target, row_max, row_sumexp, grad_out, vocab, vocab_start, n_rows);           \
+    const unsigned grid = row_kernel_grid(n_rows, false);                                                        \
+    if (grid < n_rows)                                                                                           \
+      hipLaunchKernelGGL((vocab_ce_bwd_row_kernel<T, NV, true>), dim3(grid), dim3(FU_THREADS), 0, s, (T*)logits, \
+                         target, row_max, row_sumexp, grad_out, vocab, vocab_start, n_rows);                     \
+    else                                                                                                         \
+      hipLaunchKernelGGL((vocab_ce_bwd_row_kernel<T, NV, false>), dim3(grid), dim3(FU_THREADS), 0, s, (T*)logits, \
+                         target, row_max, row_sumexp, grad_out, vocab, vocab_start, n_rows);                     \
     return;                                                                                                      \
   }
   // rows of at least a quarter of what 1024 lanes hold; shorter rows are served as well by the stepping kernel
@@ -615,8 +622,14 @@ template <typename T, int NV>
 void launch_fused(void* logits, const int64_t* target, const float* grad_rows, float grad_scale, float* loss,
                   float* row_max, float* row_sumexp, float* pred, int64_t n_rows, int64_t vocab,
                   int64_t vocab_start, hipStream_t s) {
-  hipLaunchKernelGGL((vocab_ce_fused_kernel<T, NV>), dim3(row_kernel_grid(n_rows, sizeof(T) == 2)), dim3(FU_THREADS), 0, s, (T*)logits,
-                     target, grad_rows, grad_scale, loss, row_max, row_sumexp, pred, vocab, vocab_start, n_rows);
+  // (the 20-vector instantiation has no registers left for the next row's bookkeeping: it would spill)
+  const unsigned grid = row_kernel_grid(n_rows, sizeof(T) == 2 && NV <= 16);
+  if (grid < n_rows)
+    hipLaunchKernelGGL((vocab_ce_fused_kernel<T, NV, true>), dim3(grid), dim3(FU_THREADS), 0, s, (T*)logits, target,
+                       grad_rows, grad_scale, loss, row_max, row_sumexp, pred, vocab, vocab_start, n_rows);
+  else
+    hipLaunchKernelGGL((vocab_ce_fused_kernel<T, NV, false>), dim3(grid), dim3(FU_THREADS), 0, s, (T*)logits, target,
+                       grad_rows, grad_scale, loss, row_max, row_sumexp, pred, vocab, vocab_start, n_rows);
 }
 
 template <typename T>

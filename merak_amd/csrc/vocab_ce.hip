@@ -70,13 +70,18 @@ template <> struct Elem<f16s> {  // IEEE half bits
   }
 };
 
-// Split a row of V elements starting at p into [0,head) scalar, nvec aligned
-// 16-byte vectors, and a scalar tail.
+// Split a row of V elements starting at p into [0,head) scalar, nvec 16-byte vectors, and a scalar tail.  The
+// vectors start at a 128-byte boundary, not merely a 16-byte one: a wave's 64 vectors then cover eight whole cache
+// lines, where a body that starts inside a line makes every wave's stores end in a partial line that the next
+// wave completes.  Rows whose length is not a multiple of 128 bytes start at every alignment in turn; measured on
+// [8192, 50257] fp32 the in-place gradient pass went from 625 to 580 us with line-aligned bodies (the same rows
+// padded to 50240 elements, which are line aligned by themselves: 578 us).  Reads do not care.
+// head + tail stay below 2 * 128 / sizeof(T) elements: one element per lane of the smallest workgroup.
 template <typename T>
 __device__ __forceinline__ void row_split(const T* p, int64_t V, int& head, int64_t& nvec) {
   constexpr int EPV = Elem<T>::EPV;
-  uintptr_t mis = reinterpret_cast<uintptr_t>(p) & 15u;
-  int h = mis ? (int)((16u - mis) / sizeof(T)) : 0;
+  uintptr_t mis = reinterpret_cast<uintptr_t>(p) & 127u;
+  int h = mis ? (int)((128u - mis) / sizeof(T)) : 0;
   if (h > V) h = (int)V;
   head = h;
   nvec = (V - h) / EPV;
@@ -165,7 +170,7 @@ __global__ __launch_bounds__(NT) void vocab_ce_fwd_kernel(
     Elem<T>::unpack(v, f);
     ms_accumulate<EPV>(acc, f);
   }
-  // scalar head and tail (fewer than 2*EPV elements in total)
+  // scalar head and tail (fewer than 128 / sizeof(T) + EPV elements in total: one per lane)
   {
     const int64_t tail0 = head + nvec * EPV;
     const int n_edge = head + (int)(V - tail0);

@@ -230,16 +230,18 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   // workgroups give logits that are equal to rounding, not necessarily bit for bit.)
   const int64_t rot = GUARD || (pairs % GV_MAX_WAVES) ? 0 : ((int64_t)(bx + by) * rot_mul) % pairs;
 
-  static_assert(MODE != 3 || (NB == 1 && !GUARD && D == 1), "mixed SwiGLU groups: one batch tile, K % 64 == 0, depth 1");
+  static_assert(MODE != 3 || (!GUARD && D == 1), "mixed SwiGLU groups: K % 64 == 0, depth 1");
   constexpr bool MIX = MODE == 3;
   f32x4_t acc[R][NB];
-  f32x4_t acc_up[MIX ? R : 1];   // MIX: the products with X at the up rows' k position
+  f32x4_t acc_up[MIX ? R : 1][NB];   // MIX: the products with X at the up rows' k position
 #pragma unroll
   for (int r = 0; r < R; r++)
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) acc[r][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int r = 0; r < (MIX ? R : 1); r++) acc_up[r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < (MIX ? R : 1); r++)
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) acc_up[r][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const bool low = li < 8;
 
   // D pairs (8 apart) per step: with few rows per workgroup this is what keeps enough bytes in flight.
@@ -249,7 +251,8 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   // shapes a large power of two apart, i.e. in the same memory channel and bank but another DRAM page.
   // Walking both at the same k makes the two streams evict each other's open page, so the up rows walk
   // half a row ahead (XS = 2 sets of X fragments, one per k position).
-  constexpr int XS = ((MODE == 1 || MODE == 3) && !GUARD && NB == 1) ? 2 : 1;
+  // (the mixed groups always hold two k positions; the paired groups take the shift with one batch tile only)
+  constexpr int XS = (((MODE == 1 && NB == 1) || MODE == 3) && !GUARD) ? 2 : 1;
   const int64_t up_shift = (XS == 2 && pairs % GV_WAVES == 0 && !(flags & 1)) ? ((pairs / 2) & ~(int64_t)(GV_WAVES - 1)) : 0;
   // Operand registers of one step.  PP: two such sets used in turn, the next step's requests go out before the
   // current step's operands are waited for.  Otherwise one set is rotated by copying, which the compiler folds
@@ -331,10 +334,13 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
     if constexpr (PP) {
       if (MIX) {
         // rows 0-7 (gate) belong to k position 0, rows 8-15 (up) to position 1: both products, two accumulators
-        acc[r][0] = X::mfma16(h0, bx[0][0][0], acc[r][0]);
-        acc[r][0] = X::mfma16(h1, bx[0][0][1], acc[r][0]);
-        acc_up[r] = X::mfma16(h0, bx[XS - 1][0][0], acc_up[r]);
-        acc_up[r] = X::mfma16(h1, bx[XS - 1][0][1], acc_up[r]);
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+          acc[r][nb] = X::mfma16(h0, bx[0][nb][0], acc[r][nb]);
+          acc[r][nb] = X::mfma16(h1, bx[0][nb][1], acc[r][nb]);
+          acc_up[r][nb] = X::mfma16(h0, bx[XS - 1][nb][0], acc_up[r][nb]);
+          acc_up[r][nb] = X::mfma16(h1, bx[XS - 1][nb][1], acc_up[r][nb]);
+        }
         return;
       }
       const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
@@ -345,10 +351,16 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
       }
     } else {
       if (MIX) {
-        acc[r][0] = X::mfma16(h0, bx[0][0][0], acc[r][0]);
-        acc_up[r] = X::mfma16(h0, bx[XS - 1][0][0], acc_up[r]);
-        acc[r][0] = X::mfma16(h1, bx[0][0][1], acc[r][0]);
-        acc_up[r] = X::mfma16(h1, bx[XS - 1][0][1], acc_up[r]);
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+          acc[r][nb] = X::mfma16(h0, bx[0][nb][0], acc[r][nb]);
+          acc_up[r][nb] = X::mfma16(h0, bx[XS - 1][nb][0], acc_up[r][nb]);
+        }
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+          acc[r][nb] = X::mfma16(h1, bx[0][nb][1], acc[r][nb]);
+          acc_up[r][nb] = X::mfma16(h1, bx[XS - 1][nb][1], acc_up[r][nb]);
+        }
         return;
       }
       const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
@@ -540,7 +552,9 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   if (MIX) {
     // D[i][b]: lane groups 0 and 1 hold rows 0-7 (gate, from acc), groups 2 and 3 rows 8-15 (up, from acc_up)
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r][0] = lg < 2 ? acc[r][0] : acc_up[r];
+    for (int r = 0; r < R; r++)
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) acc[r][nb] = lg < 2 ? acc[r][nb] : acc_up[r][nb];
   }
 
   // ---- sum the 8 k-slices through LDS: up to 8 tiles (row group x batch tile) per wave at a time, i.e. one
@@ -553,12 +567,15 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   for (int r0 = 0; r0 < R; r0 += GP) {
 #pragma unroll
     for (int rr = 0; rr < GP; rr++)
+      if (r0 + rr < R) {   // (the last phase of an odd number of groups is part empty)
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++)
+        for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) part_lds[wave][rr][nb][j][lane] = acc[r0 + rr][nb][j];
+          for (int j = 0; j < 4; j++) part_lds[wave][rr][nb][j][lane] = acc[r0 + rr][nb][j];
+      }
     __syncthreads();
-    for (int e = tid; e < GP * NB * 256; e += GV_THREADS) {
+    const int live = (R - r0 < GP ? R - r0 : GP) * NB * 256;
+    for (int e = tid; e < live; e += GV_THREADS) {
       const int rr = e / (NB * 256), nb = (e >> 8) % NB, j = (e >> 6) & 3, l = e & 63;
       float s = 0.f;
 #pragma unroll
@@ -977,16 +994,22 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
 // layers of 256 workgroups best, then the larger R (fewer reductions); too few workgroups are not an option.
 int pick_mixed_groups(int64_t B, int64_t N, int64_t K) {
   const int64_t half = N / 2;
-  if (B > 16 || K % 64 != 0 || (K / 64) % GV_MAX_WAVES != 0 || (half + 64) * K >= (1ll << 32)) return 0;
+  if (K % 64 != 0 || (K / 64) % GV_MAX_WAVES != 0 || (half + 64) * K >= (1ll << 32)) return 0;
   static MtpTune tune_mix("MTP_GEMV_MIX");
+  // Two batch tiles (more than 16 rows): built with seven groups, on workgroups of four waves with one operand
+  // set, and taken only when forced (MTP_GEMV_MIX = 7): 256 equal workgroups instead of 224, but twice the
+  // accumulators leave no registers for the second operand set, and 28672 x 4096 at 32 rows takes 46 us that way
+  // against 44.5 us with paired groups.
+  const int r_lo = B > 16 ? 7 : 1;
   if (tune_mix.is_set()) {
     const int r = tune_mix.get(0);
-    return r >= 1 && r <= 7 ? r : 0;
+    return r >= r_lo && r <= 7 ? r : 0;
   }
+  if (B > 16) return 0;
   const int64_t groups = (half + 7) / 8;
   int best = 0;
   double best_eff = 0.0;
-  for (int r = 1; r <= 7; r++) {
+  for (int r = r_lo; r <= 7; r++) {
     const int64_t wgs = (groups + r - 1) / r;
     if (wgs < 200) continue;
     const double eff = (double)wgs / (double)((wgs + 255) / 256 * 256);
@@ -1016,6 +1039,21 @@ int launch_gemv_mixed(const void* x, const void* w, const void* bias, void* y, i
     if (f16) GVM_T(RR, true);    \
     else GVM_T(RR, false);       \
     break
+  if (B > 16) {
+    // two batch tiles: twice the accumulators, one operand set, four waves (one workgroup per compute unit)
+    if constexpr (!NORM) {
+      if (R != 7) {
+        mtp_set_error("gemv: %d mixed row groups at %lld rows", R, (long long)B);
+        return MTP_EINVAL;
+      }
+      if (f16)
+        hipLaunchKernelGGL((gemv_kernel<7, 2, 3, false, 1, 4, true, false, false>), dim3(n_wg), dim3(4 * MTP_WAVE), 0, s, ga);
+      else
+        hipLaunchKernelGGL((gemv_kernel<7, 2, 3, false, 1, 4, false, false, false>), dim3(n_wg), dim3(4 * MTP_WAVE), 0, s, ga);
+    }
+    MTP_CHECK_LAUNCH("gemv");
+    return MTP_OK;
+  }
   switch (R) {
     GVM(1);
     GVM(2);
@@ -1125,7 +1163,8 @@ extern "C" int mtp_gemv_pair(const void* x, const void* w1, const void* bias1, v
   const int64_t half2 = N2 / 2;
   // one grid: two batch tiles, whole 64-element pairs, a second product that fills the chip with 8-group
   // workgroups by itself, 32-bit row offsets inside a workgroup's rows
-  const bool one_grid = tune_pair.get(1) != 0 && B > 16 && K % 64 == 0 && pick_gemv_cfg(B, N2, K, 1).R == 8 &&
+  const bool one_grid = tune_pair.get(1) != 0 && B > 16 && K % 64 == 0 && pick_mixed_groups(B, N2, K) == 0 &&
+                        pick_gemv_cfg(B, N2, K, 1).R == 8 &&
                         pick_gemv_cfg(B, N2, K, 1).S == 1 && 128 * K < (1ll << 31);
   if (!one_grid) {
     rc = mtp_gemv_ws(x, w1, bias1, y1, workspace, workspace_bytes, B, N1, K, bias1 ? MTP_EPI_BIAS : MTP_EPI_NONE, dtype, stream);

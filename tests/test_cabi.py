@@ -54,6 +54,20 @@ def test_argument_errors_are_reported_without_a_device():
     assert lib.mtp_gemv_fused(None, None, None, None, None, None, 0.0, 16, None, None, 0, 1, 64, 512, 3, 1, None) == -1
 
 
+def test_linear_workspace_need_is_zero_for_shapes_that_never_use_scratch():
+    lib = _lib.lib()
+    full = lib.mtp_linear_workspace_bytes()
+    # Llama-3-8B gate/up forward: whole rounds of tiles, no scratch; the Llama-70B shard's o-proj gradients (128
+    # tiles, 128 k-tiles each) are what stream-K is for; an fp32 weight gradient with few tiles is cut along k
+    assert lib.mtp_linear_workspace_need(0, 4096, 28672, 4096, _lib.MTP_BF16) == 0
+    assert lib.mtp_linear_workspace_need(3, 4096, 28672, 4096, _lib.MTP_BF16) == 0
+    assert lib.mtp_linear_workspace_need(3, 8192, 8192, 1024, _lib.MTP_BF16) == full
+    assert lib.mtp_linear_workspace_need(1, 8192, 8192, 1024, _lib.MTP_F16) == full
+    assert lib.mtp_linear_workspace_need(2, 8192, 3072, 768, _lib.MTP_F32) == 8 * (3072 * 768 + 3072) * 4
+    assert lib.mtp_linear_workspace_need(0, 8192, 3072, 768, _lib.MTP_F32) == 0
+    assert lib.mtp_linear_workspace_need(7, 8, 8, 8, _lib.MTP_BF16) == 0 and lib.mtp_linear_workspace_need(0, 0, 8, 8, 1) == 0
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setenv("MERAK_AMD_LIB", str(tmp_path / "nope.so"))
     monkeypatch.setattr(_lib, "_lib", None)

@@ -641,6 +641,23 @@ def test_every_tile_configuration_vs_oracle(gpu, set_tuning, dtype, cfg):
             assert torch.equal(out[name], again[name]), (cfg, m, n, k, name)
 
 
+def test_linear_scratch_is_allocated_only_for_shapes_that_use_it(gpu):
+    """The wrappers ask the library how much scratch a product can use and allocate none for the (many) shapes that
+    never touch it; a shape stream-K is taken for gets the buffer, per device and stream, until it is released."""
+    from merak_amd import _lib
+    ops.release_workspaces()
+    x, w, _, dy = _lin_inputs(512, 1024, 512, torch.bfloat16, 33, bias=False)      # every product has under 32 k-tiles
+    y, _ = ops.linear_fwd(x.to(gpu), w.to(gpu), None, ops.EPI_NONE)
+    ops.linear_bwd(dy.to(gpu), x.to(gpu), w.to(gpu), False)
+    assert not ops._linear_ws_cache and rel(y, F.linear(x.float(), w.float())) < TOL_BF16
+    x, w, _, _ = _lin_inputs(256, 512, 4096, torch.bfloat16, 34, bias=False)       # 2 tiles, 64 k-tiles each
+    y, _ = ops.linear_fwd(x.to(gpu), w.to(gpu), None, ops.EPI_NONE)
+    assert rel(y, F.linear(x.float(), w.float())) < TOL_BF16
+    assert [t.numel() for t in ops._linear_ws_cache.values()] == [_lib.lib().mtp_linear_workspace_bytes()]
+    ops.release_workspaces()
+    assert not ops._linear_ws_cache
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2])
 @pytest.mark.parametrize("cfg", [8, None])
 def test_stream_k_forced_vs_oracle(gpu, set_tuning, mode, cfg):
@@ -1464,10 +1481,12 @@ def test_greedy_pick_over_a_vocab_sharded_lm_head(gpu):
 
 @pytest.mark.parametrize("mix", ["1", "2", "3", "4", "5", "6", "7", None])
 @pytest.mark.parametrize("b,half,k,with_bias", [(1, 14336, 4096, False), (8, 1000, 1024, True), (16, 56, 512, False),
-                                                (3, 3584, 8192, False)])
+                                                (3, 3584, 8192, False), (32, 14336, 4096, False), (17, 1000, 1024, True),
+                                                (25, 100, 512, False)])
 def test_gemv_swiglu_mixed_row_groups(gpu, set_tuning, mix, b, half, k, with_bias):
     """SwiGLU GEMV whose 16-row tiles hold 8 gate rows and their 8 up rows, for every number of groups per
-    workgroup (forced) and for the automatic choice: same result as the oracle, ragged ends included."""
+    workgroup (forced) and for the automatic choice: same result as the oracle, ragged ends included.  Above 16
+    batch rows (two batch tiles) the form exists with seven groups; other forced values take the paired groups."""
     if mix is not None:
         set_tuning("MTP_GEMV_MIX", mix)
     g = gen(41)

@@ -316,6 +316,19 @@ def secondary(dev, timer, reps, with_cpu):
         "one_launch_speedup_over_two_launches": round((f_ms + b_ms) / o_ms, 3),
         "note": "fwd_bwd_GBs / frac_hbm_peak: the two launches of the reference's own API, three passes moved and "
                 "counted; one_launch_*: forward+backward in one kernel, two passes moved and counted"})
+    # What this board moves when a plain copy kernel reads and rewrites the same 2.1 GB in place (the backward's
+    # memory pattern with no arithmetic), and when it copies them to a second buffer: the ceiling the backward and
+    # the one-launch kernel stand against.
+    st = torch.cuda.current_stream().cuda_stream
+    nb16 = nbytes // 16 * 16
+    ip_ms = timer.run("ce.copy_in_place", lambda: _lib.check(_lib.lib().mtp_stream_copy(work.data_ptr(), work.data_ptr(), nb16, st), "copy"), reps)
+    other = torch.empty_like(work)
+    cp_ms = timer.run("ce.copy", lambda: _lib.check(_lib.lib().mtp_stream_copy(work.data_ptr(), other.data_ptr(), nb16, st), "copy"), reps)
+    del other
+    out["vocab_ce_c4"].update({
+        "copy_in_place_same_bytes_us": round(ip_ms * 1e3, 1), "copy_in_place_GBs": round(2 * nb16 / ip_ms / 1e6, 1),
+        "copy_to_second_buffer_us": round(cp_ms * 1e3, 1), "copy_to_second_buffer_GBs": round(2 * nb16 / cp_ms / 1e6, 1),
+        "bwd_rate_over_copy_in_place": round(ip_ms / b_ms, 4)})
     if with_cpu:
         # the reference's multi-pass algorithm with its three all-reduces on a 1-rank gloo group (CPU tensors)
         import torch.distributed as dist

@@ -297,12 +297,14 @@ int mtp_gemv_ws(const void* x, const void* w, const void* bias, void* y,
  *   act2 [B, N2/2] = silu(G) * U, (G | U) = x W2^T (+ bias2), W2 = [gate rows | up rows]
  * — what a block whose QKV and gate/up projections read the same rows computes
  * (the decode step of Merak/inference/text_generation_inference.py:199-203 on
- * the linears of one block).  Above 16 batch rows both products go out as one
- * grid, so that the smaller one does not start and drain the chip on its own;
- * otherwise (and for shapes the one grid does not take) the call is the two
- * launches of mtp_gemv_ws, with the same workspace rules.  act2 has the bits
- * of the separate call; y1 is summed along k in the order of the one grid's
- * larger row blocks (equal to the separate call to rounding). */
+ * the linears of one block).  Where the second product fills the chip with one
+ * workgroup per compute unit, both go out as one grid: the rows of the first
+ * product ride as one or two more row groups in the loop of the second's
+ * workgroups (or, above 16 batch rows, as a block in front of it), so that the
+ * smaller product neither starts nor drains the chip on its own.  For other
+ * shapes the call is the two launches of mtp_gemv_ws, with the same workspace
+ * rules.  Results equal those of the separate calls to rounding (other orders
+ * of the sums along k); above 16 batch rows act2 has the separate call's bits. */
 int mtp_gemv_pair(const void* x, const void* w1, const void* bias1, void* y1, int64_t N1,
                   const void* w2, const void* bias2, void* act2, int64_t N2,
                   void* workspace, int64_t workspace_bytes,

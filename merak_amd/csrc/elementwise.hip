@@ -152,7 +152,7 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(const u32x4_t* __restr
 
 // Register-resident MFMA loop.  What the matrix cores sustain depends on the operand bits, because the chip
 // runs against a power limit: `random_data` fills the four A and four B fragments with pseudo-random
-// mantissas and signs (exponents around 1.0, like N(0,1) activations); otherwise they hold small smooth
+// mantissas and signs (exponents near 1.0, like N(0,1) activations); otherwise they hold small smooth
 // values that toggle few wires.  Fragments rotate so that consecutive MFMAs see different operands.
 __global__ __launch_bounds__(256) void mfma_peak_kernel(float* __restrict__ sink, int64_t iters, int random_data) {
   const int lane = threadIdx.x & 63;

@@ -100,7 +100,9 @@ struct GemvFuse {
 // workgroups leave a quarter of the CUs with half the bytes in flight: 5.4 instead of 6.4 TB/s).  Load A fetches the
 // gate rows of a k-pair, load B the up rows half a row further along k (the two sit a large power of two apart in
 // memory, see below), so a tile mixes two k positions: it is multiplied twice, once with X at either position,
-// into two accumulators, and each lane keeps the one whose rows it owns.
+// into two accumulators, and each lane keeps the one whose rows it owns.  With two batch tiles (more than 16 batch
+// rows) the up rows walk in step with the gate rows instead: one k position, one product and one accumulator per
+// tile, which leaves the registers for a second operand set.
 // W waves split K.  Configurations whose registers allow only 8 waves per CU run as two independent workgroups of
 // 4 waves rather than one of 8: while one sums its partial tiles and writes its outputs the other keeps streaming.
 // Everything a launch hands to a workgroup.
@@ -139,8 +141,14 @@ struct GemvLds {
 };
 
 // bx, by, gy: the workgroup's place (row block, k slice) and the number of k slices; smem: GemvLds<...>::BYTES of LDS
-template <int R, int NB, int MODE, bool GUARD, int D, int W, bool F16, bool NORM, bool PP>
-__device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, const int by, const int gy, char* smem) {
+// E > 0 (mixed SwiGLU groups, gate and up rows in step): the workgroup also owns E plain 16-row groups of a second
+// matrix over the same X (xa: its weights, bias, output and row count; ebx: which block of 16 E rows), streamed in
+// the same loop as E more row groups and stored without an activation.
+template <int R, int NB, int MODE, bool GUARD, int D, int W, bool F16, bool NORM, bool PP, int E = 0>
+__device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, const int by, const int gy, char* smem,
+                                          const GemvArgs* xa = nullptr, const int ebx = 0) {
+  constexpr int RT = R + E;   // row groups in the loop
+  static_assert(E == 0 || (MODE == 3 && !NORM && !GUARD), "extra plain groups ride on mixed SwiGLU groups");
   const uint16_t* __restrict__ x = ga.x;
   const uint16_t* __restrict__ w = ga.w;
   const uint16_t* __restrict__ bias = ga.bias;
@@ -152,7 +160,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   float* __restrict__ kpart = ga.kpart;
   int32_t* __restrict__ karrived = ga.karrived;
   const GemvFuse& fz = ga.fz;
-  using L = GemvLds<R, NB, W, NORM>;
+  using L = GemvLds<RT, NB, W, NORM>;
   static_assert(!NORM || (!GUARD && MODE != 2), "the norm prologue needs K % 64 == 0 and a stored output");
   // K is the extent along k that this workgroup covers and ld the row stride of X and W: with gy > 1
   // the k range is cut into gy slices of K elements, one workgroup per (row block, slice); the
@@ -171,12 +179,16 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   // Per row group: a wave-uniform base (first row of the group) and 32-bit per-lane element offsets for
   // the two loads.  GUARD (K not a multiple of 64) keeps the plain layout: load A = first 64 bytes of the
   // pair at row li, load B = the next 64.  Rows past the end are clamped to the last row (never stored).
-  const uint16_t* wbase[R];
-  uint32_t offa[R], offb[R];
+  const uint16_t* wbase[RT];
+  uint32_t offa[RT], offb[RT];
 #pragma unroll
-  for (int r = 0; r < R; r++) {
+  for (int r = 0; r < RT; r++) {
     int64_t row0, lim;
-    if (MODE == 3) {
+    const bool extra = E > 0 && r >= R;
+    if (extra) {
+      row0 = (int64_t)ebx * (16 * E) + 16 * (r - R);
+      lim = xa->N;
+    } else if (MODE == 3) {
       row0 = (int64_t)bx * (8 * R) + 8 * r;
       lim = half;
     } else if (MODE == 1) {
@@ -189,12 +201,12 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
     }
     if (row0 >= lim) row0 = lim - 1;                 // a group entirely past the end reads the last row
     const int last = (int)(lim - 1 - row0);          // >= 0: largest valid row offset inside this group
-    wbase[r] = w + row0 * ld + koff;
+    wbase[r] = (extra ? xa->w : w) + row0 * ld + koff;
     if (GUARD) {
       const int ra = li < last ? li : last;
       offa[r] = (uint32_t)(ra * ld + 8 * lg);
       offb[r] = offa[r] + 32;
-    } else if (MODE == 3) {
+    } else if (MODE == 3 && !extra) {
       // load A: gate row row0 + li%8; load B: the up row of the same index, `half` rows further down (the host
       // checks that this offset fits 32 bits)
       const int ra = (li & 7) < last ? (li & 7) : last;
@@ -232,14 +244,15 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
 
   static_assert(MODE != 3 || (!GUARD && D == 1), "mixed SwiGLU groups: K % 64 == 0, depth 1");
   constexpr bool MIX = MODE == 3;
-  f32x4_t acc[R][NB];
-  f32x4_t acc_up[MIX ? R : 1][NB];   // MIX: the products with X at the up rows' k position
+  constexpr bool MIX2 = MIX && NB == 1 && E == 0;   // mixed groups whose up rows walk ahead of the gate rows: two products per tile
+  f32x4_t acc[RT][NB];
+  f32x4_t acc_up[MIX2 ? R : 1][NB];   // MIX2: the products with X at the up rows' k position
 #pragma unroll
-  for (int r = 0; r < R; r++)
+  for (int r = 0; r < RT; r++)
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) acc[r][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int r = 0; r < (MIX ? R : 1); r++)
+  for (int r = 0; r < (MIX2 ? R : 1); r++)
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) acc_up[r][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const bool low = li < 8;
@@ -251,14 +264,15 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   // shapes a large power of two apart, i.e. in the same memory channel and bank but another DRAM page.
   // Walking both at the same k makes the two streams evict each other's open page, so the up rows walk
   // half a row ahead (XS = 2 sets of X fragments, one per k position).
-  // (the mixed groups always hold two k positions; the paired groups take the shift with one batch tile only)
-  constexpr int XS = (((MODE == 1 && NB == 1) || MODE == 3) && !GUARD) ? 2 : 1;
+  // (with one batch tile only.  With two, gate and up rows walk in step: a mixed tile then holds one k position, needs
+  // one product and one accumulator, and its registers leave room for the second operand set)
+  constexpr int XS = ((MODE == 1 || MODE == 3) && NB == 1 && !GUARD && E == 0) ? 2 : 1;
   const int64_t up_shift = (XS == 2 && pairs % GV_WAVES == 0 && !(flags & 1)) ? ((pairs / 2) & ~(int64_t)(GV_WAVES - 1)) : 0;
   // Operand registers of one step.  PP: two such sets used in turn, the next step's requests go out before the
   // current step's operands are waited for.  Otherwise one set is rotated by copying, which the compiler folds
   // into the requests themselves: each goes out right behind the last MFMA that read its register.
-  bf16x8_t a_s0[D][R][2], b_s0[D][XS][NB][2];
-  bf16x8_t a_s1[D][R][2], b_s1[D][XS][NB][2];
+  bf16x8_t a_s0[D][RT][2], b_s0[D][XS][NB][2];
+  bf16x8_t a_s1[D][RT][2], b_s1[D][XS][NB][2];
   // NORM: RMSNorm(X) is built once per workgroup in LDS, rows padded so that the 16-byte fragment reads of four
   // batch rows fall into different banks
   constexpr int XL_PAD = L::XL_PAD;
@@ -274,14 +288,14 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
     ks[0] = pr * 64;
     ks[1] = pu * 64;
   };
-  auto load_w = [&](int64_t pq0, bf16x8_t (&a)[D][R][2]) {
+  auto load_w = [&](int64_t pq0, bf16x8_t (&a)[D][RT][2]) {
 #pragma unroll
     for (int d = 0; d < D; d++) {
       int64_t ks[2];
       pair_k(pq0, d, ks);
 #pragma unroll
-      for (int r = 0; r < R; r++) {
-        if (MIX) {   // gate rows at the pair itself, up rows at the shifted pair
+      for (int r = 0; r < RT; r++) {
+        if (MIX && r < R) {   // gate rows at the pair itself, up rows at the shifted pair
           a[d][r][0] = load_frag_nt(wbase[r] + ks[0] + offa[r], true);
           a[d][r][1] = load_frag_nt(wbase[r] + ks[1] + offb[r], true);
           continue;
@@ -310,7 +324,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
           }
     }
   };
-  auto load_set = [&](int64_t pq0, bf16x8_t (&a)[D][R][2], bf16x8_t (&b)[D][XS][NB][2]) {
+  auto load_set = [&](int64_t pq0, bf16x8_t (&a)[D][RT][2], bf16x8_t (&b)[D][XS][NB][2]) {
     load_w(pq0, a);
     load_x(pq0, b);
   };
@@ -332,7 +346,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   // products never stand next to each other inside its pinned sections)
   auto multiply_group = [&](int r, const bf16x8_t& h0, const bf16x8_t& h1, bf16x8_t (&bx)[XS][NB][2]) {
     if constexpr (PP) {
-      if (MIX) {
+      if (MIX2) {
         // rows 0-7 (gate) belong to k position 0, rows 8-15 (up) to position 1: both products, two accumulators
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
@@ -350,7 +364,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
         acc[r][nb] = X::mfma16(h1, bx[xs][nb][1], acc[r][nb]);
       }
     } else {
-      if (MIX) {
+      if (MIX2) {
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
           acc[r][nb] = X::mfma16(h0, bx[0][nb][0], acc[r][nb]);
@@ -370,11 +384,11 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
       for (int nb = 0; nb < NB; nb++) acc[r][nb] = X::mfma16(h1, bx[xs][nb][1], acc[r][nb]);
     }
   };
-  auto multiply = [&](bf16x8_t (&a_cur)[D][R][2], bf16x8_t (&b_cur)[D][XS][NB][2]) {
+  auto multiply = [&](bf16x8_t (&a_cur)[D][RT][2], bf16x8_t (&b_cur)[D][XS][NB][2]) {
 #pragma unroll
     for (int d = 0; d < D; d++)
 #pragma unroll
-      for (int r = 0; r < R; r++) {
+      for (int r = 0; r < RT; r++) {
         bf16x8_t h0, h1;
         halves(a_cur[d][r][0], a_cur[d][r][1], h0, h1);
         multiply_group(r, h0, h1, b_cur[d]);
@@ -386,7 +400,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   // while the step is multiplied.  (Left to itself the compiler gathers the selects of all groups at the top of
   // the loop behind one wait for every load: nothing in flight during the products.)  The X fragments of the
   // next step are asked for first, into the second set.
-  auto roll_step = [&](int64_t pq_next, bf16x8_t (&a)[D][R][2], bf16x8_t (&b_cur)[D][XS][NB][2],
+  auto roll_step = [&](int64_t pq_next, bf16x8_t (&a)[D][RT][2], bf16x8_t (&b_cur)[D][XS][NB][2],
                        bf16x8_t (&b_nxt)[D][XS][NB][2]) {
     load_x(pq_next, b_nxt);
 #pragma unroll
@@ -394,11 +408,11 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
       int64_t ks[2];
       pair_k(pq_next, d, ks);
 #pragma unroll
-      for (int r = 0; r < R; r++) {
+      for (int r = 0; r < RT; r++) {
         bf16x8_t h0, h1;
         halves(a[d][r][0], a[d][r][1], h0, h1);
         __builtin_amdgcn_sched_barrier(0);   // the two registers are free from here on: the requests reuse them
-        if (MIX) {
+        if (MIX && r < R) {
           a[d][r][0] = load_frag_nt(wbase[r] + ks[0] + offa[r], true);
           a[d][r][1] = load_frag_nt(wbase[r] + ks[1] + offb[r], true);
         } else {
@@ -549,7 +563,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
     }
   }
 
-  if (MIX) {
+  if (MIX2) {
     // D[i][b]: lane groups 0 and 1 hold rows 0-7 (gate, from acc), groups 2 and 3 rows 8-15 (up, from acc_up)
 #pragma unroll
     for (int r = 0; r < R; r++)
@@ -562,19 +576,19 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   // part_lds[w][group][nb][j][lane]; fin[b][local row]
   constexpr int GP = L::GP;  // row groups per phase
   float (*part_lds)[GP][NB][4][64] = reinterpret_cast<float (*)[GP][NB][4][64]>(smem + L::PART);
-  float (*fin)[16 * R + 1] = reinterpret_cast<float (*)[16 * R + 1]>(smem + L::FIN);
+  float (*fin)[16 * RT + 1] = reinterpret_cast<float (*)[16 * RT + 1]>(smem + L::FIN);
 #pragma unroll
-  for (int r0 = 0; r0 < R; r0 += GP) {
+  for (int r0 = 0; r0 < RT; r0 += GP) {
 #pragma unroll
     for (int rr = 0; rr < GP; rr++)
-      if (r0 + rr < R) {   // (the last phase of an odd number of groups is part empty)
+      if (r0 + rr < RT) {   // (the last phase of an odd number of groups is part empty)
 #pragma unroll
         for (int nb = 0; nb < NB; nb++)
 #pragma unroll
           for (int j = 0; j < 4; j++) part_lds[wave][rr][nb][j][lane] = acc[r0 + rr][nb][j];
       }
     __syncthreads();
-    const int live = (R - r0 < GP ? R - r0 : GP) * NB * 256;
+    const int live = (RT - r0 < GP ? RT - r0 : GP) * NB * 256;
     for (int e = tid; e < live; e += GV_THREADS) {
       const int rr = e / (NB * 256), nb = (e >> 8) % NB, j = (e >> 6) & 3, l = e & 63;
       float s = 0.f;
@@ -659,6 +673,19 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
         gate = X::from_bits(X::to_bits(gate));
         up = X::from_bits(X::to_bits(up));
         y[(int64_t)b * half + jn] = X::to_bits(silu_f(gate) * up);
+      }
+    }
+    if constexpr (E > 0) {
+      // the plain groups: fin[b][16 R + i] is row ebx * 16 E + i of the second matrix
+      const int64_t n0 = (int64_t)ebx * (16 * E), n_x = xa->N;
+      for (int e = tid; e < B * 16 * E; e += GV_THREADS) {
+        const int b = e / (16 * E), rl = e - b * (16 * E);
+        const int64_t n = n0 + rl;
+        if (n < n_x) {
+          float v = fin[b][16 * R + rl];
+          if (xa->bias) v += X::from_bits(xa->bias[n]);
+          xa->y[(int64_t)b * n_x + n] = X::to_bits(v);
+        }
       }
     }
   } else if (MODE == 0) {
@@ -750,14 +777,24 @@ __global__ __launch_bounds__(W * MTP_WAVE) void gemv_kernel(const GemvArgs ga) {
 // unit: a grid with more workgroups than compute units would run its last few alone).
 // Tried and dropped: the first product's row blocks as workgroups of their own in front of the second's (272
 // workgroups: 82 us against 63 us for the two launches, with one or two workgroups per compute unit alike).
-template <int R1, int R2, int MODE2, int NB, int W, bool F16>
+constexpr int gemv_pair_depth(int r1) { return r1 == 1 ? 4 : r1 == 2 ? 2 : 1; }
+// INLOOP (mixed groups only): the first n1 workgroups stream a block of 16 R1 rows of the first product in the same
+// loop as their own rows, as R1 more row groups, instead of in a pass of their own.
+template <int R1, int R2, int MODE2, int NB, int W, bool F16, bool INLOOP = false>
 __global__ __launch_bounds__(W * MTP_WAVE) void gemv_pair_kernel(const GemvArgs g1, const GemvArgs g2, const int n1) {
   using L1 = GemvLds<R1, NB, W, false>;
-  using L2 = GemvLds<R2, NB, W, false>;
+  using L2 = GemvLds<INLOOP ? R1 + R2 : R2, NB, W, false>;
   __shared__ __attribute__((aligned(16))) char smem[L1::BYTES > L2::BYTES ? L1::BYTES : L2::BYTES];
   const int bid = (int)blockIdx.x;
+  if constexpr (INLOOP) {
+    if (bid < n1) gemv_body<R2, NB, MODE2, false, 1, W, F16, false, true, R1>(g2, bid, 0, 1, smem, &g1, bid);
+    else gemv_body<R2, NB, MODE2, false, 1, W, F16, false, true>(g2, bid, 0, 1, smem);
+    return;
+  }
   if (bid < n1) {
-    gemv_body<R1, NB, 0, false, 1, W, F16, false, true>(g1, bid, 0, 1, smem);
+    // a block of few rows lives on latency: it walks several k-pairs per step instead (the host checks that every
+    // wave's share of the pairs divides)
+    gemv_body<R1, NB, 0, false, gemv_pair_depth(R1), W, F16, false, true>(g1, bid, 0, 1, smem);
     __syncthreads();   // the second product reuses the LDS
   }
   gemv_body<R2, NB, MODE2, false, 1, W, F16, false, true>(g2, bid, 0, 1, smem);
@@ -992,24 +1029,23 @@ int launch_gemv(const void* x, const void* w, const void* bias, void* y, ArgPart
 // SwiGLU with mixed row groups (MODE 3): how many groups per workgroup.  0 = this shape keeps MODE 1.
 // Every CU should hold the same number of bytes in flight: prefer the R whose workgroup count fills whole
 // layers of 256 workgroups best, then the larger R (fewer reductions); too few workgroups are not an option.
+// (28672 x 4096 at 17-32 batch rows: seven groups on 256 workgroups 41-42 us, eight paired groups on 224
+// workgroups 44.5-46 us.  The first form built for two batch tiles kept the up rows half a row ahead, i.e. twice
+// the accumulators and one operand set, and took 46 us; with 8 waves instead of 4 the present form spills and
+// takes 50 us.)
 int pick_mixed_groups(int64_t B, int64_t N, int64_t K) {
   const int64_t half = N / 2;
   if (K % 64 != 0 || (K / 64) % GV_MAX_WAVES != 0 || (half + 64) * K >= (1ll << 32)) return 0;
   static MtpTune tune_mix("MTP_GEMV_MIX");
-  // Two batch tiles (more than 16 rows): built with seven groups, on workgroups of four waves with one operand
-  // set, and taken only when forced (MTP_GEMV_MIX = 7): 256 equal workgroups instead of 224, but twice the
-  // accumulators leave no registers for the second operand set, and 28672 x 4096 at 32 rows takes 46 us that way
-  // against 44.5 us with paired groups.
-  const int r_lo = B > 16 ? 7 : 1;
   if (tune_mix.is_set()) {
     const int r = tune_mix.get(0);
-    return r >= r_lo && r <= 7 ? r : 0;
+    return r >= 1 && r <= 7 ? r : 0;
   }
-  if (B > 16) return 0;
+  (void)B;   // one or two batch tiles: the same choice (two tiles walk gate and up rows in step, see gemv_body)
   const int64_t groups = (half + 7) / 8;
   int best = 0;
   double best_eff = 0.0;
-  for (int r = r_lo; r <= 7; r++) {
+  for (int r = 1; r <= 7; r++) {
     const int64_t wgs = (groups + r - 1) / r;
     if (wgs < 200) continue;
     const double eff = (double)wgs / (double)((wgs + 255) / 256 * 256);
@@ -1040,16 +1076,28 @@ int launch_gemv_mixed(const void* x, const void* w, const void* bias, void* y, i
     else GVM_T(RR, false);       \
     break
   if (B > 16) {
-    // two batch tiles: twice the accumulators, one operand set, four waves (one workgroup per compute unit)
+    // two batch tiles: one k position per tile, two operand sets; four waves from five groups on (above 256 registers)
     if constexpr (!NORM) {
-      if (R != 7) {
-        mtp_set_error("gemv: %d mixed row groups at %lld rows", R, (long long)B);
-        return MTP_EINVAL;
+#define GVM2_T(RR, FF)                                                                                            \
+  hipLaunchKernelGGL((gemv_kernel<RR, 2, 3, false, 1, (RR >= 5 ? 4 : GV_MAX_WAVES), FF, false, true>), dim3(n_wg), \
+                     dim3((RR >= 5 ? 4 : GV_MAX_WAVES) * MTP_WAVE), 0, s, ga)
+#define GVM2(RR)                  \
+  case RR:                        \
+    if (f16) GVM2_T(RR, true);    \
+    else GVM2_T(RR, false);       \
+    break
+      switch (R) {
+        GVM2(1);
+        GVM2(2);
+        GVM2(3);
+        GVM2(4);
+        GVM2(5);
+        GVM2(6);
+        GVM2(7);
+        default: mtp_set_error("gemv: %d mixed row groups", R); return MTP_EINVAL;
       }
-      if (f16)
-        hipLaunchKernelGGL((gemv_kernel<7, 2, 3, false, 1, 4, true, false, false>), dim3(n_wg), dim3(4 * MTP_WAVE), 0, s, ga);
-      else
-        hipLaunchKernelGGL((gemv_kernel<7, 2, 3, false, 1, 4, false, false, false>), dim3(n_wg), dim3(4 * MTP_WAVE), 0, s, ga);
+#undef GVM2
+#undef GVM2_T
     }
     MTP_CHECK_LAUNCH("gemv");
     return MTP_OK;
@@ -1161,11 +1209,13 @@ extern "C" int mtp_gemv_pair(const void* x, const void* w1, const void* bias1, v
   hipStream_t s = (hipStream_t)stream;
   const bool f16 = dtype == MTP_F16;
   const int64_t half2 = N2 / 2;
-  // one grid: two batch tiles, whole 64-element pairs, a second product that fills the chip with 8-group
-  // workgroups by itself, 32-bit row offsets inside a workgroup's rows
-  const bool one_grid = tune_pair.get(1) != 0 && B > 16 && K % 64 == 0 && pick_mixed_groups(B, N2, K) == 0 &&
-                        pick_gemv_cfg(B, N2, K, 1).R == 8 &&
-                        pick_gemv_cfg(B, N2, K, 1).S == 1 && 128 * K < (1ll << 31);
+  // one grid: two batch tiles, whole 64-element pairs, a second product that fills the chip by itself with one
+  // workgroup per compute unit (seven mixed groups, or eight paired ones), 32-bit row offsets inside a workgroup's rows
+  const int mixed = pick_mixed_groups(B, N2, K);
+  const bool grid_ok = tune_pair.get(1) != 0 && K % 64 == 0 && 128 * K < (1ll << 31);
+  const bool mix_grid = grid_ok && mixed == 7 && (B > 16 || tune_pair.get(1) != 2);
+  const bool one_grid = mix_grid || (grid_ok && B > 16 && mixed == 0 && pick_gemv_cfg(B, N2, K, 1).R == 8 &&
+                                     pick_gemv_cfg(B, N2, K, 1).S == 1);
   if (!one_grid) {
     rc = mtp_gemv_ws(x, w1, bias1, y1, workspace, workspace_bytes, B, N1, K, bias1 ? MTP_EPI_BIAS : MTP_EPI_NONE, dtype, stream);
     if (rc) return rc;
@@ -1182,17 +1232,48 @@ extern "C" int mtp_gemv_pair(const void* x, const void* w1, const void* bias1, v
                     rot_mul, K, nullptr, nullptr, flags, none, 0};
   // the first product's rows in blocks of 16 R1 rows, as few rows per block as still leaves no more blocks than
   // the second product has workgroups
-  const unsigned n2 = (unsigned)((half2 + 63) / 64);
+  const unsigned n2 = mix_grid ? (unsigned)((half2 + 55) / 56) : (unsigned)((half2 + 63) / 64);
+  // mixed groups: the first product's rows as one or two more row groups in the loop of the first workgroups
+  // (MTP_GEMV_PAIR = 2 keeps the block in front of the loop)
+  if (mix_grid && tune_pair.get(1) != 2) {
+    const int e = (N1 + 15) / 16 <= (int64_t)n2 ? 1 : 2;
+    const unsigned n1e = (unsigned)((N1 + 16 * e - 1) / (16 * e));
+    if (n1e <= n2) {
+#define GVE(EE, FF)                                                                                                    \
+  do {                                                                                                                 \
+    if (B > 16)                                                                                                        \
+      hipLaunchKernelGGL((gemv_pair_kernel<EE, 7, 3, 2, 4, FF, true>), dim3(n2), dim3(4 * MTP_WAVE), 0, s, g1, g2, (int)n1e); \
+    else                                                                                                               \
+      hipLaunchKernelGGL((gemv_pair_kernel<EE, 7, 3, 1, 4, FF, true>), dim3(n2), dim3(4 * MTP_WAVE), 0, s, g1, g2, (int)n1e); \
+  } while (0)
+      if (e == 1) {
+        if (f16) GVE(1, true);
+        else GVE(1, false);
+      } else {
+        if (f16) GVE(2, true);
+        else GVE(2, false);
+      }
+#undef GVE
+      MTP_CHECK_LAUNCH("gemv_pair");
+      return MTP_OK;
+    }
+  }
   int r1 = 1;
   while (r1 < 8 && (N1 + 16 * r1 - 1) / (16 * r1) > (int64_t)n2) r1 *= 2;
+  if (B <= 16) r1 = 0;   // one batch tile: the in-loop form or two launches
   const unsigned n1 = (unsigned)((N1 + 16 * r1 - 1) / (16 * r1));
-  if (n1 > n2) {
+  if (r1 == 0 || n1 > n2 || (K / 64) % (4 * gemv_pair_depth(r1)) != 0) {
     rc = mtp_gemv_ws(x, w1, bias1, y1, workspace, workspace_bytes, B, N1, K, bias1 ? MTP_EPI_BIAS : MTP_EPI_NONE, dtype, stream);
     if (rc) return rc;
     return mtp_gemv_ws(x, w2, bias2, act2, workspace, workspace_bytes, B, N2, K, MTP_EPI_SWIGLU, dtype, stream);
   }
-#define GVP_T(RR, FF) \
-  hipLaunchKernelGGL((gemv_pair_kernel<RR, 8, 1, 2, 4, FF>), dim3(n2), dim3(4 * MTP_WAVE), 0, s, g1, g2, (int)n1)
+#define GVP_T(RR, FF)                                                                                               \
+  do {                                                                                                              \
+    if (mix_grid)                                                                                                   \
+      hipLaunchKernelGGL((gemv_pair_kernel<RR, 7, 3, 2, 4, FF>), dim3(n2), dim3(4 * MTP_WAVE), 0, s, g1, g2, (int)n1); \
+    else                                                                                                            \
+      hipLaunchKernelGGL((gemv_pair_kernel<RR, 8, 1, 2, 4, FF>), dim3(n2), dim3(4 * MTP_WAVE), 0, s, g1, g2, (int)n1); \
+  } while (0)
 #define GVP(RR)                \
   case RR:                     \
     if (f16) GVP_T(RR, true);  \

@@ -160,6 +160,21 @@ def test_gemv_and_fused_argmax_fp16(gpu, b, n, k, epi):
         ops.gemv(x.to(gpu), w.bfloat16().to(gpu))                 # mixed 16-bit dtypes
 
 
+@pytest.mark.parametrize("b", [4, 32])
+def test_gemv_pair_fp16(gpu, b):
+    """QKV-like and gate/up-like products in one grid (the first product's rows inside the loop of the mixed SwiGLU
+    groups), one and two batch tiles, ragged row counts, in IEEE half: against the oracle."""
+    g = gen(27)
+    n1, half, k = 3016, 14000, 2048
+    x = torch.randn(b, k, generator=g).to(H)
+    w1 = (torch.randn(n1, k, generator=g) * 0.02).to(H)
+    w2 = (torch.randn(2 * half, k, generator=g) * 0.02).to(H)
+    y1, a2 = ops.gemv_pair(x.to(gpu), w1.to(gpu), w2.to(gpu))
+    assert y1.dtype == H and a2.dtype == H
+    assert rel(y1, F.linear(x.float(), w1.float())) < TOL_F16
+    assert rel(a2, R.swiglu(F.linear(x.float(), w2.float()).to(H).float())) < TOL_F16
+
+
 def test_rmsnorm_rope_attention_fp16(gpu):
     from merak_amd.inference import rope_tables
     g = gen(22)

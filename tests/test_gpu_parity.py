@@ -1144,10 +1144,14 @@ def test_argmax_one_workspace_for_shapes_in_turn(gpu):
 
 @pytest.mark.parametrize("b,n1,half,k,bias", [(32, 6144, 14336, 4096, False), (17, 1000, 4096, 1024, True),
                                                (8, 6144, 14336, 4096, False), (32, 130, 200, 264, True),
-                                               (20, 1280, 3584, 8192, False)])
+                                               (20, 1280, 3584, 8192, False), (25, 6100, 14000, 4096, True),
+                                               (32, 3000, 14336, 4096, False), (5, 6100, 14000, 4096, True),
+                                               (16, 3000, 14336, 4096, False)])
 def test_gemv_pair_is_the_two_products(gpu, set_tuning, b, n1, half, k, bias):
     """mtp_gemv_pair: QKV-like and gate/up-like products over the same rows in one call — one grid above 16 rows
-    for the shapes it takes, two launches otherwise: the results of the two separate calls, and the oracle."""
+    for the shapes it takes (the first product's rows as one or two more row groups in the loop of the mixed
+    groups, ragged ends included, or as a block in front of the loop: MTP_GEMV_PAIR = 2), two launches otherwise:
+    the results of the two separate calls, and the oracle."""
     x = torch.randn(b, k, generator=gen(290)).bfloat16()
     w1 = (torch.randn(n1, k, generator=gen(291)) * 0.02).bfloat16()
     w2 = (torch.randn(2 * half, k, generator=gen(292)) * 0.02).bfloat16()
@@ -1157,12 +1161,16 @@ def test_gemv_pair_is_the_two_products(gpu, set_tuning, b, n1, half, k, bias):
     xg, w1g, w2g, b1g, b2g = dev(x), dev(w1), dev(w2), dev(b1), dev(b2)
     y1 = ops.gemv(xg, w1g, b1g, ops.EPI_BIAS if bias else ops.EPI_NONE)
     a2 = ops.gemv(xg, w2g, b2g, ops.EPI_SWIGLU)
-    for pair in (None, 0):
+    for pair in (None, 2, 0):
         set_tuning("MTP_GEMV_PAIR", pair)
         p1, p2 = ops.gemv_pair(xg, w1g, w2g, b1g, b2g)
-        # the second product runs in the configuration it has on its own: the same bits; the first one's row blocks
-        # are larger in the one grid (another order of the sums along k): the same values to rounding
-        assert torch.equal(p2, a2) and rel(p1, y1) < 3e-3, pair
+        # Above 16 rows the second product runs in the configuration it has on its own: the same bits.  Up to 16
+        # rows its up rows walk in step with the gate rows in the one grid (half a row ahead on its own), and the
+        # first product's rows are cut into other blocks in either: other orders of the sums along k, the same
+        # values to rounding.
+        assert rel(p1, y1) < 3e-3 and rel(p2, a2) < 3e-3, pair
+        if b > 16 or pair == 0:
+            assert torch.equal(p2, a2), pair
         if pair == 0:
             assert torch.equal(p1, y1)
     ref1 = F.linear(x.float(), w1.float(), None if b1 is None else b1.float())
@@ -1485,8 +1493,8 @@ def test_greedy_pick_over_a_vocab_sharded_lm_head(gpu):
                                                 (25, 100, 512, False)])
 def test_gemv_swiglu_mixed_row_groups(gpu, set_tuning, mix, b, half, k, with_bias):
     """SwiGLU GEMV whose 16-row tiles hold 8 gate rows and their 8 up rows, for every number of groups per
-    workgroup (forced) and for the automatic choice: same result as the oracle, ragged ends included.  Above 16
-    batch rows (two batch tiles) the form exists with seven groups; other forced values take the paired groups."""
+    workgroup (forced) and for the automatic choice: same result as the oracle, ragged ends included, with one
+    batch tile (up rows half a row ahead of the gate rows, two products per tile) and with two (rows in step)."""
     if mix is not None:
         set_tuning("MTP_GEMV_MIX", mix)
     g = gen(41)

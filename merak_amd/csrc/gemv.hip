@@ -907,6 +907,10 @@ GemvCfg pick_gemv_cfg(int64_t B, int64_t N, int64_t K, int mode, bool may_split 
   // care about); matrices with few row groups keep every CU busy by going deeper along k instead.
   // Measured on 128256x4096, 28672x4096, 6144x4096, 4096x14336, 8192x3584 and 1280x8192 at B = 1, 8, 32.
   GemvCfg c{B > 16 ? 8 : 4, 1, 1};
+  // The argmax form takes 8 row groups (4-wave workgroups) at every batch: 128256 x 4096 with its finishing kernel
+  // 154.5 against 155.5 us at 1 row, 154 against 157 us at 8, 152 against 159 us at 16 (half as many keys to fold,
+  // half as many reads of X).
+  if (mode == 2) c.R = 8;
   // Above 16 batch rows X is read twice per 16 R weight rows: halving R until there are enough workgroups
   // makes the L2 -> CU traffic of X a multiple of the weight stream.  With a workspace the rows stay and k is
   // cut instead (each slice reads only its part of X); every wave of a slice gets the same number of pairs.

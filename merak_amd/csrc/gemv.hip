@@ -98,11 +98,12 @@ struct GemvFuse {
 // rows, so a workgroup may own any number R of groups (8 R gate rows and their up rows) and the workgroup count can
 // be made a multiple of the CU count (R = 7 gives exactly 256 workgroups for 14336 gate rows; with R = 4 the 448
 // workgroups leave a quarter of the CUs with half the bytes in flight: 5.4 instead of 6.4 TB/s).  Load A fetches the
-// gate rows of a k-pair, load B the up rows half a row further along k (the two sit a large power of two apart in
-// memory, see below), so a tile mixes two k positions: it is multiplied twice, once with X at either position,
-// into two accumulators, and each lane keeps the one whose rows it owns.  With two batch tiles (more than 16 batch
-// rows) the up rows walk in step with the gate rows instead: one k position, one product and one accumulator per
-// tile, which leaves the registers for a second operand set.
+// gate rows of a k-pair, load B the up rows of the same pair: one product and one accumulator per tile, and two
+// operand sets in the registers.  (A first form had the up rows walk half a row ahead of the gate rows, as the
+// paired groups of MODE 1 do against the DRAM page conflicts of two streams a large power of two apart: a tile
+// then holds two k positions and is multiplied with X at both, into two accumulators.  Measured, walking in step
+// costs nothing here, and the registers it frees pay for the second operand set: 28672 x 4096 at 8 rows 39.8 ->
+// 37.4 us, at 16 rows 39.6 -> 37.5 us.)
 // W waves split K.  Configurations whose registers allow only 8 waves per CU run as two independent workgroups of
 // 4 waves rather than one of 8: while one sums its partial tiles and writes its outputs the other keeps streaming.
 // Everything a launch hands to a workgroup.
@@ -244,17 +245,11 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
 
   static_assert(MODE != 3 || (!GUARD && D == 1), "mixed SwiGLU groups: K % 64 == 0, depth 1");
   constexpr bool MIX = MODE == 3;
-  constexpr bool MIX2 = MIX && NB == 1 && E == 0;   // mixed groups whose up rows walk ahead of the gate rows: two products per tile
   f32x4_t acc[RT][NB];
-  f32x4_t acc_up[MIX2 ? R : 1][NB];   // MIX2: the products with X at the up rows' k position
 #pragma unroll
   for (int r = 0; r < RT; r++)
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) acc[r][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int r = 0; r < (MIX2 ? R : 1); r++)
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++) acc_up[r][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const bool low = li < 8;
 
   // D pairs (8 apart) per step: with few rows per workgroup this is what keeps enough bytes in flight.
@@ -264,9 +259,8 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   // shapes a large power of two apart, i.e. in the same memory channel and bank but another DRAM page.
   // Walking both at the same k makes the two streams evict each other's open page, so the up rows walk
   // half a row ahead (XS = 2 sets of X fragments, one per k position).
-  // (with one batch tile only.  With two, gate and up rows walk in step: a mixed tile then holds one k position, needs
-  // one product and one accumulator, and its registers leave room for the second operand set)
-  constexpr int XS = ((MODE == 1 || MODE == 3) && NB == 1 && !GUARD && E == 0) ? 2 : 1;
+  // (paired groups with one batch tile only; the mixed groups walk in step)
+  constexpr int XS = ((MODE == 1) && NB == 1 && !GUARD && E == 0) ? 2 : 1;
   const int64_t up_shift = (XS == 2 && pairs % GV_WAVES == 0 && !(flags & 1)) ? ((pairs / 2) & ~(int64_t)(GV_WAVES - 1)) : 0;
   // Operand registers of one step.  PP: two such sets used in turn, the next step's requests go out before the
   // current step's operands are waited for.  Otherwise one set is rotated by copying, which the compiler folds
@@ -295,7 +289,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
       pair_k(pq0, d, ks);
 #pragma unroll
       for (int r = 0; r < RT; r++) {
-        if (MIX && r < R) {   // gate rows at the pair itself, up rows at the shifted pair
+        if (MIX && r < R) {   // gate rows and up rows of the same pair
           a[d][r][0] = load_frag_nt(wbase[r] + ks[0] + offa[r], true);
           a[d][r][1] = load_frag_nt(wbase[r] + ks[1] + offb[r], true);
           continue;
@@ -346,17 +340,6 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
   // products never stand next to each other inside its pinned sections)
   auto multiply_group = [&](int r, const bf16x8_t& h0, const bf16x8_t& h1, bf16x8_t (&bx)[XS][NB][2]) {
     if constexpr (PP) {
-      if (MIX2) {
-        // rows 0-7 (gate) belong to k position 0, rows 8-15 (up) to position 1: both products, two accumulators
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-          acc[r][nb] = X::mfma16(h0, bx[0][nb][0], acc[r][nb]);
-          acc[r][nb] = X::mfma16(h1, bx[0][nb][1], acc[r][nb]);
-          acc_up[r][nb] = X::mfma16(h0, bx[XS - 1][nb][0], acc_up[r][nb]);
-          acc_up[r][nb] = X::mfma16(h1, bx[XS - 1][nb][1], acc_up[r][nb]);
-        }
-        return;
-      }
       const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
 #pragma unroll
       for (int nb = 0; nb < NB; nb++) {
@@ -364,19 +347,6 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
         acc[r][nb] = X::mfma16(h1, bx[xs][nb][1], acc[r][nb]);
       }
     } else {
-      if (MIX2) {
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-          acc[r][nb] = X::mfma16(h0, bx[0][nb][0], acc[r][nb]);
-          acc_up[r][nb] = X::mfma16(h0, bx[XS - 1][nb][0], acc_up[r][nb]);
-        }
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-          acc[r][nb] = X::mfma16(h1, bx[0][nb][1], acc[r][nb]);
-          acc_up[r][nb] = X::mfma16(h1, bx[XS - 1][nb][1], acc_up[r][nb]);
-        }
-        return;
-      }
       const int xs = (XS == 2 && r >= R / 2) ? 1 : 0;
 #pragma unroll
       for (int nb = 0; nb < NB; nb++) acc[r][nb] = X::mfma16(h0, bx[xs][nb][0], acc[r][nb]);
@@ -561,14 +531,6 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& ga, const int bx, cons
         rres[i] = (e < B * 16 * R && n < N) ? fz.residual[(int64_t)b * N + n] : (uint16_t)0;
       }
     }
-  }
-
-  if (MIX2) {
-    // D[i][b]: lane groups 0 and 1 hold rows 0-7 (gate, from acc), groups 2 and 3 rows 8-15 (up, from acc_up)
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-      for (int nb = 0; nb < NB; nb++) acc[r][nb] = lg < 2 ? acc[r][nb] : acc_up[r][nb];
   }
 
   // ---- sum the 8 k-slices through LDS: up to 8 tiles (row group x batch tile) per wave at a time, i.e. one
@@ -1045,7 +1007,7 @@ int pick_mixed_groups(int64_t B, int64_t N, int64_t K) {
     const int r = tune_mix.get(0);
     return r >= 1 && r <= 7 ? r : 0;
   }
-  (void)B;   // one or two batch tiles: the same choice (two tiles walk gate and up rows in step, see gemv_body)
+  (void)B;   // one or two batch tiles: the same choice
   const int64_t groups = (half + 7) / 8;
   int best = 0;
   double best_eff = 0.0;
@@ -1072,7 +1034,7 @@ int launch_gemv_mixed(const void* x, const void* w, const void* bias, void* y, i
   const GemvArgs ga{(const uint16_t*)x, (const uint16_t*)w, (const uint16_t*)bias, (uint16_t*)y, nullptr, (int)B, N, K,
                     rot_mul, K, nullptr, nullptr, 0, fz, 0};
 #define GVM_T(RR, FF)                                                                                              \
-  hipLaunchKernelGGL((gemv_kernel<RR, 1, 3, false, 1, GV_MAX_WAVES, FF, NORM, (RR <= 6)>), dim3(n_wg),                \
+  hipLaunchKernelGGL((gemv_kernel<RR, 1, 3, false, 1, GV_MAX_WAVES, FF, NORM, true>), dim3(n_wg),                      \
                      dim3(GV_MAX_WAVES * MTP_WAVE), 0, s, ga)
 #define GVM(RR)                  \
   case RR:                       \

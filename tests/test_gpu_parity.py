@@ -1146,7 +1146,8 @@ def test_argmax_one_workspace_for_shapes_in_turn(gpu):
                                                (8, 6144, 14336, 4096, False), (32, 130, 200, 264, True),
                                                (20, 1280, 3584, 8192, False), (25, 6100, 14000, 4096, True),
                                                (32, 3000, 14336, 4096, False), (5, 6100, 14000, 4096, True),
-                                               (16, 3000, 14336, 4096, False)])
+                                               (16, 3000, 14336, 4096, False), (32, 6090, 14336, 4096, False),
+                                               (2, 4097, 14336, 4096, True)])
 def test_gemv_pair_is_the_two_products(gpu, set_tuning, b, n1, half, k, bias):
     """mtp_gemv_pair: QKV-like and gate/up-like products over the same rows in one call — one grid above 16 rows
     for the shapes it takes (the first product's rows as one or two more row groups in the loop of the mixed

@@ -469,6 +469,35 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, AccFn accv, Rsu
   // Fast path of flush, for the blocks [JB, JB + NB) of the staged row (NB a power of two, at most 4): 16-byte
   // aligned rows of a tile that is completely inside: lane l owns chunk l % CPR of rows l / CPR, l / CPR + 64 / CPR,
   // ...; one address computation, then constant strides.
+  // Accumulating into C (C += result): the old values of block row i, one 16-byte vector per store of the fast
+  // path (piece JB holds its ITERS vectors from old_c[JB * esz] on).  They are asked for at the top of the block
+  // row, before its values are rounded and staged, so that one memory latency stands in front of the stores of a
+  // block row instead of one in front of every store (a load may not move up past the store before it).
+  constexpr int OLD_N = TJ * ESZ;
+  [[maybe_unused]] u32x4_t old_c[OLD_N];
+  const bool c_fast = tile_inside && p.C && ((reinterpret_cast<uintptr_t>(p.C) | (uintptr_t)(p.ldc * ESZ)) & 15) == 0;
+  const bool preload_c = c_fast && p.accumulate != 0;
+  auto piece_addr = [&](int i, void* out, int64_t ld, auto jb_tag, auto nb_tag, auto colfn, auto f32_tag, char*& gp,
+                        int64_t& gstride) {
+    constexpr int JB = decltype(jb_tag)::value, NB = decltype(nb_tag)::value;
+    constexpr int esz_c = decltype(f32_tag)::value ? 4 : 2;
+    constexpr int CPR = NB * 32 * esz_c / 16, RPI = 64 / CPR;
+    const int r0 = lane / CPR, cc = lane % CPR;
+    const int e0 = cc * (16 / esz_c);
+    const int col = colfn(JB + (e0 >> 5)) + (e0 & 31);
+    gp = (char*)out + ((int64_t)(m0 + blk_row(i) + r0) * ld + col) * esz_c;
+    gstride = (int64_t)RPI * ld * esz_c;
+  };
+  auto preload_piece = [&](int i, auto jb_tag, auto nb_tag, auto colfn) {
+    constexpr int JB = decltype(jb_tag)::value, NB = decltype(nb_tag)::value;
+    constexpr int CPR = NB * 32 * ESZ / 16, RPI = 64 / CPR, ITERS = 32 / RPI;
+    static_assert(JB * ESZ + ITERS <= OLD_N, "old values of a block row");
+    char* gp;
+    int64_t gstride;
+    piece_addr(i, p.C, p.ldc, jb_tag, nb_tag, colfn, std::integral_constant<bool, OUT == OUT_F32>{}, gp, gstride);
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) old_c[JB * ESZ + it] = *reinterpret_cast<const u32x4_t*>(gp + it * gstride);
+  };
   auto flush_piece = [&](int i, void* out, int64_t ld, auto jb_tag, auto nb_tag, auto colfn, auto f32_tag, bool accumulate) {
     constexpr int JB = decltype(jb_tag)::value, NB = decltype(nb_tag)::value;
     constexpr bool f32out = decltype(f32_tag)::value;
@@ -487,7 +516,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, AccFn accv, Rsu
       u32x4_t v = *reinterpret_cast<const u32x4_t*>(sp + it * RPI * PITCH);
       u32x4_t* q = reinterpret_cast<u32x4_t*>(gp + it * gstride);
       if (accumulate) {
-        const u32x4_t o = *q;
+        // (accumulation only ever goes into C, whose old values were asked for ahead)
+        const u32x4_t o = (esz_c == ESZ && JB * esz_c + it < OLD_N) ? old_c[JB * esz_c + it] : *q;
         if (f32out) {
           v.x = __float_as_uint(__uint_as_float(v.x) + __uint_as_float(o.x));
           v.y = __float_as_uint(__uint_as_float(v.y) + __uint_as_float(o.y));
@@ -579,8 +609,20 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, AccFn accv, Rsu
     }
   };
 
+  // the pieces of flush's fast path for the TJ blocks of a row of C
+  auto preload_row = [&](int i) {
+    constexpr int STEP = 4, N4 = TJ / STEP, REM = TJ % STEP;
+    static_for<N4>([&](auto t) {
+      preload_piece(i, std::integral_constant<int, decltype(t)::value * STEP>{}, std::integral_constant<int, STEP>{}, col_of_block);
+    });
+    if constexpr (REM >= 2) preload_piece(i, std::integral_constant<int, N4 * STEP>{}, std::integral_constant<int, 2>{}, col_of_block);
+    if constexpr (REM % 2 == 1)
+      preload_piece(i, std::integral_constant<int, N4 * STEP + (REM >= 2 ? 2 : 0)>{}, std::integral_constant<int, 1>{}, col_of_block);
+  };
+
 #pragma unroll
   for (int i = 0; i < TI; i++) {
+    if (preload_c) preload_row(i);
     // -- pre-activation (or plain) output: add bias, round, stage
     float pre[TJ][16];
 #pragma unroll

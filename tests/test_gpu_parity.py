@@ -607,6 +607,10 @@ def _every_product_once(gpu, dtype, m, n, k, seed):
     acc, accb = torch.ones(n, k, device=gpu), torch.ones(n, device=gpu)
     ops.linear_wgrad(dyg, xg, True, dw=acc, db=accb, accumulate=True)
     out["acc"], out["accb"] = acc, accb
+    # accumulation in the tensor dtype (how `.grad` sums micro-batches), onto a gradient of the same size
+    acc16 = out["dw"].clone()
+    ops.linear_wgrad(dyg, xg, False, dw=acc16, accumulate=True)
+    out["acc16"] = acc16
     return (x, w, b, dy), out
 
 
@@ -620,6 +624,7 @@ def _check_every_product(inputs, out, tol, what):
     rdx, rdw, rdb = R.linear_backward(x, w, dy, True)
     assert rel(out["dx"], rdx) < tol and rel(out["dw"], rdw) < tol and rel(out["db"], rdb) < tol, what
     assert rel(out["acc"] - 1, rdw) < TOL_F32 * 10 and rel(out["accb"] - 1, rdb) < TOL_F32 * 10, what
+    assert rel(out["acc16"], 2 * rdw) < tol, what
 
 
 # k, n and m multiples of 64 (every product can take the 64-deep loop), then ragged in all three

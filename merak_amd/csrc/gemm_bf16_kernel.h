@@ -640,8 +640,14 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, AccFn accv, Rsu
             }
           }
         }
+        // (without a bias there is nothing to add: x + 0 is not x for the compiler, which would keep 256 additions)
 #pragma unroll
-        for (int e = 0; e < 4; e++) pre[j][4 * g + e] = accv(i, j, g, e) + b4[e];
+        for (int e = 0; e < 4; e++) {
+          if constexpr (EPI == MTP_EPI_BIAS || EPI == MTP_EPI_BIAS_GELU || EPI == MTP_EPI_SWIGLU)
+            pre[j][4 * g + e] = accv(i, j, g, e) + b4[e];
+          else
+            pre[j][4 * g + e] = accv(i, j, g, e);
+        }
       }
     }
     if (OUT == OUT_F32) {

@@ -1175,6 +1175,8 @@ def test_gemv_pair_is_the_two_products(gpu, set_tuning, b, n1, half, k, bias):
         # first product's rows are cut into other blocks in either: other orders of the sums along k, the same
         # values to rounding.
         assert rel(p1, y1) < 3e-3 and rel(p2, a2) < 3e-3, pair
+        q1, q2 = ops.gemv_pair(xg, w1g, w2g, b1g, b2g)              # fixed summation orders: the same bits every run
+        assert torch.equal(p1, q1) and torch.equal(p2, q2), pair
         if b > 16 or pair == 0:
             assert torch.equal(p2, a2), pair
         if pair == 0:

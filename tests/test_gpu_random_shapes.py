@@ -105,6 +105,37 @@ def test_decode_products_random_shapes(gpu, seed):
 
 
 @pytest.mark.parametrize("seed", range(3))
+def test_product_pair_random_shapes(gpu, seed):
+    """mtp_gemv_pair on drawn shapes: second products that fill the chip with mixed SwiGLU groups (one grid, the
+    first product's rows as one or two more row groups in the loop, or more rows than that holds: two launches) and
+    ones that do not, every batch size class, ragged row counts, with and without biases."""
+    rng = random.Random(300 + seed)
+    g = torch.Generator(device=gpu).manual_seed(700 + seed)
+    for case in range(8):
+        dt = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+        B = rng.choice([1, 5, 8, 16, 17, 24, 32])
+        K = rng.choice([512, 1024, 2048, 1536, 520])
+        wgs = rng.choice([200, 230, 250, 256, 100])
+        half = 56 * wgs - rng.choice([0, 0, 3, 17, 55])
+        if rng.random() < 0.25:
+            half = rng.randint(1, 3000)
+        n1 = rng.choice([rng.randint(1, 16 * wgs), rng.randint(16 * wgs, 32 * wgs), rng.randint(32 * wgs, 40 * wgs)])
+        bias = rng.random() < 0.4
+        tag = f"seed {seed} case {case}: {dt} B={B} K={K} half={half} n1={n1} bias={bias}"
+        x = torch.randn(B, K, device=gpu, generator=g).to(dt)
+        w1 = (torch.randn(n1, K, device=gpu, generator=g) * 0.03).to(dt)
+        w2 = (torch.randn(2 * half, K, device=gpu, generator=g) * 0.03).to(dt)
+        b1 = (torch.randn(n1, device=gpu, generator=g) * 0.1).to(dt) if bias else None
+        b2 = (torch.randn(2 * half, device=gpu, generator=g) * 0.1).to(dt) if bias else None
+        y1, a2 = ops.gemv_pair(x, w1, w2, b1, b2)
+        assert y1.shape == (B, n1) and a2.shape == (B, half), tag
+        cpu = lambda t: None if t is None else t.cpu().float()
+        r1, _ = R.column_parallel_linear_forward(cpu(x), cpu(w1), cpu(b1))
+        pre, _ = R.column_parallel_linear_forward(cpu(x), cpu(w2), cpu(b2))
+        assert rel(y1, r1) < TOL[dt] and rel(a2, R.swiglu(pre.to(dt).float())) < TOL[dt], tag
+
+
+@pytest.mark.parametrize("seed", range(3))
 def test_cross_entropy_random_shapes(gpu, seed):
     rng = random.Random(300 + seed)
     g = torch.Generator().manual_seed(700 + seed)
